@@ -1,0 +1,189 @@
+"""Mem-cache retrieval: landmark scoring, top-k block selection, gather, attend.  TEST ORACLE.
+
+Restates the per-head, per-token branch (``aggregate is None``) of
+``LlamaAttention.forward`` in ``llama/llama_mem.py:318-430`` and the attend step
+``:447-477`` with the mask preparation of ``LlamaModel.forward`` ``:807-815``.
+
+Symbols: ``bs = mem_freq + 1`` (block), ``S`` cached tokens, ``T`` new tokens,
+``num_mems = S // bs`` complete cached blocks, ``k = min(cache_top_k, num_mems)``.
+The cache holds keys WITHOUT rotary (``:424-425``); queries and local keys come
+in already rotated (``:298``).
+
+Score contract (``:367``).  The reference computes ``matmul(q, mem_key^T) /
+sqrt(hd)`` in the model dtype: an fp32-accumulated product rounded to bf16, then
+a division rounded to bf16 again.  The accumulation order of that product is
+not defined by the reference, so this oracle fixes it to the correctly rounded
+value: dot product accumulated in fp64 -> fp32 -> bf16, then fp32 division by
+``float32(sqrt(hd))`` -> bf16.  Selection contract (``:384``): the ``k`` best
+under the total order (score descending, block index ascending), returned in
+ascending index order.  ``torch.topk`` breaks ties in an implementation-defined
+way; on rows without a tie at the k-th place both agree, which
+``tests/test_oracle_retrieval.py`` checks, together with a brute-force loop,
+the integer position formulas on hand-worked cases, and agreement of the
+bf16-faithful attend with the fp32 closed form of ``oracle/s1.py``.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .highlevel import grouped_softmax
+from .rotary import apply_rotary
+from .s1 import s1_attention
+
+
+# ------------------------------------------------------------------ positions
+def retrieval_geometry(S: int, block: int, top_k: int):
+    """Integer bookkeeping of ``llama_mem.py:321-324,358-365``.
+
+    Returns dict with ``full_len, incomplete_len, num_mems, k, prefix_len`` and
+    ``mem_pos`` (num_mems,) — the position at which each cached landmark key is
+    rotated for SCORING: every block but the newest ``k`` sits in slot 0, the
+    newest ``k`` in slots 1..k.
+    """
+    incomplete_len = S % block
+    full_len = S - incomplete_len
+    num_mems = full_len // block
+    k = min(top_k, num_mems)
+    prefix_len = full_len - (k + 1) * block
+    slot = torch.cat((torch.zeros(max(0, num_mems - k), dtype=torch.long), torch.arange(1, k + 1, dtype=torch.long)))
+    mem_pos = slot * block + (block - 1) + prefix_len
+    return dict(full_len=full_len, incomplete_len=incomplete_len, num_mems=num_mems, k=k,
+                prefix_len=prefix_len, mem_pos=mem_pos)
+
+
+def gather_positions(idx, num_mems: int, k: int, block: int, prefix_len: int):
+    """Positions at which the gathered keys are rotated (``llama_mem.py:386-388``).
+
+    idx: (..., k) ascending block indices.  Slot ``j`` (rank in the ascending
+    list) token ``t``: ``j*bs + t + (bs if idx[j] >= num_mems-k else 0) + prefix_len``.
+    Returns (..., k, bs) int64.
+    """
+    j = torch.arange(k, dtype=torch.long, device=idx.device)
+    t = torch.arange(block, dtype=torch.long, device=idx.device)
+    bump = torch.where(idx >= num_mems - k, block, 0)
+    return (j * block + bump)[..., None] + t + prefix_len
+
+
+# -------------------------------------------------------------------- scoring
+def landmark_scores(q, k_cache, cos, sin, block: int, top_k: int):
+    """Scores (B, nh, T, num_mems) in q.dtype under the score contract."""
+    S, hd = k_cache.shape[-2], k_cache.shape[-1]
+    g = retrieval_geometry(S, block, top_k)
+    lk = k_cache[..., : g["full_len"], :].unflatten(-2, (g["num_mems"], block))[..., block - 1, :]
+    lk = apply_rotary(lk, cos, sin, g["mem_pos"])                     # :366
+    dot = (q.double() @ lk.double().transpose(-1, -2)).float()        # correctly rounded fp32
+    sc = dot.to(q.dtype).float() / torch.tensor(math.sqrt(hd), dtype=torch.float32)
+    return sc.to(q.dtype)
+
+
+def select_topk(scores, k: int):
+    """Ascending indices (…, k) int64 of the k best under (score desc, index asc)."""
+    order = torch.sort(scores.float(), dim=-1, descending=True, stable=True).indices
+    return order[..., :k].sort(dim=-1).values
+
+
+def boundary_tie_rows(scores, k: int):
+    """Bool (…): rows whose k-th and (k+1)-th best scores are equal."""
+    top = torch.sort(scores.float(), dim=-1, descending=True).values
+    if top.shape[-1] <= k:
+        return torch.zeros(top.shape[:-1], dtype=torch.bool)
+    return top[..., k - 1] == top[..., k]
+
+
+# --------------------------------------------------------------------- gather
+def gather_blocks(cache, idx, block: int):
+    """``take_along_dim`` of ``llama_mem.py:393-398``: (B, nh, T, k, bs, hd)."""
+    B, nh, S, hd = cache.shape
+    num_mems = S // block
+    blocks = cache[:, :, : num_mems * block].unflatten(2, (num_mems, block))       # (B,nh,M,bs,hd)
+    T, k = idx.shape[2], idx.shape[3]
+    flat = blocks[:, :, None].expand(B, nh, T, num_mems, block, hd)
+    sel = idx[..., None, None].expand(B, nh, T, k, block, hd)
+    return torch.take_along_dim(flat, sel, dim=3)
+
+
+# ---------------------------------------------------------------- local masks
+def local_masks(is_mem_loc, T: int, dtype):
+    """Mask preparation of ``LlamaModel.forward`` (``llama_mem.py:807-815``) for a
+    chunk of ``T`` new tokens (only the last ``T`` mask columns matter on this path).
+
+    Returns additive mask (B,1,T,T) in ``dtype`` (0 / finfo.min), visible
+    landmark mask and last-section mask, both (B,1,T,T) bool.
+    """
+    low = torch.finfo(dtype).min
+    i = torch.arange(T)
+    add = torch.where(i[None, :] <= i[:, None], 0.0, low).to(dtype)[None, None]
+    add = add.expand(is_mem_loc.shape[0], 1, T, T).clone()
+    im = is_mem_loc[:, None, None, :]
+    ids = torch.where(add < -1, 0, torch.cumsum(im, -1) - im.int())
+    last_section = ids.amax(-1, keepdim=True) == ids
+    add = add.masked_fill(last_section & im, low)
+    vis = add > -1
+    return add, im & vis, last_section & vis
+
+
+# --------------------------------------------------------------------- attend
+def retrieve_and_attend(q, k_cache, v_cache, k_loc, v_loc, is_mem_loc, cos, sin, block: int, top_k: int,
+                        idx=None, n_buckets: int = 64):
+    """Whole step in the model dtype with the reference's rounding points.
+
+    q, k_loc: (B,nh,T,hd) rotated; k_cache (un-rotated), v_cache: (B,nh,S,hd) with
+    ``S % block == 0``; cos/sin: (n_pos, hd) tables in the model dtype.
+    Returns ``(out (B,nh,T,hd), idx (B,nh,T,k) int64)``.
+    """
+    B, nh, T, hd = q.shape
+    S = k_cache.shape[2]
+    g = retrieval_geometry(S, block, top_k)
+    assert g["incomplete_len"] == 0, "tail of an incomplete cached block not restated here"
+    k = g["k"]
+    if idx is None:
+        idx = select_topk(landmark_scores(q, k_cache, cos, sin, block, top_k), k)
+    pos = gather_positions(idx, g["num_mems"], k, block, g["prefix_len"])           # (B,nh,T,k,bs)
+    ksel = apply_rotary(gather_blocks(k_cache, idx, block), cos, sin, pos)          # :408-410
+    vsel = gather_blocks(v_cache, idx, block)
+    ksel = ksel.flatten(3, 4)                                                       # (B,nh,T,k*bs,hd)
+    vsel = vsel.flatten(3, 4)
+    div = math.sqrt(hd)
+    prefix = (q.unsqueeze(3) @ ksel.transpose(3, 4)).squeeze(3) / div               # :412
+    add, im_loc, ls_loc = local_masks(is_mem_loc, T, q.dtype)
+    local = (q @ k_loc.transpose(2, 3)) / div + add                                 # :448,460
+    local = torch.max(local, torch.tensor(torch.finfo(q.dtype).min, dtype=q.dtype)) # :461
+    x = torch.cat((prefix, local), dim=-1)
+    im_prefix = torch.zeros(k * block, dtype=torch.bool)
+    im_prefix[block - 1 :: block] = True                                            # :415
+    im = torch.cat((im_prefix.expand(B, 1, T, -1), im_loc), dim=-1).expand(B, nh, T, -1)
+    ls = torch.cat((torch.zeros(B, 1, T, k * block, dtype=torch.bool), ls_loc), dim=-1).expand(B, nh, T, -1)
+    w = grouped_softmax(x, im, ls, n_buckets).to(q.dtype)                           # :469
+    w_prefix, w_loc = w[..., : k * block], w[..., k * block :]
+    out = w_loc @ v_loc + (w_prefix.unsqueeze(3) @ vsel).squeeze(3)                 # :472-474
+    return out, idx
+
+
+def retrieve_and_attend_s1(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block: int, top_k: int, idx,
+                           heads=None, tokens=None):
+    """Same step as fp32 closed form: the ``k`` retrieved blocks (rotated at their
+    slot positions) act as history blocks in front of the local chunk, whose
+    landmarks sit at fixed stride.  Evaluated for selected heads / tokens of
+    batch 0..B-1; returns dict {(b, h, t): out (hd,) fp32}."""
+    B, nh, T, hd = q.shape
+    S = k_cache.shape[2]
+    g = retrieval_geometry(S, block, top_k)
+    k = g["k"]
+    heads = range(nh) if heads is None else heads
+    tokens = range(T) if tokens is None else tokens
+    res = {}
+    for b in range(B):
+        for h in heads:
+            blocks_k = k_cache[b, h, : g["full_len"]].unflatten(0, (g["num_mems"], block))
+            blocks_v = v_cache[b, h, : g["full_len"]].unflatten(0, (g["num_mems"], block))
+            for t in tokens:
+                sel = idx[b, h, t]
+                pos = gather_positions(sel, g["num_mems"], k, block, g["prefix_len"])
+                ks = apply_rotary(blocks_k[sel], cos, sin, pos).flatten(0, 1)
+                vs = blocks_v[sel].flatten(0, 1)
+                kk = torch.cat((ks, k_loc[b, h]), 0).float()
+                vv = torch.cat((vs, v_loc[b, h]), 0).float()
+                res[(b, h, t)] = s1_attention(q[b, h].float(), kk, vv, block, rows=[t])[0]
+    return res

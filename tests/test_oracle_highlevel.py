@@ -1,0 +1,67 @@
+"""The scatter/gather restatement and the closed form are two independently
+written statements of the same mathematics; they must agree."""
+import math
+
+import pytest
+import torch
+
+from oracle import highlevel, s1
+
+
+def _rand(*shape, seed=0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=torch.float32).to(dtype)
+
+
+@pytest.mark.parametrize("lq,lk,block", [(24, 24, 8), (16, 32, 8), (32, 32, 4), (20, 20, 8)])
+def test_fixed_stride_case_equals_closed_form(lq, lk, block):
+    q, k, v = _rand(2, 2, lq, 8, seed=1), _rand(2, 2, lk, 8, seed=2), _rand(2, 2, lk, 8, seed=3)
+    a = highlevel.attention_fixed_stride(q, k, v, block)
+    b = s1.s1_attention(q, k, v, block)
+    assert torch.isfinite(a).all()
+    assert torch.allclose(a, b, atol=1e-12)
+
+
+def test_fixed_stride_with_exactly_as_many_buckets_as_blocks():
+    # the llama flavour fixes 64 buckets (llama_mem.py:228); 64 blocks just fit.
+    block, nb = 4, 6
+    L = block * nb
+    q, k, v = _rand(1, 1, L, 4, seed=4), _rand(1, 1, L, 4, seed=5), _rand(1, 1, L, 4, seed=6)
+    a = highlevel.attention_fixed_stride(q, k, v, block, n_buckets=nb)
+    assert torch.allclose(a, s1.s1_attention(q, k, v, block), atol=1e-12)
+
+
+def test_lm_benchmark_flavour_equals_closed_form():
+    # BASELINE config 0 in miniature: landmark after every `mem_freq` tokens.
+    B, H, T, d, block = 2, 2, 40, 8, 5
+    q, k, v = _rand(B, H, T, d, seed=7), _rand(B, H, T, d, seed=8), _rand(B, H, T, d, seed=9)
+    is_mem = (torch.arange(T) % block == block - 1)[None].expand(B, T)
+    a = highlevel.attention_lm_benchmark(q, k, v, is_mem, n_buckets=T // block + 3)
+    assert torch.allclose(a, s1.s1_attention(q, k, v, block), atol=1e-12)
+
+
+def test_gradients_through_restatement_equal_closed_form():
+    block = 4
+    q, k, v = _rand(1, 2, 16, 8, seed=10), _rand(1, 2, 16, 8, seed=11), _rand(1, 2, 16, 8, seed=12)
+    do = _rand(1, 2, 16, 8, seed=13)
+    grads = []
+    for fn in (lambda a, b, c: highlevel.attention_fixed_stride(a, b, c, block),
+               lambda a, b, c: s1.s1_attention(a, b, c, block)):
+        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+        grads.append(torch.autograd.grad((fn(qq, kk, vv) * do).sum(), [qq, kk, vv]))
+    for a, b in zip(*grads):
+        assert torch.allclose(a, b, atol=1e-12)
+
+
+def test_irregular_landmarks_row_sums_and_block_structure():
+    # lm_benchmark allows arbitrary landmark positions; rows must still be distributions,
+    # and a row in the first section must be plain causal softmax over non-landmark keys.
+    B, H, T, d = 1, 1, 12, 4
+    q, k = _rand(B, H, T, d, seed=14), _rand(B, H, T, d, seed=15)
+    is_mem = torch.zeros(B, T, dtype=torch.bool)
+    is_mem[0, [2, 6, 9]] = True          # no two adjacent: an empty block would swallow its landmark's mass
+    w = highlevel.attention_lm_benchmark(q, k, torch.eye(T, dtype=torch.float64)[None, None], is_mem, n_buckets=8)
+    assert torch.allclose(w.sum(-1), torch.ones(B, H, T, dtype=torch.float64), atol=1e-12)
+    s = (q[0, 0, 1] @ k[0, 0, :2].T) / math.sqrt(d)
+    assert torch.allclose(w[0, 0, 1, :2], torch.softmax(s, 0), atol=1e-12)
+    assert (w[0, 0][:, is_mem[0]] == 0).all()         # landmark columns never carry weight

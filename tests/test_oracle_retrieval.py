@@ -1,0 +1,132 @@
+"""Pins oracle/rotary.py and oracle/retrieval.py."""
+import math
+
+import pytest
+import torch
+
+from oracle import retrieval, rotary
+
+
+def _rand(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float32) * scale).to(dtype)
+
+
+# ------------------------------------------------------------------ rotary
+def test_rotary_identity_norm_and_relative_property():
+    d = 16
+    cos, sin = rotary.rotary_tables(64, d, torch.float64)
+    x, y = _rand(5, d, seed=1, dtype=torch.float64), _rand(5, d, seed=2, dtype=torch.float64)
+    assert torch.equal(rotary.apply_rotary(x, cos, sin, torch.zeros(5, dtype=torch.long)), x)
+    pos = torch.tensor([6, 9, 17, 40, 63])
+    xr = rotary.apply_rotary(x, cos, sin, pos)
+    pair = lambda t: t[..., : d // 2] ** 2 + t[..., d // 2 :] ** 2
+    assert torch.allclose(pair(xr), pair(x), atol=1e-12)
+    # <rot(x, m), rot(y, n)> depends only on m - n
+    a = (rotary.apply_rotary(x, cos, sin, pos) * rotary.apply_rotary(y, cos, sin, pos - 3)).sum(-1)
+    b = (rotary.apply_rotary(x, cos, sin, pos - 2) * rotary.apply_rotary(y, cos, sin, pos - 5)).sum(-1)
+    assert torch.allclose(a, b, atol=1e-10)
+    # first pair rotates by the full angle: (x0, x_{d/2}) at position 1 turns by 1 radian
+    e = torch.zeros(1, d, dtype=torch.float64)
+    e[0, 0] = 1.0
+    r = rotary.apply_rotary(e, cos, sin, torch.tensor([1]))
+    assert abs(r[0, 0] - math.cos(1.0)) < 1e-7 and abs(r[0, d // 2] - math.sin(1.0)) < 1e-7
+
+
+def test_rotary_equals_torch_bf16_elementwise():
+    d = 32
+    cos, sin = rotary.rotary_tables(128, d, torch.bfloat16)
+    x = _rand(2, 3, 7, d, seed=3, dtype=torch.bfloat16)
+    pos = torch.tensor([0, 5, 31, 64, 99, 100, 127])
+    ours = rotary.apply_rotary(x, cos, sin, pos)
+    theirs = x * cos[pos] + rotary.rotate_half(x) * sin[pos]         # torch rounds after every op
+    assert torch.equal(ours, theirs)
+
+
+# ---------------------------------------------------------------- geometry
+def test_geometry_hand_worked():
+    # 10 cached blocks of 4, top-3: prefix_len = 40 - 16 = 24; older blocks all at slot 0.
+    g = retrieval.retrieval_geometry(40, 4, 3)
+    assert (g["num_mems"], g["k"], g["prefix_len"], g["incomplete_len"]) == (10, 3, 24, 0)
+    assert g["mem_pos"].tolist() == [27] * 7 + [31, 35, 39]          # newest three keep their true positions
+    # BASELINE config 4 numbers
+    g = retrieval.retrieval_geometry(32768, 32, 4)
+    assert g["prefix_len"] == 32608
+    assert g["mem_pos"][:1020].unique().tolist() == [32639]
+    assert g["mem_pos"][1020:].tolist() == [32671, 32703, 32735, 32767]
+    # fewer cached blocks than top_k
+    g = retrieval.retrieval_geometry(8, 4, 5)
+    assert (g["k"], g["prefix_len"]) == (2, -4) and g["mem_pos"].tolist() == [3, 7]
+    # incomplete tail
+    g = retrieval.retrieval_geometry(43, 4, 3)
+    assert (g["full_len"], g["incomplete_len"], g["num_mems"]) == (40, 3, 10)
+
+
+def test_gather_positions_hand_worked():
+    idx = torch.tensor([1, 4, 8, 9])                                  # 10 blocks, k=4: blocks >= 6 are "new"
+    pos = retrieval.gather_positions(idx, 10, 4, 4, 20)
+    assert pos[:, 0].tolist() == [20, 24, 28 + 4, 32 + 4]
+    assert pos[2].tolist() == [32, 33, 34, 35]
+
+
+# --------------------------------------------------------------- selection
+def test_select_topk_brute_force_and_torch_topk_on_untied_rows():
+    g = torch.Generator().manual_seed(4)
+    sc = torch.randn(64, 40, generator=g).to(torch.bfloat16)          # bf16 -> plenty of ties
+    k = 4
+    got = retrieval.select_topk(sc, k)
+    for r in range(sc.shape[0]):
+        row = sc[r].float().tolist()
+        order = sorted(range(len(row)), key=lambda j: (-row[j], j))
+        assert got[r].tolist() == sorted(order[:k])
+    ties = retrieval.boundary_tie_rows(sc, k)
+    assert ties.any() and not ties.all()
+    tk = sc.float().topk(k, dim=-1).indices.sort(-1).values
+    assert torch.equal(got[~ties], tk[~ties])
+
+
+def test_score_contract_rounding_points():
+    B, nh, T, hd, bs, nm = 1, 2, 5, 16, 4, 6
+    q = _rand(B, nh, T, hd, seed=5, dtype=torch.bfloat16, scale=0.5)
+    kc = _rand(B, nh, nm * bs, hd, seed=6, dtype=torch.bfloat16, scale=0.5)
+    cos, sin = rotary.rotary_tables(64, hd, torch.bfloat16)
+    sc = retrieval.landmark_scores(q, kc, cos, sin, bs, 2)
+    g = retrieval.retrieval_geometry(nm * bs, bs, 2)
+    # recompute one entry by hand with python floats
+    b, h, t, m = 0, 1, 3, 4
+    lk = kc[b, h, m * bs + bs - 1]
+    lkr = rotary.apply_rotary(lk[None], cos, sin, g["mem_pos"][m : m + 1])[0]
+    dot = sum(float(a) * float(c) for a, c in zip(q[b, h, t], lkr))
+    two = torch.tensor(dot, dtype=torch.float64).float().bfloat16().float() / torch.tensor(math.sqrt(hd)).float()
+    assert sc[b, h, t, m] == two.bfloat16()
+    assert sc.dtype == torch.bfloat16 and sc.shape == (B, nh, T, nm)
+
+
+# ------------------------------------------------------------------ attend
+def test_gather_blocks_is_a_copy_of_the_selected_blocks():
+    B, nh, T, hd, bs, nm = 1, 2, 3, 4, 4, 5
+    cache = _rand(B, nh, nm * bs, hd, seed=7)
+    idx = torch.tensor([[0, 3], [1, 4], [2, 3]])[None, None].expand(B, nh, T, 2)
+    got = retrieval.gather_blocks(cache, idx, bs)
+    for t in range(T):
+        for j in range(2):
+            blk = int(idx[0, 0, t, j])
+            assert torch.equal(got[0, 1, t, j], cache[0, 1, blk * bs : (blk + 1) * bs])
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+def test_attend_in_model_dtype_equals_fp32_closed_form(dtype, tol):
+    B, nh, T, hd, bs, nm, k = 1, 2, 16, 16, 8, 6, 3
+    S = nm * bs
+    q = _rand(B, nh, T, hd, seed=8, dtype=dtype, scale=0.5)
+    kc = _rand(B, nh, S, hd, seed=9, dtype=dtype, scale=0.5)
+    vc = _rand(B, nh, S, hd, seed=10, dtype=dtype, scale=0.5)
+    kl = _rand(B, nh, T, hd, seed=11, dtype=dtype, scale=0.5)
+    vl = _rand(B, nh, T, hd, seed=12, dtype=dtype, scale=0.5)
+    is_mem = (torch.arange(T) % bs == bs - 1)[None]
+    cos, sin = rotary.rotary_tables(S + T, hd, dtype)
+    out, idx = retrieval.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, bs, k)
+    assert idx.shape == (B, nh, T, k) and (idx[..., 1:] > idx[..., :-1]).all()
+    ref = retrieval.retrieve_and_attend_s1(q, kc, vc, kl, vl, cos, sin, bs, k, idx)
+    for (b, h, t), o in ref.items():
+        assert (out[b, h, t].float() - o).abs().max() < tol, (b, h, t)
