@@ -1,0 +1,66 @@
+/* liblandmark_hip.so — C ABI of the MI355X (gfx950) landmark-attention kernels.
+ *
+ * Plain pointers and sizes only; the caller (the Python shim in
+ * landmark_hip/, or any other host) owns every buffer, passes device pointers
+ * and the HIP stream to run on.  Nothing is allocated, nothing synchronises.
+ *
+ * Return value of every entry point:  0 = launched;  < 0 = argument error
+ * detected on the host before any GPU work (LMK_ERR_*, testable without a GPU);
+ * > 0 = a hipError_t from the launch.
+ *
+ * Tensors are 16-bit (bf16 or fp16), logical shape (B, H, L, D) with element
+ * strides (stride_b, stride_h, stride_row) and unit stride along D.  Every base
+ * pointer and every stride*2 bytes must be a multiple of 16 bytes.
+ */
+#ifndef LMK_H
+#define LMK_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LMK_DTYPE_BF16 0
+#define LMK_DTYPE_F16 1
+
+#define LMK_OK 0
+#define LMK_ERR_NULL (-1)        /* a required pointer is NULL */
+#define LMK_ERR_SHAPE (-2)       /* non-positive or inconsistent sizes */
+#define LMK_ERR_UNSUPPORTED (-3) /* head dim / block size / dtype outside the built set */
+#define LMK_ERR_ALIGN (-4)       /* pointer or stride not 16-byte aligned */
+#define LMK_ERR_HISTORY (-5)     /* Lk - Lq is not n_prefix * block */
+#define LMK_ERR_PARTIAL (-6)     /* backward needs Lq and Lk to be whole blocks */
+#define LMK_ERR_SCALE (-7)       /* softmax scale must be finite and > 0 */
+#define LMK_ERR_WORKSPACE (-8)   /* workspace too small */
+
+typedef struct lmk_tensor4 {
+  void* ptr;          /* device pointer */
+  int64_t stride_b;   /* element strides */
+  int64_t stride_h;
+  int64_t stride_row;
+} lmk_tensor4;
+
+/* Human-readable text for a return code (static storage). */
+const char* lmk_strerror(int code);
+
+/* Library / build identification: "landmark_hip <version> gfx950". */
+const char* lmk_version(void);
+
+/* Forward pass.  Replaces the launch of `_fwd_kernel` in
+ * FusedLandmarkAttention.forward (llama/ltriton/flash_landmark_attention.py:311-353,
+ * kernel :6-122).
+ *   q, o: (B,H,Lq,D); k, v: (B,H,Lk,D); L, M: (B*H, Lq) fp32, contiguous.
+ *   block: landmark block size (landmark = last key of each block); 32, 64 or 128.
+ *   n_prefix: number of history blocks, (Lk - Lq) / block  (:396-398).
+ *   L = sum exp(s - M), M = max of the scaled scores over the query's global bucket
+ *   (natural-log units, as the reference stores them, :116-119).
+ * Lq need not be a multiple of block (the reference masks partial tiles, :44,:118-122). */
+int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                 float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
+                 int n_prefix, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LMK_H */

@@ -1,0 +1,73 @@
+// C ABI of liblandmark_hip.so: argument validation on the host, then dispatch
+// to the kernel launchers.  Declarations and the contract live in include/lmk.h.
+#include <cmath>
+
+#include "lmk_launch.hpp"
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+bool stride_ok(int64_t s) { return (s & 7) == 0; }  // 8 elements x 2 bytes = 16 bytes
+
+int check_tensor(const lmk_tensor4* t) {
+  if (t == nullptr || t->ptr == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(t->ptr) || !stride_ok(t->stride_b) || !stride_ok(t->stride_h) || !stride_ok(t->stride_row))
+    return LMK_ERR_ALIGN;
+  return LMK_OK;
+}
+
+int check_common(int B, int H, int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype) {
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || n_prefix < 0) return LMK_ERR_SHAPE;
+  if (!(D == 64 || D == 128)) return LMK_ERR_UNSUPPORTED;
+  if (!(block == 32 || block == 64 || block == 128)) return LMK_ERR_UNSUPPORTED;
+  if (!(dtype == LMK_DTYPE_BF16 || dtype == LMK_DTYPE_F16)) return LMK_ERR_UNSUPPORTED;
+  if (Lk < Lq || (int64_t)Lk - Lq != (int64_t)n_prefix * block) return LMK_ERR_HISTORY;
+  if (!std::isfinite(sm_scale) || !(sm_scale > 0.f)) return LMK_ERR_SCALE;
+  return LMK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* lmk_strerror(int code) {
+  switch (code) {
+    case LMK_OK: return "ok";
+    case LMK_ERR_NULL: return "a required pointer is NULL";
+    case LMK_ERR_SHAPE: return "non-positive or inconsistent sizes";
+    case LMK_ERR_UNSUPPORTED: return "unsupported head dim (64,128), block size (32,64,128) or dtype (bf16,f16)";
+    case LMK_ERR_ALIGN: return "pointer or stride not 16-byte aligned";
+    case LMK_ERR_HISTORY: return "Lk - Lq must equal n_prefix * block";
+    case LMK_ERR_PARTIAL: return "backward supported only for full blocks";
+    case LMK_ERR_SCALE: return "softmax scale must be finite and > 0";
+    case LMK_ERR_WORKSPACE: return "workspace too small";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  return "unknown error";
+}
+
+const char* lmk_version(void) { return "landmark_hip 0.1 gfx950"; }
+
+int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                 float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
+                 int n_prefix, int dtype, void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o))) return rc;
+  if (L == nullptr || M == nullptr) return LMK_ERR_NULL;
+  if ((rc = check_common(B, H, Lq, Lk, D, sm_scale, block, n_prefix, dtype))) return rc;
+  lmk::FwdParams p;
+  p.q = q->ptr; p.k = k->ptr; p.v = v->ptr; p.o = o->ptr;
+  p.L = L; p.M = M;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
+  p.n_prefix = n_prefix;
+  p.n_qtiles = (Lq + 127) / 128;
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.ks_b = k->stride_b; p.ks_h = k->stride_h; p.ks_r = k->stride_row;
+  p.vs_b = v->stride_b; p.vs_h = v->stride_h; p.vs_r = v->stride_row;
+  p.os_b = o->stride_b; p.os_h = o->stride_h; p.os_r = o->stride_row;
+  p.scale_log2 = sm_scale * 1.4426950408889634f;
+  return lmk::launch_fwd(p, D, block, dtype, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,152 @@
+// Shared device helpers for the gfx950 (CDNA4) landmark-attention kernels.
+//
+// Everything here is written for wave64 and the 32x32x16 bf16/f16 MFMA:
+//   A (32 x 16): lane l holds row  l%32, k = 8*(l/32) .. +7   (8 x 16 bit = 4 VGPRs)
+//   B (16 x 32): lane l holds col  l%32, k = 8*(l/32) .. +7
+//   C (32 x 32): lane l holds col  l%32, rows 8*(r/4) + 4*(l/32) + r%4 for r = 0..15
+// The kernels compute S^T = K Q^T so that a query owns one lane pair (l, l^32):
+// a softmax over the 32 keys of a tile is 16 in-lane values plus one
+// v_permlane32_swap.  The C registers r = 8j .. 8j+7 of a lane then hold keys
+// 16j + {0..3, 8..11} + 4*(l/32), which is used directly as the B operand of the
+// next product with the same key permutation applied to its A operand.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lmk {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
+
+struct bf16_t {};  // element tags
+struct f16_t {};
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// ---- MFMA ---------------------------------------------------------------
+template <class T>
+__device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c);
+template <>
+__device__ __forceinline__ f32x16_t mfma32<bf16_t>(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x16_t mfma32<f16_t>(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+
+// ---- fp32 <-> 16-bit ------------------------------------------------------
+template <class T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <>
+__device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) {
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));  // v_cvt_pk_bf16_f32 (RNE)
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi) {
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+}
+
+template <class T>
+__device__ __forceinline__ float unpack_lo(uint32_t u);
+template <class T>
+__device__ __forceinline__ float unpack_hi(uint32_t u);
+template <>
+__device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t u) { return __uint_as_float(u << 16); }
+template <>
+__device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+template <>
+__device__ __forceinline__ float unpack_lo<f16_t>(uint32_t u) {
+  return (float)__builtin_bit_cast(f16x2_t, u)[0];
+}
+template <>
+__device__ __forceinline__ float unpack_hi<f16_t>(uint32_t u) {
+  return (float)__builtin_bit_cast(f16x2_t, u)[1];
+}
+
+// ---- lane-pair (l, l^32) exchange ----------------------------------------
+// v_permlane32_swap exchanges the upper half of its first operand with the lower
+// half of its second; with both operands equal the two results are, for every
+// lane, the value held by the low lane and by the high lane of its pair.
+__device__ __forceinline__ float pair_max(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float pair_hi(float x) {  // value of the lane with l >= 32
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float pair_lo(float x) {  // value of the lane with l < 32
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// ---- LDS tile addressing ---------------------------------------------------
+// Tiles are stored row-major, ROWB = 2*D bytes per key row, in 16-byte chunks whose
+// index is XOR-swizzled with the row so that both access patterns below spread
+// over all banks.
+//   K tiles: read as MFMA A operand, lane -> (row l%32, 16 B at d = 16*ks + 8*(l/32));
+//            swizzle chunk ^= row & (CH-1) (CH = chunks per row, capped at 16).
+//   V tiles: read with ds_read_b64_tr_b16 (4 rows x 16 columns per 16-lane group);
+//            swizzle chunk ^= (row & 3) << 2 keeps the four rows of a group apart.
+template <int D>
+__device__ __forceinline__ int k_tile_off(int row, int chunk) {
+  constexpr int CH = D / 8;
+  return row * (2 * D) + ((chunk ^ (row & (CH - 1) & 15)) << 4);
+}
+template <int D>
+__device__ __forceinline__ int v_tile_off(int row, int chunk) {
+  constexpr int CH = D / 8;
+  return row * (2 * D) + ((chunk ^ (((row & 3) << 2) & (CH - 1))) << 4);
+}
+
+typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
+
+// Transposed LDS read: inside each group of 16 lanes, lane i supplies the address of
+// 4 consecutive 16-bit columns of row i/4 (columns 4*(i%4)..+3 of a 4 x 16 patch) and
+// receives the 4 rows of column i.
+__device__ __forceinline__ u32x2_t lds_read_tr(const unsigned char* p) {
+  s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+  return __builtin_bit_cast(u32x2_t, v);
+}
+
+// V^T fragment (A operand, rows = 32 head dims of chunk dc, k = 16 keys of step j of the
+// 32-key tile at LDS row base rb) in the key order of the C layout.
+template <int D>
+__device__ __forceinline__ u32x4_t load_vt_frag(const unsigned char* vbuf, int rb, int j, int dc, int lane) {
+  const int h = lane >> 5, i = lane & 15, g2 = (lane >> 4) & 1;
+  const int col = 32 * dc + 16 * g2 + 4 * (i & 3);
+  const int row0 = rb + 16 * j + 4 * h + (i >> 2);
+  u32x2_t a = lds_read_tr(vbuf + v_tile_off<D>(row0, col >> 3) + ((col >> 2) & 1) * 8);
+  u32x2_t b = lds_read_tr(vbuf + v_tile_off<D>(row0 + 8, col >> 3) + ((col >> 2) & 1) * 8);
+  u32x4_t r = {a[0], a[1], b[0], b[1]};
+  return r;
+}
+
+// K fragment (A operand, rows = 32 keys of the tile at LDS row base rb, k = head dims
+// 16*ks + 8*(l/32) .. +7).
+template <int D>
+__device__ __forceinline__ u32x4_t load_k_frag(const unsigned char* kbuf, int rb, int ks, int lane) {
+  const int row = rb + (lane & 31);
+  return *(const u32x4_t*)(kbuf + k_tile_off<D>(row, 2 * ks + (lane >> 5)));
+}
+
+}  // namespace lmk

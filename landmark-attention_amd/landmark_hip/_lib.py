@@ -1,0 +1,74 @@
+"""ctypes binding of liblandmark_hip.so (C ABI declared in include/lmk.h).
+
+The library is the only compute path: if it is missing or a call fails the
+caller gets an exception, never a fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblandmark_hip.so")
+
+DTYPE_CODES = {torch.bfloat16: 0, torch.float16: 1}
+
+
+class LmkError(RuntimeError):
+    def __init__(self, code: int, text: str):
+        super().__init__(f"liblandmark_hip: {text} (code {code})")
+        self.code = code
+
+
+class Tensor4(ctypes.Structure):
+    """``lmk_tensor4`` of include/lmk.h."""
+
+    _fields_ = [("ptr", ctypes.c_void_p), ("stride_b", ctypes.c_int64), ("stride_h", ctypes.c_int64),
+                ("stride_row", ctypes.c_int64)]
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} not found: build it with `python landmark-attention_amd/build.py` "
+                "(hipcc --offload-arch=gfx950); there is no fallback path")
+        L = ctypes.CDLL(LIB_PATH)
+        L.lmk_strerror.restype = ctypes.c_char_p
+        L.lmk_strerror.argtypes = [ctypes.c_int]
+        L.lmk_version.restype = ctypes.c_char_p
+        T4 = ctypes.POINTER(Tensor4)
+        i, f, vp = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+        L.lmk_attn_fwd.restype = i
+        L.lmk_attn_fwd.argtypes = [T4, T4, T4, T4, vp, vp, i, i, i, i, i, f, i, i, i, vp]
+        _lib = L
+    return _lib
+
+
+def check(code: int) -> None:
+    if code != 0:
+        raise LmkError(code, lib().lmk_strerror(code).decode())
+
+
+def tensor4(t: torch.Tensor) -> Tensor4:
+    """Describe a (B, H, L, D) tensor with unit stride along D."""
+    assert t.dim() == 4 and t.stride(3) == 1
+    return Tensor4(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def kernel_ready(t: torch.Tensor) -> torch.Tensor:
+    """Return ``t`` itself when the kernels can read it in place (unit stride along D,
+    16-byte aligned base and strides), otherwise a contiguous copy."""
+    if (t.stride(3) == 1 and t.data_ptr() % 16 == 0 and all(t.stride(i) % 8 == 0 for i in range(3))):
+        return t
+    return t.contiguous()
+
+
+def current_stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

@@ -1,0 +1,85 @@
+"""``fused_landmark_attention`` with the reference's call surface
+(``llama/ltriton/flash_landmark_attention.py:308-403``), backed by the HIP kernels.
+
+Differences a caller can observe, all of them relaxations:
+* ``is_mem=None`` is accepted and means "landmarks at fixed stride" (the reference's
+  README promises this, its code dereferences ``is_mem.shape``, ``:393``);
+* q/k/v views with arbitrary batch/head/row strides are read in place when their last
+  dim is dense and 16-byte aligned (the reference always copies, ``:312-314``).
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+SUPPORTED_BLOCKS = (32, 64, 128)
+SUPPORTED_HEAD_DIMS = (64, 128)
+
+
+def _launch_fwd(q, k, v, n_prefix, sm_scale, block):
+    B, H, Lq, D = q.shape
+    Lk = k.shape[2]
+    o = torch.empty((B, H, Lq, D), device=q.device, dtype=q.dtype)
+    L = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+    M = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+    rc = _lib.lib().lmk_attn_fwd(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o),
+                                 L.data_ptr(), M.data_ptr(), B, H, Lq, Lk, D, float(sm_scale), int(block),
+                                 int(n_prefix), _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+    _lib.check(rc)
+    return o, L, M
+
+
+class FusedLandmarkAttention(torch.autograd.Function):
+    """Same ``forward(ctx, q, k, v, n_prefix_q, sm_scale, block_size)`` /
+    ``backward(ctx, do) -> (dq, dk, dv, None, None, None)`` contract as the reference
+    (``flash_landmark_attention.py:308-389``)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, n_prefix_q, sm_scale, block_size):
+        batch, nheads, seqlen_q, d = q.shape
+        seqlen_k = k.shape[2]
+        assert k.shape == (batch, nheads, seqlen_k, d)
+        assert v.shape == (batch, nheads, seqlen_k, d)
+        assert d <= 128, "FlashAttention only support head dimensions up to 128"
+        assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+        assert q.is_cuda and k.is_cuda and v.is_cuda
+        assert q.dtype in _lib.DTYPE_CODES, "HIP kernels are built for bf16 and fp16"
+        assert d in SUPPORTED_HEAD_DIMS, f"HIP kernels are built for head dims {SUPPORTED_HEAD_DIMS}"
+        assert block_size in SUPPORTED_BLOCKS, f"HIP kernels are built for block sizes {SUPPORTED_BLOCKS}"
+        q, k, v = _lib.kernel_ready(q), _lib.kernel_ready(k), _lib.kernel_ready(v)
+        with torch.cuda.device(q.device):
+            o, L, m = _launch_fwd(q, k, v, n_prefix_q, sm_scale, block_size)
+        ctx.save_for_backward(q, k, v, o, L, m)
+        ctx.sm_scale = sm_scale
+        ctx.N_PREFIX_Q = n_prefix_q
+        ctx.BLOCK = block_size
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        raise NotImplementedError("backward kernels not built yet")
+
+
+def fused_landmark_attention(q, k, v, is_mem, sm_scale=None, block_size=64):
+    """Landmark grouped-softmax causal attention, landmarks at every ``block_size``-th key.
+
+    q: (B, H, Lq, D); k, v: (B, H, Lk, D) with ``Lk - Lq`` a whole number of blocks of
+    history.  ``is_mem`` (bool, last dim Lk) must mark exactly the positions
+    ``j % block_size == block_size - 1`` (checked as in the reference, ``:393-394``, which
+    costs one device->host sync); pass ``None`` to skip the check.
+    """
+    if is_mem is not None:
+        expected_is_mem = torch.arange(0, is_mem.shape[-1], device=is_mem.device) % block_size == (block_size - 1)
+        assert (is_mem == expected_is_mem).all()
+
+    n_history_kv = k.shape[-2] - q.shape[-2]
+    assert n_history_kv % block_size == 0
+    n_history_blocks = n_history_kv // block_size
+
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(q.size(-1))
+
+    return FusedLandmarkAttention.apply(q, k, v, n_history_blocks, sm_scale, block_size)
