@@ -15,6 +15,7 @@
 #ifndef LMK_H
 #define LMK_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -59,6 +60,24 @@ const char* lmk_version(void);
 int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                  float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
                  int n_prefix, int dtype, void* stream);
+
+/* Bytes of device workspace lmk_attn_bwd needs (0 for invalid sizes):
+ * 2*(B*H*Lq) floats of per-row terms + 2*(B*H*(Lk/block)*Lq) floats of per-(row, block)
+ * terms handed from the dQ kernel to the dK/dV kernel. */
+size_t lmk_attn_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int block);
+
+/* Backward pass.  Replaces the launches of `_bwd_preprocess` and `_bwd_kernel` in
+ * FusedLandmarkAttention.backward (llama/ltriton/flash_landmark_attention.py:356-389,
+ * kernels :125-149 and :152-305).
+ *   inputs: q, k, v, o (forward output), dout (gradient of o), L, M (forward statistics);
+ *   outputs: dq (B,H,Lq,D), dk, dv (B,H,Lk,D) in the tensors' 16-bit dtype (accumulated in
+ *   fp32, rounded once); every element is written, nothing needs zeroing.
+ *   workspace: 16-byte aligned device memory of at least lmk_attn_bwd_workspace_bytes().
+ * Lq and Lk must be multiples of block (as in the reference, :359-360). */
+int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                 const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                 const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B, int H,
+                 int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

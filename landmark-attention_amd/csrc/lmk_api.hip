@@ -70,4 +70,51 @@ int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
   return lmk::launch_fwd(p, D, block, dtype, (hipStream_t)stream);
 }
 
+size_t lmk_attn_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int block) {
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || block <= 0) return 0;
+  const size_t rows = (size_t)B * H * Lq;
+  const size_t nb = (size_t)(Lk / block);
+  return sizeof(float) * (2 * rows + 2 * rows * nb);
+}
+
+int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                 const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                 const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B, int H,
+                 int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype, void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o)) ||
+      (rc = check_tensor(dout)) || (rc = check_tensor(dq)) || (rc = check_tensor(dk)) || (rc = check_tensor(dv)))
+    return rc;
+  if (L == nullptr || M == nullptr || workspace == nullptr) return LMK_ERR_NULL;
+  if ((rc = check_common(B, H, Lq, Lk, D, sm_scale, block, n_prefix, dtype))) return rc;
+  if (Lq % block != 0 || Lk % block != 0) return LMK_ERR_PARTIAL;
+  if (!aligned16(workspace)) return LMK_ERR_ALIGN;
+  if (workspace_bytes < lmk_attn_bwd_workspace_bytes(B, H, Lq, Lk, block)) return LMK_ERR_WORKSPACE;
+  lmk::BwdParams p;
+  p.q = q->ptr; p.k = k->ptr; p.v = v->ptr; p.o = o->ptr; p.dout = dout->ptr;
+  p.dq = dq->ptr; p.dk = dk->ptr; p.dv = dv->ptr;
+  p.L = L; p.M = M;
+  const size_t rows = (size_t)B * H * Lq;
+  const size_t nb = (size_t)(Lk / block);
+  float* w = static_cast<float*>(workspace);
+  p.delta = w;
+  p.mhat = w + rows;
+  p.stat_a = w + 2 * rows;
+  p.stat_n = w + 2 * rows + rows * nb;
+  p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
+  p.n_prefix = n_prefix; p.n_blocks = (int)nb;
+  p.n_qtiles = (Lq + 127) / 128; p.n_kvtiles = (Lk + 127) / 128;
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.ks_b = k->stride_b; p.ks_h = k->stride_h; p.ks_r = k->stride_row;
+  p.vs_b = v->stride_b; p.vs_h = v->stride_h; p.vs_r = v->stride_row;
+  p.os_b = o->stride_b; p.os_h = o->stride_h; p.os_r = o->stride_row;
+  p.dos_b = dout->stride_b; p.dos_h = dout->stride_h; p.dos_r = dout->stride_row;
+  p.dqs_b = dq->stride_b; p.dqs_h = dq->stride_h; p.dqs_r = dq->stride_row;
+  p.dks_b = dk->stride_b; p.dks_h = dk->stride_h; p.dks_r = dk->stride_row;
+  p.dvs_b = dv->stride_b; p.dvs_h = dv->stride_h; p.dvs_r = dv->stride_row;
+  p.scale = sm_scale;
+  p.scale_log2 = sm_scale * 1.4426950408889634f;
+  return lmk::launch_bwd(p, D, block, dtype, (hipStream_t)stream);
+}
+
 }  // extern "C"

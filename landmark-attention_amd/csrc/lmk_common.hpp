@@ -98,24 +98,22 @@ __device__ __forceinline__ float pair_lo(float x) {  // value of the lane with l
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
 // ---- LDS tile addressing ---------------------------------------------------
-// Tiles are stored row-major, ROWB = 2*D bytes per key row, in 16-byte chunks whose
-// index is XOR-swizzled with the row so that both access patterns below spread
-// over all banks.
-//   K tiles: read as MFMA A operand, lane -> (row l%32, 16 B at d = 16*ks + 8*(l/32));
-//            swizzle chunk ^= row & (CH-1) (CH = chunks per row, capped at 16).
-//   V tiles: read with ds_read_b64_tr_b16 (4 rows x 16 columns per 16-lane group);
-//            swizzle chunk ^= (row & 3) << 2 keeps the four rows of a group apart.
+// Tiles are stored row-major, 2*D bytes per row, in 16-byte chunks whose index is
+// XOR-swizzled with f(row) = ((row & 3) << 2) | ((row >> 2) & 3).  One layout serves
+// both ways a tile is read:
+//   * as an MFMA operand with the head dim along k: lane -> (row l%32, one 16-byte chunk);
+//     f is a bijection on 16 consecutive rows, so 16 lanes cover all 16 chunk columns;
+//   * transposed, with ds_read_b64_tr_b16: a 16-lane group touches 4 consecutive rows x
+//     32 bytes; the (row & 3) << 2 term sends the four rows to four different 64-byte
+//     column groups.
 template <int D>
-__device__ __forceinline__ int k_tile_off(int row, int chunk) {
+__device__ __forceinline__ int tile_off(int row, int chunk) {
   constexpr int CH = D / 8;
-  return row * (2 * D) + ((chunk ^ (row & (CH - 1) & 15)) << 4);
-}
-template <int D>
-__device__ __forceinline__ int v_tile_off(int row, int chunk) {
-  constexpr int CH = D / 8;
-  return row * (2 * D) + ((chunk ^ (((row & 3) << 2) & (CH - 1))) << 4);
+  const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (CH - 1);
+  return row * (2 * D) + ((chunk ^ f) << 4);
 }
 
 typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
@@ -128,25 +126,26 @@ __device__ __forceinline__ u32x2_t lds_read_tr(const unsigned char* p) {
   return __builtin_bit_cast(u32x2_t, v);
 }
 
-// V^T fragment (A operand, rows = 32 head dims of chunk dc, k = 16 keys of step j of the
-// 32-key tile at LDS row base rb) in the key order of the C layout.
+// Transposed fragment of a row-major tile (A operand, rows = 32 head dims of chunk dc,
+// k = 16 tile rows of step j of the 32-row tile at LDS row base rb) in the row order of
+// the C layout: register pair 0 holds rows 16j + 4h + {0..3}, pair 1 rows 16j + 8 + 4h + {0..3}.
 template <int D>
-__device__ __forceinline__ u32x4_t load_vt_frag(const unsigned char* vbuf, int rb, int j, int dc, int lane) {
+__device__ __forceinline__ u32x4_t load_tr_frag(const unsigned char* vbuf, int rb, int j, int dc, int lane) {
   const int h = lane >> 5, i = lane & 15, g2 = (lane >> 4) & 1;
   const int col = 32 * dc + 16 * g2 + 4 * (i & 3);
   const int row0 = rb + 16 * j + 4 * h + (i >> 2);
-  u32x2_t a = lds_read_tr(vbuf + v_tile_off<D>(row0, col >> 3) + ((col >> 2) & 1) * 8);
-  u32x2_t b = lds_read_tr(vbuf + v_tile_off<D>(row0 + 8, col >> 3) + ((col >> 2) & 1) * 8);
+  u32x2_t a = lds_read_tr(vbuf + tile_off<D>(row0, col >> 3) + ((col >> 2) & 1) * 8);
+  u32x2_t b = lds_read_tr(vbuf + tile_off<D>(row0 + 8, col >> 3) + ((col >> 2) & 1) * 8);
   u32x4_t r = {a[0], a[1], b[0], b[1]};
   return r;
 }
 
-// K fragment (A operand, rows = 32 keys of the tile at LDS row base rb, k = head dims
+// Row fragment (A operand, rows = the 32 rows of the tile at LDS row base rb, k = head dims
 // 16*ks + 8*(l/32) .. +7).
 template <int D>
-__device__ __forceinline__ u32x4_t load_k_frag(const unsigned char* kbuf, int rb, int ks, int lane) {
+__device__ __forceinline__ u32x4_t load_row_frag(const unsigned char* kbuf, int rb, int ks, int lane) {
   const int row = rb + (lane & 31);
-  return *(const u32x4_t*)(kbuf + k_tile_off<D>(row, 2 * ks + (lane >> 5)));
+  return *(const u32x4_t*)(kbuf + tile_off<D>(row, 2 * ks + (lane >> 5)));
 }
 
 }  // namespace lmk

@@ -95,8 +95,8 @@ __global__ __launch_bounds__(256, (BS >= 128 ? 1 : 2)) void lmk_fwd_kernel(FwdPa
 #pragma unroll
     for (int i = 0; i < C::NCH; ++i) {
       const int id = tid + 256 * i, row = id / C::CH, ch = id % C::CH;
-      *(u32x4_t*)(kb + k_tile_off<D>(row, ch)) = kreg[i];
-      *(u32x4_t*)(vb + v_tile_off<D>(row, ch)) = vreg[i];
+      *(u32x4_t*)(kb + tile_off<D>(row, ch)) = kreg[i];
+      *(u32x4_t*)(vb + tile_off<D>(row, ch)) = vreg[i];
     }
   };
 
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256, (BS >= 128 ? 1 : 2)) void lmk_fwd_kernel(FwdPa
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(load_k_frag<D>(kb, rb, ks, lane), qf[ks], s);
+    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(load_row_frag<D>(kb, rb, ks, lane), qf[ks], s);
     return s;
   };
   auto pv_tile = [&](const unsigned char* vb, int rb, const float* w) {
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256, (BS >= 128 ? 1 : 2)) void lmk_fwd_kernel(FwdPa
       u32x4_t wf = {pack2<T>(w[8 * j + 0], w[8 * j + 1]), pack2<T>(w[8 * j + 2], w[8 * j + 3]),
                     pack2<T>(w[8 * j + 4], w[8 * j + 5]), pack2<T>(w[8 * j + 6], w[8 * j + 7])};
 #pragma unroll
-      for (int dc = 0; dc < C::DC; ++dc) acc[dc] = mfma32<T>(load_vt_frag<D>(vb, rb, j, dc, lane), wf, acc[dc]);
+      for (int dc = 0; dc < C::DC; ++dc) acc[dc] = mfma32<T>(load_tr_frag<D>(vb, rb, j, dc, lane), wf, acc[dc]);
     }
   };
   auto rescale = [&](float alpha) {

@@ -22,4 +22,20 @@ struct FwdParams {
 
 int launch_fwd(const FwdParams& p, int D, int BS, int dtype, hipStream_t stream);
 
+struct BwdParams {
+  const void *q, *k, *v, *o, *dout;
+  void *dq, *dk, *dv;
+  const float *L, *M;            // forward statistics, (B*H, Lq)
+  float *delta, *mhat;           // (B*H, Lq) each, written by the pre kernel
+  float *stat_a, *stat_n;        // (B*H, n_blocks, Lq) each, written by the dq kernel
+  int B, H, Lq, Lk;
+  int n_prefix, n_blocks;        // history blocks; Lk / block
+  int n_qtiles, n_kvtiles;       // ceil(Lq / 128), ceil(Lk / 128)
+  int64_t qs_b, qs_h, qs_r, ks_b, ks_h, ks_r, vs_b, vs_h, vs_r, os_b, os_h, os_r, dos_b, dos_h, dos_r;
+  int64_t dqs_b, dqs_h, dqs_r, dks_b, dks_h, dks_r, dvs_b, dvs_h, dvs_r;
+  float scale, scale_log2;
+};
+
+int launch_bwd(const BwdParams& p, int D, int BS, int dtype, hipStream_t stream);
+
 }  // namespace lmk

@@ -32,6 +32,23 @@ def _launch_fwd(q, k, v, n_prefix, sm_scale, block):
     return o, L, M
 
 
+def _launch_bwd(q, k, v, o, do, L, M, n_prefix, sm_scale, block):
+    B, H, Lq, D = q.shape
+    Lk = k.shape[2]
+    lib = _lib.lib()
+    dq = torch.empty((B, H, Lq, D), device=q.device, dtype=q.dtype)
+    dk = torch.empty((B, H, Lk, D), device=q.device, dtype=q.dtype)
+    dv = torch.empty((B, H, Lk, D), device=q.device, dtype=q.dtype)
+    nbytes = lib.lmk_attn_bwd_workspace_bytes(B, H, Lq, Lk, int(block))
+    ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+    rc = lib.lmk_attn_bwd(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o), _lib.tensor4(do),
+                          L.data_ptr(), M.data_ptr(), _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv),
+                          ws.data_ptr(), nbytes, B, H, Lq, Lk, D, float(sm_scale), int(block), int(n_prefix),
+                          _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+    _lib.check(rc)
+    return dq, dk, dv
+
+
 class FusedLandmarkAttention(torch.autograd.Function):
     """Same ``forward(ctx, q, k, v, n_prefix_q, sm_scale, block_size)`` /
     ``backward(ctx, do) -> (dq, dk, dv, None, None, None)`` contract as the reference
@@ -60,7 +77,14 @@ class FusedLandmarkAttention(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do):
-        raise NotImplementedError("backward kernels not built yet")
+        BLOCK = ctx.BLOCK
+        q, k, v, o, l, m = ctx.saved_tensors
+        assert q.shape[2] % BLOCK == 0, "Backward supported only for full blocks"
+        assert k.shape[2] % BLOCK == 0, "Backward supported only for full blocks"
+        do = _lib.kernel_ready(do)
+        with torch.cuda.device(q.device):
+            dq, dk, dv = _launch_bwd(q, k, v, o, do, l, m, ctx.N_PREFIX_Q, ctx.sm_scale, BLOCK)
+        return dq, dk, dv, None, None, None
 
 
 def fused_landmark_attention(q, k, v, is_mem, sm_scale=None, block_size=64):
