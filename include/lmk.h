@@ -34,6 +34,9 @@ extern "C" {
 #define LMK_ERR_PARTIAL (-6)     /* backward needs Lq and Lk to be whole blocks */
 #define LMK_ERR_SCALE (-7)       /* softmax scale must be finite and > 0 */
 #define LMK_ERR_WORKSPACE (-8)   /* workspace too small */
+#define LMK_ERR_CACHE (-9)       /* cached length is not a positive whole number of blocks */
+#define LMK_ERR_TOPK (-10)       /* top_k outside 1..64 */
+#define LMK_ERR_TABLE (-11)      /* rotary tables hold fewer positions than the cache */
 
 typedef struct lmk_tensor4 {
   void* ptr;          /* device pointer */
@@ -78,6 +81,40 @@ int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
                  const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
                  const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B, int H,
                  int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype, void* stream);
+
+/* ---- mem-cache retrieval (inference) --------------------------------------------------
+ * The reference has no function boundary here: scoring, selection and gather are inline in
+ * LlamaAttention.forward (llama/llama_mem.py:318-430) and the attend step follows at :447-477.
+ * Conventions kept from there: the cache tuple is (K without rotary, V), each (B,H,S,D)
+ * (:424-430); a block is mem_freq+1 tokens whose last token is the landmark; queries arrive
+ * rotated; cos/sin are (n_pos, D) tables in the model dtype with the half-split layout of
+ * LlamaRotaryEmbedding (:95-124) and `table_stride_row` elements between rows.
+ * S must be a positive multiple of block (no incomplete cached block). */
+
+/* Bytes of device workspace lmk_retrieve_topk needs: rotated landmark keys and their norms,
+ * plus two fp32 score planes of B*H*T*(S/block). */
+size_t lmk_retrieve_workspace_bytes(int B, int H, int T, int S, int D, int block);
+
+/* Landmark scoring + top-k selection (llama_mem.py:344-384, aggregate=None branch).
+ *   idx_out: (B,H,T,k) int64, k = min(top_k, S/block), block indices in ascending order.
+ * Score of (query, block) = fp32 dot product accumulated sequentially over the head dim,
+ * rounded to the model dtype, divided by sqrt(D) in fp32 and rounded again; the k best
+ * under (score descending, index ascending) are selected. */
+int lmk_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table, const void* sin_table,
+                      int64_t table_stride_row, int64_t n_pos, int64_t* idx_out, void* workspace,
+                      size_t workspace_bytes, int B, int H, int T, int S, int D, int block, int top_k, int dtype,
+                      void* stream);
+
+/* Gather of the selected K/V blocks with rotary at their slot positions and attention over
+ * them (llama_mem.py:386-412), merged with the attention over the local chunk (:447-477).
+ *   o_loc, L_loc, M_loc: output and statistics of lmk_attn_fwd run on the local chunk
+ *   (q against the T new keys/values); out: (B,H,T,D) final attention output.
+ * Blocks are read in place from the cache; nothing of size (T, k*block, D) is materialised.
+ * Built for D = 128 and block 32 or 64. */
+int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+                      const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
+                      const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, const lmk_tensor4* out, int B,
+                      int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

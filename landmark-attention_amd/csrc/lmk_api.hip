@@ -26,6 +26,42 @@ int check_common(int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
   return LMK_OK;
 }
 
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+struct RetrLayout {
+  size_t lk_rot, lk_norm, approx, exact, total;
+};
+
+RetrLayout retr_layout(int B, int H, int T, int S, int D, int block) {
+  const size_t bh = (size_t)B * H, nm = (size_t)(S / block);
+  RetrLayout l;
+  l.lk_rot = 0;
+  l.lk_norm = align256(l.lk_rot + bh * nm * D * 2);
+  l.approx = align256(l.lk_norm + bh * nm * 4);
+  l.exact = align256(l.approx + bh * T * nm * 4);
+  l.total = align256(l.exact + bh * T * nm * 4);
+  return l;
+}
+
+int check_retrieval(int B, int H, int T, int S, int D, int block, int top_k, int dtype, int64_t n_pos) {
+  if (B <= 0 || H <= 0 || T <= 0 || S <= 0) return LMK_ERR_SHAPE;
+  if (!(D == 64 || D == 128)) return LMK_ERR_UNSUPPORTED;
+  if (block < 2 || block > 4096) return LMK_ERR_UNSUPPORTED;
+  if (!(dtype == LMK_DTYPE_BF16 || dtype == LMK_DTYPE_F16)) return LMK_ERR_UNSUPPORTED;
+  if (S < block || S % block != 0) return LMK_ERR_CACHE;
+  if (top_k < 1 || top_k > 64) return LMK_ERR_TOPK;
+  if (n_pos < S) return LMK_ERR_TABLE;
+  return LMK_OK;
+}
+
+void fill_retr_common(lmk::RetrParams& p, int B, int H, int T, int S, int D, int block, int top_k) {
+  p.B = B; p.H = H; p.T = T; p.S = S; p.block = block;
+  p.num_mems = S / block;
+  p.k = top_k < p.num_mems ? top_k : p.num_mems;
+  p.prefix_len = (int64_t)S - (int64_t)(p.k + 1) * block;
+  p.sqrt_hd = (float)std::sqrt((double)D);
+}
+
 }  // namespace
 
 extern "C" {
@@ -41,6 +77,9 @@ const char* lmk_strerror(int code) {
     case LMK_ERR_PARTIAL: return "backward supported only for full blocks";
     case LMK_ERR_SCALE: return "softmax scale must be finite and > 0";
     case LMK_ERR_WORKSPACE: return "workspace too small";
+    case LMK_ERR_CACHE: return "cache must hold at least one whole block and no incomplete block";
+    case LMK_ERR_TOPK: return "top_k must be in 1..64";
+    case LMK_ERR_TABLE: return "rotary tables shorter than the cached length";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -115,6 +154,66 @@ int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
   p.scale = sm_scale;
   p.scale_log2 = sm_scale * 1.4426950408889634f;
   return lmk::launch_bwd(p, D, block, dtype, (hipStream_t)stream);
+}
+
+size_t lmk_retrieve_workspace_bytes(int B, int H, int T, int S, int D, int block) {
+  if (B <= 0 || H <= 0 || T <= 0 || S <= 0 || D <= 0 || block <= 0) return 0;
+  return retr_layout(B, H, T, S, D, block).total;
+}
+
+int lmk_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table, const void* sin_table,
+                      int64_t table_stride_row, int64_t n_pos, int64_t* idx_out, void* workspace,
+                      size_t workspace_bytes, int B, int H, int T, int S, int D, int block, int top_k, int dtype,
+                      void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache))) return rc;
+  if (cos_table == nullptr || sin_table == nullptr || idx_out == nullptr || workspace == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row) || !aligned16(workspace))
+    return LMK_ERR_ALIGN;
+  if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
+  const RetrLayout l = retr_layout(B, H, T, S, D, block);
+  if (workspace_bytes < l.total) return LMK_ERR_WORKSPACE;
+  lmk::RetrParams p = {};
+  fill_retr_common(p, B, H, T, S, D, block, top_k);
+  p.q = q->ptr; p.kcache = kcache->ptr; p.cos = cos_table; p.sin = sin_table; p.idx = idx_out;
+  char* w = static_cast<char*>(workspace);
+  p.lk_rot = w + l.lk_rot;
+  p.lk_norm = reinterpret_cast<float*>(w + l.lk_norm);
+  p.approx = reinterpret_cast<float*>(w + l.approx);
+  p.exact = reinterpret_cast<float*>(w + l.exact);
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
+  p.cs_r = table_stride_row;
+  return lmk::launch_retrieve_topk(p, D, dtype, (hipStream_t)stream);
+}
+
+int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+                      const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
+                      const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, const lmk_tensor4* out, int B,
+                      int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache)) || (rc = check_tensor(vcache)) ||
+      (rc = check_tensor(o_loc)) || (rc = check_tensor(out)))
+    return rc;
+  if (cos_table == nullptr || sin_table == nullptr || idx == nullptr || L_loc == nullptr || M_loc == nullptr)
+    return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
+  if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
+  if (D != 128 || !(block == 32 || block == 64)) return LMK_ERR_UNSUPPORTED;
+  if (!std::isfinite(sm_scale) || !(sm_scale > 0.f)) return LMK_ERR_SCALE;
+  lmk::RetrParams p = {};
+  fill_retr_common(p, B, H, T, S, D, block, top_k);
+  p.q = q->ptr; p.kcache = kcache->ptr; p.vcache = vcache->ptr; p.cos = cos_table; p.sin = sin_table;
+  p.idx = const_cast<int64_t*>(idx);
+  p.o_loc = o_loc->ptr; p.L_loc = L_loc; p.M_loc = M_loc; p.out = out->ptr;
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
+  p.vcs_b = vcache->stride_b; p.vcs_h = vcache->stride_h; p.vcs_r = vcache->stride_row;
+  p.ols_b = o_loc->stride_b; p.ols_h = o_loc->stride_h; p.ols_r = o_loc->stride_row;
+  p.outs_b = out->stride_b; p.outs_h = out->stride_h; p.outs_r = out->stride_row;
+  p.cs_r = table_stride_row;
+  p.scale_log2 = sm_scale * 1.4426950408889634f;
+  return lmk::launch_gather_attend(p, D, block, dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -38,4 +38,23 @@ struct BwdParams {
 
 int launch_bwd(const BwdParams& p, int D, int BS, int dtype, hipStream_t stream);
 
+struct RetrParams {
+  const void *q, *kcache, *vcache, *cos, *sin;   // q rotated; caches un-rotated; tables (n_pos, D)
+  const void* o_loc;                              // attention over the local chunk (gather step)
+  const float *L_loc, *M_loc;
+  void* out;
+  int64_t* idx;                                   // (B, H, T, k) ascending block indices
+  void* lk_rot;                                   // (B*H, num_mems, D) rotated landmark keys
+  float* lk_norm;                                 // (B*H, num_mems)
+  float *approx, *exact;                          // (B*H*T, num_mems) each
+  int B, H, T, S, block, num_mems, k;
+  int64_t prefix_len;                             // full_len - (k + 1) * block, may be -block
+  int64_t qs_b, qs_h, qs_r, kcs_b, kcs_h, kcs_r, vcs_b, vcs_h, vcs_r, cs_r;
+  int64_t ols_b, ols_h, ols_r, outs_b, outs_h, outs_r;
+  float sqrt_hd, scale_log2;
+};
+
+int launch_retrieve_topk(const RetrParams& p, int D, int dtype, hipStream_t stream);
+int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream);
+
 }  // namespace lmk

@@ -1,0 +1,458 @@
+// Mem-cache retrieval for gfx950: landmark scoring, top-k block selection, gather + attend.
+//
+// Replaces the inline retrieval of LlamaAttention.forward (llama/llama_mem.py:344-412) and
+// the attend step over retrieved blocks (:447-477) for the per-head, per-token branch.
+//
+// Selection must be reproducible bit for bit, so the score of (query, landmark) is defined
+// as: fp32 dot product accumulated sequentially over the head dim with one fma per element,
+// rounded to the model dtype, divided in fp32 by sqrt(hd), rounded again (the two roundings of
+// `matmul(...) / math.sqrt(head_dim)`, :367).  Evaluating that for every pair on the vector
+// ALU would dominate the step, so the work is split:
+//   lk      rotate every cached landmark key at its slot position (:359-366), exactly as the
+//           model dtype would round it, into a dense side array, with its 2-norm
+//   score   MFMA product q . lk^T -> approximate fp32 scores
+//   select  per query: bracket every score by the accumulation-error bound
+//           eps = 2^-14 |q| |k|, push both ends through the (monotone) rounding contract, find
+//           the k-th best lower end, and re-evaluate in the defined order only the "contenders"
+//           whose upper end reaches it; then pick the k best under (score desc, index asc)
+//           and write them in ascending order as int64 (:384).
+//   gather  per query: stream the k selected K/V blocks straight from the cache, rotate keys at
+//           their gather positions (:386-388, :408-410), local softmax per block gated by its
+//           landmark, and merge with the attention over the local chunk (computed by the fused
+//           forward kernel) through the shared global softmax bucket.
+#include "lmk_common.hpp"
+#include "lmk_launch.hpp"
+
+namespace lmk {
+
+template <class T>
+__device__ __forceinline__ float round_to(float x) {  // fp32 -> T (RNE) -> fp32
+  return unpack_lo<T>(pack2<T>(x, 0.f));
+}
+
+// rotary on 8 consecutive head dims held as 4 packed dwords; `other` holds the chunk D/2 away
+template <class T>
+__device__ __forceinline__ void rotate_chunk(const u32x4_t x, const u32x4_t other, const u32x4_t c, const u32x4_t s,
+                                             bool upper_half, float* out) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float x0 = unpack_lo<T>(x[i]), x1 = unpack_hi<T>(x[i]);
+    float r0 = unpack_lo<T>(other[i]), r1 = unpack_hi<T>(other[i]);
+    if (!upper_half) {  // rotate_half: first half gets -x[d + D/2], second half gets x[d - D/2]
+      r0 = -r0;
+      r1 = -r1;
+    }
+    const float a0 = round_to<T>(x0 * unpack_lo<T>(c[i])), a1 = round_to<T>(x1 * unpack_hi<T>(c[i]));
+    const float b0 = round_to<T>(r0 * unpack_lo<T>(s[i])), b1 = round_to<T>(r1 * unpack_hi<T>(s[i]));
+    out[2 * i] = round_to<T>(a0 + b0);
+    out[2 * i + 1] = round_to<T>(a1 + b1);
+  }
+}
+
+__device__ __forceinline__ u32x4_t shfl_xor4(u32x4_t v, int mask) {
+  u32x4_t r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = (uint32_t)__shfl_xor((int)v[i], mask, 64);
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// lk: rotated landmark keys (dense) and their norms
+// ---------------------------------------------------------------------------
+template <class T, int D>
+__global__ __launch_bounds__(256) void lmk_landmark_keys_kernel(RetrParams p) {
+  constexpr int LPR = D / 8;
+  constexpr int RPW = 256 / LPR;
+  const int tid = threadIdx.x, j = tid % LPR;
+  const int64_t row = (int64_t)blockIdx.x * RPW + tid / LPR;      // (bh, m)
+  const int64_t total = (int64_t)p.B * p.H * p.num_mems;
+  float nrm = 0.f;
+  if (row < total) {
+    const int bh = (int)(row / p.num_mems), m = (int)(row % p.num_mems);
+    const int b = bh / p.H, hh = bh % p.H;
+    const int slot = (m < p.num_mems - p.k) ? 0 : m - (p.num_mems - p.k) + 1;
+    const int64_t pos = (int64_t)slot * p.block + (p.block - 1) + p.prefix_len;
+    const char* src = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h + ((int64_t)m * p.block + p.block - 1) * p.kcs_r);
+    const u32x4_t x = *(const u32x4_t*)(src + 16 * j);
+    const u32x4_t other = *(const u32x4_t*)(src + 16 * (j ^ (LPR / 2)));
+    const u32x4_t c = *(const u32x4_t*)((const char*)p.cos + 2 * (pos * p.cs_r) + 16 * j);
+    const u32x4_t s = *(const u32x4_t*)((const char*)p.sin + 2 * (pos * p.cs_r) + 16 * j);
+    float r[8];
+    rotate_chunk<T>(x, other, c, s, j >= LPR / 2, r);
+    u32x4_t o = {pack2<T>(r[0], r[1]), pack2<T>(r[2], r[3]), pack2<T>(r[4], r[5]), pack2<T>(r[6], r[7])};
+    *(u32x4_t*)((char*)p.lk_rot + 2 * (row * D) + 16 * j) = o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) nrm += r[i] * r[i];
+  }
+#pragma unroll
+  for (int msk = LPR / 2; msk >= 1; msk >>= 1) nrm += __shfl_xor(nrm, msk, 64);
+  if (row < total && j == 0) p.lk_norm[row] = sqrtf(nrm) * 1.000001f;
+}
+
+// ---------------------------------------------------------------------------
+// score: approximate fp32 scores with MFMA, S^T layout (lane = query, registers = landmarks)
+// ---------------------------------------------------------------------------
+template <class T, int D>
+__global__ __launch_bounds__(256) void lmk_score_kernel(RetrParams p) {
+  constexpr int KS = D / 16;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ql = lane & 31, h = lane >> 5;
+  const int n_qt = (p.T + 127) / 128;
+  const int bh = blockIdx.x / n_qt, qt = blockIdx.x % n_qt;
+  const int b = bh / p.H, hh = bh % p.H;
+  const int q0 = qt * 128 + wave * 32;
+  if (q0 >= p.T) return;
+  const int qrow = q0 + ql;
+  const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h);
+  u32x4_t qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    u32x4_t z = {0, 0, 0, 0};
+    qf[ks] = z;
+    if (qrow < p.T) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
+  }
+  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * p.num_mems * D);
+  float* out = p.approx + ((int64_t)bh * p.T + qrow) * p.num_mems;
+  for (int m0 = 0; m0 < p.num_mems; m0 += 32) {
+    const int m = m0 + ql;
+    f32x16_t s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4_t a = {0, 0, 0, 0};
+      if (m < p.num_mems) a = *(const u32x4_t*)(lk + 2 * ((int64_t)m * D + 16 * ks + 8 * h));
+      s = mfma32<T>(a, qf[ks], s);
+    }
+    if (qrow < p.T) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int mm = m0 + 8 * (r >> 2) + 4 * h + (r & 3);
+        if (mm < p.num_mems) out[mm] = s[r];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// select: exact top-k per query row, one wave per row
+// ---------------------------------------------------------------------------
+template <class T>
+__device__ __forceinline__ float contract(float dot, float sqrt_hd) {
+  return round_to<T>(__fdiv_rn(round_to<T>(dot), sqrt_hd));
+}
+
+// wave-wide arg-best under (value desc, index asc); every lane gets the winner
+__device__ __forceinline__ void wave_best(float& v, int& i) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    const float ov = __shfl_xor(v, m, 64);
+    const int oi = __shfl_xor(i, m, 64);
+    if (ov > v || (ov == v && oi < i)) {
+      v = ov;
+      i = oi;
+    }
+  }
+}
+
+constexpr int kSelSeg = 1024;   // landmarks handled per sweep of the contender list
+
+template <class T, int D>
+__global__ __launch_bounds__(256) void lmk_select_kernel(RetrParams p) {
+  __shared__ __align__(16) float q_lds[4][D];
+  __shared__ int cand[4][kSelSeg];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;             // (bh, t)
+  const int64_t total = (int64_t)p.B * p.H * p.T;
+  if (row >= total) return;                                       // whole wave leaves; no block-wide barrier below
+  const int bh = (int)(row / p.T), t = (int)(row % p.T);
+  const int b = bh / p.H, hh = bh % p.H;
+  const int NM = p.num_mems;
+
+  // q row -> fp32 in LDS (read back as a broadcast), and its norm
+  const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
+  float qn = 0.f;
+  for (int d = 2 * lane; d < D; d += 128) {
+    const uint32_t u = *(const uint32_t*)(qp + 2 * d);
+    const float x0 = unpack_lo<T>(u), x1 = unpack_hi<T>(u);
+    q_lds[wave][d] = x0;
+    q_lds[wave][d + 1] = x1;
+    qn += x0 * x0 + x1 * x1;
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) qn += __shfl_xor(qn, m, 64);
+  const float eps_q = sqrtf(qn) * 1.000001f * (1.0f / 16384.0f);
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_s_waitcnt(0xc07f);                             // LDS writes of this wave visible (lgkmcnt 0)
+
+  const float* approx = p.approx + row * NM;
+  float* exact = p.exact + row * NM;
+  const float* lkn = p.lk_norm + (int64_t)bh * NM;
+  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * NM * D);
+  const float sq = p.sqrt_hd;
+
+  // ---- tau = k-th best lower end
+  float tau = INFINITY;
+  {
+    float pv = INFINITY;
+    int pi = -1;
+    for (int j = 0; j < p.k; ++j) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      for (int m = lane; m < NM; m += 64) {
+        const float lo = contract<T>(approx[m] - eps_q * lkn[m], sq);
+        const bool after = (lo < pv) || (lo == pv && m > pi);     // strictly after the previous pick
+        if (after && (lo > bv || (lo == bv && m < bi))) {
+          bv = lo;
+          bi = m;
+        }
+      }
+      wave_best(bv, bi);
+      pv = bv;
+      pi = bi;
+    }
+    tau = pv;
+  }
+
+  // ---- contenders: upper end reaches tau -> exact score in the defined order; others -inf
+  for (int seg = 0; seg < NM; seg += kSelSeg) {
+    int count = 0;
+    for (int m0 = seg; m0 < min(NM, seg + kSelSeg); m0 += 64) {
+      const int m = m0 + lane;
+      bool is_c = false;
+      if (m < NM) {
+        const float hi = contract<T>(approx[m] + eps_q * lkn[m], sq);
+        is_c = hi >= tau;
+        if (!is_c) exact[m] = -INFINITY;
+      }
+      const uint64_t bal = __ballot(is_c);
+      if (is_c) cand[wave][count + __popcll(bal & ((1ull << lane) - 1))] = m;
+      count += __popcll(bal);
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    for (int c0 = 0; c0 < count; c0 += 64) {
+      if (c0 + lane < count) {
+        const int m = cand[wave][c0 + lane];
+        const char* kr = lk + 2 * ((int64_t)m * D);
+        float acc = 0.f;
+#pragma unroll 4
+        for (int d8 = 0; d8 < D / 8; ++d8) {
+          const u32x4_t kk = *(const u32x4_t*)(kr + 16 * d8);
+          const float4 qa = *(const float4*)&q_lds[wave][8 * d8];
+          const float4 qb = *(const float4*)&q_lds[wave][8 * d8 + 4];
+          acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
+          acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
+          acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
+          acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
+          acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
+          acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
+          acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
+          acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
+        }
+        exact[m] = contract<T>(acc, sq);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  __threadfence_block();
+
+  // ---- k best exact scores, then ascending order
+  int mine = -1;                                                 // lane j keeps the j-th pick
+  {
+    float pv = INFINITY;
+    int pi = -1;
+    for (int j = 0; j < p.k; ++j) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      for (int m = lane; m < NM; m += 64) {
+        const float x = exact[m];
+        const bool after = (x < pv) || (x == pv && m > pi);
+        if (after && (x > bv || (x == bv && m < bi))) {
+          bv = x;
+          bi = m;
+        }
+      }
+      wave_best(bv, bi);
+      pv = bv;
+      pi = bi;
+      if (lane == j) mine = bi;
+    }
+  }
+  int rank = 0;
+  for (int j = 0; j < p.k; ++j) {
+    const int o = __shfl(mine, j, 64);
+    rank += (o < mine) ? 1 : 0;
+  }
+  if (lane < p.k) p.idx[row * p.k + rank] = (int64_t)mine;
+}
+
+// ---------------------------------------------------------------------------
+// gather + attend over the selected blocks, merged with the local-chunk attention
+// ---------------------------------------------------------------------------
+template <class T, int D, int BS>
+__global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
+  static_assert(D == 128, "lane mapping below assumes 16 chunks of 8 head dims per row");
+  constexpr int KPG = BS / 4;                                     // keys per 16-lane group per block
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int j = lane & 15, g = lane >> 4;                          // head-dim chunk, key group
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;             // (bh, t)
+  const int64_t total = (int64_t)p.B * p.H * p.T;
+  if (row >= total) return;
+  const int bh = (int)(row / p.T), t = (int)(row % p.T);
+  const int b = bh / p.H, hh = bh % p.H;
+
+  float qv[8];
+  {
+    const u32x4_t u = *(const u32x4_t*)((const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r) + 16 * j);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      qv[2 * i] = unpack_lo<T>(u[i]);
+      qv[2 * i + 1] = unpack_hi<T>(u[i]);
+    }
+  }
+  const char* kc = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h);
+  const char* vc = (const char*)p.vcache + 2 * (b * p.vcs_b + hh * p.vcs_h);
+  const float c2 = p.scale_log2;
+
+  float Mrun = -INFINITY, lrun = 0.f;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+
+  for (int js = 0; js < p.k; ++js) {
+    const int blk = (int)p.idx[row * p.k + js];
+    const int64_t pos0 = (int64_t)js * BS + ((blk >= p.num_mems - p.k) ? BS : 0) + p.prefix_len;
+    const int64_t key0 = (int64_t)blk * BS;
+    // this group's keys: kk = g + 4*i
+    u32x4_t kx[KPG], vx[KPG];
+#pragma unroll
+    for (int i = 0; i < KPG; ++i) {
+      const int kk = g + 4 * i;
+      kx[i] = *(const u32x4_t*)(kc + 2 * ((key0 + kk) * p.kcs_r) + 16 * j);
+      vx[i] = *(const u32x4_t*)(vc + 2 * ((key0 + kk) * p.vcs_r) + 16 * j);
+    }
+    float sc[KPG];
+#pragma unroll
+    for (int i = 0; i < KPG; ++i) {
+      const int kk = g + 4 * i;
+      const u32x4_t c = *(const u32x4_t*)((const char*)p.cos + 2 * ((pos0 + kk) * p.cs_r) + 16 * j);
+      const u32x4_t s = *(const u32x4_t*)((const char*)p.sin + 2 * ((pos0 + kk) * p.cs_r) + 16 * j);
+      const u32x4_t other = shfl_xor4(kx[i], 8);
+      float r[8];
+      rotate_chunk<T>(kx[i], other, c, s, j >= 8, r);
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) d = __builtin_fmaf(qv[e], r[e], d);
+      d += __shfl_xor(d, 1, 64);
+      d += __shfl_xor(d, 2, 64);
+      d += __shfl_xor(d, 4, 64);
+      d += __shfl_xor(d, 8, 64);
+      sc[i] = d * c2;                                             // log2 domain
+    }
+    // landmark = key BS-1 = group 3, i = KPG-1
+    const float t_lm = __shfl(sc[KPG - 1], 48, 64);
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < KPG; ++i)
+      if (!(i == KPG - 1 && g == 3)) mx = fmaxf(mx, sc[i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float den = 0.f;
+#pragma unroll
+    for (int i = 0; i < KPG; ++i) {
+      float e = fast_exp2(sc[i] - mx);
+      if (i == KPG - 1 && g == 3) e = 0.f;
+      sc[i] = e;
+      den += e;
+    }
+    den += __shfl_xor(den, 16, 64);
+    den += __shfl_xor(den, 32, 64);
+    const float Mnew = fmaxf(Mrun, t_lm);
+    const float alpha = fast_exp2(Mrun - Mnew);
+    const float gate = fast_exp2(t_lm - Mnew);
+    lrun = lrun * alpha + gate;
+    Mrun = Mnew;
+    const float f = gate / den;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+#pragma unroll
+    for (int i = 0; i < KPG; ++i) {
+      const float w = round_to<T>(sc[i] * f);                     // weights enter PV in the model dtype
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[2 * e] = __builtin_fmaf(w, unpack_lo<T>(vx[i][e]), acc[2 * e]);
+        acc[2 * e + 1] = __builtin_fmaf(w, unpack_hi<T>(vx[i][e]), acc[2 * e + 1]);
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    acc[e] += __shfl_xor(acc[e], 16, 64);
+    acc[e] += __shfl_xor(acc[e], 32, 64);
+  }
+  // merge with the local chunk: out_loc (normalised), L_loc, M_loc (natural-log units)
+  const float Ml = p.M_loc[row] * kLog2e, Ll = p.L_loc[row];
+  const float Mt = fmaxf(Mrun, Ml);
+  const float wr = fast_exp2(Mrun - Mt), wl = fast_exp2(Ml - Mt) * Ll;
+  const float inv = 1.0f / (lrun * wr + wl);
+  if (g == 0) {
+    const u32x4_t ol = *(const u32x4_t*)((const char*)p.o_loc + 2 * (b * p.ols_b + hh * p.ols_h + (int64_t)t * p.ols_r) + 16 * j);
+    float o[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[2 * i] = (acc[2 * i] * wr + unpack_lo<T>(ol[i]) * wl) * inv;
+      o[2 * i + 1] = (acc[2 * i + 1] * wr + unpack_hi<T>(ol[i]) * wl) * inv;
+    }
+    u32x4_t ov = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
+    *(u32x4_t*)((char*)p.out + 2 * (b * p.outs_b + hh * p.outs_h + (int64_t)t * p.outs_r) + 16 * j) = ov;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// launchers
+// ---------------------------------------------------------------------------
+template <class T, int D>
+static int launch_topk_t(const RetrParams& p, hipStream_t stream) {
+  constexpr int RPW = 256 / (D / 8);
+  const int64_t lkrows = (int64_t)p.B * p.H * p.num_mems;
+  hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
+  int rc;
+  if ((rc = (int)hipGetLastError())) return rc;
+  const int n_qt = (p.T + 127) / 128;
+  hipLaunchKernelGGL((lmk_score_kernel<T, D>), dim3(p.B * p.H * n_qt), dim3(256), 0, stream, p);
+  if ((rc = (int)hipGetLastError())) return rc;
+  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  hipLaunchKernelGGL((lmk_select_kernel<T, D>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+int launch_retrieve_topk(const RetrParams& p, int D, int dtype, hipStream_t stream) {
+  if (dtype == LMK_DTYPE_BF16) {
+    if (D == 128) return launch_topk_t<bf16_t, 128>(p, stream);
+    if (D == 64) return launch_topk_t<bf16_t, 64>(p, stream);
+  } else if (dtype == LMK_DTYPE_F16) {
+    if (D == 128) return launch_topk_t<f16_t, 128>(p, stream);
+    if (D == 64) return launch_topk_t<f16_t, 64>(p, stream);
+  }
+  return LMK_ERR_UNSUPPORTED;
+}
+
+template <class T>
+static int launch_gather_t(const RetrParams& p, int BS, hipStream_t stream) {
+  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  const dim3 grid((unsigned)((rows + 3) / 4));
+  if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 32>), grid, dim3(256), 0, stream, p);
+  else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 64>), grid, dim3(256), 0, stream, p);
+  else return LMK_ERR_UNSUPPORTED;
+  return (int)hipGetLastError();
+}
+
+int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream) {
+  if (D != 128) return LMK_ERR_UNSUPPORTED;
+  if (dtype == LMK_DTYPE_BF16) return launch_gather_t<bf16_t>(p, BS, stream);
+  if (dtype == LMK_DTYPE_F16) return launch_gather_t<f16_t>(p, BS, stream);
+  return LMK_ERR_UNSUPPORTED;
+}
+
+}  // namespace lmk

@@ -52,6 +52,14 @@ def lib() -> ctypes.CDLL:
         L.lmk_attn_bwd.restype = i
         L.lmk_attn_bwd.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, ctypes.c_size_t,
                                    i, i, i, i, i, f, i, i, i, vp]
+        i64, sz = ctypes.c_int64, ctypes.c_size_t
+        L.lmk_retrieve_workspace_bytes.restype = sz
+        L.lmk_retrieve_workspace_bytes.argtypes = [i, i, i, i, i, i]
+        L.lmk_retrieve_topk.restype = i
+        L.lmk_retrieve_topk.argtypes = [T4, T4, vp, vp, i64, i64, vp, vp, sz, i, i, i, i, i, i, i, i, vp]
+        L.lmk_gather_attend.restype = i
+        L.lmk_gather_attend.argtypes = [T4, T4, T4, vp, vp, vp, i64, i64, T4, vp, vp, T4,
+                                        i, i, i, i, i, f, i, i, i, vp]
         _lib = L
     return _lib
 

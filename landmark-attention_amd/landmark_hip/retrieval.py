@@ -1,0 +1,90 @@
+"""Mem-cache retrieval at inference: landmark scoring, top-k block selection and
+attention over the gathered blocks, on the HIP kernels.
+
+Mirrors the per-head, per-token branch of ``LlamaAttention.forward``
+(``llama/llama_mem.py:318-430`` retrieval, ``:447-477`` attend) with the reference's own
+conventions: ``past_key_value = (K_without_rotary, V)`` each ``(B, nh, S, hd)`` (``:424-430``),
+``block = mem_freq + 1`` with the landmark as the last token of a block, queries and local
+keys already rotated (``:298``), ``cos/sin`` the model-dtype tables of
+``LlamaRotaryEmbedding`` (``:121-124``).  The cached length must be a whole number of blocks.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+from .attention import _launch_fwd
+
+
+def _tables(cos, sin, dtype):
+    cos = cos.reshape(-1, cos.shape[-1])
+    sin = sin.reshape(-1, sin.shape[-1])
+    assert cos.dtype == sin.dtype == dtype, "rotary tables must be in the model dtype (llama_mem.py:121-124)"
+    assert cos.shape == sin.shape
+    if cos.stride(1) != 1 or cos.stride(0) % 8 or cos.data_ptr() % 16:
+        cos = cos.contiguous()
+    if sin.stride(1) != 1 or sin.stride(0) != cos.stride(0) or sin.data_ptr() % 16:
+        sin = sin.contiguous()
+        cos = cos.contiguous()
+    return cos, sin
+
+
+def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int):
+    """Indices ``(B, nh, T, k)`` int64, ascending, of the ``k = min(top_k, S // block)`` cached
+    blocks whose landmark keys score highest against each query (``llama_mem.py:344-384``).
+
+    Equivalent to ``(q @ rot(landmark_keys)^T / sqrt(hd)).topk(k).indices.sort()`` with the
+    product accumulated sequentially in fp32 and ties broken towards the lower index."""
+    B, H, T, D = q.shape
+    S = k_cache.shape[2]
+    assert k_cache.shape == (B, H, S, D) and q.dtype == k_cache.dtype and q.is_cuda and k_cache.is_cuda
+    q, k_cache = _lib.kernel_ready(q), _lib.kernel_ready(k_cache)
+    cos, sin = _tables(cos, sin, q.dtype)
+    lib = _lib.lib()
+    k = min(top_k, S // block)
+    idx = torch.empty((B, H, T, k), device=q.device, dtype=torch.int64)
+    nbytes = lib.lmk_retrieve_workspace_bytes(B, H, T, S, D, int(block))
+    with torch.cuda.device(q.device):
+        ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+        rc = lib.lmk_retrieve_topk(_lib.tensor4(q), _lib.tensor4(k_cache), cos.data_ptr(), sin.data_ptr(),
+                                   cos.stride(0), cos.shape[0], idx.data_ptr(), ws.data_ptr(), nbytes,
+                                   B, H, T, S, D, int(block), int(top_k), _lib.DTYPE_CODES[q.dtype],
+                                   _lib.current_stream(q.device))
+    _lib.check(rc)
+    return idx
+
+
+def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
+    """Attention output ``(B, nh, T, hd)`` over the blocks ``idx`` selects plus the local chunk
+    (``llama_mem.py:386-412,447-477``).  The local chunk is attended with the fused forward
+    kernel; the gather kernel reads the selected blocks in place and merges both parts."""
+    B, H, T, D = q.shape
+    S = k_cache.shape[2]
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    q, k_cache, v_cache, k_loc, v_loc = (_lib.kernel_ready(t) for t in (q, k_cache, v_cache, k_loc, v_loc))
+    cos, sin = _tables(cos, sin, q.dtype)
+    with torch.cuda.device(q.device):
+        o_loc, L_loc, M_loc = _launch_fwd(q, k_loc, v_loc, 0, sm_scale, block)
+        out = torch.empty_like(o_loc)
+        rc = _lib.lib().lmk_gather_attend(
+            _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), idx.data_ptr(), cos.data_ptr(),
+            sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(o_loc), L_loc.data_ptr(), M_loc.data_ptr(),
+            _lib.tensor4(out), B, H, T, S, D, float(sm_scale), int(block), int(top_k), _lib.DTYPE_CODES[q.dtype],
+            _lib.current_stream(q.device))
+    _lib.check(rc)
+    return out
+
+
+def retrieve_and_attend(q, past_key_value, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
+    """One inference step of the mem-cache path: returns ``(out, idx)``.
+
+    ``past_key_value = (K_without_rotary, V)``; ``k_loc`` rotated, ``v_loc``: the new chunk.
+    The caller appends the un-rotated new keys and values to the cache afterwards
+    (``llama_mem.py:424-430``)."""
+    k_cache, v_cache = past_key_value[0], past_key_value[1]
+    idx = retrieve_topk(q, k_cache, cos, sin, block, top_k)
+    out = gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
+    return out, idx

@@ -10,13 +10,16 @@ The cache holds keys WITHOUT rotary (``:424-425``); queries and local keys come
 in already rotated (``:298``).
 
 Score contract (``:367``).  The reference computes ``matmul(q, mem_key^T) /
-sqrt(hd)`` in the model dtype: an fp32-accumulated product rounded to bf16, then
-a division rounded to bf16 again.  The accumulation order of that product is
-not defined by the reference, so this oracle fixes it to the correctly rounded
-value: dot product accumulated in fp64 -> fp32 -> bf16, then fp32 division by
-``float32(sqrt(hd))`` -> bf16.  Selection contract (``:384``): the ``k`` best
-under the total order (score descending, block index ascending), returned in
-ascending index order.  ``torch.topk`` breaks ties in an implementation-defined
+sqrt(hd)`` in the model dtype: an fp32-accumulated product rounded to the model
+dtype, then a division rounded again.  The reference leaves the accumulation
+order of that product to the BLAS library, so it has to be fixed for indices to
+be reproducible bit for bit.  This build fixes it to the plain sequential order:
+``acc = fma(q[d], k[d], acc)`` in fp32 for ``d = 0 .. hd-1`` (a product of two
+16-bit floats is exact in fp32, so every step is one correctly rounded fp32
+addition, which numpy reproduces exactly), then ``acc -> model dtype``, then fp32
+division by ``float32(sqrt(hd))`` ``-> model dtype``.  Selection contract
+(``:384``): the ``k`` best under the total order (score descending, block index
+ascending), returned in ascending index order.  ``torch.topk`` breaks ties in an implementation-defined
 way; on rows without a tie at the k-th place both agree, which
 ``tests/test_oracle_retrieval.py`` checks, together with a brute-force loop,
 the integer position formulas on hand-worked cases, and agreement of the
@@ -26,6 +29,7 @@ from __future__ import annotations
 
 import math
 
+import numpy as np
 import torch
 
 from .highlevel import grouped_softmax
@@ -67,13 +71,26 @@ def gather_positions(idx, num_mems: int, k: int, block: int, prefix_len: int):
 
 
 # -------------------------------------------------------------------- scoring
+def sequential_dot_fp32(q, keys):
+    """(…, T, M) fp32: ``sum_d q[t,d]*keys[m,d]`` accumulated in fp32 in the order
+    d = 0, 1, … with one rounding per step (the score contract above).  q: (…, T, hd),
+    keys: (…, M, hd), both holding 16-bit float values."""
+    qf = q.float().numpy()
+    kf = keys.float().numpy()
+    acc = np.zeros(qf.shape[:-1] + (kf.shape[-2],), dtype=np.float32)
+    for d in range(qf.shape[-1]):
+        prod = qf[..., :, None, d] * kf[..., None, :, d]          # exact in fp32
+        acc = (acc + prod).astype(np.float32)
+    return torch.from_numpy(acc)
+
+
 def landmark_scores(q, k_cache, cos, sin, block: int, top_k: int):
     """Scores (B, nh, T, num_mems) in q.dtype under the score contract."""
     S, hd = k_cache.shape[-2], k_cache.shape[-1]
     g = retrieval_geometry(S, block, top_k)
     lk = k_cache[..., : g["full_len"], :].unflatten(-2, (g["num_mems"], block))[..., block - 1, :]
     lk = apply_rotary(lk, cos, sin, g["mem_pos"])                     # :366
-    dot = (q.double() @ lk.double().transpose(-1, -2)).float()        # correctly rounded fp32
+    dot = sequential_dot_fp32(q, lk)
     sc = dot.to(q.dtype).float() / torch.tensor(math.sqrt(hd), dtype=torch.float32)
     return sc.to(q.dtype)
 

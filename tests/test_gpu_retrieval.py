@@ -1,0 +1,108 @@
+"""Retrieval parity: top-k block indices bit-exact against the oracle's score/selection
+contract, and gather+attend output within 2e-2 of the oracle (both the model-dtype
+restatement of the reference and the fp32 closed form)."""
+import pytest
+import torch
+
+from oracle import retrieval as oret
+from oracle import rotary as orot
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(B, H, T, S, D, seed, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.5).to(dtype)
+    q, kc, vc, kl, vl = mk(B, H, T, D), mk(B, H, S, D), mk(B, H, S, D), mk(B, H, T, D), mk(B, H, T, D)
+    cos, sin = orot.rotary_tables(S + T, D, dtype)
+    return q, kc, vc, kl, vl, cos, sin
+
+
+CASES = [
+    # B, H, T, S, D, block, top_k
+    (1, 2, 8, 64 * 32, 128, 32, 4),
+    (2, 3, 40, 20 * 32, 128, 32, 5),
+    (1, 2, 16, 3 * 32, 128, 32, 5),        # fewer cached blocks than top_k
+    (1, 2, 130, 33 * 32, 128, 32, 1),      # ragged landmark tile, ragged query tile
+    (1, 2, 64, 40 * 64, 128, 64, 4),
+    (1, 2, 32, 50 * 32, 64, 32, 4),
+    (1, 2, 16, 70 * 16, 128, 16, 3),       # selection does not depend on the block size set of the attend kernels
+]
+
+
+@pytest.mark.parametrize("B,H,T,S,D,block,top_k", CASES)
+def test_topk_indices_bit_exact(B, H, T, S, D, block, top_k):
+    from landmark_hip.retrieval import retrieve_topk
+    print(f"case B{B} H{H} T{T} S{S} D{D} bs{block} k{top_k}", flush=True)
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=S + T)
+    sc = oret.landmark_scores(q, kc, cos, sin, block, top_k)
+    want = oret.select_topk(sc, min(top_k, S // block))
+    got = retrieve_topk(q.cuda(), kc.cuda(), cos.cuda(), sin.cuda(), block, top_k)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.int64 and got.shape == want.shape
+    assert torch.equal(got.cpu(), want)
+
+
+def test_topk_with_massive_ties():
+    # identical landmark keys in many blocks: every score ties, the lowest indices must win
+    from landmark_hip.retrieval import retrieve_topk
+    B, H, T, S, D, block, top_k = 1, 2, 8, 2100 * 32, 128, 32, 4    # > 1024 landmarks: two list sweeps
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=3)
+    kc[:, :, block - 1::block] = kc[:, :, block - 1:block]
+    sc = oret.landmark_scores(q, kc, cos, sin, block, top_k)
+    want = oret.select_topk(sc, top_k)
+    got = retrieve_topk(q.cuda(), kc.cuda(), cos.cuda(), sin.cuda(), block, top_k)
+    assert torch.equal(got.cpu(), want)
+
+
+def test_fp16_indices_bit_exact():
+    from landmark_hip.retrieval import retrieve_topk
+    B, H, T, S, D, block, top_k = 1, 2, 24, 48 * 32, 128, 32, 4
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=4, dtype=torch.float16)
+    want = oret.select_topk(oret.landmark_scores(q, kc, cos, sin, block, top_k), top_k)
+    got = retrieve_topk(q.cuda(), kc.cuda(), cos.cuda(), sin.cuda(), block, top_k)
+    assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("B,H,T,S,block,top_k", [(1, 2, 64, 24 * 32, 32, 4), (1, 2, 128, 12 * 64, 64, 3),
+                                                  (2, 2, 96, 3 * 32, 32, 5)])
+def test_gather_attend_matches_oracle(B, H, T, S, block, top_k):
+    from landmark_hip.retrieval import retrieve_and_attend
+    D = 128
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=S + T + 1)
+    is_mem = (torch.arange(T) % block == block - 1)[None].expand(B, T)
+    ref_bf16, idx_ref = oret.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, block, top_k)
+    dev = lambda t: t.cuda()
+    out, idx = retrieve_and_attend(dev(q), (dev(kc), dev(vc)), dev(kl), dev(vl), dev(cos), dev(sin), block, top_k)
+    torch.cuda.synchronize()
+    assert torch.equal(idx.cpu(), idx_ref)
+    out = out.float().cpu()
+    assert (out - ref_bf16.float()).abs().max().item() <= 2e-2
+    ref32 = oret.retrieve_and_attend_s1(q, kc, vc, kl, vl, cos, sin, block, top_k, idx_ref,
+                                        heads=[0, H - 1], tokens=[0, 1, block - 2, block - 1, block, T - 1])
+    for (b, h, t), o in ref32.items():
+        assert (out[b, h, t] - o).abs().max().item() <= 2e-2, (b, h, t)
+
+
+def test_baseline_config4_full_size():
+    # BASELINE config 4: H32 D128, 32768 cached tokens = 1024 blocks of 32, 256 queries, top-4
+    from landmark_hip.retrieval import retrieve_and_attend
+    B, H, T, S, D, block, top_k = 1, 32, 256, 32768, 128, 32, 4
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=0)
+    sc = oret.landmark_scores(q, kc, cos, sin, block, top_k)
+    want = oret.select_topk(sc, top_k)
+    ties = oret.boundary_tie_rows(sc, top_k)
+    dev = lambda t: t.cuda()
+    out, idx = retrieve_and_attend(dev(q), (dev(kc), dev(vc)), dev(kl), dev(vl), dev(cos), dev(sin), block, top_k)
+    torch.cuda.synchronize()
+    print("config4 rows", ties.numel(), "rows with a tie at the 4th place", int(ties.sum()), flush=True)
+    assert torch.equal(idx.cpu(), want)
+    # torch.topk agrees wherever the k-th place is not tied
+    tk = sc.float().topk(top_k, dim=-1).indices.sort(-1).values
+    assert torch.equal(idx.cpu()[~ties], tk[~ties])
+    # attend: fp32 closed form on sampled (head, token) pairs
+    ref32 = oret.retrieve_and_attend_s1(q, kc, vc, kl, vl, cos, sin, block, top_k, want,
+                                        heads=[0, 13, 31], tokens=[0, 30, 31, 32, 100, 255])
+    out = out.float().cpu()
+    for (b, h, t), o in ref32.items():
+        assert (out[b, h, t] - o).abs().max().item() <= 2e-2, (b, h, t)

@@ -96,9 +96,15 @@ def test_score_contract_rounding_points():
     b, h, t, m = 0, 1, 3, 4
     lk = kc[b, h, m * bs + bs - 1]
     lkr = rotary.apply_rotary(lk[None], cos, sin, g["mem_pos"][m : m + 1])[0]
-    dot = sum(float(a) * float(c) for a, c in zip(q[b, h, t], lkr))
-    two = torch.tensor(dot, dtype=torch.float64).float().bfloat16().float() / torch.tensor(math.sqrt(hd)).float()
+    import numpy as np
+    acc = np.float32(0.0)
+    for a, c in zip(q[b, h, t].float().tolist(), lkr.float().tolist()):
+        acc = np.float32(acc + np.float32(np.float32(a) * np.float32(c)))     # one fp32 rounding per step
+    two = torch.tensor(float(acc)).bfloat16().float() / torch.tensor(math.sqrt(hd)).float()
     assert sc[b, h, t, m] == two.bfloat16()
+    # and the sequential sum stays within fp32 accumulation error of the exact dot product
+    exact = sum(float(a) * float(c) for a, c in zip(q[b, h, t], lkr))
+    assert abs(float(acc) - exact) < 1e-5
     assert sc.dtype == torch.bfloat16 and sc.shape == (B, nh, T, nm)
 
 
