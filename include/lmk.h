@@ -82,6 +82,21 @@ int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
                  const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B, int H,
                  int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype, void* stream);
 
+/* Same as lmk_attn_bwd but runs only the kernels selected by `phases` (LMK_BWD_PRE: row terms,
+ * LMK_BWD_DQ: dQ and the per-block terms, LMK_BWD_DKDV: dK and dV), in that order.  Each phase
+ * consumes what the earlier ones left in `workspace`, so a subset is only meaningful after a
+ * full run on the same arguments; it exists to time and profile the kernels one by one.
+ * No counterpart in the reference (its backward is a single launch, :373-388). */
+#define LMK_BWD_PRE 1
+#define LMK_BWD_DQ 2
+#define LMK_BWD_DKDV 4
+#define LMK_BWD_ALL 7
+int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                        const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
+                        int H, int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype, int phases,
+                        void* stream);
+
 /* ---- mem-cache retrieval (inference) --------------------------------------------------
  * The reference has no function boundary here: scoring, selection and gather are inline in
  * LlamaAttention.forward (llama/llama_mem.py:318-430) and the attend step follows at :447-477.

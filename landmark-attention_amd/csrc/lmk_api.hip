@@ -120,7 +120,17 @@ int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
                  const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
                  const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B, int H,
                  int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype, void* stream) {
+  return lmk_attn_bwd_phases(q, k, v, o, dout, L, M, dq, dk, dv, workspace, workspace_bytes, B, H, Lq, Lk, D,
+                             sm_scale, block, n_prefix, dtype, LMK_BWD_ALL, stream);
+}
+
+int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                        const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
+                        int H, int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype, int phases,
+                        void* stream) {
   int rc;
+  if (phases <= 0 || phases > LMK_BWD_ALL) return LMK_ERR_SHAPE;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o)) ||
       (rc = check_tensor(dout)) || (rc = check_tensor(dq)) || (rc = check_tensor(dk)) || (rc = check_tensor(dv)))
     return rc;
@@ -153,7 +163,7 @@ int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
   p.dvs_b = dv->stride_b; p.dvs_h = dv->stride_h; p.dvs_r = dv->stride_row;
   p.scale = sm_scale;
   p.scale_log2 = sm_scale * 1.4426950408889634f;
-  return lmk::launch_bwd(p, D, block, dtype, (hipStream_t)stream);
+  return lmk::launch_bwd(p, D, block, dtype, phases, (hipStream_t)stream);
 }
 
 size_t lmk_retrieve_workspace_bytes(int B, int H, int T, int S, int D, int block) {

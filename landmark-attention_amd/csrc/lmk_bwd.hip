@@ -489,15 +489,15 @@ static int set_lds(K kern, int bytes) {
 }
 
 template <class T, int D, int BS>
-static int launch_bwd_t(const BwdParams& p, hipStream_t stream) {
+static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
   int rc;
-  {
+  if (phases & 1) {
     constexpr int RPW = 256 / (D / 8);
     const int64_t rows = (int64_t)p.B * p.H * p.Lq;
     hipLaunchKernelGGL((lmk_bwd_pre_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
   }
-  {
+  if (phases & 2) {
     using C = DqCfg<T, D, BS>;
     auto kern = lmk_bwd_dq_kernel<T, D, BS>;
     static bool done = false;
@@ -508,7 +508,7 @@ static int launch_bwd_t(const BwdParams& p, hipStream_t stream) {
     hipLaunchKernelGGL(kern, dim3(p.n_qtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
   }
-  {
+  if (phases & 4) {
     using C = DkvCfg<T, D, BS>;
     auto kern = lmk_bwd_dkdv_kernel<T, D, BS>;
     static bool done = false;
@@ -523,22 +523,22 @@ static int launch_bwd_t(const BwdParams& p, hipStream_t stream) {
 }
 
 template <class T>
-static int launch_bwd_d(const BwdParams& p, int D, int BS, hipStream_t stream) {
+static int launch_bwd_d(const BwdParams& p, int D, int BS, int phases, hipStream_t stream) {
   if (D == 128) {
-    if (BS == 32) return launch_bwd_t<T, 128, 32>(p, stream);
-    if (BS == 64) return launch_bwd_t<T, 128, 64>(p, stream);
-    if (BS == 128) return launch_bwd_t<T, 128, 128>(p, stream);
+    if (BS == 32) return launch_bwd_t<T, 128, 32>(p, phases, stream);
+    if (BS == 64) return launch_bwd_t<T, 128, 64>(p, phases, stream);
+    if (BS == 128) return launch_bwd_t<T, 128, 128>(p, phases, stream);
   } else if (D == 64) {
-    if (BS == 32) return launch_bwd_t<T, 64, 32>(p, stream);
-    if (BS == 64) return launch_bwd_t<T, 64, 64>(p, stream);
-    if (BS == 128) return launch_bwd_t<T, 64, 128>(p, stream);
+    if (BS == 32) return launch_bwd_t<T, 64, 32>(p, phases, stream);
+    if (BS == 64) return launch_bwd_t<T, 64, 64>(p, phases, stream);
+    if (BS == 128) return launch_bwd_t<T, 64, 128>(p, phases, stream);
   }
   return LMK_ERR_UNSUPPORTED;
 }
 
-int launch_bwd(const BwdParams& p, int D, int BS, int dtype, hipStream_t stream) {
-  if (dtype == LMK_DTYPE_BF16) return launch_bwd_d<bf16_t>(p, D, BS, stream);
-  if (dtype == LMK_DTYPE_F16) return launch_bwd_d<f16_t>(p, D, BS, stream);
+int launch_bwd(const BwdParams& p, int D, int BS, int dtype, int phases, hipStream_t stream) {
+  if (dtype == LMK_DTYPE_BF16) return launch_bwd_d<bf16_t>(p, D, BS, phases, stream);
+  if (dtype == LMK_DTYPE_F16) return launch_bwd_d<f16_t>(p, D, BS, phases, stream);
   return LMK_ERR_UNSUPPORTED;
 }
 

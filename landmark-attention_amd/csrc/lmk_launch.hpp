@@ -36,7 +36,8 @@ struct BwdParams {
   float scale, scale_log2;
 };
 
-int launch_bwd(const BwdParams& p, int D, int BS, int dtype, hipStream_t stream);
+// phases: bit 0 = pre, bit 1 = dq, bit 2 = dkdv
+int launch_bwd(const BwdParams& p, int D, int BS, int dtype, int phases, hipStream_t stream);
 
 struct RetrParams {
   const void *q, *kcache, *vcache, *cos, *sin;   // q rotated; caches un-rotated; tables (n_pos, D)

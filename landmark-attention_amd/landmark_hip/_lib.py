@@ -52,6 +52,9 @@ def lib() -> ctypes.CDLL:
         L.lmk_attn_bwd.restype = i
         L.lmk_attn_bwd.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, ctypes.c_size_t,
                                    i, i, i, i, i, f, i, i, i, vp]
+        L.lmk_attn_bwd_phases.restype = i
+        L.lmk_attn_bwd_phases.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, ctypes.c_size_t,
+                                          i, i, i, i, i, f, i, i, i, i, vp]
         i64, sz = ctypes.c_int64, ctypes.c_size_t
         L.lmk_retrieve_workspace_bytes.restype = sz
         L.lmk_retrieve_workspace_bytes.argtypes = [i, i, i, i, i, i]

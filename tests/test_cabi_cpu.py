@@ -1,0 +1,119 @@
+"""CPU-side checks of the C ABI: the shared library loads without a GPU, exports every
+symbol include/lmk.h declares, and rejects bad arguments on the host before any launch."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "lmk.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from landmark_hip import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("lmk_build", os.path.join(ROOT, "landmark-attention_amd", "build.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        mod.build()
+    return _lib.lib()
+
+
+def _declared():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(lmk_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = _declared()
+    assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_strerror"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_version_and_strerror(lib):
+    assert b"gfx950" in lib.lmk_version()
+    assert lib.lmk_strerror(0) == b"ok"
+    for code in range(-11, 0):
+        assert lib.lmk_strerror(code) not in (b"", b"unknown error")
+
+
+def _t4(ptr=0x1000, sb=0, sh=0, sr=128):
+    from landmark_hip._lib import Tensor4
+    return Tensor4(ptr, sb, sh, sr)
+
+
+def _fwd(lib, q=None, k=None, v=None, o=None, L=0x2000, M=0x3000, B=1, H=1, Lq=64, Lk=64, D=128, scale=0.1,
+         block=32, n_prefix=0, dtype=0):
+    t = _t4()
+    return lib.lmk_attn_fwd(q or t, k or t, v or t, o or t, L, M, B, H, Lq, Lk, D, scale, block, n_prefix, dtype, None)
+
+
+def test_forward_argument_errors(lib):
+    # every call here fails validation, so nothing is launched and no GPU is needed
+    assert _fwd(lib, q=_t4(ptr=0)) == -1                      # NULL
+    assert _fwd(lib, L=0) == -1
+    assert _fwd(lib, q=_t4(ptr=0x1008)) == -4                 # misaligned pointer
+    assert _fwd(lib, k=_t4(sr=130)) == -4                     # misaligned row stride
+    assert _fwd(lib, B=0) == -2
+    assert _fwd(lib, D=96) == -3
+    assert _fwd(lib, block=48) == -3
+    assert _fwd(lib, dtype=7) == -3
+    assert _fwd(lib, Lq=64, Lk=96, n_prefix=0) == -5          # history not declared
+    assert _fwd(lib, Lq=64, Lk=80, n_prefix=1) == -5          # history not whole blocks
+    assert _fwd(lib, Lq=96, Lk=64) == -5
+    assert _fwd(lib, scale=0.0) == -7
+    assert _fwd(lib, scale=float("nan")) == -7
+
+
+def test_backward_argument_errors(lib):
+    t = _t4()
+    args = lambda **kw: dict(dict(ws=0x4000, wsb=1 << 30, B=1, H=1, Lq=64, Lk=64, D=128, scale=0.1, block=32,
+                                  n_prefix=0, dtype=0), **kw)
+
+    def call(**kw):
+        a = args(**kw)
+        return lib.lmk_attn_bwd(t, t, t, t, t, 0x2000, 0x3000, t, t, t, a["ws"], a["wsb"], a["B"], a["H"], a["Lq"],
+                                a["Lk"], a["D"], a["scale"], a["block"], a["n_prefix"], a["dtype"], None)
+
+    assert call(ws=0) == -1
+    assert call(Lq=48, Lk=48) == -6                           # partial blocks
+    assert call(wsb=16) == -8                                 # workspace too small
+    assert call(block=16) == -3
+    need = lib.lmk_attn_bwd_workspace_bytes(2, 32, 2048, 2048, 32)
+    assert need == 4 * (2 * 2 * 32 * 2048 + 2 * 2 * 32 * 2048 * 64)
+    assert lib.lmk_attn_bwd_workspace_bytes(0, 1, 1, 1, 1) == 0
+
+
+def test_retrieval_argument_errors(lib):
+    t = _t4()
+
+    def topk(S=64, block=32, top_k=4, n_pos=4096, ws=0x4000, wsb=1 << 30, cos=0x5000, D=128):
+        return lib.lmk_retrieve_topk(t, t, cos, 0x6000, 128, n_pos, 0x7000, ws, wsb, 1, 1, 8, S, D, block, top_k, 0, None)
+
+    assert topk(cos=0) == -1
+    assert topk(S=70) == -9                                   # incomplete cached block
+    assert topk(S=16) == -9                                   # less than one block
+    assert topk(top_k=0) == -10 and topk(top_k=65) == -10
+    assert topk(n_pos=32) == -11
+    assert topk(wsb=64) == -8
+    assert topk(D=96) == -3
+    assert lib.lmk_retrieve_workspace_bytes(1, 32, 256, 32768, 128, 32) >= 32 * 1024 * 128 * 2 + 2 * 32 * 256 * 1024 * 4
+    # gather+attend is built for D=128 and blocks of 32/64 only
+    rc = lib.lmk_gather_attend(t, t, t, 0x7000, 0x5000, 0x6000, 128, 4096, t, 0x2000, 0x3000, t, 1, 1, 8, 64, 64, 0.1,
+                               32, 4, 0, None)
+    assert rc == -3
+
+
+def test_python_shim_rejects_what_the_reference_rejects():
+    import torch
+    from ltriton.flash_landmark_attention import FusedLandmarkAttention, fused_landmark_attention
+    q = torch.zeros(1, 1, 32, 128, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):                       # CPU tensors (flash_landmark_attention.py:324)
+        fused_landmark_attention(q, q, q, None, block_size=32)
+    with pytest.raises(AssertionError):                       # history not whole blocks (:397)
+        fused_landmark_attention(q, torch.zeros(1, 1, 40, 128, dtype=torch.bfloat16), q, None, block_size=32)
+    assert issubclass(FusedLandmarkAttention, torch.autograd.Function)
