@@ -65,7 +65,7 @@ int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
                  int n_prefix, int dtype, void* stream);
 
 /* Bytes of device workspace lmk_attn_bwd needs (0 for invalid sizes):
- * 2*(B*H*Lq) floats of per-row terms + 2*(B*H*(Lk/block)*Lq) floats of per-(row, block)
+ * 2*(B*H*Lq) floats of per-row terms + 3*(B*H*(Lk/block)*Lq) floats of per-(row, block)
  * terms handed from the dQ kernel to the dK/dV kernel. */
 size_t lmk_attn_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int block);
 

@@ -113,7 +113,7 @@ size_t lmk_attn_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int block) {
   if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || block <= 0) return 0;
   const size_t rows = (size_t)B * H * Lq;
   const size_t nb = (size_t)(Lk / block);
-  return sizeof(float) * (2 * rows + 2 * rows * nb);
+  return sizeof(float) * (2 * rows + 3 * rows * nb);
 }
 
 int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
@@ -150,6 +150,7 @@ int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
   p.mhat = w + rows;
   p.stat_a = w + 2 * rows;
   p.stat_n = w + 2 * rows + rows * nb;
+  p.stat_l = w + 2 * rows + 2 * rows * nb;
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
   p.n_prefix = n_prefix; p.n_blocks = (int)nb;
   p.n_qtiles = (Lq + 127) / 128; p.n_kvtiles = (Lk + 127) / 128;

@@ -8,13 +8,17 @@
 //   pre    delta = rowsum(O * dO),  mhat = M*log2(e) + log2(L)          (per query row)
 //   dq     query-stationary, S^T layout (lane = query): recomputes the local softmax of
 //          every earlier block, the gate, nD = rowsum(P * dP), forms dS and accumulates
-//          dQ^T = K^T dS^T.  It also writes, per (query, earlier block), the two numbers
-//          the third kernel needs:  a  with  gate*P = exp2(s*c - a),  and  nD.
+//          dQ^T = K^T dS^T.  It also writes, per (query, earlier block), the three numbers
+//          the third kernel needs:  a  with  gate*P = exp2(s*c - a),  nD,  and dS at the
+//          block's landmark key.
 //   dkdv   key-stationary, S layout (lane = key): purely elementwise between its four
 //          products S = Q K^T, dP = dO V^T, dV^T += dO^T W, dK^T += Q^T dS.
 //
 // All probabilities are used normalised (exp2(s*c - mhat) already divides by L), so dO is
 // consumed as is; the reference's rescaled copy dO/L (:147) is not needed.
+#include <cstdlib>
+#include <type_traits>
+
 #include "lmk_common.hpp"
 #include "lmk_launch.hpp"
 
@@ -218,6 +222,7 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dq_kernel(BwdParams p) {
             const int64_t si = ((int64_t)bh * p.n_blocks + blk) * p.Lq + qrow;
             p.stat_a[si] = mloc + fast_log2(den) - glog;
             p.stat_n[si] = nD;
+            p.stat_l[si] = g * (nD - delta);              // dS at the block's landmark key
           }
 #pragma unroll
           for (int u = 0; u < C::NT; ++u) {
@@ -507,6 +512,9 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
     }
     hipLaunchKernelGGL(kern, dim3(p.n_qtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
+  }
+  if ((phases & 4) && BS == 32 && getenv("LMK_DKDV_GENERIC") == nullptr) {
+    return launch_bwd_dkdv32(p, D, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream);
   }
   if (phases & 4) {
     using C = DkvCfg<T, D, BS>;

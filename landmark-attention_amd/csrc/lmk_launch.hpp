@@ -21,13 +21,14 @@ struct FwdParams {
 };
 
 int launch_fwd(const FwdParams& p, int D, int BS, int dtype, hipStream_t stream);
+int launch_fwd32(const FwdParams& p, int D, int dtype, hipStream_t stream);   // block 32 specialisation
 
 struct BwdParams {
   const void *q, *k, *v, *o, *dout;
   void *dq, *dk, *dv;
   const float *L, *M;            // forward statistics, (B*H, Lq)
   float *delta, *mhat;           // (B*H, Lq) each, written by the pre kernel
-  float *stat_a, *stat_n;        // (B*H, n_blocks, Lq) each, written by the dq kernel
+  float *stat_a, *stat_n, *stat_l;   // (B*H, n_blocks, Lq) each, written by the dq kernel
   int B, H, Lq, Lk;
   int n_prefix, n_blocks;        // history blocks; Lk / block
   int n_qtiles, n_kvtiles;       // ceil(Lq / 128), ceil(Lk / 128)
@@ -38,6 +39,7 @@ struct BwdParams {
 
 // phases: bit 0 = pre, bit 1 = dq, bit 2 = dkdv
 int launch_bwd(const BwdParams& p, int D, int BS, int dtype, int phases, hipStream_t stream);
+int launch_bwd_dkdv32(const BwdParams& p, int D, int dtype, hipStream_t stream);   // block 32 specialisation
 
 struct RetrParams {
   const void *q, *kcache, *vcache, *cos, *sin;   // q rotated; caches un-rotated; tables (n_pos, D)

@@ -84,7 +84,7 @@ def test_backward_argument_errors(lib):
     assert call(wsb=16) == -8                                 # workspace too small
     assert call(block=16) == -3
     need = lib.lmk_attn_bwd_workspace_bytes(2, 32, 2048, 2048, 32)
-    assert need == 4 * (2 * 2 * 32 * 2048 + 2 * 2 * 32 * 2048 * 64)
+    assert need == 4 * (2 * 2 * 32 * 2048 + 3 * 2 * 32 * 2048 * 64)
     assert lib.lmk_attn_bwd_workspace_bytes(0, 1, 1, 1, 1) == 0
 
 
