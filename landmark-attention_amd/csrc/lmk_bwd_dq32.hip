@@ -33,8 +33,7 @@ struct Dq32Cfg {
   static constexpr int ROWB = 2 * D;
   static constexpr int BLK_BYTES = 32 * ROWB;              // one block of K (or of V)
   static constexpr int BUF_BYTES = 2 * BLK_BYTES;          // K then V
-  static constexpr int NBUF = 4;                           // ring slots: 2 in use, 2 in flight
-  static constexpr int DIST = 2;
+  static constexpr int NBUF = 4;                           // ring slots: blocks k, k+1 in use, k+2, k+3 in flight
   static constexpr int RPD = 1024 / ROWB;                  // block rows covered by one 1 KB request
   static constexpr int NREQ = 2 * (32 / RPD);              // requests per block (K and V)
   static constexpr int PER_TILE = NREQ / NW;               // requests per wave and block
@@ -43,7 +42,6 @@ struct Dq32Cfg {
   static constexpr int GO_OFF = NBUF * BUF_BYTES;          // per wave: its 32 rows of dO (B operand of dP^T)
   static constexpr int STAT_OFF = GO_OFF + NW * BLK_BYTES;
   static constexpr int LDS_BYTES = STAT_OFF + NW * STAT_WAVE;
-  static constexpr bool SKEW = false;
 };
 
 __device__ __forceinline__ void dq_dma16(const void* base_uniform, uint32_t voff, uint32_t lds_off) {
@@ -103,20 +101,21 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   const float mhat = rowok ? p.mhat[(int64_t)bh * p.Lq + qrow] : 0.f;
   const float delta = rowok ? p.delta[(int64_t)bh * p.Lq + qrow] : 0.f;
 
-  int koff[C::KS];
-#pragma unroll
-  for (int ks = 0; ks < C::KS; ++ks) koff[ks] = tile_off<D>(ql, 2 * ks + h);
-  int voff[C::DC][2];
+  // row fragment ks of a tile sits at tile_off(ql, 2 ks + h) = tile_off(ql, h) ^ (32 ks): the swizzle
+  // is an XOR on the 16-byte chunk index and 2 ks only touches bits the row term leaves zero
+  const int koff0 = tile_off<D>(ql, h);
+  auto koff = [&](int ks) __attribute__((always_inline)) { return koff0 ^ (ks << 5); };
+  // transposed fragments: lane reads 8 bytes of row 4h + i/4 (+ 8 for the second half) at column
+  // 32 dc + 16 g2 + 4 (i%4).  dc moves the chunk index by 4 dc (address bits 6, 7); row + 8 flips
+  // bit 1 of the swizzle term (address bit 5) and adds 8 rows.  All of these are XORs on the
+  // dc = 0, first-half offset because the bits involved are independent of the rest.
+  int voff0;
   {
     const int i = lane & 15, g2 = (lane >> 4) & 1;
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc) {
-      const int col = 32 * dc + 16 * g2 + 4 * (i & 3);
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf)
-        voff[dc][hf] = tile_off<D>(4 * h + (i >> 2) + 8 * hf, col >> 3) + ((col >> 2) & 1) * 8;
-    }
+    const int col = 16 * g2 + 4 * (i & 3);
+    voff0 = tile_off<D>(4 * h + (i >> 2), col >> 3) + ((col >> 2) & 1) * 8;
   }
+  constexpr int VOFF_HI = (8 * C::ROWB) | 32;
 
   // ---- requests: wave w issues request n = w*PER_TILE + d of each block (K first, then V)
   uint32_t r_vo[C::PER_TILE];
@@ -134,7 +133,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
     r_vo[d] = (uint32_t)(2 * (row * rs + 8 * (chp ^ f)));
     r_lds[d] = (r_isv[d] ? C::BLK_BYTES : 0) + part * 1024;
   }
-  auto request = [&](int slot_bytes, int blk) {
+  auto request = [&](int slot_bytes, int blk) __attribute__((always_inline)) {
     const int bb = min(blk, nkb - 1);                      // past the end: re-read the last block (never used)
 #pragma unroll
     for (int d = 0; d < C::PER_TILE; ++d) {
@@ -149,104 +148,179 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dc][r] = 0.f;
 
-  unsigned char* stat_lds = smem + C::STAT_OFF + wave * C::STAT_WAVE;   // [plane 3][FL][32] floats
-  auto flush = [&](int blast) {                            // write blocks 8*(blast/8) .. blast of this wave's terms
-    const int b0 = blast & ~(C::FL - 1), bi = lane >> 3, part = lane & 7;
-    if (b0 + bi <= blast) {
-      const int64_t dst = ((int64_t)bh * p.n_blocks + b0 + bi) * p.Lq + q0 + 4 * part;
-      *(float4*)(p.stat_a + dst) = *(const float4*)(stat_lds + ((0 * C::FL + bi) * 32 + 4 * part) * 4);
-      *(float4*)(p.stat_n + dst) = *(const float4*)(stat_lds + ((1 * C::FL + bi) * 32 + 4 * part) * 4);
-      *(float4*)(p.stat_l + dst) = *(const float4*)(stat_lds + ((2 * C::FL + bi) * 32 + 4 * part) * 4);
+  // per-wave staging of the per-block terms in LDS: [plane 3][FL][32] floats at STAT_OFF + wave * STAT_WAVE
+  auto lane_now = []() __attribute__((always_inline)) {     // lane id without a long-lived register
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+  };
+  // flush: lane -> (block fl_bi of the group, queries 4 fl_part ..); wave-uniform base in SGPRs, one
+  // 32-bit lane offset shared by the three planes.  Lane-only values are recomputed at each use
+  // (see `fresh` below): held across the loop they cost registers the loop does not have.
+  auto flush = [&](int blast) __attribute__((always_inline)) {   // blocks FL*(blast/FL) .. blast of this wave's terms
+    const int ln = lane_now();
+    const int fl_bi = ln >> 3, fl_part = ln & 7;
+    const uint32_t fl_off = 4u * (uint32_t)(fl_bi * p.Lq + 4 * fl_part);
+    const int fl_lds = C::STAT_OFF + wave * C::STAT_WAVE + (fl_bi * 32 + 4 * fl_part) * 4;
+    const int b0 = __builtin_amdgcn_readfirstlane(blast & ~(C::FL - 1));
+    const int64_t ub = ((int64_t)bh * p.n_blocks + b0) * p.Lq + q0;
+    if (b0 + fl_bi <= blast) {
+#pragma unroll
+      for (int pl = 0; pl < 3; ++pl) {
+        const float* base = (pl == 0 ? p.stat_a : pl == 1 ? p.stat_n : p.stat_l) + ub;
+        const u32x4_t val = *(const u32x4_t*)(smem + fl_lds + pl * C::FL * 128);
+        asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(fl_off), "v"(val), "s"(base) : "memory");
+      }
     }
   };
 
-  // ---- the three stages
-  f32x16_t sc, dp;
-  u32x4_t dsf[2];                                           // packed dS^T of the block: keys 0..15, 16..31
-  auto stage_x = [&](int slot) {
+  // ---- the stages
+  // addresses that depend only on the lane are recomputed where they are used: kept across the
+  // loop they would push the wave past its register budget
+  auto fresh = [](int x) __attribute__((always_inline)) {
+    asm volatile("" : "+v"(x));
+    return x;
+  };
+  const int goff = C::GO_OFF + wave * C::BLK_BYTES;
+  const int gk0 = goff + koff0;                             // this wave's dO row fragments: gk0 ^ (32 ks)
+  auto zero16 = [](f32x16_t& x) __attribute__((always_inline)) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      sc[r] = 0.f;
-      dp[r] = 0.f;
-    }
+    for (int r = 0; r < 16; ++r) x[r] = 0.f;
+  };
+  u32x4_t dsf[2];                                           // packed dS^T of the block: keys 0..15, 16..31
+  auto stage_x = [&](int slot_bytes, f32x16_t& s, f32x16_t& d) __attribute__((always_inline)) {
+    zero16(s);
+    zero16(d);
+    const int kb = fresh(koff0 + slot_bytes), gb = fresh(gk0);
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) {
-      sc = mfma32<T>(*(const u32x4_t*)(smem + slot + koff[ks]), qf[ks], sc);
-      dp = mfma32<T>(*(const u32x4_t*)(smem + slot + C::BLK_BYTES + koff[ks]),
-                     *(const u32x4_t*)(smem + C::GO_OFF + wave * C::BLK_BYTES + koff[ks]), dp);
+      const int ka = kb ^ (ks << 5);
+      s = mfma32<T>(*(const u32x4_t*)(smem + ka), qf[ks], s);
+      d = mfma32<T>(*(const u32x4_t*)(smem + ka + C::BLK_BYTES), *(const u32x4_t*)(smem + (gb ^ (ks << 5))), d);
     }
   };
-  auto pack_ds = [&](const float* ds) {
+  auto zbase = [&](int slot_bytes, int* zb) __attribute__((always_inline)) {
+    const int b = fresh(voff0 + slot_bytes);
+#pragma unroll
+    for (int dc = 0; dc < C::DC; ++dc) {
+      zb[2 * dc] = b ^ (dc << 6);
+      zb[2 * dc + 1] = b ^ ((dc << 6) | VOFF_HI);
+    }
+  };
+  auto ztr = [&](const int* zb, int n) __attribute__((always_inline)) {   // A operand of the n-th dQ^T MFMA: K^T, keys 16 j ..
+    const int j = n / C::DC, dc = n % C::DC;
+    const u32x2_t a0 = lds_read_tr(smem + 16 * j * C::ROWB + zb[2 * dc]);
+    const u32x2_t a1 = lds_read_tr(smem + 16 * j * C::ROWB + zb[2 * dc + 1]);
+    const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
+    return a;
+  };
+  auto stage_z = [&](int slot_bytes) __attribute__((always_inline)) {     // dQ^T += K^T dS^T
+    int zb[2 * C::DC];
+    zbase(slot_bytes, zb);
+#pragma unroll
+    for (int n = 0; n < 2 * C::DC; ++n) acc[n % C::DC] = mfma32<T>(ztr(zb, n), dsf[n / C::DC], acc[n % C::DC]);
+  };
+  // X of the next block interleaved with Y of an earlier block `blk`.  The wave issues in order, so
+  // the instruction stream is the schedule: each MFMA is followed by a slice of Y that runs while
+  // the matrix pipe is busy.  Key of register r is 8*(r/4) + 4h + r%4; the landmark is r = 15, h = 1.
+  auto stage_xy = [&](int nslot, int blk, f32x16_t& s, f32x16_t& d, f32x16_t& sn, f32x16_t& dn)
+                      __attribute__((always_inline)) {
+    zero16(sn);
+    zero16(dn);
+    constexpr int NX = 2 * C::KS;
+    const int kb = fresh(koff0 + nslot), gb = fresh(gk0);
+    u32x4_t fk[C::KS], fv[C::KS], fg[C::KS];
+    auto frags = [&](int ks) __attribute__((always_inline)) {
+      fk[ks] = *(const u32x4_t*)(smem + (kb ^ (ks << 5)));
+      fv[ks] = *(const u32x4_t*)(smem + (kb ^ (ks << 5)) + C::BLK_BYTES);
+      fg[ks] = *(const u32x4_t*)(smem + (gb ^ (ks << 5)));
+    };
+    frags(0);
+    const float s_last = s[15];
+    float mx = 0.f, mloc = 0.f, t_lm = 0.f, den = 0.f, spd = 0.f, nD = 0.f, f = 0.f, fn = 0.f, dslm = 0.f;
+    float ds[16];
+    auto ywork = [&](int u) __attribute__((always_inline)) {
+      if (u == 0) {
+        mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+        mx = fmaxf(fmaxf(mx, s[3]), s[4]);
+        mx = fmaxf(fmaxf(mx, s[5]), s[6]);
+        mx = fmaxf(fmaxf(mx, s[7]), s[8]);
+      } else if (u == 1) {
+        mx = fmaxf(fmaxf(mx, s[9]), s[10]);
+        mx = fmaxf(fmaxf(mx, s[11]), s[12]);
+        mx = fmaxf(fmaxf(mx, s[13]), s[14]);
+        mx = fmaxf(mx, (h == 0) ? s_last : -INFINITY);
+        mx = pair_max(mx);
+        t_lm = pair_hi(s_last) * c2;
+        mloc = mx * c2;
+      } else if (u < 10) {
+#pragma unroll
+        for (int r = 2 * (u - 2); r < 2 * (u - 2) + 2; ++r) {
+          float x = fast_exp2(__builtin_fmaf(s[r], c2, -mloc));
+          if (r == 15) x = (h == 0) ? x : 0.f;
+          s[r] = x;
+          den += x;
+          spd = __builtin_fmaf(x, d[r], spd);
+        }
+      } else if (u == 10) {
+        den = pair_sum(den);
+        spd = pair_sum(spd);
+      } else if (u == 11) {
+        const float invden = fast_rcp(den);
+        nD = spd * invden;
+        const float glog = t_lm - mhat;                    // log2 of the normalised gate
+        const float g = fast_exp2(glog);
+        f = g * invden;
+        fn = f * nD;
+        dslm = g * (nD - delta);
+        const int ln = lane_now();
+        if (ln < 32) {                                     // h == 0: lane = query
+          const int bi = blk & (C::FL - 1);
+          unsigned char* sp = smem + C::STAT_OFF + wave * C::STAT_WAVE + bi * 128 + ln * 4;
+          *(float*)(sp + 0 * C::FL * 128) = mloc + fast_log2(den) - glog;
+          *(float*)(sp + 1 * C::FL * 128) = nD;
+          *(float*)(sp + 2 * C::FL * 128) = dslm;
+        }
+      } else {
+#pragma unroll
+        for (int r = 4 * (u - 12); r < 4 * (u - 12) + 4; ++r) {
+          ds[r] = s[r] * __builtin_fmaf(f, d[r], -fn);
+          if (r == 15) ds[r] = (h == 1) ? dslm : ds[r];
+          if (r & 1) dsf[r >> 3][(r >> 1) & 3] = pack2<T>(ds[r - 1], ds[r]);
+        }
+      }
+    };
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < NX; ++m) {
+      const int ks = m >> 1;
+      if ((m & 1) == 0 && ks + 1 < C::KS) frags(ks + 1);
+      if ((m & 1) == 0) sn = mfma32<T>(fk[ks], qf[ks], sn);
+      else dn = mfma32<T>(fv[ks], fg[ks], dn);
+#pragma unroll
+      for (int u = (m * 16) / NX; u < ((m + 1) * 16) / NX; ++u) ywork(u);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if ((blk & (C::FL - 1)) == C::FL - 1 || blk == cblk - 1) flush(blk);
+  };
+  auto stage_y_diag = [&](const f32x16_t& s, const f32x16_t& d) __attribute__((always_inline)) {   // the wave's own block
+    float ds[16];
+    const int lim = ql - ((ql == 31) ? 1 : 0);             // the landmark query looks one to the left
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = 8 * (r >> 2) + 4 * h + (r & 3);
+      const float pr = (key <= lim) ? fast_exp2(__builtin_fmaf(s[r], c2, -mhat)) : 0.f;
+      ds[r] = pr * (d[r] - delta);
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      u32x4_t f = {pack2<T>(ds[8 * j + 0], ds[8 * j + 1]), pack2<T>(ds[8 * j + 2], ds[8 * j + 3]),
-                   pack2<T>(ds[8 * j + 4], ds[8 * j + 5]), pack2<T>(ds[8 * j + 6], ds[8 * j + 7])};
-      dsf[j] = f;
+      u32x4_t fr = {pack2<T>(ds[8 * j + 0], ds[8 * j + 1]), pack2<T>(ds[8 * j + 2], ds[8 * j + 3]),
+                    pack2<T>(ds[8 * j + 4], ds[8 * j + 5]), pack2<T>(ds[8 * j + 6], ds[8 * j + 7])};
+      dsf[j] = fr;
     }
-  };
-  auto stage_y = [&](int blk) {
-    float ds[16];
-    if (blk < cblk) {
-      // earlier block: key of register r is 8*(r/4) + 4h + r%4; the landmark is (r = 15, h = 1)
-      const float s_last = sc[15];
-      float mx = (h == 0) ? s_last : -INFINITY;
-#pragma unroll
-      for (int r = 0; r < 15; ++r) mx = fmaxf(mx, sc[r]);
-      mx = pair_max(mx);
-      const float t_lm = pair_hi(s_last) * c2;
-      const float mloc = mx * c2;
-      float den = 0.f, spd = 0.f;
-      float e[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float x = fast_exp2(__builtin_fmaf(sc[r], c2, -mloc));
-        if (r == 15) x = (h == 0) ? x : 0.f;
-        e[r] = x;
-        den += x;
-        spd = __builtin_fmaf(x, dp[r], spd);
-      }
-      den = pair_sum(den);
-      spd = pair_sum(spd);
-      const float invden = fast_rcp(den);
-      const float nD = spd * invden;
-      const float glog = t_lm - mhat;                      // log2 of the normalised gate
-      const float g = fast_exp2(glog);
-      const float f = g * invden;
-      const float dslm = g * (nD - delta);
-      if (h == 0) {
-        const int bi = blk & (C::FL - 1);
-        *(float*)(stat_lds + ((0 * C::FL + bi) * 32 + ql) * 4) = mloc + fast_log2(den) - glog;
-        *(float*)(stat_lds + ((1 * C::FL + bi) * 32 + ql) * 4) = nD;
-        *(float*)(stat_lds + ((2 * C::FL + bi) * 32 + ql) * 4) = dslm;
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) ds[r] = e[r] * f * (dp[r] - nD);
-      if (h == 1) ds[15] = dslm;
-      if ((blk & (C::FL - 1)) == C::FL - 1 || blk == cblk - 1) flush(blk);
-    } else {
-      const int lim = ql - ((ql == 31) ? 1 : 0);           // the landmark query looks one to the left
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = 8 * (r >> 2) + 4 * h + (r & 3);
-        const float pr = (key <= lim) ? fast_exp2(__builtin_fmaf(sc[r], c2, -mhat)) : 0.f;
-        ds[r] = pr * (dp[r] - delta);
-      }
-    }
-    pack_ds(ds);
-  };
-  auto stage_z = [&](int slot) {
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int dc = 0; dc < C::DC; ++dc) {
-        const u32x2_t a0 = lds_read_tr(smem + slot + 16 * j * C::ROWB + voff[dc][0]);
-        const u32x2_t a1 = lds_read_tr(smem + slot + 16 * j * C::ROWB + voff[dc][1]);
-        const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
-        acc[dc] = mfma32<T>(a, dsf[j], acc[dc]);
-      }
   };
 
-  // ---- prologue: this wave's dO rows -> LDS; blocks 0 .. DIST-1 requested; block 0 must have landed
+  // ---- prologue: this wave's dO rows -> LDS; blocks 0 .. 2 requested; blocks 0 and 1 must have landed
   {
     const int qb = min(q0, p.Lq - 32);                     // inactive waves re-read valid rows (never used)
     const char* gt = gp + 2 * ((int64_t)qb * p.dos_r);
@@ -254,45 +328,44 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
     for (int n = 0; n < 32 / C::RPD; ++n) {
       const int row = C::RPD * n + lane / C::CH, chp = lane % C::CH;
       const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
-      dq_dma16(gt, (uint32_t)(2 * (row * p.dos_r + 8 * (chp ^ f))), C::GO_OFF + wave * C::BLK_BYTES + n * 1024);
+      dq_dma16(gt, (uint32_t)(2 * (row * p.dos_r + 8 * (chp ^ f))), goff + n * 1024);
     }
   }
 #pragma unroll
-  for (int t = 0; t < C::DIST; ++t) request(t * C::BUF_BYTES, t);
-  dq_wait_vmcnt<(C::DIST - 1) * C::PER_TILE>();
+  for (int t = 0; t < C::NBUF - 1; ++t) request(t * C::BUF_BYTES, t);
+  dq_wait_vmcnt<C::PER_TILE>();
   __syncthreads();
 
-  const bool late = C::SKEW && wave >= C::NW / 2;          // upper waves run half a period behind
-  const int periods = nblk + 1;
-  auto period = [&](auto Rc, int k) {
+  f32x16_t sA, dA, sB, dB;                                  // S^T, dP^T of the even / odd blocks
+  zero16(sB);
+  zero16(dB);
+  stage_x(0, sA, dA);
+
+  auto period = [&](auto Rc, int k) __attribute__((always_inline)) {
     constexpr int R = decltype(Rc)::value;
-    constexpr int CUR = R * C::BUF_BYTES, PRV = ((R + C::NBUF - 1) % C::NBUF) * C::BUF_BYTES;
-    request(((R + C::DIST) % C::NBUF) * C::BUF_BYTES, k + C::DIST);   // into the slot block k-2 has left
-    if (!late) {
-      if (k < nblk && k <= cblk && rowok) {
-        stage_x(CUR);
-        stage_y(k);
-        stage_z(CUR);
-      }
-    } else {
-      if (k >= 1 && k - 1 <= cblk && rowok) stage_z(PRV);
-      if (k < nblk && k <= cblk && rowok) {
-        stage_x(CUR);
-        stage_y(k);
-      }
+    constexpr int CUR = R * C::BUF_BYTES, NXT = ((R + 1) % C::NBUF) * C::BUF_BYTES;
+    request(((R + 3) % C::NBUF) * C::BUF_BYTES, k + 3);    // into the slot block k-1 has left
+    if (rowok && k <= cblk) {
+      f32x16_t& s = (R & 1) ? sB : sA;
+      f32x16_t& d = (R & 1) ? dB : dA;
+      f32x16_t& sn = (R & 1) ? sA : sB;
+      f32x16_t& dn = (R & 1) ? dA : dB;
+      if (k < cblk) stage_xy(NXT, k, s, d, sn, dn);
+      else stage_y_diag(s, d);
+      stage_z(CUR);
     }
-    dq_wait_vmcnt<(C::DIST - 1) * C::PER_TILE>();          // block k+1 has landed (k+2 may be in flight)
+    dq_wait_vmcnt<C::PER_TILE>();                          // block k+2 has landed (k+3 may be in flight)
     __syncthreads();
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
-  for (int k = 0; k < periods; k += 4) {
+  for (int k = 0; k < nblk; k += 4) {
     period(I0{}, k);
-    if (k + 1 < periods) period(I1{}, k + 1);
-    if (k + 2 < periods) period(I2{}, k + 2);
-    if (k + 3 < periods) period(I3{}, k + 3);
+    if (k + 1 < nblk) period(I1{}, k + 1);
+    if (k + 2 < nblk) period(I2{}, k + 2);
+    if (k + 3 < nblk) period(I3{}, k + 3);
   }
   dq_wait_vmcnt<0>();                                      // nothing may still be writing LDS when the wave ends
 
