@@ -1,21 +1,25 @@
 // dK/dV kernel of the backward pass, landmark block = 32 keys.
 //
-// Key-stationary: a workgroup is 4 waves, one per SIMD, each owning one 32-key tile whose K and V
-// fragments stay in registers as B operands.  Query tiles (32 rows of Q and of dO) and the terms
-// the elementwise step needs (per row: mhat, delta; per (row, block): a, nD, dS at the landmark,
-// left behind by the dQ kernel) stream through a ring of five LDS slots filled by direct
-// global->LDS loads (global_load_lds_dwordx4): tile j+4 is requested while tile j is computed, no
-// registers are tied up by data in flight, and vmcnt is counted by hand (five requests per wave
-// and tile).  The LDS swizzle is applied on the source side: lane i of a request lands at
+// Key-stationary.  A workgroup is 8 waves = 4 key tiles of 32 keys x 2 roles; the two waves of a
+// key tile sit on the same SIMD (waves t and t+4) and split the work so that each holds one
+// accumulator and both pipes of the SIMD have work from two instruction streams at once:
+//     wave V (t):    S = Q K^T,  W = exp2(S c - x)  (the attention weights),  dV^T += dO^T W
+//     wave K (t+4):  dP = dO V^T,  dS = W (dP - y) + z,                       dK^T += Q^T dS
+// W goes from wave V to wave K through LDS as packed 16-bit values, lane for lane (both waves hold
+// the same accumulator layout: lane = key, register r = query row 8*(r/4) + 4*(l/32) + r%4), and
+// wave K runs one query tile behind wave V, so one barrier per query tile orders everything.
+// Within a wave the products of the next tile are interleaved with the elementwise work of the
+// current one (the wave issues in order, so the instruction stream is the schedule).
+//
+// Query tiles (32 rows of Q and of dO) and the terms the elementwise steps need (per row: mhat,
+// delta; per (row, block): a, nD, dS at the landmark, left behind by the dQ kernel) stream through
+// a ring of six LDS slots filled by direct global->LDS loads (global_load_lds_dwordx4): tile i+4 is
+// requested while tile i is computed, no registers are tied up by data in flight, and vmcnt is
+// counted by hand.  The LDS swizzle is applied on the source side: lane i of a request lands at
 // +16*i, so it fetches the chunk that belongs there.
-// With one wave per SIMD the schedule is the instruction stream (see `body`):
-//     S, dP of tile j+1 (16 MFMA)  ||  elementwise W, dS of tile j (VALU)
-//     dV^T += dO^T W, dK^T += Q^T dS of tile j (16 MFMA)
-// Layout: S = Q K^T in the accumulator layout, lane = key, register r = query row
-// 8*(r/4) + 4*(l/32) + r%4 of the tile.  Everything between the products is elementwise:
-//     earlier block (query tile past the key tile):  W = exp2(s*c - a),  dS = W (dP - nD);
-//         at the block's landmark key W = 0 and dS is the value stored by the dQ kernel
-//     own block / not yet visible:  W = [key <= lim] exp2(s*c - mhat),  dS = W (dP - delta)
+//     earlier block (query tile past the key tile):  x = a, y = nD, z = 0; at the block's landmark
+//         key W = 0 (x = 1e30) and z = the dS stored by the dQ kernel
+//     own block / not yet visible:  W = [key <= lim] exp2(s*c - mhat),  y = delta, z = 0
 #include <type_traits>
 
 #include "lmk_common.hpp"
@@ -25,20 +29,24 @@ namespace lmk {
 
 template <class T, int D>
 struct Dkv32Cfg {
-  static constexpr int NW = 4;
+  static constexpr int NKT = 4;                            // key tiles per workgroup
+  static constexpr int NW = 2 * NKT;
   static constexpr int NTHR = 64 * NW;
   static constexpr int CH = D / 8;
   static constexpr int KS = D / 16;
   static constexpr int DC = D / 32;
   static constexpr int ROWB = 2 * D;
   static constexpr int TILE_BYTES = 32 * ROWB;             // one query tile of Q (or of dO)
-  static constexpr int STAT_BYTES = 1024 * NW;             // per wave: a, nD, dslm, mhat, delta (128 B each) + pad
+  static constexpr int STAT_BYTES = 1024 * NKT;            // per key tile: a, nD, dslm, mhat, delta (128 B each) + pad
   static constexpr int BUF_BYTES = 2 * TILE_BYTES + STAT_BYTES;   // Q, dO, terms
-  static constexpr int NBUF = 5;                           // ring slots: 2 in use, 3 in flight
+  static constexpr int NBUF = 6;                           // ring slots: tiles i-1, i, i+1 in use, i+2 .. i+4 in flight
   static constexpr int RPD = 1024 / ROWB;                  // tile rows covered by one 1 KB request
-  static constexpr int NDMA = 32 / RPD / NW;               // requests per wave, tile and tensor
-  static constexpr int PER_TILE = 2 * NDMA + 1;            // requests per wave and ring slot
-  static constexpr int CONST_OFF = NBUF * BUF_BYTES;       // 32 x 1e30f, then 32 x 0.0f
+  static constexpr int NDMA = 32 / RPD / NKT;              // requests per K-role wave, tile and tensor
+  static constexpr int PER_TILE_K = 2 * NDMA;              // K-role waves fetch Q and dO
+  static constexpr int PER_TILE_V = 1;                     // V-role waves fetch their key tile's terms
+  static constexpr int XCH_OFF = NBUF * BUF_BYTES;         // W hand-over: [parity 2][key tile][piece 2][lane][16 B]
+  static constexpr int XCH_TILE = 2048;
+  static constexpr int CONST_OFF = XCH_OFF + 2 * NKT * XCH_TILE;   // 32 x 1e30f, then 32 x 0.0f
   static constexpr int LDS_BYTES = CONST_OFF + 256;
 };
 
@@ -57,11 +65,16 @@ __device__ __forceinline__ void wait_vmcnt() {             // s_waitcnt vmcnt(N)
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
+#define LMK_INL __attribute__((always_inline))
+
 template <class T, int D>
-__global__ __launch_bounds__(256, 1) void lmk_bwd_dkdv32_kernel(BwdParams p) {
+__global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   using C = Dkv32Cfg<T, D>;
   extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tile = wave & (C::NKT - 1);                    // key tile inside the workgroup
+  const bool role_k = wave >= C::NKT;                      // false: S, W, dV; true: dP, dS, dK
   const int ql = lane & 31, h = lane >> 5;
 
   int bh, kvt;                                             // (batch*head, 128-key tile); most work first
@@ -78,14 +91,10 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   }
   const int b_ = bh / p.H, hh = bh % p.H;
   const char* qp = (const char*)p.q + 2 * (b_ * p.qs_b + hh * p.qs_h);
-  const char* kp = (const char*)p.k + 2 * (b_ * p.ks_b + hh * p.ks_h);
-  const char* vp = (const char*)p.v + 2 * (b_ * p.vs_b + hh * p.vs_h);
   const char* gp = (const char*)p.dout + 2 * (b_ * p.dos_b + hh * p.dos_h);
-  char* dkp = (char*)p.dk + 2 * (b_ * p.dks_b + hh * p.dks_h);
-  char* dvp = (char*)p.dv + 2 * (b_ * p.dvs_b + hh * p.dvs_h);
 
   const int nkt = p.Lk >> 5;                               // key tiles (= landmark blocks)
-  const int kt = kvt * 4 + wave;
+  const int kt = kvt * C::NKT + tile;
   const bool active = kt < nkt;
   const int krow = kt * 32 + ql;
   const bool lm_lane = (ql == 31);                         // this lane's key is its block's landmark
@@ -93,17 +102,7 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   const int nq = p.Lq >> 5;
   const float c2 = p.scale_log2;
 
-  u32x4_t kf[C::KS], vf[C::KS];
-#pragma unroll
-  for (int ks = 0; ks < C::KS; ++ks) {
-    u32x4_t z = {0, 0, 0, 0};
-    kf[ks] = z;
-    vf[ks] = z;
-    if (active) {
-      kf[ks] = *(const u32x4_t*)(kp + 2 * ((int64_t)krow * p.ks_r + 16 * ks + 8 * h));
-      vf[ks] = *(const u32x4_t*)(vp + 2 * ((int64_t)krow * p.vs_r + 16 * ks + 8 * h));
-    }
-  }
+  u32x4_t bf[C::KS];                                       // stationary operand, loaded after the first requests
 
   int koff[C::KS];
 #pragma unroll
@@ -120,12 +119,13 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     }
   }
 
-  // ---- loaders: per ring slot every wave issues NDMA requests for Q, NDMA for dO and one for its terms
-  const int j_first = max(0, kvt * 4 - PT);                // first query tile any wave here can see
+  // ---- loaders.  K-role wave b fetches rows RPD*(b*NDMA + d) .. of Q and of dO; V-role wave t
+  // fetches the terms of key tile t.
+  const int j_first = max(0, kvt * C::NKT - PT);           // first query tile any wave here can see
   uint32_t q_vo[C::NDMA], g_vo[C::NDMA];                   // per-lane source offsets inside a tile (bytes)
 #pragma unroll
   for (int d = 0; d < C::NDMA; ++d) {
-    const int n = wave * C::NDMA + d;                      // request n covers tile rows RPD*n ..
+    const int n = tile * C::NDMA + d;
     const int row = C::RPD * n + lane / C::CH, chp = lane % C::CH;
     const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
     q_vo[d] = (uint32_t)(2 * (row * p.qs_r + 8 * (chp ^ f)));   // the chunk that belongs at LDS position chp
@@ -140,204 +140,237 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dkdv32_kernel(BwdParams p) {
              : (arr == 3) ? p.mhat + head_row : p.delta + head_row;
     st_src += 4 * part;
   }
-  auto request = [&](int slot_bytes, int j) {              // everything of query tile j -> ring slot at slot_bytes
+  auto request = [&](int slot_bytes, int j) LMK_INL {      // this wave's share of query tile j -> ring slot
     const int jj = min(j, nq - 1);                         // past the end: re-read the last tile (never used)
-    const char* qt = qp + 2 * ((int64_t)jj * 32 * p.qs_r);
-    const char* gt = gp + 2 * ((int64_t)jj * 32 * p.dos_r);
+    if (role_k) {
+      const char* qt = qp + 2 * ((int64_t)jj * 32 * p.qs_r);
+      const char* gt = gp + 2 * ((int64_t)jj * 32 * p.dos_r);
 #pragma unroll
-    for (int d = 0; d < C::NDMA; ++d) {
-      dma16_s(qt, q_vo[d], slot_bytes + (wave * C::NDMA + d) * 1024);
-      dma16_s(gt, g_vo[d], slot_bytes + C::TILE_BYTES + (wave * C::NDMA + d) * 1024);
+      for (int d = 0; d < C::NDMA; ++d) {
+        dma16_s(qt, q_vo[d], slot_bytes + (tile * C::NDMA + d) * 1024);
+        dma16_s(gt, g_vo[d], slot_bytes + C::TILE_BYTES + (tile * C::NDMA + d) * 1024);
+      }
+    } else {
+      dma16_v(st_src + 32 * jj, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
     }
-    dma16_v(st_src + 32 * jj, slot_bytes + 2 * C::TILE_BYTES + wave * 1024);
+  };
+  auto wait_tiles = [&]() LMK_INL {                        // all but this wave's two newest tiles have landed
+    if (role_k) wait_vmcnt<2 * C::PER_TILE_K>();
+    else wait_vmcnt<2 * C::PER_TILE_V>();
   };
 
-  f32x16_t dkacc[C::DC], dvacc[C::DC];
+  auto zero16 = [](f32x16_t& x) LMK_INL {
 #pragma unroll
-  for (int dc = 0; dc < C::DC; ++dc)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      dkacc[dc][r] = 0.f;
-      dvacc[dc][r] = 0.f;
-    }
-
-  auto row_tile = [&](int tileoff, const u32x4_t* bf) {    // (32 rows of the LDS tile) x (this wave's 32 keys)
-    f32x16_t s;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) s[r] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(*(const u32x4_t*)(smem + tileoff + koff[ks]), bf[ks], s);
-    return s;
+    for (int r = 0; r < 16; ++r) x[r] = 0.f;
   };
-
-  // ---- prologue: tiles j_first .. +3 requested; the first two must have landed
-  request(0 * C::BUF_BYTES, j_first);
-  request(1 * C::BUF_BYTES, j_first + 1);
-  request(2 * C::BUF_BYTES, j_first + 2);
-  request(3 * C::BUF_BYTES, j_first + 3);
-  if (tid < 64) ((float*)(smem + C::CONST_OFF))[tid] = (tid < 32) ? 1e30f : 0.f;
-  wait_vmcnt<2 * C::PER_TILE>();
-  __syncthreads();
-
-  f32x16_t s_cur = row_tile(0, kf), dp_cur = row_tile(C::TILE_BYTES, vf);
-
-  // One iteration = one query tile j against this wave's key tile.  The wave issues in order, so
-  // the instruction stream itself is the schedule: every MFMA is followed by a few independent
-  // instructions that run while the matrix pipe is busy (a 32x32x16 MFMA occupies it for ~33
-  // cycles, a VALU instruction of a lone wave issues every ~5.5); sched_barrier(0) pins the order.
-  //   phase A   16 MFMA: S and dP of tile j+1        + elementwise registers 0..11 of tile j
-  //   phase B1   8 MFMA: dV, dK from rows 0..15      + elementwise registers 12..15
-  //   phase B2   8 MFMA: dV, dK from rows 16..31
-  // MASKED = false: the query tile lies in a later block than the keys (the common case): every key
-  //   is visible, W = exp2(s*c - a), dS = W (dP - nD); the landmark lane reads 1e30 for `a` (W = 0)
-  //   and the stored dS as addend.
-  // MASKED = true: own block or not yet visible: W = [key <= lim] exp2(s*c - mhat), dS = W (dP - delta).
-  auto body = [&](auto Rc, auto Mc, int j) {
-    constexpr int R = decltype(Rc)::value;
-    constexpr bool MASKED = decltype(Mc)::value;
-    constexpr int CUR = R * C::BUF_BYTES, NXT = ((R + 1) % C::NBUF) * C::BUF_BYTES;
-    const int CST = CUR + 2 * C::TILE_BYTES + wave * 1024;  // this wave's terms: a, nD, dslm, mhat, delta
-
-    const int dtq = PT + j;                                // the tile's own landmark block
-    const int krel = 32 * (kt - dtq) + ql;                 // key position relative to the query tile's first row
-    // x: exponent offset, y: subtrahend of dP, z: addend of dS  (byte offsets of 32-float arrays)
-    const int xoff = (MASKED ? CST + 384 : (lm_lane ? C::CONST_OFF : CST)) + 16 * h;
-    const int yoff = (MASKED ? CST + 512 : CST + 128) + 16 * h;
-    const int zoff = (lm_lane ? CST + 256 : C::CONST_OFF + 128) + 16 * h;
-    float4 x4[4], y4[4], z4[4];                            // fetched one register group ahead of their use
-    auto load_xyz = [&](int g) {
-      x4[g] = *(const float4*)(smem + xoff + 32 * g);
-      y4[g] = *(const float4*)(smem + yoff + 32 * g);
-      if (!MASKED) z4[g] = *(const float4*)(smem + zoff + 32 * g);
-    };
-    load_xyz(0);
-    float w[16], ds[16];
-    u32x4_t wf[2], df[2];                                  // packed B operands: rows 0..15 and 16..31
-    auto elementwise = [&](int r) {                        // register r <-> query row 8*(r/4) + 4h + r%4
-      const int g = r >> 2, e = r & 3;
-      if (e == 0 && g < 3) load_xyz(g + 1);
-      const float xa = (e == 0) ? x4[g].x : (e == 1) ? x4[g].y : (e == 2) ? x4[g].z : x4[g].w;
-      const float ya = (e == 0) ? y4[g].x : (e == 1) ? y4[g].y : (e == 2) ? y4[g].z : y4[g].w;
-      float ex = fast_exp2(__builtin_fmaf(s_cur[r], c2, -xa));
-      if (MASKED) {
-        // key visible to this query row?  the landmark row of a block looks one position to the left
-        const int qloc = 8 * g + 4 * h + e;
-        ex = (krel <= qloc - ((qloc == 31) ? 1 : 0)) ? ex : 0.f;
-        ds[r] = ex * (dp_cur[r] - ya);
-      } else {
-        const float za = (e == 0) ? z4[g].x : (e == 1) ? z4[g].y : (e == 2) ? z4[g].z : z4[g].w;
-        ds[r] = __builtin_fmaf(ex, dp_cur[r] - ya, za);
-      }
-      w[r] = ex;
-      if (r & 1) {                                         // pack pairs as soon as they exist
-        wf[r >> 3][(r >> 1) & 3] = pack2<T>(w[r - 1], w[r]);
-        df[r >> 3][(r >> 1) & 3] = pack2<T>(ds[r - 1], ds[r]);
-      }
-    };
-
-    // ---- phase A
-    f32x16_t s_next, dp_next;
+  auto row_tile = [&](int tile_bytes, f32x16_t& s) LMK_INL {   // (32 rows of the LDS tile) x (this wave's 32 keys)
+    zero16(s);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      s_next[r] = 0.f;
-      dp_next[r] = 0.f;
-    }
-    constexpr int NA = 2 * C::KS;                          // MFMAs in phase A (16 for D = 128, 8 for D = 64)
-    auto frag = [&](int i) {
-      return *(const u32x4_t*)(smem + NXT + (i < C::KS ? 0 : C::TILE_BYTES) + koff[i < C::KS ? i : i - C::KS]);
-    };
-    constexpr int PF = 4;                                  // LDS reads in flight ahead of their MFMA
-    u32x4_t fr[NA + PF];
-#pragma unroll
-    for (int i = 0; i < PF; ++i) fr[i] = frag(i);
-    __builtin_amdgcn_sched_barrier(0);
-    constexpr int EA = 12;                                 // elementwise registers done under phase A
-#pragma unroll
-    for (int i = 0; i < NA; ++i) {
-      if (i + PF < NA) fr[i + PF] = frag(i + PF);
-      if (i < C::KS) s_next = mfma32<T>(fr[i], kf[i], s_next);
-      else dp_next = mfma32<T>(fr[i], vf[i - C::KS], dp_next);
-#pragma unroll
-      for (int r = (i * EA) / NA; r < ((i + 1) * EA) / NA; ++r) elementwise(r);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-
-    // ---- phase B: dV^T += dO^T W, dK^T += Q^T dS
-    constexpr int NB = 4 * C::DC;                          // MFMAs in phase B (16 for D = 128, 8 for D = 64)
-    auto trindex = [&](int n) {                            // n-th MFMA -> j2 (row half), t (0: dO, 1: Q), dc
-      const int j2 = n / (2 * C::DC), t = (n / C::DC) & 1, dc = n % C::DC;
-      return (j2 << 3) | (t << 2) | dc;
-    };
-    auto trfrag = [&](int m) {
-      const int dc = m & 3, t = (m >> 2) & 1, j2 = m >> 3;
-      const int base = CUR + (t == 0 ? C::TILE_BYTES : 0) + 16 * j2 * C::ROWB;
+    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(*(const u32x4_t*)(smem + tile_bytes + koff[ks]), bf[ks], s);
+  };
+  // second product of a tile: acc[dc] += (tile at tile_bytes)^T x (packed B operands: rows 0..15, 16..31)
+  auto tr_product = [&](int tile_bytes, const u32x4_t* pk, f32x16_t* acc) LMK_INL {
+    constexpr int NB = 2 * C::DC, PF = 2;
+    auto trfrag = [&](int n) LMK_INL {
+      const int j2 = n / C::DC, dc = n % C::DC;
+      const int base = tile_bytes + 16 * j2 * C::ROWB;
       const u32x2_t a0 = lds_read_tr(smem + base + voff[dc][0]), a1 = lds_read_tr(smem + base + voff[dc][1]);
       const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
       return a;
     };
     u32x4_t tf[NB + PF];
 #pragma unroll
-    for (int n = 0; n < PF; ++n) tf[n] = trfrag(trindex(n));
-    __builtin_amdgcn_sched_barrier(0);
+    for (int n = 0; n < PF; ++n) tf[n] = trfrag(n);
 #pragma unroll
     for (int n = 0; n < NB; ++n) {
-      if (n + PF < NB) tf[n + PF] = trfrag(trindex(n + PF));
-      const int m = trindex(n);
-      const int dc = m & 3, t = (m >> 2) & 1, j2 = m >> 3;
-      if (t == 0) dvacc[dc] = mfma32<T>(tf[n], wf[j2], dvacc[dc]);
-      else dkacc[dc] = mfma32<T>(tf[n], df[j2], dkacc[dc]);
-      if (n < NB / 2) {                                    // remaining elementwise registers under the first half
+      if (n + PF < NB) tf[n + PF] = trfrag(n + PF);
+      acc[n % C::DC] = mfma32<T>(tf[n], pk[n / C::DC], acc[n % C::DC]);
+    }
+  };
+
+  // ---- V role: one query tile i.  S of tile i+1 (slot nslot) is interleaved with W of tile i.
+  auto body_v = [&](auto Mc, int i, int cslot, int nslot, int par, f32x16_t& s, f32x16_t& sn, f32x16_t* acc) LMK_INL {
+    constexpr bool MASKED = decltype(Mc)::value;
+    const int CST = cslot + 2 * C::TILE_BYTES + tile * 1024;   // this key tile's terms: a, nD, dslm, mhat, delta
+    const int krel = 32 * (kt - (PT + i)) + ql;            // key position relative to the query tile's first row
+    const int xoff = (MASKED ? CST + 384 : (lm_lane ? C::CONST_OFF : CST)) + 16 * h;
+    float4 x4[4];
 #pragma unroll
-        for (int r = EA + (n * (16 - EA)) / (NB / 2); r < EA + ((n + 1) * (16 - EA)) / (NB / 2); ++r) elementwise(r);
+    for (int g = 0; g < 4; ++g) x4[g] = *(const float4*)(smem + xoff + 32 * g);
+    u32x4_t wf[2];
+    float w[16];
+    auto elementwise = [&](int r) LMK_INL {                // register r <-> query row 8*(r/4) + 4h + r%4
+      const int g = r >> 2, e = r & 3;
+      const float xa = (e == 0) ? x4[g].x : (e == 1) ? x4[g].y : (e == 2) ? x4[g].z : x4[g].w;
+      float ex = fast_exp2(__builtin_fmaf(s[r], c2, -xa));
+      if (MASKED) {
+        // key visible to this query row?  the landmark row of a block looks one position to the left
+        const int qloc = 8 * g + 4 * h + e;
+        ex = (krel <= qloc - ((qloc == 31) ? 1 : 0)) ? ex : 0.f;
       }
+      w[r] = ex;
+      if (r & 1) {
+        uint32_t pk = pack2<T>(w[r - 1], w[r]);
+        asm volatile("" : "+v"(pk));                       // pins this slice between its two MFMAs
+        wf[r >> 3][(r >> 1) & 3] = pk;
+      }
+    };
+    zero16(sn);
+    constexpr int PF = 2;
+    u32x4_t fr[C::KS + PF];
+#pragma unroll
+    for (int m = 0; m < PF; ++m) fr[m] = *(const u32x4_t*)(smem + nslot + koff[m]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < C::KS; ++m) {
+      if (m + PF < C::KS) fr[m + PF] = *(const u32x4_t*)(smem + nslot + koff[m + PF]);
+      sn = mfma32<T>(fr[m], bf[m], sn);
+#pragma unroll
+      for (int r = (m * 16) / C::KS; r < ((m + 1) * 16) / C::KS; ++r) elementwise(r);
       __builtin_amdgcn_sched_barrier(0);
     }
-    s_cur = s_next;
-    dp_cur = dp_next;
-  };
-  auto iter = [&](auto Rc, int j) {
-    constexpr int R = decltype(Rc)::value;
-    request(((R + 4) % C::NBUF) * C::BUF_BYTES, j + 4);    // into the slot tile j-1 has left
-    if (PT + j > kt) body(Rc, std::false_type{}, j);       // wave-uniform choice
-    else body(Rc, std::true_type{}, j);
-    wait_vmcnt<2 * C::PER_TILE>();                         // tile j+2 has landed (tiles j+3, j+4 may be in flight)
-    __syncthreads();
+    unsigned char* xp = smem + C::XCH_OFF + (par * C::NKT + tile) * C::XCH_TILE + lane * 16;
+    *(u32x4_t*)(xp) = wf[0];
+    *(u32x4_t*)(xp + 1024) = wf[1];
+    tr_product(cslot + C::TILE_BYTES, wf, acc);            // dV^T += dO^T W
   };
 
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
-  using I3 = std::integral_constant<int, 3>;
-  using I4 = std::integral_constant<int, 4>;
-  int j = j_first;
-  for (; j + 4 < nq; j += 5) {
-    iter(I0{}, j);
-    iter(I1{}, j + 1);
-    iter(I2{}, j + 2);
-    iter(I3{}, j + 3);
-    iter(I4{}, j + 4);
+  // ---- K role: dP of tile i (slot cslot) interleaved with dS of tile i-1 (slot pslot), then dK of tile i-1.
+  auto body_k = [&](int i, int cslot, int pslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc) LMK_INL {
+    const bool masked = PT + (i - 1) <= kt;                // tile i-1: own block or not yet visible
+    const int CST = pslot + 2 * C::TILE_BYTES + tile * 1024;
+    // y: subtrahend of dP, z: addend of dS  (byte offsets of 32-float arrays)
+    const int yoff = (masked ? CST + 512 : CST + 128) + 16 * h;
+    const int zoff = ((!masked && lm_lane) ? CST + 256 : C::CONST_OFF + 128) + 16 * h;
+    float4 y4[4], z4[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      y4[g] = *(const float4*)(smem + yoff + 32 * g);
+      z4[g] = *(const float4*)(smem + zoff + 32 * g);
+    }
+    const unsigned char* xp = smem + C::XCH_OFF + (par_prev * C::NKT + tile) * C::XCH_TILE + lane * 16;
+    u32x4_t wv[2] = {*(const u32x4_t*)(xp), *(const u32x4_t*)(xp + 1024)};
+    u32x4_t df[2];
+    float ds[16];
+    auto elementwise = [&](int r) LMK_INL {
+      const int g = r >> 2, e = r & 3;
+      const float ya = (e == 0) ? y4[g].x : (e == 1) ? y4[g].y : (e == 2) ? y4[g].z : y4[g].w;
+      const float za = (e == 0) ? z4[g].x : (e == 1) ? z4[g].y : (e == 2) ? z4[g].z : z4[g].w;
+      const uint32_t pk = wv[r >> 3][(r >> 1) & 3];
+      const float wr = (r & 1) ? unpack_hi<T>(pk) : unpack_lo<T>(pk);
+      ds[r] = __builtin_fmaf(wr, dpp[r] - ya, za);
+      if (r & 1) {
+        uint32_t pd = pack2<T>(ds[r - 1], ds[r]);
+        asm volatile("" : "+v"(pd));                       // pins this slice between its two MFMAs
+        df[r >> 3][(r >> 1) & 3] = pd;
+      }
+    };
+    zero16(dpn);
+    constexpr int PF = 2;
+    u32x4_t fr[C::KS + PF];
+#pragma unroll
+    for (int m = 0; m < PF; ++m) fr[m] = *(const u32x4_t*)(smem + cslot + C::TILE_BYTES + koff[m]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < C::KS; ++m) {
+      if (m + PF < C::KS) fr[m + PF] = *(const u32x4_t*)(smem + cslot + C::TILE_BYTES + koff[m + PF]);
+      dpn = mfma32<T>(fr[m], bf[m], dpn);
+#pragma unroll
+      for (int r = (m * 16) / C::KS; r < ((m + 1) * 16) / C::KS; ++r) elementwise(r);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    tr_product(pslot, df, acc);                            // dK^T += Q^T dS
+  };
+
+  // ---- prologue: tiles j_first .. +3 requested; the first two must have landed
+#pragma unroll
+  for (int t = 0; t < 4; ++t) request(t * C::BUF_BYTES, j_first + t);
+  if (tid < 64) ((float*)(smem + C::CONST_OFF))[tid] = (tid < 32) ? 1e30f : 0.f;
+  // this wave's stationary operand: K fragments (V role) or V fragments (K role), lane = key
+  {
+    const char* src = role_k ? (const char*)p.v + 2 * (b_ * p.vs_b + hh * p.vs_h)
+                             : (const char*)p.k + 2 * (b_ * p.ks_b + hh * p.ks_h);
+    const int64_t rs = role_k ? p.vs_r : p.ks_r;
+#pragma unroll
+    for (int ks = 0; ks < C::KS; ++ks) {
+      u32x4_t z = {0, 0, 0, 0};
+      bf[ks] = z;
+      if (active) bf[ks] = *(const u32x4_t*)(src + 2 * ((int64_t)krow * rs + 16 * ks + 8 * h));
+    }
+    // consume them here: the wait the compiler puts in front of this also covers the requests above,
+    // and no wait for these loads can then end up inside the loop, where it would drain the ring
+#pragma unroll
+    for (int ks = 0; ks < C::KS; ++ks) asm volatile("" : "+v"(bf[ks]));
   }
-  if (j < nq) iter(I0{}, j);
-  if (j + 1 < nq) iter(I1{}, j + 1);
-  if (j + 2 < nq) iter(I2{}, j + 2);
-  if (j + 3 < nq) iter(I3{}, j + 3);
-  wait_vmcnt<0>();                                         // nothing may still be writing LDS when the wave ends
 
-  if (active) {
-    const float scl = p.scale;
+  wait_tiles();
+  __syncthreads();
+
+  // Iteration i = j_first .. nq, one barrier each, in both roles.  V role: tiles i (W, dV) and i+1 (S).
+  // K role: tiles i (dP) and i-1 (dS, dK); it has nothing to finish in the first iteration and only
+  // finishes in the last.  The ring slot of tile i is a wave-uniform counter.
+  auto wrap = [](int x) LMK_INL { return x >= C::NBUF ? x - C::NBUF : x; };
+  auto store_acc = [&](const f32x16_t* acc, char* dst, int64_t rs, float scl) LMK_INL {
 #pragma unroll
     for (int dc = 0; dc < C::DC; ++dc)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        u32x2_t k2 = {pack2<T>(dkacc[dc][4 * g + 0] * scl, dkacc[dc][4 * g + 1] * scl),
-                      pack2<T>(dkacc[dc][4 * g + 2] * scl, dkacc[dc][4 * g + 3] * scl)};
-        u32x2_t v2 = {pack2<T>(dvacc[dc][4 * g + 0], dvacc[dc][4 * g + 1]),
-                      pack2<T>(dvacc[dc][4 * g + 2], dvacc[dc][4 * g + 3])};
-        *(u32x2_t*)(dkp + 2 * ((int64_t)krow * p.dks_r + 32 * dc + 8 * g + 4 * h)) = k2;
-        *(u32x2_t*)(dvp + 2 * ((int64_t)krow * p.dvs_r + 32 * dc + 8 * g + 4 * h)) = v2;
+        u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * scl, acc[dc][4 * g + 1] * scl),
+                      pack2<T>(acc[dc][4 * g + 2] * scl, acc[dc][4 * g + 3] * scl)};
+        *(u32x2_t*)(dst + 2 * ((int64_t)krow * rs + 32 * dc + 8 * g + 4 * h)) = o2;
       }
+  };
+  if (!role_k) {
+    f32x16_t acc[C::DC];                                   // dV^T: rows = d, lane = key
+#pragma unroll
+    for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
+    f32x16_t cur, nxt;                                      // S of tiles i and i+1
+    row_tile(0, cur);                                       // S of the first tile
+    int sc = 0;
+    auto step = [&](auto Mc, int i) LMK_INL {
+      request(wrap(sc + 4) * C::BUF_BYTES, i + 4);          // into the slot tile i-2 has left
+      body_v(Mc, i, sc * C::BUF_BYTES, wrap(sc + 1) * C::BUF_BYTES, (i - j_first) & 1, cur, nxt, acc);
+      cur = nxt;
+      wait_vmcnt<2 * C::PER_TILE_V>();                      // tile i+2 has landed (tiles i+3, i+4 may be in flight)
+      __syncthreads();
+      sc = wrap(sc + 1);
+    };
+    // own block and tiles that cannot see these keys yet come first, then every later tile sees all keys:
+    // two loops, so that each has one code path and the accumulators stay where they are
+    int i = j_first;
+    const int i_full = min(nq, max(j_first, kt - PT + 1));
+    for (; i < i_full; ++i) step(std::true_type{}, i);
+    for (; i < nq; ++i) step(std::false_type{}, i);
+    request(wrap(sc + 4) * C::BUF_BYTES, nq + 4);           // the K role finishes tile nq-1 in one more iteration
+    wait_vmcnt<2 * C::PER_TILE_V>();
+    __syncthreads();
+    wait_vmcnt<0>();                                       // nothing may still be writing LDS when the wave ends
+    if (active) store_acc(acc, (char*)p.dv + 2 * (b_ * p.dvs_b + hh * p.dvs_h), p.dvs_r, 1.f);
+  } else {
+    f32x16_t acc[C::DC];                                   // dK^T: rows = d, lane = key
+#pragma unroll
+    for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
+    f32x16_t prv, cur;                                      // dP of tiles i-1 and i
+    int sc = 0;
+    request(wrap(sc + 4) * C::BUF_BYTES, j_first + 4);
+    row_tile(C::TILE_BYTES, prv);                           // dP of the first tile
+    wait_vmcnt<2 * C::PER_TILE_K>();
+    __syncthreads();
+    sc = 1;
+    for (int i = j_first + 1; i <= nq; ++i) {
+      request(wrap(sc + 4) * C::BUF_BYTES, i + 4);
+      body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc);
+      prv = cur;
+      wait_vmcnt<2 * C::PER_TILE_K>();
+      __syncthreads();
+      sc = wrap(sc + 1);
+    }
+    wait_vmcnt<0>();
+    if (active) store_acc(acc, (char*)p.dk + 2 * (b_ * p.dks_b + hh * p.dks_h), p.dks_r, p.scale);
   }
 }
+
+#undef LMK_INL
 
 template <class T, int D>
 static int launch_dkdv32_t(const BwdParams& p, hipStream_t stream) {
