@@ -160,9 +160,9 @@ def main():
     t_dkdv = _time_launches(lambda: phase(4), n_k, 3)
     # algorithmic share of each kernel under the 5-product backward convention (S, dP, dQ | dK, dV)
     kernels = {
-        "lmk_fwd_kernel": (t_fwd, fwd_flops),
-        "lmk_bwd_dq_kernel": (t_dq, 1.5 * fwd_flops),
-        "lmk_bwd_dkdv_kernel": (t_dkdv, 1.0 * fwd_flops),
+        "lmk_fwd32_kernel": (t_fwd, fwd_flops),
+        "lmk_bwd_dq32_kernel": (t_dq, 1.5 * fwd_flops),
+        "lmk_bwd_dkdv32_kernel": (t_dkdv, 1.0 * fwd_flops),
     }
     dom = max(kernels, key=lambda n: kernels[n][0])
     t_dom, f_dom = kernels[dom]
@@ -179,8 +179,8 @@ def main():
                                "block=32, q,k,v ~ N(0,1)*0.5, dO ~ N(0,1), seed 0"},
         "frac_of_mfma_peak": value / PEAK_BF16_TFLOPS,
         "tokens_per_s": B * L / (ms_per_step * 1e-3),
-        "kernel_ms": {"lmk_fwd_kernel": t_fwd, "lmk_bwd_pre_kernel": t_pre, "lmk_bwd_dq_kernel": t_dq,
-                      "lmk_bwd_dkdv_kernel": t_dkdv, "event_ms_per_step": ms, "wall_ms_per_step": wall_ms},
+        "kernel_ms": {"lmk_fwd32_kernel": t_fwd, "lmk_bwd_pre_kernel": t_pre, "lmk_bwd_dq32_kernel": t_dq,
+                      "lmk_bwd_dkdv32_kernel": t_dkdv, "event_ms_per_step": ms, "wall_ms_per_step": wall_ms},
         "forward_only": {"TFLOPs": fwd_flops / (t_fwd * 1e-3) / 1e12, "frac": fwd_flops / (t_fwd * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
         "roofline": roofline,
     }

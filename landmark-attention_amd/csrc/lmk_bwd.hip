@@ -502,7 +502,7 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
     hipLaunchKernelGGL((lmk_bwd_pre_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
   }
-  if ((phases & 2) && BS == 32 && getenv("LMK_DQ_GENERIC") == nullptr) {
+  if ((phases & 2) && BS == 32) {
     if ((rc = launch_bwd_dq32(p, D, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream))) return rc;
   } else if (phases & 2) {
     using C = DqCfg<T, D, BS>;
@@ -515,7 +515,7 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
     hipLaunchKernelGGL(kern, dim3(p.n_qtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
   }
-  if ((phases & 4) && BS == 32 && getenv("LMK_DKDV_GENERIC") == nullptr) {
+  if ((phases & 4) && BS == 32) {
     return launch_bwd_dkdv32(p, D, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream);
   }
   if (phases & 4) {

@@ -280,7 +280,7 @@ static int launch_fwd_d(const FwdParams& p, int D, int BS, hipStream_t stream) {
 }
 
 int launch_fwd(const FwdParams& p, int D, int BS, int dtype, hipStream_t stream) {
-  if (BS == 32 && getenv("LMK_FWD_GENERIC") == nullptr) return launch_fwd32(p, D, dtype, stream);
+  if (BS == 32) return launch_fwd32(p, D, dtype, stream);
   if (dtype == LMK_DTYPE_BF16) return launch_fwd_d<bf16_t>(p, D, BS, stream);
   if (dtype == LMK_DTYPE_F16) return launch_fwd_d<f16_t>(p, D, BS, stream);
   return LMK_ERR_UNSUPPORTED;
