@@ -57,7 +57,8 @@ __device__ __forceinline__ void dq_wait_vmcnt() {          // s_waitcnt vmcnt(N)
 template <class T, int D>
 __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   using C = Dq32Cfg<T, D>;
-  extern __shared__ __align__(16) unsigned char smem[];
+  extern __shared__ __align__(16) unsigned char smem[];   // used through LDS byte addresses (it starts at 0)
+  (void)smem;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ql = lane & 31, h = lane >> 5;
@@ -168,7 +169,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
 #pragma unroll
       for (int pl = 0; pl < 3; ++pl) {
         const float* base = (pl == 0 ? p.stat_a : pl == 1 ? p.stat_n : p.stat_l) + ub;
-        const u32x4_t val = *(const u32x4_t*)(smem + fl_lds + pl * C::FL * 128);
+        const u32x4_t val = lds_ld128(fl_lds + pl * C::FL * 128);
         asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(fl_off), "v"(val), "s"(base) : "memory");
       }
     }
@@ -182,7 +183,14 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
     return x;
   };
   const int goff = C::GO_OFF + wave * C::BLK_BYTES;
-  const int gk0 = goff + koff0;                             // this wave's dO row fragments: gk0 ^ (32 ks)
+  // row-fragment addresses of a tile at LDS address 0 (K, V: the slot is added as an immediate) and
+  // of this wave's dO rows
+  int kx[C::KS], gx[C::KS];
+#pragma unroll
+  for (int ks = 0; ks < C::KS; ++ks) {
+    kx[ks] = koff0 ^ (ks << 5);
+    gx[ks] = goff + kx[ks];
+  }
   auto zero16 = [](f32x16_t& x) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) x[r] = 0.f;
@@ -191,12 +199,10 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   auto stage_x = [&](int slot_bytes, f32x16_t& s, f32x16_t& d) __attribute__((always_inline)) {
     zero16(s);
     zero16(d);
-    const int kb = fresh(koff0 + slot_bytes), gb = fresh(gk0);
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) {
-      const int ka = kb ^ (ks << 5);
-      s = mfma32<T>(*(const u32x4_t*)(smem + ka), qf[ks], s);
-      d = mfma32<T>(*(const u32x4_t*)(smem + ka + C::BLK_BYTES), *(const u32x4_t*)(smem + (gb ^ (ks << 5))), d);
+      s = mfma32<T>(lds_ld128(kx[ks] + slot_bytes), qf[ks], s);
+      d = mfma32<T>(lds_ld128(kx[ks] + slot_bytes + C::BLK_BYTES), lds_ld128(gx[ks]), d);
     }
   };
   auto zbase = [&](int slot_bytes, int* zb) __attribute__((always_inline)) {
@@ -209,8 +215,8 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   };
   auto ztr = [&](const int* zb, int n) __attribute__((always_inline)) {   // A operand of the n-th dQ^T MFMA: K^T, keys 16 j ..
     const int j = n / C::DC, dc = n % C::DC;
-    const u32x2_t a0 = lds_read_tr(smem + 16 * j * C::ROWB + zb[2 * dc]);
-    const u32x2_t a1 = lds_read_tr(smem + 16 * j * C::ROWB + zb[2 * dc + 1]);
+    const u32x2_t a0 = lds_ld_tr(16 * j * C::ROWB + zb[2 * dc]);
+    const u32x2_t a1 = lds_ld_tr(16 * j * C::ROWB + zb[2 * dc + 1]);
     const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
     return a;
   };
@@ -228,12 +234,11 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
     zero16(sn);
     zero16(dn);
     constexpr int NX = 2 * C::KS;
-    const int kb = fresh(koff0 + nslot), gb = fresh(gk0);
     u32x4_t fk[C::KS], fv[C::KS], fg[C::KS];
     auto frags = [&](int ks) __attribute__((always_inline)) {
-      fk[ks] = *(const u32x4_t*)(smem + (kb ^ (ks << 5)));
-      fv[ks] = *(const u32x4_t*)(smem + (kb ^ (ks << 5)) + C::BLK_BYTES);
-      fg[ks] = *(const u32x4_t*)(smem + (gb ^ (ks << 5)));
+      fk[ks] = lds_ld128(kx[ks] + nslot);
+      fv[ks] = lds_ld128(kx[ks] + nslot + C::BLK_BYTES);
+      fg[ks] = lds_ld128(gx[ks]);
     };
     frags(0);
     const float s_last = s[15];
@@ -276,10 +281,10 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
         const int ln = lane_now();
         if (ln < 32) {                                     // h == 0: lane = query
           const int bi = blk & (C::FL - 1);
-          unsigned char* sp = smem + C::STAT_OFF + wave * C::STAT_WAVE + bi * 128 + ln * 4;
-          *(float*)(sp + 0 * C::FL * 128) = mloc + fast_log2(den) - glog;
-          *(float*)(sp + 1 * C::FL * 128) = nD;
-          *(float*)(sp + 2 * C::FL * 128) = dslm;
+          const int sp = C::STAT_OFF + wave * C::STAT_WAVE + bi * 128 + ln * 4;
+          lds_st32(sp + 0 * C::FL * 128, mloc + fast_log2(den) - glog);
+          lds_st32(sp + 1 * C::FL * 128, nD);
+          lds_st32(sp + 2 * C::FL * 128, dslm);
         }
       } else {
 #pragma unroll

@@ -126,6 +126,20 @@ __device__ __forceinline__ u32x2_t lds_read_tr(const unsigned char* p) {
   return __builtin_bit_cast(u32x2_t, v);
 }
 
+// LDS access by byte address.  A kernel whose only LDS is its dynamic array sees that array at LDS
+// address 0 (the direct global->LDS loads rely on the same fact), so offsets into it are LDS
+// addresses.  Going through an integer keeps the compiler from adding the array's (zero) base to
+// every address with a vector instruction.
+typedef __attribute__((address_space(3))) u32x4_t* lds_u32x4_ptr;
+typedef __attribute__((address_space(3))) float* lds_f32_ptr;
+__device__ __forceinline__ u32x4_t lds_ld128(int addr) { return *(lds_u32x4_ptr)(uint32_t)addr; }
+__device__ __forceinline__ void lds_st128(int addr, u32x4_t v) { *(lds_u32x4_ptr)(uint32_t)addr = v; }
+__device__ __forceinline__ void lds_st32(int addr, float v) { *(lds_f32_ptr)(uint32_t)addr = v; }
+__device__ __forceinline__ u32x2_t lds_ld_tr(int addr) {
+  s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(uint32_t)addr);
+  return __builtin_bit_cast(u32x2_t, v);
+}
+
 // Transposed fragment of a row-major tile (A operand, rows = 32 head dims of chunk dc,
 // k = 16 tile rows of step j of the 32-row tile at LDS row base rb) in the row order of
 // the C layout: register pair 0 holds rows 16j + 4h + {0..3}, pair 1 rows 16j + 8 + 4h + {0..3}.
