@@ -142,17 +142,36 @@ __device__ __forceinline__ float contract(float dot, float sqrt_hd) {
   return round_to<T>(__fdiv_rn(round_to<T>(dot), sqrt_hd));
 }
 
-// wave-wide arg-best under (value desc, index asc); every lane gets the winner
+// wave-wide arg-best under (value desc, index asc); every lane gets the winner.  Inside a row of 16
+// lanes the exchange partners come from DPP (no LDS round trip); the four row results are then read
+// as scalars.
+template <int CTRL>
+__device__ __forceinline__ void best_step_dpp(float& v, int& i) {
+  const float ov = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+  const int oi = __builtin_amdgcn_update_dpp(0, i, CTRL, 0xf, 0xf, false);
+  if (ov > v || (ov == v && oi < i)) {
+    v = ov;
+    i = oi;
+  }
+}
 __device__ __forceinline__ void wave_best(float& v, int& i) {
+  best_step_dpp<0xB1>(v, i);                                      // quad_perm [1,0,3,2]
+  best_step_dpp<0x4E>(v, i);                                      // quad_perm [2,3,0,1]
+  best_step_dpp<0x141>(v, i);                                     // row_half_mirror
+  best_step_dpp<0x140>(v, i);                                     // row_mirror: every lane has its row's best
+  float bv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+  int bi = __builtin_amdgcn_readlane(i, 0);
 #pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) {
-    const float ov = __shfl_xor(v, m, 64);
-    const int oi = __shfl_xor(i, m, 64);
-    if (ov > v || (ov == v && oi < i)) {
-      v = ov;
-      i = oi;
+  for (int r = 1; r < 4; ++r) {
+    const float ov = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16 * r));
+    const int oi = __builtin_amdgcn_readlane(i, 16 * r);
+    if (ov > bv || (ov == bv && oi < bi)) {
+      bv = ov;
+      bi = oi;
     }
   }
+  v = bv;
+  i = bi;
 }
 
 constexpr int kSelSeg = 1024;   // landmarks handled per sweep of the contender list
@@ -288,6 +307,231 @@ __global__ __launch_bounds__(256) void lmk_select_kernel(RetrParams p) {
 }
 
 // ---------------------------------------------------------------------------
+// fused score + select for caches of at most kFusedMaxMems landmark blocks: the approximate scores
+// of 32 query rows never leave the CU
+// ---------------------------------------------------------------------------
+// A workgroup (4 waves) owns 32 consecutive query rows of one (batch, head).
+//   score   the waves split the landmarks; S = Q LK^T by MFMA with the landmark in the lane, so a
+//           register (= one query row) lands in 32 consecutive LDS words
+//   select  each wave takes 8 of the rows in turn; a lane holds the 16 scores m = 64 j + lane of the
+//           row in registers: bracket, k-th best lower end, exact re-evaluation of the contenders
+//           (written back over their approximate score), k best, ascending order
+// The bracket uses a cheap monotone over-/under-estimate of the rounding contract: round_T(x) / sqrt(hd)
+// is replaced by a multiplication by the rounded reciprocal, pushed outwards by 2^-21 relative (the
+// product is within 2^-22 of the correctly rounded quotient) before the final rounding.  That only
+// adds contenders; the ranking itself uses the exact contract.
+constexpr int kFusedMaxMems = 1024;
+constexpr int kFusedRows = 32;
+constexpr int kFusedWaves = 16;
+constexpr int kFusedList = 128;                                   // contender list per wave: flushed at 64, a ballot adds <= 64
+
+template <class T, int D>
+__global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrParams p) {
+  constexpr int KS = D / 16;
+  constexpr int NJ = kFusedMaxMems / 64;                          // scores per lane and row
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int NM = p.num_mems;
+  const int NMr = (NM + 63) & ~63;                                // columns read by the select phase
+  const int NMp = NMr + 32;                                       // row stride (words): the two half-waves of a store
+                                                                  // then hit different banks
+  float* sc = (float*)smem;                                       // [32][NMp]
+  float* q_lds = sc + kFusedRows * NMp;                           // [waves][D]
+  int* cand = (int*)(q_lds + kFusedWaves * D);                    // [waves][kFusedList]
+  unsigned char* q_raw = (unsigned char*)(cand + kFusedWaves * kFusedList);   // [32][D] in the model dtype
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ql = lane & 31, h = lane >> 5;
+  const int n_qt = (p.T + kFusedRows - 1) / kFusedRows;
+  const int bh = blockIdx.x / n_qt, t0 = (blockIdx.x % n_qt) * kFusedRows;
+  const int b = bh / p.H, hh = bh % p.H;
+  const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h);
+  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * NM * D);
+  const float* lkn = p.lk_norm + (int64_t)bh * NM;
+
+  // ---- the 32 query rows -> LDS (the select phase reads them from there)
+  for (int c = tid; c < kFusedRows * (D / 8); c += 64 * kFusedWaves) {
+    const int r = c / (D / 8), ch = c % (D / 8);
+    u32x4_t v = {0, 0, 0, 0};
+    if (t0 + r < p.T) v = *(const u32x4_t*)(qp + 2 * ((int64_t)(t0 + r) * p.qs_r + 8 * ch));
+    *(u32x4_t*)(q_raw + r * 2 * D + 16 * ch) = v;
+  }
+  // ---- score: A = query rows (lane -> row), B = landmark keys (lane -> landmark)
+  {
+    u32x4_t qf[KS];
+    const int qrow = t0 + ql;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4_t z = {0, 0, 0, 0};
+      qf[ks] = z;
+      if (qrow < p.T) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
+    }
+    for (int m0 = 32 * wave; m0 < NMr; m0 += 32 * kFusedWaves) {
+      const int m = m0 + ql;
+      u32x4_t kf[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        u32x4_t z = {0, 0, 0, 0};
+        kf[ks] = z;
+        if (m < NM) kf[ks] = *(const u32x4_t*)(lk + 2 * ((int64_t)m * D + 16 * ks + 8 * h));
+      }
+      f32x16_t s;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) s = mfma32<T>(qf[ks], kf[ks], s);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[(8 * (r >> 2) + 4 * h + (r & 3)) * NMp + m] = (m < NM) ? s[r] : -INFINITY;
+    }
+  }
+  __syncthreads();
+
+  // ---- select
+  float nrm[NJ];                                                  // |k_m| of this lane's landmarks
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const int m = 64 * j + lane;
+    nrm[j] = (m < NM) ? lkn[m] : 0.f;
+  }
+  const float sq = p.sqrt_hd, inv_sq = 1.0f / sq;
+  float* qrow_lds = q_lds + wave * D;
+  int* cnd = cand + wave * kFusedList;
+  const int nj = NMr >> 6;                                        // slices in use (wave-uniform)
+
+  // wave-wide arg-best of v[] under (value desc, index asc); the winner's slot is set to -inf
+  auto take_best = [&](float* v, float& bv_out, int& bi_out) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+      if (j < nj && v[j] > bv) {                                  // ascending j = ascending index: strict > keeps the first
+        bv = v[j];
+        bi = 64 * j + lane;
+      }
+    wave_best(bv, bi);
+    const int win = __builtin_amdgcn_readfirstlane(bi);
+    const bool owner = lane == (win & 63);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) v[j] = (owner && j == (win >> 6)) ? -INFINITY : v[j];
+    bv_out = bv;
+    bi_out = win;
+  };
+
+  for (int qi = wave; qi < kFusedRows; qi += kFusedWaves) {
+    const int t = t0 + qi;
+    if (t >= p.T) break;                                          // wave-uniform
+    const int64_t row = (int64_t)bh * p.T + t;
+    // q row -> fp32 in LDS (read back as a broadcast), and its norm
+    const unsigned char* qr = q_raw + qi * 2 * D;
+    float qn = 0.f;
+    for (int d = 2 * lane; d < D; d += 128) {
+      const uint32_t u = *(const uint32_t*)(qr + 2 * d);
+      const float x0 = unpack_lo<T>(u), x1 = unpack_hi<T>(u);
+      qrow_lds[d] = x0;
+      qrow_lds[d + 1] = x1;
+      qn += x0 * x0 + x1 * x1;
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) qn += __shfl_xor(qn, m, 64);
+    const float eps_q = sqrtf(qn) * 1.000001f * (1.0f / 16384.0f);
+
+    float* srow = sc + qi * NMp;
+    float lo[NJ], hi[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      lo[j] = -INFINITY;
+      hi[j] = -INFINITY;
+      if (j < nj) {
+        const float a = srow[64 * j + lane];
+        if (a > -INFINITY) {
+          const float e = eps_q * nrm[j];
+          const float cl = round_to<T>(a - e) * inv_sq, ch = round_to<T>(a + e) * inv_sq;
+          lo[j] = round_to<T>(cl - fabsf(cl) * 4.76837158203125e-7f);
+          hi[j] = round_to<T>(ch + fabsf(ch) * 4.76837158203125e-7f);
+        }
+      }
+    }
+    // tau = k-th best lower end
+    float tau = -INFINITY;
+    for (int j = 0; j < p.k; ++j) {
+      int bi;
+      take_best(lo, tau, bi);
+    }
+    // contenders: upper end reaches tau.  They are collected in a short list and evaluated exactly,
+    // one lane per contender, whenever the list holds a wave's worth (and at the end).
+    auto evaluate = [&](int count) {
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);                         // this wave's LDS writes (q row, list) are visible
+      for (int c0 = 0; c0 < count; c0 += 64) {
+        if (c0 + lane < count) {
+          const int m = cnd[c0 + lane];
+          const char* kr = lk + 2 * ((int64_t)m * D);
+          float acc = 0.f;
+#pragma unroll
+          for (int g = 0; g < D / 64; ++g) {                      // 8 loads in flight, then their 64 dependent fmas
+            u32x4_t kv[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) kv[i] = *(const u32x4_t*)(kr + 16 * (8 * g + i));
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              const u32x4_t kk = kv[i];
+              const float4 qa = *(const float4*)&qrow_lds[8 * (8 * g + i)];
+              const float4 qb = *(const float4*)&qrow_lds[8 * (8 * g + i) + 4];
+              acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
+              acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
+              acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
+              acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
+              acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
+              acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
+              acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
+              acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
+            }
+          }
+          srow[m] = contract<T>(acc, sq);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+    };
+    uint32_t is_c = 0;
+    int count = 0;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      if (j < nj) {
+        const bool c = hi[j] >= tau && hi[j] > -INFINITY;
+        const uint64_t bal = __ballot(c);
+        if (c) {
+          cnd[count + __popcll(bal & ((1ull << lane) - 1))] = 64 * j + lane;
+          is_c |= 1u << j;
+        }
+        count += __popcll(bal);
+        if (count >= 64) {                                        // wave-uniform
+          evaluate(count);
+          count = 0;
+        }
+      }
+    }
+    if (count > 0) evaluate(count);
+    // k best exact scores, then ascending order
+    float x[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) x[j] = (j < nj && ((is_c >> j) & 1)) ? srow[64 * j + lane] : -INFINITY;
+    int mine = -1;                                               // lane j keeps the j-th pick
+    for (int j = 0; j < p.k; ++j) {
+      float bv;
+      int bi;
+      take_best(x, bv, bi);
+      if (lane == j) mine = bi;
+    }
+    int rank = 0;
+    for (int j = 0; j < p.k; ++j) {
+      const int o = __shfl(mine, j, 64);
+      rank += (o < mine) ? 1 : 0;
+    }
+    if (lane < p.k) p.idx[row * p.k + rank] = (int64_t)mine;
+    __builtin_amdgcn_wave_barrier();                              // the next row reuses the q row and the list
+  }
+}
+
+// ---------------------------------------------------------------------------
 // gather + attend over the selected blocks, merged with the local-chunk attention
 // ---------------------------------------------------------------------------
 template <class T, int D, int BS>
@@ -419,6 +663,21 @@ static int launch_topk_t(const RetrParams& p, hipStream_t stream) {
   hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
   int rc;
   if ((rc = (int)hipGetLastError())) return rc;
+  if (p.num_mems <= kFusedMaxMems) {
+    const int NMr = (p.num_mems + 63) & ~63;
+    const int lds = (kFusedRows * (NMr + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
+    auto kern = lmk_topk_fused_kernel<T, D>;
+    static bool attr_done = false;
+    if (!attr_done) {
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (kFusedRows * (kFusedMaxMems + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D);
+      if (e != hipSuccess) return (int)e;
+      attr_done = true;
+    }
+    const int n_rt = (p.T + kFusedRows - 1) / kFusedRows;
+    hipLaunchKernelGGL(kern, dim3(p.B * p.H * n_rt), dim3(64 * kFusedWaves), lds, stream, p);
+    return (int)hipGetLastError();
+  }
   const int n_qt = (p.T + 127) / 128;
   hipLaunchKernelGGL((lmk_score_kernel<T, D>), dim3(p.B * p.H * n_qt), dim3(256), 0, stream, p);
   if ((rc = (int)hipGetLastError())) return rc;

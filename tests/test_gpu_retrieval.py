@@ -55,6 +55,24 @@ def test_topk_with_massive_ties():
     assert torch.equal(got.cpu(), want)
 
 
+@pytest.mark.parametrize("n_mems,top_k", [(700, 4), (1024, 64), (130, 7)])
+def test_topk_ties_inside_one_workgroup(n_mems, top_k):
+    # at most 1024 landmarks: scores stay on the CU; identical landmark keys make every block a
+    # contender, so the contender list is flushed several times, and a large top_k runs many rounds
+    from landmark_hip.retrieval import retrieve_topk
+    B, H, T, D, block = 1, 2, 40, 128, 32
+    S = n_mems * block
+    print(f"case ties n_mems{n_mems} k{top_k}", flush=True)
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=n_mems)
+    kc[:, :, block - 1::block] = kc[:, :, block - 1:block]
+    if n_mems == 1024:                                   # half tied, half distinct
+        kc[:, :, block - 1::2 * block] = (torch.randn(B, H, n_mems // 2, D) * 0.5).to(kc.dtype)
+    sc = oret.landmark_scores(q, kc, cos, sin, block, top_k)
+    want = oret.select_topk(sc, top_k)
+    got = retrieve_topk(q.cuda(), kc.cuda(), cos.cuda(), sin.cuda(), block, top_k)
+    assert torch.equal(got.cpu(), want)
+
+
 def test_fp16_indices_bit_exact():
     from landmark_hip.retrieval import retrieve_topk
     B, H, T, S, D, block, top_k = 1, 2, 24, 48 * 32, 128, 32, 4
