@@ -534,82 +534,133 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
 // ---------------------------------------------------------------------------
 // gather + attend over the selected blocks, merged with the local-chunk attention
 // ---------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float sum8(float d) {                  // sum over the 8 lanes of a key group (lane & 7)
+  d += dpp_f<0xB1>(d);                                            // quad_perm [1,0,3,2]
+  d += dpp_f<0x4E>(d);                                            // quad_perm [2,3,0,1]
+  d += dpp_f<0x141>(d);                                           // row_half_mirror
+  return d;
+}
+
+// One wave per query row.  Eight lanes share a key: lane j of the group holds head dims 8j..8j+7 and
+// 64+8j..64+8j+7, i.e. both partners of the rotary pair, so the rotation needs no exchange between
+// lanes; the eight key groups of the wave take keys g, g+8, .. of a block.  Rotation and scores are
+// evaluated in fp32 from the 16-bit cache and table values (the reference rounds the rotated key to
+// the model dtype first; the difference is far inside the 2e-2 bound of this step, and selection --
+// where bits matter -- does not go through here).
 template <class T, int D, int BS>
 __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   static_assert(D == 128, "lane mapping below assumes 16 chunks of 8 head dims per row");
-  constexpr int KPG = BS / 4;                                     // keys per 16-lane group per block
+  constexpr int KPG = BS / 8;                                     // keys per 8-lane group per block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int j = lane & 15, g = lane >> 4;                          // head-dim chunk, key group
+  const int j = lane & 7, g = lane >> 3;                           // head-dim chunk pair, key group
   const int64_t row = (int64_t)blockIdx.x * 4 + wave;             // (bh, t)
   const int64_t total = (int64_t)p.B * p.H * p.T;
   if (row >= total) return;
   const int bh = (int)(row / p.T), t = (int)(row % p.T);
   const int b = bh / p.H, hh = bh % p.H;
 
-  float qv[8];
-  {
-    const u32x4_t u = *(const u32x4_t*)((const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r) + 16 * j);
+  auto unpack8 = [](const u32x4_t u, float* o) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      qv[2 * i] = unpack_lo<T>(u[i]);
-      qv[2 * i + 1] = unpack_hi<T>(u[i]);
+      o[2 * i] = unpack_lo<T>(u[i]);
+      o[2 * i + 1] = unpack_hi<T>(u[i]);
     }
+  };
+  float qlo[8], qhi[8];
+  {
+    const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
+    unpack8(*(const u32x4_t*)(qp + 16 * j), qlo);
+    unpack8(*(const u32x4_t*)(qp + 128 + 16 * j), qhi);
   }
   const char* kc = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h);
   const char* vc = (const char*)p.vcache + 2 * (b * p.vcs_b + hh * p.vcs_h);
   const float c2 = p.scale_log2;
 
   float Mrun = -INFINITY, lrun = 0.f;
-  float acc[8];
+  float alo[8], ahi[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  for (int i = 0; i < 8; ++i) {
+    alo[i] = 0.f;
+    ahi[i] = 0.f;
+  }
 
-  for (int js = 0; js < p.k; ++js) {
-    const int blk = (int)p.idx[row * p.k + js];
-    const int64_t pos0 = (int64_t)js * BS + ((blk >= p.num_mems - p.k) ? BS : 0) + p.prefix_len;
+  // K/V of block js+1 are requested before block js is worked on: a wave keeps two blocks in flight
+  u32x4_t klo[KPG], khi[KPG], vlo[KPG], vhi[KPG], nklo[KPG], nkhi[KPG], nvlo[KPG], nvhi[KPG];
+  auto fetch = [&](int blk, u32x4_t* a, u32x4_t* bq, u32x4_t* c, u32x4_t* dq) {
     const int64_t key0 = (int64_t)blk * BS;
-    // this group's keys: kk = g + 4*i
-    u32x4_t kx[KPG], vx[KPG];
 #pragma unroll
     for (int i = 0; i < KPG; ++i) {
-      const int kk = g + 4 * i;
-      kx[i] = *(const u32x4_t*)(kc + 2 * ((key0 + kk) * p.kcs_r) + 16 * j);
-      vx[i] = *(const u32x4_t*)(vc + 2 * ((key0 + kk) * p.vcs_r) + 16 * j);
+      const int kk = g + 8 * i;                                   // this group's keys
+      const char* kr = kc + 2 * ((key0 + kk) * p.kcs_r) + 16 * j;
+      const char* vr = vc + 2 * ((key0 + kk) * p.vcs_r) + 16 * j;
+      a[i] = *(const u32x4_t*)(kr);
+      bq[i] = *(const u32x4_t*)(kr + 128);
+      c[i] = *(const u32x4_t*)(vr);
+      dq[i] = *(const u32x4_t*)(vr + 128);
+    }
+  };
+  int blk_next = (int)p.idx[row * p.k];
+  fetch(blk_next, nklo, nkhi, nvlo, nvhi);
+  for (int js = 0; js < p.k; ++js) {
+    const int blk = blk_next;
+    const int64_t pos0 = (int64_t)js * BS + ((blk >= p.num_mems - p.k) ? BS : 0) + p.prefix_len;
+#pragma unroll
+    for (int i = 0; i < KPG; ++i) {
+      klo[i] = nklo[i];
+      khi[i] = nkhi[i];
+      vlo[i] = nvlo[i];
+      vhi[i] = nvhi[i];
+    }
+    if (js + 1 < p.k) {
+      blk_next = (int)p.idx[row * p.k + js + 1];
+      fetch(blk_next, nklo, nkhi, nvlo, nvhi);
     }
     float sc[KPG];
 #pragma unroll
     for (int i = 0; i < KPG; ++i) {
-      const int kk = g + 4 * i;
-      const u32x4_t c = *(const u32x4_t*)((const char*)p.cos + 2 * ((pos0 + kk) * p.cs_r) + 16 * j);
-      const u32x4_t s = *(const u32x4_t*)((const char*)p.sin + 2 * ((pos0 + kk) * p.cs_r) + 16 * j);
-      const u32x4_t other = shfl_xor4(kx[i], 8);
-      float r[8];
-      rotate_chunk<T>(kx[i], other, c, s, j >= 8, r);
+      const int kk = g + 8 * i;
+      const char* cr = (const char*)p.cos + 2 * ((pos0 + kk) * p.cs_r) + 16 * j;
+      const char* sr = (const char*)p.sin + 2 * ((pos0 + kk) * p.cs_r) + 16 * j;
+      float kl[8], kh[8], cl[8], ch[8], sl[8], sh[8];
+      unpack8(klo[i], kl);
+      unpack8(khi[i], kh);
+      unpack8(*(const u32x4_t*)(cr), cl);
+      unpack8(*(const u32x4_t*)(cr + 128), ch);
+      unpack8(*(const u32x4_t*)(sr), sl);
+      unpack8(*(const u32x4_t*)(sr + 128), sh);
       float d = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) d = __builtin_fmaf(qv[e], r[e], d);
-      d += __shfl_xor(d, 1, 64);
-      d += __shfl_xor(d, 2, 64);
-      d += __shfl_xor(d, 4, 64);
-      d += __shfl_xor(d, 8, 64);
-      sc[i] = d * c2;                                             // log2 domain
+      for (int e = 0; e < 8; ++e) {
+        // rotate_half: the first half pairs with -x[d + D/2], the second with x[d - D/2]
+        const float rl = __builtin_fmaf(kl[e], cl[e], -kh[e] * sl[e]);
+        const float rh = __builtin_fmaf(kh[e], ch[e], kl[e] * sh[e]);
+        d = __builtin_fmaf(qlo[e], rl, d);
+        d = __builtin_fmaf(qhi[e], rh, d);
+      }
+      sc[i] = sum8(d) * c2;                                       // log2 domain
     }
-    // landmark = key BS-1 = group 3, i = KPG-1
-    const float t_lm = __shfl(sc[KPG - 1], 48, 64);
+    // landmark = key BS-1 = group 7, i = KPG-1
+    const float t_lm = __shfl(sc[KPG - 1], 56, 64);
     float mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < KPG; ++i)
-      if (!(i == KPG - 1 && g == 3)) mx = fmaxf(mx, sc[i]);
+      if (!(i == KPG - 1 && g == 7)) mx = fmaxf(mx, sc[i]);
+    mx = fmaxf(mx, dpp_f<0x128>(mx));                             // row_ror 8: the other key group of the row
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     float den = 0.f;
 #pragma unroll
     for (int i = 0; i < KPG; ++i) {
       float e = fast_exp2(sc[i] - mx);
-      if (i == KPG - 1 && g == 3) e = 0.f;
+      if (i == KPG - 1 && g == 7) e = 0.f;
       sc[i] = e;
       den += e;
     }
+    den += dpp_f<0x128>(den);
     den += __shfl_xor(den, 16, 64);
     den += __shfl_xor(den, 32, 64);
     const float Mnew = fmaxf(Mrun, t_lm);
@@ -619,21 +670,30 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     Mrun = Mnew;
     const float f = gate / den;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+    for (int e = 0; e < 8; ++e) {
+      alo[e] *= alpha;
+      ahi[e] *= alpha;
+    }
 #pragma unroll
     for (int i = 0; i < KPG; ++i) {
       const float w = round_to<T>(sc[i] * f);                     // weights enter PV in the model dtype
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        acc[2 * e] = __builtin_fmaf(w, unpack_lo<T>(vx[i][e]), acc[2 * e]);
-        acc[2 * e + 1] = __builtin_fmaf(w, unpack_hi<T>(vx[i][e]), acc[2 * e + 1]);
+        alo[2 * e] = __builtin_fmaf(w, unpack_lo<T>(vlo[i][e]), alo[2 * e]);
+        alo[2 * e + 1] = __builtin_fmaf(w, unpack_hi<T>(vlo[i][e]), alo[2 * e + 1]);
+        ahi[2 * e] = __builtin_fmaf(w, unpack_lo<T>(vhi[i][e]), ahi[2 * e]);
+        ahi[2 * e + 1] = __builtin_fmaf(w, unpack_hi<T>(vhi[i][e]), ahi[2 * e + 1]);
       }
     }
   }
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    acc[e] += __shfl_xor(acc[e], 16, 64);
-    acc[e] += __shfl_xor(acc[e], 32, 64);
+  for (int e = 0; e < 8; ++e) {                                   // sum over the eight key groups
+    alo[e] += dpp_f<0x128>(alo[e]);
+    ahi[e] += dpp_f<0x128>(ahi[e]);
+    alo[e] += __shfl_xor(alo[e], 16, 64);
+    ahi[e] += __shfl_xor(ahi[e], 16, 64);
+    alo[e] += __shfl_xor(alo[e], 32, 64);
+    ahi[e] += __shfl_xor(ahi[e], 32, 64);
   }
   // merge with the local chunk: out_loc (normalised), L_loc, M_loc (natural-log units)
   const float Ml = p.M_loc[row] * kLog2e, Ll = p.L_loc[row];
@@ -641,15 +701,19 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   const float wr = fast_exp2(Mrun - Mt), wl = fast_exp2(Ml - Mt) * Ll;
   const float inv = 1.0f / (lrun * wr + wl);
   if (g == 0) {
-    const u32x4_t ol = *(const u32x4_t*)((const char*)p.o_loc + 2 * (b * p.ols_b + hh * p.ols_h + (int64_t)t * p.ols_r) + 16 * j);
-    float o[8];
+    const char* olp = (const char*)p.o_loc + 2 * (b * p.ols_b + hh * p.ols_h + (int64_t)t * p.ols_r) + 16 * j;
+    char* outp = (char*)p.out + 2 * (b * p.outs_b + hh * p.outs_h + (int64_t)t * p.outs_r) + 16 * j;
+    float ol[8], o[8];
+    unpack8(*(const u32x4_t*)(olp), ol);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      o[2 * i] = (acc[2 * i] * wr + unpack_lo<T>(ol[i]) * wl) * inv;
-      o[2 * i + 1] = (acc[2 * i + 1] * wr + unpack_hi<T>(ol[i]) * wl) * inv;
-    }
+    for (int i = 0; i < 8; ++i) o[i] = (alo[i] * wr + ol[i] * wl) * inv;
     u32x4_t ov = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
-    *(u32x4_t*)((char*)p.out + 2 * (b * p.outs_b + hh * p.outs_h + (int64_t)t * p.outs_r) + 16 * j) = ov;
+    *(u32x4_t*)(outp) = ov;
+    unpack8(*(const u32x4_t*)(olp + 128), ol);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (ahi[i] * wr + ol[i] * wl) * inv;
+    u32x4_t ov2 = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
+    *(u32x4_t*)(outp + 128) = ov2;
   }
 }
 
