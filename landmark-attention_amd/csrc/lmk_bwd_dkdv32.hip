@@ -168,28 +168,24 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(*(const u32x4_t*)(smem + tile_bytes + koff[ks]), bf[ks], s);
   };
-  // second product of a tile: acc[dc] += (tile at tile_bytes)^T x (packed B operands: rows 0..15, 16..31)
-  auto tr_product = [&](int tile_bytes, const u32x4_t* pk, f32x16_t* acc) LMK_INL {
-    constexpr int NB = 2 * C::DC, PF = 2;
-    auto trfrag = [&](int n) LMK_INL {
-      const int j2 = n / C::DC, dc = n % C::DC;
-      const int base = tile_bytes + 16 * j2 * C::ROWB;
-      const u32x2_t a0 = lds_read_tr(smem + base + voff[dc][0]), a1 = lds_read_tr(smem + base + voff[dc][1]);
-      const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
-      return a;
-    };
-    u32x4_t tf[NB + PF];
+  // second product of a tile: acc[dc] += (tile at tile_bytes)^T x (packed B operands: rows 0..15, 16..31).
+  // Its A operands do not depend on anything computed in the iteration, so they are fetched from LDS
+  // during the first product (trfrag), one per MFMA slot, and are in registers when it starts.
+  constexpr int NB = 2 * C::DC;
+  auto trfrag = [&](int tile_bytes, int n) LMK_INL {
+    const int j2 = n / C::DC, dc = n % C::DC;
+    const int base = tile_bytes + 16 * j2 * C::ROWB;
+    const u32x2_t a0 = lds_read_tr(smem + base + voff[dc][0]), a1 = lds_read_tr(smem + base + voff[dc][1]);
+    const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
+    return a;
+  };
+  auto tr_product = [&](const u32x4_t* tf, const u32x4_t* pk, f32x16_t* acc) LMK_INL {
 #pragma unroll
-    for (int n = 0; n < PF; ++n) tf[n] = trfrag(n);
-#pragma unroll
-    for (int n = 0; n < NB; ++n) {
-      if (n + PF < NB) tf[n + PF] = trfrag(n + PF);
-      acc[n % C::DC] = mfma32<T>(tf[n], pk[n / C::DC], acc[n % C::DC]);
-    }
+    for (int n = 0; n < NB; ++n) acc[n % C::DC] = mfma32<T>(tf[n], pk[n / C::DC], acc[n % C::DC]);
   };
 
   // ---- V role: one query tile i.  S of tile i+1 (slot nslot) is interleaved with W of tile i.
-  auto body_v = [&](auto Mc, int i, int cslot, int nslot, int par, f32x16_t& s, f32x16_t& sn, f32x16_t* acc) LMK_INL {
+  auto body_v = [&](auto Mc, int i, int cslot, int nslot, int par, f32x16_t& s, f32x16_t& sn, f32x16_t* acc, auto sync) LMK_INL {
     constexpr bool MASKED = decltype(Mc)::value;
     const int CST = cslot + 2 * C::TILE_BYTES + tile * 1024;   // this key tile's terms: a, nD, dslm, mhat, delta
     const int krel = 32 * (kt - (PT + i)) + ql;            // key position relative to the query tile's first row
@@ -217,13 +213,15 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     };
     zero16(sn);
     constexpr int PF = 2;
-    u32x4_t fr[C::KS + PF];
+    u32x4_t fr[C::KS + PF], tf[NB];
 #pragma unroll
     for (int m = 0; m < PF; ++m) fr[m] = *(const u32x4_t*)(smem + nslot + koff[m]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < C::KS; ++m) {
       if (m + PF < C::KS) fr[m + PF] = *(const u32x4_t*)(smem + nslot + koff[m + PF]);
+#pragma unroll
+      for (int n = (m * NB) / C::KS; n < ((m + 1) * NB) / C::KS; ++n) tf[n] = trfrag(cslot + C::TILE_BYTES, n);
       sn = mfma32<T>(fr[m], bf[m], sn);
 #pragma unroll
       for (int r = (m * 16) / C::KS; r < ((m + 1) * 16) / C::KS; ++r) elementwise(r);
@@ -232,11 +230,12 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     unsigned char* xp = smem + C::XCH_OFF + (par * C::NKT + tile) * C::XCH_TILE + lane * 16;
     *(u32x4_t*)(xp) = wf[0];
     *(u32x4_t*)(xp + 1024) = wf[1];
-    tr_product(cslot + C::TILE_BYTES, wf, acc);            // dV^T += dO^T W
+    sync();                                                // the iteration's barrier: what follows needs no LDS
+    tr_product(tf, wf, acc);                               // dV^T += dO^T W
   };
 
   // ---- K role: dP of tile i (slot cslot) interleaved with dS of tile i-1 (slot pslot), then dK of tile i-1.
-  auto body_k = [&](int i, int cslot, int pslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc) LMK_INL {
+  auto body_k = [&](int i, int cslot, int pslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc, auto sync) LMK_INL {
     const bool masked = PT + (i - 1) <= kt;                // tile i-1: own block or not yet visible
     const int CST = pslot + 2 * C::TILE_BYTES + tile * 1024;
     // y: subtrahend of dP, z: addend of dS  (byte offsets of 32-float arrays)
@@ -267,19 +266,22 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     };
     zero16(dpn);
     constexpr int PF = 2;
-    u32x4_t fr[C::KS + PF];
+    u32x4_t fr[C::KS + PF], tf[NB];
 #pragma unroll
     for (int m = 0; m < PF; ++m) fr[m] = *(const u32x4_t*)(smem + cslot + C::TILE_BYTES + koff[m]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < C::KS; ++m) {
       if (m + PF < C::KS) fr[m + PF] = *(const u32x4_t*)(smem + cslot + C::TILE_BYTES + koff[m + PF]);
+#pragma unroll
+      for (int n = (m * NB) / C::KS; n < ((m + 1) * NB) / C::KS; ++n) tf[n] = trfrag(pslot, n);
       dpn = mfma32<T>(fr[m], bf[m], dpn);
 #pragma unroll
       for (int r = (m * 16) / C::KS; r < ((m + 1) * 16) / C::KS; ++r) elementwise(r);
       __builtin_amdgcn_sched_barrier(0);
     }
-    tr_product(pslot, df, acc);                            // dK^T += Q^T dS
+    sync();
+    tr_product(tf, df, acc);                               // dK^T += Q^T dS
   };
 
   // ---- prologue: tiles j_first .. +3 requested; the first two must have landed
@@ -329,10 +331,14 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     int sc = 0;
     auto step = [&](auto Mc, int i) LMK_INL {
       request(wrap(sc + 4) * C::BUF_BYTES, i + 4);          // into the slot tile i-2 has left
-      body_v(Mc, i, sc * C::BUF_BYTES, wrap(sc + 1) * C::BUF_BYTES, (i - j_first) & 1, cur, nxt, acc);
+      // the barrier sits between the two products: the second one has its operands in registers, so
+      // its MFMAs run while the workgroup's stragglers arrive and the next tile's operands are fetched
+      auto sync = [&]() LMK_INL {
+        wait_vmcnt<2 * C::PER_TILE_V>();                    // tile i+2 has landed (tiles i+3, i+4 may be in flight)
+        __syncthreads();
+      };
+      body_v(Mc, i, sc * C::BUF_BYTES, wrap(sc + 1) * C::BUF_BYTES, (i - j_first) & 1, cur, nxt, acc, sync);
       cur = nxt;
-      wait_vmcnt<2 * C::PER_TILE_V>();                      // tile i+2 has landed (tiles i+3, i+4 may be in flight)
-      __syncthreads();
       sc = wrap(sc + 1);
     };
     // own block and tiles that cannot see these keys yet come first, then every later tile sees all keys:
@@ -359,10 +365,12 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     sc = 1;
     for (int i = j_first + 1; i <= nq; ++i) {
       request(wrap(sc + 4) * C::BUF_BYTES, i + 4);
-      body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc);
+      auto sync = [&]() LMK_INL {
+        wait_vmcnt<2 * C::PER_TILE_K>();
+        __syncthreads();
+      };
+      body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc, sync);
       prv = cur;
-      wait_vmcnt<2 * C::PER_TILE_K>();
-      __syncthreads();
       sc = wrap(sc + 1);
     }
     wait_vmcnt<0>();
