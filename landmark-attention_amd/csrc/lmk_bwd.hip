@@ -496,7 +496,8 @@ static int set_lds(K kern, int bytes) {
 template <class T, int D, int BS>
 static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
   int rc;
-  if (phases & 1) {
+  // block 32: the dQ kernel computes delta and mhat itself, so the separate pass only runs when asked for alone
+  if ((phases & 1) && !(BS == 32 && (phases & 2))) {
     constexpr int RPW = 256 / (D / 8);
     const int64_t rows = (int64_t)p.B * p.H * p.Lq;
     hipLaunchKernelGGL((lmk_bwd_pre_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);

@@ -99,8 +99,20 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
     qf[ks] = z;
     if (rowok) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
   }
-  const float mhat = rowok ? p.mhat[(int64_t)bh * p.Lq + qrow] : 0.f;
-  const float delta = rowok ? p.delta[(int64_t)bh * p.Lq + qrow] : 0.f;
+  // delta = rowsum(O * dO) and mhat = M log2(e) + log2(L) of this lane's query row are computed here,
+  // after the prologue (dO comes from LDS), and left in the workspace for the dK/dV kernel
+  // (`_bwd_preprocess`, llama/ltriton/flash_landmark_attention.py:125-149)
+  float mhat = 0.f, delta = 0.f;
+  u32x4_t of[C::KS];                                        // this lane's part of its O row
+  {
+    const char* op = (const char*)p.o + 2 * (b_ * p.os_b + hh * p.os_h);
+#pragma unroll
+    for (int ks = 0; ks < C::KS; ++ks) {
+      u32x4_t z = {0, 0, 0, 0};
+      of[ks] = z;
+      if (rowok) of[ks] = *(const u32x4_t*)(op + 2 * ((int64_t)qrow * p.os_r + 16 * ks + 8 * h));
+    }
+  }
 
   // row fragment ks of a tile sits at tile_off(ql, 2 ks + h) = tile_off(ql, h) ^ (32 ks): the swizzle
   // is an XOR on the 16-byte chunk index and 2 ks only touches bits the row term leaves zero
@@ -340,6 +352,26 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   for (int t = 0; t < C::NBUF - 1; ++t) request(t * C::BUF_BYTES, t);
   dq_wait_vmcnt<C::PER_TILE>();
   __syncthreads();
+  {
+    float dsum = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < C::KS; ++ks) {
+      const u32x4_t g4 = lds_ld128(gx[ks]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        dsum += unpack_lo<T>(of[ks][i]) * unpack_lo<T>(g4[i]) + unpack_hi<T>(of[ks][i]) * unpack_hi<T>(g4[i]);
+    }
+    delta = pair_sum(dsum);
+    if (rowok) {
+      const int64_t r = (int64_t)bh * p.Lq + qrow;
+      mhat = p.M[r] * kLog2e + fast_log2(p.L[r]);
+      if (h == 0) {
+        p.delta[r] = delta;
+        p.mhat[r] = mhat;
+      }
+    }
+    asm volatile("" : "+v"(mhat), "+v"(delta));             // their loads are waited for here, not in the loop
+  }
 
   f32x16_t sA, dA, sB, dB;                                  // S^T, dP^T of the even / odd blocks
   zero16(sB);
