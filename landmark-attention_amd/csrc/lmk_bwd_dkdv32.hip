@@ -140,19 +140,36 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
              : (arr == 3) ? p.mhat + head_row : p.delta + head_row;
     st_src += 4 * part;
   }
-  auto request = [&](int slot_bytes, int j) LMK_INL {      // this wave's share of query tile j -> ring slot
-    const int jj = min(j, nq - 1);                         // past the end: re-read the last tile (never used)
+  // Requests go out in tile order (j_first, j_first+1, ..), so the source position is a running
+  // offset: one vector add per request instead of 64-bit scalar multiplies per iteration.  Past the
+  // last tile it stops advancing and the last tile is re-read (never used).
+  int j_req = j_first;                                     // tile the next request fetches
+  const uint32_t q_step = (uint32_t)(2 * 32 * p.qs_r), g_step = (uint32_t)(2 * 32 * p.dos_r);
+#pragma unroll
+  for (int d = 0; d < C::NDMA; ++d) {
+    q_vo[d] += (uint32_t)j_first * q_step;
+    g_vo[d] += (uint32_t)j_first * g_step;
+  }
+  st_src += 32 * (int64_t)j_first;
+  auto request = [&](int slot_bytes) LMK_INL {             // this wave's share of query tile j_req -> ring slot
     if (role_k) {
-      const char* qt = qp + 2 * ((int64_t)jj * 32 * p.qs_r);
-      const char* gt = gp + 2 * ((int64_t)jj * 32 * p.dos_r);
 #pragma unroll
       for (int d = 0; d < C::NDMA; ++d) {
-        dma16_s(qt, q_vo[d], slot_bytes + (tile * C::NDMA + d) * 1024);
-        dma16_s(gt, g_vo[d], slot_bytes + C::TILE_BYTES + (tile * C::NDMA + d) * 1024);
+        dma16_s(qp, q_vo[d], slot_bytes + (tile * C::NDMA + d) * 1024);
+        dma16_s(gp, g_vo[d], slot_bytes + C::TILE_BYTES + (tile * C::NDMA + d) * 1024);
       }
     } else {
-      dma16_v(st_src + 32 * jj, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
+      dma16_v(st_src, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
     }
+    const bool more = j_req < nq - 1;                      // wave-uniform
+    const uint32_t qs = more ? q_step : 0u, gs = more ? g_step : 0u;
+#pragma unroll
+    for (int d = 0; d < C::NDMA; ++d) {
+      q_vo[d] += qs;
+      g_vo[d] += gs;
+    }
+    st_src += more ? 32 : 0;
+    j_req += more ? 1 : 0;
   };
   auto wait_tiles = [&]() LMK_INL {                        // all but this wave's two newest tiles have landed
     if (role_k) wait_vmcnt<2 * C::PER_TILE_K>();
@@ -286,7 +303,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 
   // ---- prologue: tiles j_first .. +3 requested; the first two must have landed
 #pragma unroll
-  for (int t = 0; t < 4; ++t) request(t * C::BUF_BYTES, j_first + t);
+  for (int t = 0; t < 4; ++t) request(t * C::BUF_BYTES);
   if (tid < 64) ((float*)(smem + C::CONST_OFF))[tid] = (tid < 32) ? 1e30f : 0.f;
   // this wave's stationary operand: K fragments (V role) or V fragments (K role), lane = key
   {
@@ -330,7 +347,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     row_tile(0, cur);                                       // S of the first tile
     int sc = 0;
     auto step = [&](auto Mc, int i) LMK_INL {
-      request(wrap(sc + 4) * C::BUF_BYTES, i + 4);          // into the slot tile i-2 has left
+      request(wrap(sc + 4) * C::BUF_BYTES);                 // tile i+4, into the slot tile i-2 has left
       // the barrier sits between the two products: the second one has its operands in registers, so
       // its MFMAs run while the workgroup's stragglers arrive and the next tile's operands are fetched
       auto sync = [&]() LMK_INL {
@@ -347,7 +364,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     const int i_full = min(nq, max(j_first, kt - PT + 1));
     for (; i < i_full; ++i) step(std::true_type{}, i);
     for (; i < nq; ++i) step(std::false_type{}, i);
-    request(wrap(sc + 4) * C::BUF_BYTES, nq + 4);           // the K role finishes tile nq-1 in one more iteration
+    request(wrap(sc + 4) * C::BUF_BYTES);                   // the K role finishes tile nq-1 in one more iteration
     wait_vmcnt<2 * C::PER_TILE_V>();
     __syncthreads();
     wait_vmcnt<0>();                                       // nothing may still be writing LDS when the wave ends
@@ -358,13 +375,13 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
     f32x16_t prv, cur;                                      // dP of tiles i-1 and i
     int sc = 0;
-    request(wrap(sc + 4) * C::BUF_BYTES, j_first + 4);
+    request(wrap(sc + 4) * C::BUF_BYTES);
     row_tile(C::TILE_BYTES, prv);                           // dP of the first tile
     wait_vmcnt<2 * C::PER_TILE_K>();
     __syncthreads();
     sc = 1;
     for (int i = j_first + 1; i <= nq; ++i) {
-      request(wrap(sc + 4) * C::BUF_BYTES, i + 4);
+      request(wrap(sc + 4) * C::BUF_BYTES);
       auto sync = [&]() LMK_INL {
         wait_vmcnt<2 * C::PER_TILE_K>();
         __syncthreads();
