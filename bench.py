@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A step is one forward + backward of fused landmark attention at BASELINE config 2
+A step is one forward + backward of fused landmark attention at benchmark config 2
 (B=2, H=32, L=2048, D=128, block 32, bf16, synthetic N(0,1)*0.5 inputs, dO ~ N(0,1)) through
 the autograd Function, inputs resident in HBM.  Prints ONE JSON line: the headline metric in
 TFLOP/s (conventional causal count: fwd = 4*B*H*L*L*D/2, bwd = 2.5*fwd), the roofline of the
@@ -70,7 +70,7 @@ def cpu_baseline(sample_heads=4):
 
 
 def retrieval_bench(n=20, warm=3):
-    """BASELINE config 4: retrieval + gather + attend; algorithmic bytes 547.6 MB per step."""
+    """benchmark config 4: retrieval + gather + attend; algorithmic bytes 547.6 MB per step."""
     import torch
     from landmark_hip.retrieval import gather_attend, retrieve_topk
     dev = torch.device("cuda:0")
@@ -189,7 +189,7 @@ def main():
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "BASELINE config 2: fused_landmark_attention forward+backward, B=2 H=32 L=2048 D=128 "
+        "config": {"workload": "benchmark config 2: fused_landmark_attention forward+backward, B=2 H=32 L=2048 D=128 "
                                "block=32, q,k,v ~ N(0,1)*0.5, dO ~ N(0,1), seed 0"},
         "frac_of_mfma_peak": value / PEAK_BF16_TFLOPS,
         "tokens_per_s": B * L / (ms_per_step * 1e-3),

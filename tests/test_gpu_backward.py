@@ -105,7 +105,7 @@ def test_backward_deterministic_bitwise():
 
 
 def test_baseline_config2_full_size():
-    # BASELINE config 2: B2 H32 L2048 D128 block 32, dO ~ N(0,1)
+    # benchmark config 2: B2 H32 L2048 D128 block 32, dO ~ N(0,1)
     B, H, L, D, block = 2, 32, 2048, 128, 32
     q, k, v = make_qkv(B, H, L, L, D, seed=0)
     do = torch.randn(B, H, L, D, generator=torch.Generator().manual_seed(1)).bfloat16()

@@ -111,7 +111,7 @@ def test_deterministic_bitwise():
 
 
 def test_baseline_config1_full_size():
-    # BASELINE config 1: B2 H32 L2048 D128 block 32
+    # benchmark config 1: B2 H32 L2048 D128 block 32
     B, H, L, D, block = 2, 32, 2048, 128, 32
     q, k, v = make_qkv(B, H, L, L, D, seed=0)
     out = _run(q, k, v, block).float().cpu()

@@ -103,7 +103,7 @@ def test_gather_attend_matches_oracle(B, H, T, S, block, top_k):
 
 
 def test_baseline_config4_full_size():
-    # BASELINE config 4: H32 D128, 32768 cached tokens = 1024 blocks of 32, 256 queries, top-4
+    # benchmark config 4: H32 D128, 32768 cached tokens = 1024 blocks of 32, 256 queries, top-4
     from landmark_hip.retrieval import retrieve_and_attend
     B, H, T, S, D, block, top_k = 1, 32, 256, 32768, 128, 32, 4
     q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=0)

@@ -32,7 +32,7 @@ def test_fixed_stride_with_exactly_as_many_buckets_as_blocks():
 
 
 def test_lm_benchmark_flavour_equals_closed_form():
-    # BASELINE config 0 in miniature: landmark after every `mem_freq` tokens.
+    # benchmark config 0 in miniature: landmark after every `mem_freq` tokens.
     B, H, T, d, block = 2, 2, 40, 8, 5
     q, k, v = _rand(B, H, T, d, seed=7), _rand(B, H, T, d, seed=8), _rand(B, H, T, d, seed=9)
     is_mem = (torch.arange(T) % block == block - 1)[None].expand(B, T)

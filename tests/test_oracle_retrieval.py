@@ -49,7 +49,7 @@ def test_geometry_hand_worked():
     g = retrieval.retrieval_geometry(40, 4, 3)
     assert (g["num_mems"], g["k"], g["prefix_len"], g["incomplete_len"]) == (10, 3, 24, 0)
     assert g["mem_pos"].tolist() == [27] * 7 + [31, 35, 39]          # newest three keep their true positions
-    # BASELINE config 4 numbers
+    # benchmark config 4 numbers
     g = retrieval.retrieval_geometry(32768, 32, 4)
     assert g["prefix_len"] == 32608
     assert g["mem_pos"][:1020].unique().tolist() == [32639]
