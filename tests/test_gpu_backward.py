@@ -32,6 +32,10 @@ CASES = [
     (1, 8, 384, 384, 128, 32, torch.bfloat16),
     (1, 2, 128, 256, 128, 32, torch.bfloat16),     # history prefix
     (1, 2, 96, 160, 128, 32, torch.bfloat16),      # ragged workgroup tails
+    (1, 2, 64, 96, 128, 32, torch.bfloat16),       # odd history (1 block)
+    (1, 2, 160, 256, 128, 32, torch.bfloat16),     # odd history (3 blocks), 5 query blocks
+    (1, 2, 544, 544, 128, 32, torch.bfloat16),     # 17 blocks: the LDS rings wrap at every phase
+    (1, 2, 544, 544, 64, 32, torch.float16),
     (1, 2, 256, 256, 128, 64, torch.bfloat16),
     (1, 2, 128, 320, 128, 64, torch.bfloat16),
     (1, 2, 512, 512, 128, 128, torch.bfloat16),

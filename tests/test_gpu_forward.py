@@ -35,6 +35,8 @@ CASES = [
     (1, 8, 384, 384, 128, 32, torch.bfloat16),    # XCD-aware mapping, 3 query tiles
     (1, 2, 128, 256, 128, 32, torch.bfloat16),    # history prefix of 4 blocks
     (1, 2, 100, 100, 128, 32, torch.bfloat16),    # partial last block (forward only)
+    (1, 2, 160, 256, 128, 32, torch.bfloat16),    # odd history (3 blocks)
+    (1, 2, 544, 544, 128, 32, torch.bfloat16),    # 17 blocks: the LDS ring wraps at every phase
     (1, 2, 40, 104, 128, 32, torch.bfloat16),     # partial + history
     (1, 2, 256, 256, 128, 64, torch.bfloat16),
     (1, 2, 256, 384, 128, 64, torch.bfloat16),
