@@ -248,6 +248,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     *(u32x4_t*)(xp) = wf[0];
     *(u32x4_t*)(xp + 1024) = wf[1];
     sync();                                                // the iteration's barrier: what follows needs no LDS
+    __builtin_amdgcn_sched_barrier(0);                     // keeps the MFMAs below behind the barrier
     tr_product(tf, wf, acc);                               // dV^T += dO^T W
   };
 
@@ -298,6 +299,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       __builtin_amdgcn_sched_barrier(0);
     }
     sync();
+    __builtin_amdgcn_sched_barrier(0);
     tr_product(tf, df, acc);                               // dK^T += Q^T dS
   };
 
