@@ -34,7 +34,7 @@ extern "C" {
 #define LMK_ERR_PARTIAL (-6)     /* backward needs Lq and Lk to be whole blocks */
 #define LMK_ERR_SCALE (-7)       /* softmax scale must be finite and > 0 */
 #define LMK_ERR_WORKSPACE (-8)   /* workspace too small */
-#define LMK_ERR_CACHE (-9)       /* cached length is not a positive whole number of blocks */
+#define LMK_ERR_CACHE (-9)       /* cache holds no complete block (or, for lmk_local_window, no tail) */
 #define LMK_ERR_TOPK (-10)       /* top_k outside 1..64 */
 #define LMK_ERR_TABLE (-11)      /* rotary tables hold fewer positions than the cache */
 
@@ -106,7 +106,10 @@ int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
  * (:424-430); a block is mem_freq+1 tokens whose last token is the landmark; queries arrive
  * rotated; cos/sin are (n_pos, D) tables in the model dtype with the half-split layout of
  * LlamaRotaryEmbedding (:95-124) and `table_stride_row` elements between rows.
- * S must be a positive multiple of block (no incomplete cached block). */
+ * The cache must hold at least one complete block.  When it ends in an incomplete block
+ * (S % block != 0, the state between two landmarks while decoding, :321-324) retrieval works on
+ * the S - S % block tokens of the complete blocks, and the tail joins the local window of the
+ * attend step (:329-342; see lmk_local_window). */
 
 /* Bytes of device workspace lmk_retrieve_topk needs: rotated landmark keys and their norms,
  * plus two fp32 score planes of B*H*T*(S/block). */
@@ -132,6 +135,22 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
                       const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
                       const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, const lmk_tensor4* out, int B,
                       int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, void* stream);
+
+/* Local window of the attend step when the cache ends in an incomplete block of
+ * inc = S % block tokens (llama_mem.py:329-342; needs inc > 0 and T + inc <= block, the
+ * reference's assert at :330).  Writes, each (B,H,inc+T,D):
+ *   k_win = [tail keys rotated at positions S-inc .. S-1 (:337-338) ; k_loc]   (:339)
+ *   v_win = [tail values ; v_loc]                                               (:340)
+ *   q_win = [inc zero rows ; q]
+ * lmk_attn_fwd on (q_win, k_win, v_win) with Lq = Lk = inc + T and n_prefix = 0 then holds, in
+ * its last T rows (o, L, M), the attention of the new tokens over the window: the o_loc, L_loc,
+ * M_loc that lmk_gather_attend takes.  Replaces the torch.cat / apply_rotary_pos_emb calls of
+ * :337-340; the mask rows :331-335 give the tail no landmark and put it in every query's last
+ * section, which is what the forward kernel's own block does with rows in front of the queries. */
+int lmk_local_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,
+                     const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
+                     int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win, const lmk_tensor4* k_win,
+                     const lmk_tensor4* v_win, int B, int H, int T, int S, int D, int block, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

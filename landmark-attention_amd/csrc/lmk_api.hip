@@ -48,7 +48,7 @@ int check_retrieval(int B, int H, int T, int S, int D, int block, int top_k, int
   if (!(D == 64 || D == 128)) return LMK_ERR_UNSUPPORTED;
   if (block < 2 || block > 4096) return LMK_ERR_UNSUPPORTED;
   if (!(dtype == LMK_DTYPE_BF16 || dtype == LMK_DTYPE_F16)) return LMK_ERR_UNSUPPORTED;
-  if (S < block || S % block != 0) return LMK_ERR_CACHE;
+  if (S < block) return LMK_ERR_CACHE;          // at least one complete block; a shorter tail behind it is fine
   if (top_k < 1 || top_k > 64) return LMK_ERR_TOPK;
   if (n_pos < S) return LMK_ERR_TABLE;
   return LMK_OK;
@@ -56,9 +56,9 @@ int check_retrieval(int B, int H, int T, int S, int D, int block, int top_k, int
 
 void fill_retr_common(lmk::RetrParams& p, int B, int H, int T, int S, int D, int block, int top_k) {
   p.B = B; p.H = H; p.T = T; p.S = S; p.block = block;
-  p.num_mems = S / block;
+  p.num_mems = S / block;                         // complete blocks; the S % block newest tokens are the tail
   p.k = top_k < p.num_mems ? top_k : p.num_mems;
-  p.prefix_len = (int64_t)S - (int64_t)(p.k + 1) * block;
+  p.prefix_len = (int64_t)p.num_mems * block - (int64_t)(p.k + 1) * block;   // llama_mem.py:361 with full_len
   p.sqrt_hd = (float)std::sqrt((double)D);
 }
 
@@ -77,7 +77,7 @@ const char* lmk_strerror(int code) {
     case LMK_ERR_PARTIAL: return "backward supported only for full blocks";
     case LMK_ERR_SCALE: return "softmax scale must be finite and > 0";
     case LMK_ERR_WORKSPACE: return "workspace too small";
-    case LMK_ERR_CACHE: return "cache must hold at least one whole block and no incomplete block";
+    case LMK_ERR_CACHE: return "cache must hold at least one whole block";
     case LMK_ERR_TOPK: return "top_k must be in 1..64";
     case LMK_ERR_TABLE: return "rotary tables shorter than the cached length";
     default: break;
@@ -225,6 +225,39 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
   p.cs_r = table_stride_row;
   p.scale_log2 = sm_scale * 1.4426950408889634f;
   return lmk::launch_gather_attend(p, D, block, dtype, (hipStream_t)stream);
+}
+
+int lmk_local_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,
+                     const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
+                     int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win, const lmk_tensor4* k_win,
+                     const lmk_tensor4* v_win, int B, int H, int T, int S, int D, int block, int dtype, void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache)) || (rc = check_tensor(vcache)) ||
+      (rc = check_tensor(k_loc)) || (rc = check_tensor(v_loc)) || (rc = check_tensor(q_win)) ||
+      (rc = check_tensor(k_win)) || (rc = check_tensor(v_win)))
+    return rc;
+  if (cos_table == nullptr || sin_table == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
+  if ((rc = check_retrieval(B, H, T, S, D, block, 1, dtype, n_pos))) return rc;
+  const int inc = S % block;
+  if (inc == 0) return LMK_ERR_CACHE;             // no tail: the new chunk alone is the window
+  if (T + inc > block) return LMK_ERR_SHAPE;      // llama_mem.py:330
+  lmk::WindowParams p = {};
+  p.q = q->ptr; p.kcache = kcache->ptr; p.vcache = vcache->ptr; p.k_loc = k_loc->ptr; p.v_loc = v_loc->ptr;
+  p.cos = cos_table; p.sin = sin_table;
+  p.q_win = q_win->ptr; p.k_win = k_win->ptr; p.v_win = v_win->ptr;
+  p.B = B; p.H = H; p.T = T; p.inc = inc;
+  p.full_len = (int64_t)S - inc;
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
+  p.vcs_b = vcache->stride_b; p.vcs_h = vcache->stride_h; p.vcs_r = vcache->stride_row;
+  p.kls_b = k_loc->stride_b; p.kls_h = k_loc->stride_h; p.kls_r = k_loc->stride_row;
+  p.vls_b = v_loc->stride_b; p.vls_h = v_loc->stride_h; p.vls_r = v_loc->stride_row;
+  p.qws_b = q_win->stride_b; p.qws_h = q_win->stride_h; p.qws_r = q_win->stride_row;
+  p.kws_b = k_win->stride_b; p.kws_h = k_win->stride_h; p.kws_r = k_win->stride_row;
+  p.vws_b = v_win->stride_b; p.vws_h = v_win->stride_h; p.vws_r = v_win->stride_row;
+  p.cs_r = table_stride_row;
+  return lmk::launch_local_window(p, D, dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

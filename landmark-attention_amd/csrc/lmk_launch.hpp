@@ -58,7 +58,18 @@ struct RetrParams {
   float sqrt_hd, scale_log2;
 };
 
+// local window of the attend step when the cache ends in an incomplete block of `inc` tokens
+struct WindowParams {
+  const void *q, *kcache, *vcache, *k_loc, *v_loc, *cos, *sin;
+  void *q_win, *k_win, *v_win;                    // (B, H, inc + T, D) each
+  int B, H, T, inc;
+  int64_t full_len;                               // first cached row of the tail = its rotary position
+  int64_t qs_b, qs_h, qs_r, kcs_b, kcs_h, kcs_r, vcs_b, vcs_h, vcs_r, kls_b, kls_h, kls_r, vls_b, vls_h, vls_r;
+  int64_t qws_b, qws_h, qws_r, kws_b, kws_h, kws_r, vws_b, vws_h, vws_r, cs_r;
+};
+
 int launch_retrieve_topk(const RetrParams& p, int D, int dtype, hipStream_t stream);
+int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t stream);
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream);
 
 }  // namespace lmk

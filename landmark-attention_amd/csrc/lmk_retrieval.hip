@@ -771,6 +771,66 @@ static int launch_gather_t(const RetrParams& p, int BS, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// local window: [cached tail | new chunk] when the cache ends in an incomplete block
+// (llama_mem.py:321-342).  One 16-byte chunk per thread:
+//   k_win = [rot(tail keys, positions full_len ..) ; k_loc]     (:337-339)
+//   v_win = [tail values ; v_loc]                                (:340)
+//   q_win = [zero rows ; q]   -- rows in front of the queries so that the fused forward kernel,
+//           run square on the window, yields the new tokens' attention in its last T rows
+// ---------------------------------------------------------------------------
+template <class T, int D>
+__global__ __launch_bounds__(256) void lmk_local_window_kernel(WindowParams p) {
+  constexpr int LPR = D / 8;
+  constexpr int RPW = 256 / LPR;
+  const int tid = threadIdx.x, j = tid % LPR;
+  const int W = p.inc + p.T;
+  const int64_t row = (int64_t)blockIdx.x * RPW + tid / LPR;      // (bh, r)
+  if (row >= (int64_t)p.B * p.H * W) return;
+  const int bh = (int)(row / W), r = (int)(row % W);
+  const int b = bh / p.H, hh = bh % p.H;
+  u32x4_t qo = {0, 0, 0, 0}, ko, vo;
+  if (r < p.inc) {
+    const int64_t pos = p.full_len + r;
+    const char* src = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h + pos * p.kcs_r);
+    const u32x4_t x = *(const u32x4_t*)(src + 16 * j);
+    const u32x4_t other = *(const u32x4_t*)(src + 16 * (j ^ (LPR / 2)));
+    const u32x4_t c = *(const u32x4_t*)((const char*)p.cos + 2 * (pos * p.cs_r) + 16 * j);
+    const u32x4_t s = *(const u32x4_t*)((const char*)p.sin + 2 * (pos * p.cs_r) + 16 * j);
+    float o[8];
+    rotate_chunk<T>(x, other, c, s, j >= LPR / 2, o);
+    ko = u32x4_t{pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
+    vo = *(const u32x4_t*)((const char*)p.vcache + 2 * (b * p.vcs_b + hh * p.vcs_h + pos * p.vcs_r) + 16 * j);
+  } else {
+    const int t = r - p.inc;
+    qo = *(const u32x4_t*)((const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + t * p.qs_r) + 16 * j);
+    ko = *(const u32x4_t*)((const char*)p.k_loc + 2 * (b * p.kls_b + hh * p.kls_h + t * p.kls_r) + 16 * j);
+    vo = *(const u32x4_t*)((const char*)p.v_loc + 2 * (b * p.vls_b + hh * p.vls_h + t * p.vls_r) + 16 * j);
+  }
+  *(u32x4_t*)((char*)p.q_win + 2 * (b * p.qws_b + hh * p.qws_h + r * p.qws_r) + 16 * j) = qo;
+  *(u32x4_t*)((char*)p.k_win + 2 * (b * p.kws_b + hh * p.kws_h + r * p.kws_r) + 16 * j) = ko;
+  *(u32x4_t*)((char*)p.v_win + 2 * (b * p.vws_b + hh * p.vws_h + r * p.vws_r) + 16 * j) = vo;
+}
+
+template <class T, int D>
+static int launch_window_t(const WindowParams& p, hipStream_t stream) {
+  constexpr int RPW = 256 / (D / 8);
+  const int64_t rows = (int64_t)p.B * p.H * (p.inc + p.T);
+  hipLaunchKernelGGL((lmk_local_window_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t stream) {
+  if (dtype == LMK_DTYPE_BF16) {
+    if (D == 128) return launch_window_t<bf16_t, 128>(p, stream);
+    if (D == 64) return launch_window_t<bf16_t, 64>(p, stream);
+  } else if (dtype == LMK_DTYPE_F16) {
+    if (D == 128) return launch_window_t<f16_t, 128>(p, stream);
+    if (D == 64) return launch_window_t<f16_t, 64>(p, stream);
+  }
+  return LMK_ERR_UNSUPPORTED;
+}
+
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream) {
   if (D != 128) return LMK_ERR_UNSUPPORTED;
   if (dtype == LMK_DTYPE_BF16) return launch_gather_t<bf16_t>(p, BS, stream);

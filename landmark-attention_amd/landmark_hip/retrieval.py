@@ -6,7 +6,9 @@ Mirrors the per-head, per-token branch of ``LlamaAttention.forward``
 conventions: ``past_key_value = (K_without_rotary, V)`` each ``(B, nh, S, hd)`` (``:424-430``),
 ``block = mem_freq + 1`` with the landmark as the last token of a block, queries and local
 keys already rotated (``:298``), ``cos/sin`` the model-dtype tables of
-``LlamaRotaryEmbedding`` (``:121-124``).  The cached length must be a whole number of blocks.
+``LlamaRotaryEmbedding`` (``:121-124``).  The cache may end in an incomplete block (the state
+between two landmarks while decoding): retrieval then covers the complete blocks and the tail
+joins the local window (``:321-342``).
 """
 from __future__ import annotations
 
@@ -43,7 +45,7 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int):
     q, k_cache = _lib.kernel_ready(q), _lib.kernel_ready(k_cache)
     cos, sin = _tables(cos, sin, q.dtype)
     lib = _lib.lib()
-    k = min(top_k, S // block)
+    k = min(top_k, S // block)                      # complete blocks only (llama_mem.py:321-324,358-359)
     idx = torch.empty((B, H, T, k), device=q.device, dtype=torch.int64)
     nbytes = lib.lmk_retrieve_workspace_bytes(B, H, T, S, D, int(block))
     with torch.cuda.device(q.device):
@@ -57,18 +59,33 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int):
 
 
 def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
-    """Attention output ``(B, nh, T, hd)`` over the blocks ``idx`` selects plus the local chunk
-    (``llama_mem.py:386-412,447-477``).  The local chunk is attended with the fused forward
-    kernel; the gather kernel reads the selected blocks in place and merges both parts."""
+    """Attention output ``(B, nh, T, hd)`` over the blocks ``idx`` selects plus the local window
+    (``llama_mem.py:386-412,447-477``).  The local window -- the new chunk, behind the tail of
+    an incomplete cached block if there is one (``:329-342``) -- is attended with the fused
+    forward kernel; the gather kernel reads the selected blocks in place and merges both parts."""
     B, H, T, D = q.shape
     S = k_cache.shape[2]
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
     q, k_cache, v_cache, k_loc, v_loc = (_lib.kernel_ready(t) for t in (q, k_cache, v_cache, k_loc, v_loc))
     cos, sin = _tables(cos, sin, q.dtype)
+    inc = S % block
     with torch.cuda.device(q.device):
-        o_loc, L_loc, M_loc = _launch_fwd(q, k_loc, v_loc, 0, sm_scale, block)
-        out = torch.empty_like(o_loc)
+        if inc == 0:
+            o_loc, L_loc, M_loc = _launch_fwd(q, k_loc, v_loc, 0, sm_scale, block)
+        else:
+            assert T + inc <= block, "new chunk and cached tail must fit one block (llama_mem.py:330)"
+            q_win, k_win, v_win = (torch.empty((B, H, inc + T, D), device=q.device, dtype=q.dtype) for _ in range(3))
+            _lib.check(_lib.lib().lmk_local_window(
+                _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), _lib.tensor4(k_loc), _lib.tensor4(v_loc),
+                cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(q_win), _lib.tensor4(k_win),
+                _lib.tensor4(v_win), B, H, T, S, D, int(block), _lib.DTYPE_CODES[q.dtype],
+                _lib.current_stream(q.device)))
+            o_win, L_win, M_win = _launch_fwd(q_win, k_win, v_win, 0, sm_scale, block)
+            o_loc = o_win[:, :, inc:]                                   # a strided view: read in place
+            L_loc = L_win.view(B * H, inc + T)[:, inc:].contiguous()
+            M_loc = M_win.view(B * H, inc + T)[:, inc:].contiguous()
+        out = torch.empty_like(q)
         rc = _lib.lib().lmk_gather_attend(
             _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), idx.data_ptr(), cos.data_ptr(),
             sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(o_loc), L_loc.data_ptr(), M_loc.data_ptr(),

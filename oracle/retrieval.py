@@ -6,6 +6,9 @@ Restates the per-head, per-token branch (``aggregate is None``) of
 
 Symbols: ``bs = mem_freq + 1`` (block), ``S`` cached tokens, ``T`` new tokens,
 ``num_mems = S // bs`` complete cached blocks, ``k = min(cache_top_k, num_mems)``.
+When the cache ends in an incomplete block (``S % bs`` tokens, ``:321-324``) those tokens
+are not retrieved from: they are rotated at their own positions and put in front of the
+new chunk (``:329-342``), visible to every query, in no landmark group.
 The cache holds keys WITHOUT rotary (``:424-425``); queries and local keys come
 in already rotated (``:298``).
 
@@ -121,6 +124,18 @@ def gather_blocks(cache, idx, block: int):
     return torch.take_along_dim(flat, sel, dim=3)
 
 
+def local_window(k_cache, v_cache, k_loc, v_loc, cos, sin, block: int):
+    """Keys and values of the local window when the cache ends in an incomplete block
+    (``llama_mem.py:337-340``): the tail's keys rotated at positions ``full_len ..`` in front of
+    the new chunk's, the tail's values in front of the new chunk's."""
+    S = k_cache.shape[2]
+    inc = S % block
+    full_len = S - inc
+    pos = torch.arange(full_len, S, dtype=torch.long)
+    k_tail = apply_rotary(k_cache[:, :, full_len:], cos, sin, pos)
+    return torch.cat((k_tail, k_loc), dim=2), torch.cat((v_cache[:, :, full_len:], v_loc), dim=2)
+
+
 # ---------------------------------------------------------------- local masks
 def local_masks(is_mem_loc, T: int, dtype):
     """Mask preparation of ``LlamaModel.forward`` (``llama_mem.py:807-815``) for a
@@ -146,15 +161,18 @@ def retrieve_and_attend(q, k_cache, v_cache, k_loc, v_loc, is_mem_loc, cos, sin,
                         idx=None, n_buckets: int = 64):
     """Whole step in the model dtype with the reference's rounding points.
 
-    q, k_loc: (B,nh,T,hd) rotated; k_cache (un-rotated), v_cache: (B,nh,S,hd) with
-    ``S % block == 0``; cos/sin: (n_pos, hd) tables in the model dtype.
+    q, k_loc: (B,nh,T,hd) rotated; k_cache (un-rotated), v_cache: (B,nh,S,hd);
+    cos/sin: (n_pos, hd) tables in the model dtype.
     Returns ``(out (B,nh,T,hd), idx (B,nh,T,k) int64)``.
     """
     B, nh, T, hd = q.shape
     S = k_cache.shape[2]
     g = retrieval_geometry(S, block, top_k)
-    assert g["incomplete_len"] == 0, "tail of an incomplete cached block not restated here"
+    inc = g["incomplete_len"]
     k = g["k"]
+    if inc:
+        assert T + inc <= block                                                     # :330
+        k_loc, v_loc = local_window(k_cache, v_cache, k_loc, v_loc, cos, sin, block)
     if idx is None:
         idx = select_topk(landmark_scores(q, k_cache, cos, sin, block, top_k), k)
     pos = gather_positions(idx, g["num_mems"], k, block, g["prefix_len"])           # (B,nh,T,k,bs)
@@ -165,6 +183,10 @@ def retrieve_and_attend(q, k_cache, v_cache, k_loc, v_loc, is_mem_loc, cos, sin,
     div = math.sqrt(hd)
     prefix = (q.unsqueeze(3) @ ksel.transpose(3, 4)).squeeze(3) / div               # :412
     add, im_loc, ls_loc = local_masks(is_mem_loc, T, q.dtype)
+    if inc:                                                                         # :331-335 and the mask slice of :460
+        add = torch.cat((torch.zeros(B, 1, T, inc, dtype=add.dtype), add), dim=-1)
+        im_loc = torch.cat((torch.zeros(B, 1, T, inc, dtype=torch.bool).expand(im_loc.shape[0], 1, T, inc), im_loc), dim=-1)
+        ls_loc = torch.cat((torch.ones(B, 1, T, inc, dtype=torch.bool).expand(ls_loc.shape[0], 1, T, inc), ls_loc), dim=-1)
     local = (q @ k_loc.transpose(2, 3)) / div + add                                 # :448,460
     local = torch.max(local, torch.tensor(torch.finfo(q.dtype).min, dtype=q.dtype)) # :461
     x = torch.cat((prefix, local), dim=-1)
@@ -188,6 +210,10 @@ def retrieve_and_attend_s1(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block: i
     S = k_cache.shape[2]
     g = retrieval_geometry(S, block, top_k)
     k = g["k"]
+    inc = g["incomplete_len"]
+    if inc:                       # the tail opens the current block; zero rows stand in for its queries
+        k_loc, v_loc = local_window(k_cache, v_cache, k_loc, v_loc, cos, sin, block)
+        q = torch.cat((torch.zeros(B, nh, inc, hd, dtype=q.dtype), q), dim=2)
     heads = range(nh) if heads is None else heads
     tokens = range(T) if tokens is None else tokens
     res = {}
@@ -202,5 +228,5 @@ def retrieve_and_attend_s1(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block: i
                 vs = blocks_v[sel].flatten(0, 1)
                 kk = torch.cat((ks, k_loc[b, h]), 0).float()
                 vv = torch.cat((vs, v_loc[b, h]), 0).float()
-                res[(b, h, t)] = s1_attention(q[b, h].float(), kk, vv, block, rows=[t])[0]
+                res[(b, h, t)] = s1_attention(q[b, h].float(), kk, vv, block, rows=[inc + t])[0]
     return res

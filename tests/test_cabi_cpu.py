@@ -29,7 +29,8 @@ def _declared():
 
 def test_every_declared_symbol_is_exported(lib):
     names = _declared()
-    assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_strerror"} <= set(names)
+    assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
+            "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
 
@@ -95,8 +96,7 @@ def test_retrieval_argument_errors(lib):
         return lib.lmk_retrieve_topk(t, t, cos, 0x6000, 128, n_pos, 0x7000, ws, wsb, 1, 1, 8, S, D, block, top_k, 0, None)
 
     assert topk(cos=0) == -1
-    assert topk(S=70) == -9                                   # incomplete cached block
-    assert topk(S=16) == -9                                   # less than one block
+    assert topk(S=16) == -9                                   # less than one complete block
     assert topk(top_k=0) == -10 and topk(top_k=65) == -10
     assert topk(n_pos=32) == -11
     assert topk(wsb=64) == -8
@@ -106,6 +106,14 @@ def test_retrieval_argument_errors(lib):
     rc = lib.lmk_gather_attend(t, t, t, 0x7000, 0x5000, 0x6000, 128, 4096, t, 0x2000, 0x3000, t, 1, 1, 8, 64, 64, 0.1,
                                32, 4, 0, None)
     assert rc == -3
+
+    # window of an incomplete cached block: needs a tail, and tail + new chunk within one block (llama_mem.py:330)
+    def window(S, T):
+        return lib.lmk_local_window(t, t, t, t, t, 0x5000, 0x6000, 128, 4096, t, t, t, 1, 1, T, S, 128, 32, 0, None)
+
+    assert window(64, 4) == -9
+    assert window(70, 27) == -2
+    assert window(20, 4) == -9
 
 
 def test_python_shim_rejects_what_the_reference_rejects():

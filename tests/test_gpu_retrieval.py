@@ -102,6 +102,56 @@ def test_gather_attend_matches_oracle(B, H, T, S, block, top_k):
         assert (out[b, h, t] - o).abs().max().item() <= 2e-2, (b, h, t)
 
 
+# cache ending in an incomplete block: the state between two landmarks while decoding
+# (llama_mem.py:321-342).  inc = S % block cached tail tokens, T new tokens, T + inc <= block.
+@pytest.mark.parametrize("n_mems,inc,T,block,top_k", [
+    (20, 7, 1, 32, 4),          # decode by one token
+    (20, 31, 1, 32, 4),         # the new token is the block's landmark: it does not see itself
+    (20, 1, 31, 32, 4),         # a chunk that completes the block
+    (20, 10, 12, 32, 4),
+    (3, 5, 2, 32, 5),           # fewer complete blocks than top_k
+    (12, 40, 24, 64, 3),        # block 64, ends on the landmark
+    (12, 17, 1, 64, 3),
+])
+def test_incomplete_cached_block(n_mems, inc, T, block, top_k):
+    from landmark_hip.retrieval import retrieve_and_attend
+    B, H, D = 2, 3, 128
+    S = n_mems * block + inc
+    print(f"case tail n_mems{n_mems} inc{inc} T{T} bs{block} k{top_k}", flush=True)
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=S + T + 2)
+    is_mem = ((torch.arange(T) + inc) % block == block - 1)[None].expand(B, T)
+    ref_bf16, idx_ref = oret.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, block, top_k)
+    dev = lambda t: t.cuda()
+    out, idx = retrieve_and_attend(dev(q), (dev(kc), dev(vc)), dev(kl), dev(vl), dev(cos), dev(sin), block, top_k)
+    torch.cuda.synchronize()
+    assert torch.equal(idx.cpu(), idx_ref)
+    out = out.float().cpu()
+    assert (out - ref_bf16.float()).abs().max().item() <= 2e-2
+    ref32 = oret.retrieve_and_attend_s1(q, kc, vc, kl, vl, cos, sin, block, top_k, idx_ref,
+                                        heads=[0, H - 1], tokens=sorted({0, T // 2, T - 1}))
+    for (b, h, t), o in ref32.items():
+        assert (out[b, h, t] - o).abs().max().item() <= 2e-2, (b, h, t)
+
+
+def test_local_window_rows_bit_exact():
+    # the window builder alone: rotated tail keys bit for bit, values and new rows copied, zero query rows
+    from landmark_hip import _lib
+    B, H, T, D, block, inc = 1, 2, 3, 128, 32, 6
+    S = 4 * block + inc
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=77)
+    k_ref, v_ref = oret.local_window(kc, vc, kl, vl, cos, sin, block)
+    dev = lambda t: t.cuda()
+    qd, kcd, vcd, kld, vld, cd, sd = map(dev, (q, kc, vc, kl, vl, cos, sin))
+    qw, kw, vw = (torch.full((B, H, inc + T, D), 3.0, device="cuda:0", dtype=q.dtype) for _ in range(3))
+    T4 = _lib.tensor4
+    _lib.check(_lib.lib().lmk_local_window(T4(qd), T4(kcd), T4(vcd), T4(kld), T4(vld), cd.data_ptr(), sd.data_ptr(),
+                                           cd.stride(0), cd.shape[0], T4(qw), T4(kw), T4(vw), B, H, T, S, D, block, 0,
+                                           _lib.current_stream(qd.device)))
+    torch.cuda.synchronize()
+    assert torch.equal(kw.cpu(), k_ref) and torch.equal(vw.cpu(), v_ref)
+    assert torch.equal(qw.cpu()[:, :, inc:], q) and (qw.cpu()[:, :, :inc] == 0).all()
+
+
 def test_baseline_config4_full_size():
     # benchmark config 4: H32 D128, 32768 cached tokens = 1024 blocks of 32, 256 queries, top-4
     from landmark_hip.retrieval import retrieve_and_attend

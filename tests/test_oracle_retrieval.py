@@ -136,3 +136,67 @@ def test_attend_in_model_dtype_equals_fp32_closed_form(dtype, tol):
     ref = retrieval.retrieve_and_attend_s1(q, kc, vc, kl, vl, cos, sin, bs, k, idx)
     for (b, h, t), o in ref.items():
         assert (out[b, h, t].float() - o).abs().max() < tol, (b, h, t)
+
+
+# ------------------------------------------------- incomplete cached block (decode between landmarks)
+def _tail_case(dtype, inc, T, bs=8, nm=5, k=2, hd=16, nh=2, seed=20):
+    S = nm * bs + inc
+    q = _rand(1, nh, T, hd, seed=seed, dtype=dtype, scale=0.5)
+    kc = _rand(1, nh, S, hd, seed=seed + 1, dtype=dtype, scale=0.5)
+    vc = _rand(1, nh, S, hd, seed=seed + 2, dtype=dtype, scale=0.5)
+    kl = _rand(1, nh, T, hd, seed=seed + 3, dtype=dtype, scale=0.5)
+    vl = _rand(1, nh, T, hd, seed=seed + 4, dtype=dtype, scale=0.5)
+    is_mem = ((torch.arange(T) + inc) % bs == bs - 1)[None]          # the block's landmark, if the chunk reaches it
+    cos, sin = rotary.rotary_tables(S + T, hd, dtype)
+    return q, kc, vc, kl, vl, is_mem, cos, sin, bs, k
+
+
+def test_geometry_ignores_the_tail():
+    # 5 complete blocks of 8 and 3 tail tokens: positions as for S = 40 (llama_mem.py:321-324,358-365)
+    a, b = retrieval.retrieval_geometry(43, 8, 2), retrieval.retrieval_geometry(40, 8, 2)
+    assert (a["full_len"], a["incomplete_len"], a["num_mems"], a["prefix_len"]) == (40, 3, 5, 16)
+    assert torch.equal(a["mem_pos"], b["mem_pos"])
+
+
+@pytest.mark.parametrize("inc,T", [(3, 1), (1, 6), (5, 3), (7, 1)])     # (5,3) and (7,1) end on the landmark
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+def test_attend_with_incomplete_cached_block_equals_closed_form(dtype, tol, inc, T):
+    q, kc, vc, kl, vl, is_mem, cos, sin, bs, k = _tail_case(dtype, inc, T)
+    out, idx = retrieval.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, bs, k)
+    # selection sees the complete blocks only
+    full = kc[:, :, : kc.shape[2] - inc]
+    assert torch.equal(idx, retrieval.select_topk(retrieval.landmark_scores(q, full, cos, sin, bs, k), k))
+    ref = retrieval.retrieve_and_attend_s1(q, kc, vc, kl, vl, cos, sin, bs, k, idx)
+    for (b, h, t), o in ref.items():
+        assert (out[b, h, t].float() - o).abs().max() < tol, (b, h, t)
+
+
+def test_incomplete_cached_block_literal_row():
+    """One query written out by hand in float64: global bucket = landmarks of the retrieved blocks,
+    the tail, the new tokens up to the query (the landmark query not itself); every retrieved block
+    contributes its own softmax over its non-landmark keys, weighted by its landmark's share."""
+    inc, T = 5, 3
+    q, kc, vc, kl, vl, is_mem, cos, sin, bs, k = _tail_case(torch.float32, inc, T)
+    out, idx = retrieval.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, bs, k)
+    g = retrieval.retrieval_geometry(kc.shape[2], bs, k)
+    hd = q.shape[-1]
+    for h in range(q.shape[1]):
+        for t in range(T):
+            qq = q[0, h, t].double()
+            sel = idx[0, h, t]
+            pos = retrieval.gather_positions(sel, g["num_mems"], k, bs, g["prefix_len"])
+            blocks = [(rotary.apply_rotary(kc[0, h, b * bs : (b + 1) * bs], cos, sin, pos[j]).double(),
+                       vc[0, h, b * bs : (b + 1) * bs].double()) for j, b in enumerate(sel.tolist())]
+            tail_pos = torch.arange(g["full_len"], g["full_len"] + inc)
+            wk = torch.cat((rotary.apply_rotary(kc[0, h, g["full_len"] :], cos, sin, tail_pos), kl[0, h])).double()
+            wv = torch.cat((vc[0, h, g["full_len"] :], vl[0, h])).double()
+            last = inc + t - (1 if (inc + t) % bs == bs - 1 else 0)      # the landmark query does not see itself
+            s_win = (wk[: last + 1] @ qq) / math.sqrt(hd)
+            s_lm = torch.stack([(kb[bs - 1] @ qq) / math.sqrt(hd) for kb, _ in blocks])
+            z = torch.cat((s_lm, s_win))
+            w = torch.softmax(z, 0)
+            o = w[k:] @ wv[: last + 1]
+            for j, (kb, vb) in enumerate(blocks):
+                loc = torch.softmax((kb[: bs - 1] @ qq) / math.sqrt(hd), 0)
+                o = o + w[j] * (loc @ vb[: bs - 1])
+            assert (out[0, h, t].double() - o).abs().max() < 2e-5, (h, t)
