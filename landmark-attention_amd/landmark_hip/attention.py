@@ -22,7 +22,8 @@ SUPPORTED_HEAD_DIMS = (64, 128)
 def _launch_fwd(q, k, v, n_prefix, sm_scale, block):
     B, H, Lq, D = q.shape
     Lk = k.shape[2]
-    o = torch.empty((B, H, Lq, D), device=q.device, dtype=q.dtype)
+    o = torch.empty_like(q)        # keeps q's memory layout: a (B,L,H,D)-backed q gives an output whose
+    #                                transpose(1, 2).reshape(B, L, H*D) for o_proj (llama_mem.py:484-486) is a view
     L = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
     M = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
     rc = _lib.lib().lmk_attn_fwd(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o),
@@ -36,9 +37,7 @@ def _launch_bwd(q, k, v, o, do, L, M, n_prefix, sm_scale, block):
     B, H, Lq, D = q.shape
     Lk = k.shape[2]
     lib = _lib.lib()
-    dq = torch.empty((B, H, Lq, D), device=q.device, dtype=q.dtype)
-    dk = torch.empty((B, H, Lk, D), device=q.device, dtype=q.dtype)
-    dv = torch.empty((B, H, Lk, D), device=q.device, dtype=q.dtype)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)     # each in its input's layout
     nbytes = lib.lmk_attn_bwd_workspace_bytes(B, H, Lq, Lk, int(block))
     ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
     rc = lib.lmk_attn_bwd(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o), _lib.tensor4(do),

@@ -71,12 +71,13 @@ def test_landmark_value_rows_get_zero_gradient_and_last_landmark_key_too():
     assert gk[:, :, block - 1].abs().max() > 0
 
 
-def test_reference_script_loss_and_blhd_layout():
+@pytest.mark.parametrize("block", [64, 32])
+def test_reference_script_loss_and_blhd_layout(block):
     # the reference's own check: grads of (out**2).sum() on (B,L,H,D)-backed views
     # (test_flash_landmark_attention.py:91-94,156-157)
     from ltriton.flash_landmark_attention import fused_landmark_attention
     from oracle import s1
-    B, H, L, D, block = 2, 4, 256, 128, 64
+    B, H, L, D = 2, 4, 256, 128
     q, k, v = make_qkv(B, H, L, L, D, seed=11, layout="blhd")
     dev = torch.device("cuda:0")
     qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
@@ -87,6 +88,7 @@ def test_reference_script_loss_and_blhd_layout():
     r = torch.autograd.grad((s1.s1_attention(qc, kc, vc, block) ** 2).sum(), [qc, kc, vc])
     for a, b_ in zip(g, r):
         assert (a.float().cpu() - b_).abs().max().item() <= 4e-2
+        assert a.transpose(1, 2).is_contiguous()             # gradients come back in their input's layout
 
 
 def test_partial_block_backward_is_rejected():

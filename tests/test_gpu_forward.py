@@ -80,6 +80,8 @@ def test_noncontiguous_blhd_inputs_and_custom_scale():
     ref, _, _ = oracle_forward(q, k, v, block, scale=0.05)
     out = _run(q, k, v, block, scale=0.05)
     assert (out.float().cpu() - ref).abs().max().item() <= TOL
+    # the output keeps the inputs' layout, so the caller's transpose + reshape for o_proj is a view
+    assert out.transpose(1, 2).is_contiguous()
 
 
 def test_is_mem_none_and_bad_is_mem():
