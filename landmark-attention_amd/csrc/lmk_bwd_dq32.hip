@@ -103,6 +103,11 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   // after the prologue (dO comes from LDS), and left in the workspace for the dK/dV kernel
   // (`_bwd_preprocess`, llama/ltriton/flash_landmark_attention.py:125-149)
   float mhat = 0.f, delta = 0.f;
+  float row_M = 0.f, row_L = 1.f;                           // fetched here, with everything else the prologue waits for
+  if (rowok) {
+    row_M = p.M[(int64_t)bh * p.Lq + qrow];
+    row_L = p.L[(int64_t)bh * p.Lq + qrow];
+  }
   u32x4_t of[C::KS];                                        // this lane's part of its O row
   {
     const char* op = (const char*)p.o + 2 * (b_ * p.os_b + hh * p.os_h);
@@ -235,8 +240,18 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   auto stage_z = [&](int slot_bytes) __attribute__((always_inline)) {     // dQ^T += K^T dS^T
     int zb[2 * C::DC];
     zbase(slot_bytes, zb);
+    // operands are fetched PFZ MFMAs ahead: a fetch that is awaited at once costs the LDS latency per MFMA
+    constexpr int NZ = 2 * C::DC, PFZ = 2;
+    u32x4_t zf[NZ];
 #pragma unroll
-    for (int n = 0; n < 2 * C::DC; ++n) acc[n % C::DC] = mfma32<T>(ztr(zb, n), dsf[n / C::DC], acc[n % C::DC]);
+    for (int n = 0; n < PFZ; ++n) zf[n] = ztr(zb, n);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < NZ; ++n) {
+      if (n + PFZ < NZ) zf[n + PFZ] = ztr(zb, n + PFZ);
+      acc[n % C::DC] = mfma32<T>(zf[n], dsf[n / C::DC], acc[n % C::DC]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
   // X of the next block interleaved with Y of an earlier block `blk`.  The wave issues in order, so
   // the instruction stream is the schedule: each MFMA is followed by a slice of Y that runs while
@@ -364,7 +379,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
     delta = pair_sum(dsum);
     if (rowok) {
       const int64_t r = (int64_t)bh * p.Lq + qrow;
-      mhat = p.M[r] * kLog2e + fast_log2(p.L[r]);
+      mhat = row_M * kLog2e + fast_log2(row_L);
       if (h == 0) {
         p.delta[r] = delta;
         p.mhat[r] = mhat;
