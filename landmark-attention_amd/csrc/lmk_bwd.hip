@@ -488,11 +488,6 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dkdv_kernel(BwdParams p) {
 // ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
-template <class K>
-static int set_lds(K kern, int bytes) {
-  return (int)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-}
-
 template <class T, int D, int BS>
 static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
   int rc;
@@ -508,11 +503,8 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
   } else if (phases & 2) {
     using C = DqCfg<T, D, BS>;
     auto kern = lmk_bwd_dq_kernel<T, D, BS>;
-    static bool done = false;
-    if (!done) {
-      if ((rc = set_lds(kern, C::LDS_BYTES))) return rc;
-      done = true;
-    }
+    static std::atomic<uint64_t> lds_ok{0};
+    if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
     hipLaunchKernelGGL(kern, dim3(p.n_qtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
   }
@@ -522,11 +514,8 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
   if (phases & 4) {
     using C = DkvCfg<T, D, BS>;
     auto kern = lmk_bwd_dkdv_kernel<T, D, BS>;
-    static bool done = false;
-    if (!done) {
-      if ((rc = set_lds(kern, C::LDS_BYTES))) return rc;
-      done = true;
-    }
+    static std::atomic<uint64_t> lds_ok{0};
+    if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
     hipLaunchKernelGGL(kern, dim3(p.n_kvtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
   }

@@ -403,12 +403,8 @@ template <class T, int D>
 static int launch_dkdv32_t(const BwdParams& p, hipStream_t stream) {
   using C = Dkv32Cfg<T, D>;
   auto kern = lmk_bwd_dkdv32_kernel<T, D>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) return (int)e;
-    attr_done = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   hipLaunchKernelGGL(kern, dim3(p.n_kvtiles * p.B * p.H), dim3(C::NTHR), C::LDS_BYTES, stream, p);
   return (int)hipGetLastError();
 }

@@ -254,12 +254,8 @@ template <class T, int D, int BS>
 static int launch_fwd_t(const FwdParams& p, hipStream_t stream) {
   using C = FwdCfg<T, D, BS>;
   auto kern = lmk_fwd_kernel<T, D, BS>;
-  static bool attr_done = false;  // the attribute is per function, setting it twice is harmless
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) return (int)e;
-    attr_done = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   const int grid = p.n_qtiles * p.B * p.H;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), C::LDS_BYTES, stream, p);
   return (int)hipGetLastError();

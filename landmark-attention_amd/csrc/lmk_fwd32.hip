@@ -295,12 +295,8 @@ template <class T, int D>
 static int launch_fwd32_t(const FwdParams& p, hipStream_t stream) {
   using C = Fwd32Cfg<T, D>;
   auto kern = lmk_fwd32_kernel<T, D>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) return (int)e;
-    attr_done = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   const int n_qt = (p.Lq + C::QT - 1) / C::QT;
   hipLaunchKernelGGL(kern, dim3(n_qt * p.B * p.H), dim3(C::NTHR), C::LDS_BYTES, stream, p);
   return (int)hipGetLastError();

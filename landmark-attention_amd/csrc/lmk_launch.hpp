@@ -5,9 +5,27 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/lmk.h"
 
 namespace lmk {
+
+// A kernel's dynamic-LDS limit is an attribute of the function ON ONE DEVICE: it is raised once per
+// (kernel instantiation, device); `done` is that instantiation's bit mask of devices already served.
+// Returns 0 or a hipError_t.
+template <class K>
+inline int allow_dynamic_lds(K kern, int bytes, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return 0;
+  e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return (int)e;
+  done.fetch_or(bit, std::memory_order_release);
+  return 0;
+}
 
 struct FwdParams {
   const void *q, *k, *v;

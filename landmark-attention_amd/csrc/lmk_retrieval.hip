@@ -731,13 +731,9 @@ static int launch_topk_t(const RetrParams& p, hipStream_t stream) {
     const int NMr = (p.num_mems + 63) & ~63;
     const int lds = (kFusedRows * (NMr + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
     auto kern = lmk_topk_fused_kernel<T, D>;
-    static bool attr_done = false;
-    if (!attr_done) {
-      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (kFusedRows * (kFusedMaxMems + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D);
-      if (e != hipSuccess) return (int)e;
-      attr_done = true;
-    }
+    static std::atomic<uint64_t> lds_ok{0};
+    constexpr int lds_max = (kFusedRows * (kFusedMaxMems + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
+    if (int rc = allow_dynamic_lds(kern, lds_max, lds_ok)) return rc;
     const int n_rt = (p.T + kFusedRows - 1) / kFusedRows;
     hipLaunchKernelGGL(kern, dim3(p.B * p.H * n_rt), dim3(64 * kFusedWaves), lds, stream, p);
     return (int)hipGetLastError();
