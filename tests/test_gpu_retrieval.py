@@ -83,7 +83,9 @@ def test_fp16_indices_bit_exact():
 
 
 @pytest.mark.parametrize("B,H,T,S,block,top_k", [(1, 2, 64, 24 * 32, 32, 4), (1, 2, 128, 12 * 64, 64, 3),
-                                                  (2, 2, 96, 3 * 32, 32, 5)])
+                                                  (2, 2, 96, 3 * 32, 32, 5),
+                                                  (1, 2, 1, 24 * 32, 32, 4),      # decode: first token of a new block
+                                                  (1, 2, 5, 12 * 64, 64, 3)])
 def test_gather_attend_matches_oracle(B, H, T, S, block, top_k):
     from landmark_hip.retrieval import retrieve_and_attend
     D = 128
@@ -97,7 +99,8 @@ def test_gather_attend_matches_oracle(B, H, T, S, block, top_k):
     out = out.float().cpu()
     assert (out - ref_bf16.float()).abs().max().item() <= 2e-2
     ref32 = oret.retrieve_and_attend_s1(q, kc, vc, kl, vl, cos, sin, block, top_k, idx_ref,
-                                        heads=[0, H - 1], tokens=[0, 1, block - 2, block - 1, block, T - 1])
+                                        heads=[0, H - 1],
+                                        tokens=sorted({t for t in (0, 1, block - 2, block - 1, block, T - 1) if 0 <= t < T}))
     for (b, h, t), o in ref32.items():
         assert (out[b, h, t] - o).abs().max().item() <= 2e-2, (b, h, t)
 
