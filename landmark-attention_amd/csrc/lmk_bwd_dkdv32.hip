@@ -41,9 +41,9 @@ struct Dkv32Cfg {
   static constexpr int BUF_BYTES = 2 * TILE_BYTES + STAT_BYTES;   // Q, dO, terms
   static constexpr int NBUF = 6;                           // ring slots: tiles i-1, i, i+1 in use, i+2 .. i+4 in flight
   static constexpr int RPD = 1024 / ROWB;                  // tile rows covered by one 1 KB request
-  static constexpr int NDMA = 32 / RPD / NKT;              // requests per K-role wave, tile and tensor
-  static constexpr int PER_TILE_K = 2 * NDMA;              // K-role waves fetch Q and dO
-  static constexpr int PER_TILE_V = 1;                     // V-role waves fetch their key tile's terms
+  static constexpr int NDMA = 32 / RPD / NKT;              // requests per wave and tile for one tensor
+  static constexpr int PER_TILE_K = NDMA;                  // K-role waves fetch dO (the role with more arithmetic)
+  static constexpr int PER_TILE_V = NDMA + 1;              // V-role waves fetch Q and their key tile's terms
   static constexpr int XCH_OFF = NBUF * BUF_BYTES;         // W hand-over: [parity 2][key tile][piece 2][lane][16 B]
   static constexpr int XCH_TILE = 2048;
   static constexpr int CONST_OFF = XCH_OFF + 2 * NKT * XCH_TILE;   // 32 x 1e30f, then 32 x 0.0f
@@ -119,17 +119,21 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     }
   }
 
-  // ---- loaders.  K-role wave b fetches rows RPD*(b*NDMA + d) .. of Q and of dO; V-role wave t
-  // fetches the terms of key tile t.
+  // ---- loaders.  Wave pair t fetches rows RPD*(t*NDMA + d) .. of a query tile: the V-role wave those
+  // of Q plus the terms of key tile t, the K-role wave those of dO.
   const int j_first = max(0, kvt * C::NKT - PT);           // first query tile any wave here can see
-  uint32_t q_vo[C::NDMA], g_vo[C::NDMA];                   // per-lane source offsets inside a tile (bytes)
-#pragma unroll
-  for (int d = 0; d < C::NDMA; ++d) {
-    const int n = tile * C::NDMA + d;
-    const int row = C::RPD * n + lane / C::CH, chp = lane % C::CH;
-    const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
-    q_vo[d] = (uint32_t)(2 * (row * p.qs_r + 8 * (chp ^ f)));   // the chunk that belongs at LDS position chp
-    g_vo[d] = (uint32_t)(2 * (row * p.dos_r + 8 * (chp ^ f)));
+  static_assert(C::NDMA <= 2, "two running offsets per wave");
+  // per-lane source offset (bytes) of this wave's requests 0 and 1 inside its tensor: Q for the V role, dO for the K role
+  uint32_t src_vo0, src_vo1 = 0;
+  const char* src_base = role_k ? gp : qp;                 // wave-uniform
+  const int64_t src_rs = role_k ? p.dos_r : p.qs_r;
+  {
+    const int chp = lane % C::CH;
+    const int row0 = C::RPD * (tile * C::NDMA) + lane / C::CH, row1 = row0 + C::RPD;
+    const int f0 = (((row0 & 3) << 2) | ((row0 >> 2) & 3)) & (C::CH - 1);
+    const int f1 = (((row1 & 3) << 2) | ((row1 >> 2) & 3)) & (C::CH - 1);
+    src_vo0 = (uint32_t)(2 * (row0 * src_rs + 8 * (chp ^ f0)));   // the chunk that belongs at LDS position chp
+    if (C::NDMA > 1) src_vo1 = (uint32_t)(2 * (row1 * src_rs + 8 * (chp ^ f1)));
   }
   const float* st_src;                                     // this lane's 16 bytes of terms for query tile 0
   {
@@ -144,32 +148,38 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   // offset: one vector add per request instead of 64-bit scalar multiplies per iteration.  Past the
   // last tile it stops advancing and the last tile is re-read (never used).
   int j_req = j_first;                                     // tile the next request fetches
-  const uint32_t q_step = (uint32_t)(2 * 32 * p.qs_r), g_step = (uint32_t)(2 * 32 * p.dos_r);
-#pragma unroll
-  for (int d = 0; d < C::NDMA; ++d) {
-    q_vo[d] += (uint32_t)j_first * q_step;
-    g_vo[d] += (uint32_t)j_first * g_step;
-  }
+  const uint32_t src_step = (uint32_t)(2 * 32 * src_rs);
+  src_vo0 += (uint32_t)j_first * src_step;
+  src_vo1 += (uint32_t)j_first * src_step;
   st_src += 32 * (int64_t)j_first;
-  auto request = [&](int slot_bytes) LMK_INL {             // this wave's share of query tile j_req -> ring slot
-    if (role_k) {
-#pragma unroll
-      for (int d = 0; d < C::NDMA; ++d) {
-        dma16_s(qp, q_vo[d], slot_bytes + (tile * C::NDMA + d) * 1024);
-        dma16_s(gp, g_vo[d], slot_bytes + C::TILE_BYTES + (tile * C::NDMA + d) * 1024);
-      }
-    } else {
-      dma16_v(st_src, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
-    }
+  // One piece of this wave's share of query tile j_req -> ring slot.  A tile's pieces go out one per MFMA
+  // slot of the first product rather than together: all eight waves asking at once queue up in front of
+  // the address unit.  V role: pieces 0 .. NDMA-1 fetch Q rows, piece NDMA the terms; K role: dO rows.
+  const int dst_off = (role_k ? C::TILE_BYTES : 0) + tile * C::NDMA * 1024;   // this wave's rows inside a slot
+  auto request_piece = [&](int slot_bytes, auto Pc) LMK_INL {
+    constexpr int P = decltype(Pc)::value;
     const bool more = j_req < nq - 1;                      // wave-uniform
-    const uint32_t qs = more ? q_step : 0u, gs = more ? g_step : 0u;
-#pragma unroll
-    for (int d = 0; d < C::NDMA; ++d) {
-      q_vo[d] += qs;
-      g_vo[d] += gs;
+    if constexpr (P < C::NDMA) {
+      uint32_t& vo = (P == 0) ? src_vo0 : src_vo1;
+      dma16_s(src_base, vo, slot_bytes + dst_off + P * 1024);
+      vo += more ? src_step : 0u;
+      if (P == C::NDMA - 1 && role_k) j_req += more ? 1 : 0;
+    } else if constexpr (P == C::NDMA) {
+      if (!role_k) {
+        dma16_v(st_src, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
+        st_src += more ? 32 : 0;
+        j_req += more ? 1 : 0;
+      }
     }
-    st_src += more ? 32 : 0;
-    j_req += more ? 1 : 0;
+  };
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  using P2 = std::integral_constant<int, 2>;
+  static_assert(C::PER_TILE_V <= 3, "a tile's pieces are P0 .. P2");
+  auto request = [&](int slot_bytes) LMK_INL {             // the whole share at once (prologue, last iterations)
+    request_piece(slot_bytes, P0{});
+    request_piece(slot_bytes, P1{});
+    request_piece(slot_bytes, P2{});
   };
   auto wait_tiles = [&]() LMK_INL {                        // all but this wave's two newest tiles have landed
     if (role_k) wait_vmcnt<2 * C::PER_TILE_K>();
@@ -202,7 +212,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   };
 
   // ---- V role: one query tile i.  S of tile i+1 (slot nslot) is interleaved with W of tile i.
-  auto body_v = [&](auto Mc, int i, int cslot, int nslot, int par, f32x16_t& s, f32x16_t& sn, f32x16_t* acc, auto sync) LMK_INL {
+  auto body_v = [&](auto Mc, int i, int cslot, int nslot, int rslot, int par, f32x16_t& s, f32x16_t& sn, f32x16_t* acc, auto sync) LMK_INL {
     constexpr bool MASKED = decltype(Mc)::value;
     const int CST = cslot + 2 * C::TILE_BYTES + tile * 1024;   // this key tile's terms: a, nD, dslm, mhat, delta
     const int krel = 32 * (kt - (PT + i)) + ql;            // key position relative to the query tile's first row
@@ -239,6 +249,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       if (m + PF < C::KS) fr[m + PF] = *(const u32x4_t*)(smem + nslot + koff[m + PF]);
 #pragma unroll
       for (int n = (m * NB) / C::KS; n < ((m + 1) * NB) / C::KS; ++n) tf[n] = trfrag(cslot + C::TILE_BYTES, n);
+      if (m == 0) request_piece(rslot, P0{});              // tile i+4, into the slot tile i-2 has left
+      if (m == 2) request_piece(rslot, P1{});
+      if (m == 4) request_piece(rslot, P2{});
       sn = mfma32<T>(fr[m], bf[m], sn);
 #pragma unroll
       for (int r = (m * 16) / C::KS; r < ((m + 1) * 16) / C::KS; ++r) elementwise(r);
@@ -253,7 +266,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   };
 
   // ---- K role: dP of tile i (slot cslot) interleaved with dS of tile i-1 (slot pslot), then dK of tile i-1.
-  auto body_k = [&](int i, int cslot, int pslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc, auto sync) LMK_INL {
+  auto body_k = [&](int i, int cslot, int pslot, int rslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc, auto sync) LMK_INL {
     const bool masked = PT + (i - 1) <= kt;                // tile i-1: own block or not yet visible
     const int CST = pslot + 2 * C::TILE_BYTES + tile * 1024;
     // y: subtrahend of dP, z: addend of dS  (byte offsets of 32-float arrays)
@@ -293,14 +306,19 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       if (m + PF < C::KS) fr[m + PF] = *(const u32x4_t*)(smem + cslot + C::TILE_BYTES + koff[m + PF]);
 #pragma unroll
       for (int n = (m * NB) / C::KS; n < ((m + 1) * NB) / C::KS; ++n) tf[n] = trfrag(pslot, n);
+      if (m == 1) request_piece(rslot, P0{});
+      if (m == 3) request_piece(rslot, P1{});
       dpn = mfma32<T>(fr[m], bf[m], dpn);
 #pragma unroll
       for (int r = (m * 16) / C::KS; r < ((m + 1) * 16) / C::KS; ++r) elementwise(r);
       __builtin_amdgcn_sched_barrier(0);
     }
-    sync();
-    __builtin_amdgcn_sched_barrier(0);
+    // The two roles meet the iteration's barrier in opposite phases: this role has its second product
+    // (operands in registers, matrix pipe only) in front of the barrier, the V role behind it, so one
+    // wave's MFMA-only stretch coincides with the other's LDS-and-vector stretch on their shared SIMD.
     tr_product(tf, df, acc);                               // dK^T += Q^T dS
+    __builtin_amdgcn_sched_barrier(0);
+    sync();
   };
 
   // ---- prologue: tiles j_first .. +3 requested; the first two must have landed
@@ -349,14 +367,13 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     row_tile(0, cur);                                       // S of the first tile
     int sc = 0;
     auto step = [&](auto Mc, int i) LMK_INL {
-      request(wrap(sc + 4) * C::BUF_BYTES);                 // tile i+4, into the slot tile i-2 has left
       // the barrier sits between the two products: the second one has its operands in registers, so
       // its MFMAs run while the workgroup's stragglers arrive and the next tile's operands are fetched
       auto sync = [&]() LMK_INL {
         wait_vmcnt<2 * C::PER_TILE_V>();                    // tile i+2 has landed (tiles i+3, i+4 may be in flight)
         __syncthreads();
       };
-      body_v(Mc, i, sc * C::BUF_BYTES, wrap(sc + 1) * C::BUF_BYTES, (i - j_first) & 1, cur, nxt, acc, sync);
+      body_v(Mc, i, sc * C::BUF_BYTES, wrap(sc + 1) * C::BUF_BYTES, wrap(sc + 4) * C::BUF_BYTES, (i - j_first) & 1, cur, nxt, acc, sync);
       cur = nxt;
       sc = wrap(sc + 1);
     };
@@ -383,12 +400,11 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     __syncthreads();
     sc = 1;
     for (int i = j_first + 1; i <= nq; ++i) {
-      request(wrap(sc + 4) * C::BUF_BYTES);
       auto sync = [&]() LMK_INL {
         wait_vmcnt<2 * C::PER_TILE_K>();
         __syncthreads();
       };
-      body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc, sync);
+      body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, wrap(sc + 4) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc, sync);
       prv = cur;
       sc = wrap(sc + 1);
     }
