@@ -217,9 +217,12 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     const int CST = cslot + 2 * C::TILE_BYTES + tile * 1024;   // this key tile's terms: a, nD, dslm, mhat, delta
     const int krel = 32 * (kt - (PT + i)) + ql;            // key position relative to the query tile's first row
     const int xoff = (MASKED ? CST + 384 : (lm_lane ? C::CONST_OFF : CST)) + 16 * h;
+    // terms of rows 8g + 4h .. +3, fetched two MFMA slots ahead of the slice that uses them (slot m works
+    // on registers r with r / 4 == grp(m)): at the top of the iteration only what the first MFMA and the
+    // first slice need is asked for, in that order, because LDS answers a wave in order
     float4 x4[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) x4[g] = *(const float4*)(smem + xoff + 32 * g);
+    auto ldx = [&](int g) LMK_INL { x4[g] = *(const float4*)(smem + xoff + 32 * g); };
+    auto grp = [](int m) LMK_INL { return ((m * 16) / C::KS) >> 2; };
     u32x4_t wf[2];
     float w[16];
     auto elementwise = [&](int r) LMK_INL {                // register r <-> query row 8*(r/4) + 4h + r%4
@@ -244,9 +247,13 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 #pragma unroll
     for (int m = 0; m < PF; ++m) fr[m] = *(const u32x4_t*)(smem + nslot + koff[m]);
     __builtin_amdgcn_sched_barrier(0);
+    ldx(0);
+    if (grp(1) != 0) ldx(grp(1));
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < C::KS; ++m) {
       if (m + PF < C::KS) fr[m + PF] = *(const u32x4_t*)(smem + nslot + koff[m + PF]);
+      if (m + 2 < C::KS && grp(m + 2) != grp(m + 1)) ldx(grp(m + 2));
 #pragma unroll
       for (int n = (m * NB) / C::KS; n < ((m + 1) * NB) / C::KS; ++n) tf[n] = trfrag(cslot + C::TILE_BYTES, n);
       if (m == 0) request_piece(rslot, P0{});              // tile i+4, into the slot tile i-2 has left
@@ -272,14 +279,14 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     // y: subtrahend of dP, z: addend of dS  (byte offsets of 32-float arrays)
     const int yoff = (masked ? CST + 512 : CST + 128) + 16 * h;
     const int zoff = ((!masked && lm_lane) ? CST + 256 : C::CONST_OFF + 128) + 16 * h;
-    float4 y4[4], z4[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
+    float4 y4[4], z4[4];                                   // fetched two MFMA slots ahead, as in the V role
+    auto ldyz = [&](int g) LMK_INL {
       y4[g] = *(const float4*)(smem + yoff + 32 * g);
       z4[g] = *(const float4*)(smem + zoff + 32 * g);
-    }
+    };
+    auto grp = [](int m) LMK_INL { return ((m * 16) / C::KS) >> 2; };
     const unsigned char* xp = smem + C::XCH_OFF + (par_prev * C::NKT + tile) * C::XCH_TILE + lane * 16;
-    u32x4_t wv[2] = {*(const u32x4_t*)(xp), *(const u32x4_t*)(xp + 1024)};
+    u32x4_t wv[2];
     u32x4_t df[2];
     float ds[16];
     auto elementwise = [&](int r) LMK_INL {
@@ -301,9 +308,15 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 #pragma unroll
     for (int m = 0; m < PF; ++m) fr[m] = *(const u32x4_t*)(smem + cslot + C::TILE_BYTES + koff[m]);
     __builtin_amdgcn_sched_barrier(0);
+    wv[0] = *(const u32x4_t*)(xp);
+    ldyz(0);
+    if (grp(1) != 0) ldyz(grp(1));
+    wv[1] = *(const u32x4_t*)(xp + 1024);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < C::KS; ++m) {
       if (m + PF < C::KS) fr[m + PF] = *(const u32x4_t*)(smem + cslot + C::TILE_BYTES + koff[m + PF]);
+      if (m + 2 < C::KS && grp(m + 2) != grp(m + 1)) ldyz(grp(m + 2));
 #pragma unroll
       for (int n = (m * NB) / C::KS; n < ((m + 1) * NB) / C::KS; ++n) tf[n] = trfrag(pslot, n);
       if (m == 1) request_piece(rslot, P0{});
