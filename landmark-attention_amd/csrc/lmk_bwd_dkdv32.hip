@@ -334,10 +334,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     sync();
   };
 
-  // ---- prologue: tiles j_first .. +3 requested; the first two must have landed
-#pragma unroll
-  for (int t = 0; t < 4; ++t) request(t * C::BUF_BYTES);
-  if (tid < 64) ((float*)(smem + C::CONST_OFF))[tid] = (tid < 32) ? 1e30f : 0.f;
+  // ---- prologue.  The stationary operand and the first two tiles are asked for first and awaited; tiles
+  // j_first+2, +3 go out behind that wait, so the workgroup does not sit through four tiles' worth of
+  // traffic (every workgroup of a launch round starts at the same moment) before its first product.
   // this wave's stationary operand: K fragments (V role) or V fragments (K role), lane = key
   {
     const char* src = role_k ? (const char*)p.v + 2 * (b_ * p.vs_b + hh * p.vs_h)
@@ -349,10 +348,16 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       bf[ks] = z;
       if (active) bf[ks] = *(const u32x4_t*)(src + 2 * ((int64_t)krow * rs + 16 * ks + 8 * h));
     }
-    // consume them here: the wait the compiler puts in front of this also covers the requests above,
-    // and no wait for these loads can then end up inside the loop, where it would drain the ring
+    request(0);
+    request(C::BUF_BYTES);
+    if (tid < 64) ((float*)(smem + C::CONST_OFF))[tid] = (tid < 32) ? 1e30f : 0.f;
+    // consume the operand here: no wait for these loads can then end up inside the loop, where it would
+    // drain the ring; the explicit wait covers the two requests, which the compiler does not count
+    wait_vmcnt<0>();
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) asm volatile("" : "+v"(bf[ks]));
+    request(2 * C::BUF_BYTES);
+    request(3 * C::BUF_BYTES);
   }
 
   wait_tiles();
