@@ -1,20 +1,23 @@
 // Forward kernel of fused landmark attention, landmark block = 32 keys (one MFMA tile).
 //
 // Same mathematics and layout as lmk_fwd.hip (S^T = K Q^T in the accumulator layout, lane =
-// query), organised around memory latency and pipe overlap:
-//   * a workgroup is 8 waves = 256 query rows sharing one K/V stream (wave w owns landmark block
-//     c0 + w), so a head's K/V is read from L2 once per 256 queries;
-//   * K/V blocks (32 keys) move global -> registers -> LDS through a ring of four LDS buffers and
-//     four register sets: the load of block b+6 is issued while block b is computed, which covers
-//     the L2/HBM latency that a one-block lookahead leaves exposed;
-//   * the S^T product of block b+1 is issued before the softmax of block b, so the matrix pipe
-//     works while the VALU does the exponentials; all LDS addresses are lane constants plus
-//     immediates (the ring is unrolled by four);
-//   * the running maximum is lazy: the reference value Mref only moves when a landmark score
-//     exceeds it by 2^8, so the accumulator is rescaled a handful of times per query instead of
-//     once per block; the true maximum is tracked on the side for the saved statistics.
-// Blocks below c0 are "earlier" for all eight waves (straight-line main loop); blocks c0 .. c0+7
-// are handled per wave (earlier / own / not visible).
+// query).  A workgroup is 8 waves = 256 query rows sharing one K/V stream, two waves per SIMD;
+// wave w owns landmark block c0 + w and keeps its Q fragments (B operands) and its O^T accumulator
+// in registers.  K/V blocks stream through a ring of four LDS slots filled by direct global->LDS
+// loads (block k+3 is requested while block k is computed; vmcnt is counted by hand).
+//
+// The softmax over the global bucket (the landmarks of the earlier blocks and the keys of the own
+// block) needs a reference maximum.  Only landmark scores enter it from the earlier blocks, so it
+// is known before the main loop at 1/32 of the cost of the scores: a first pass multiplies the
+// queries with the landmark keys alone (32 landmarks per MFMA tile) and keeps the row maximum R.
+// With R fixed the main loop has no running maximum, no rescaling of the accumulator and no
+// branch; per block a wave does
+//     X  S^T = K Q^T of the next block                        8 MFMA, row fragments from LDS
+//     Y  local softmax of the block, gate exp2(s_lm - R)       vector ALU only, interleaved with X
+//     Z  O^T += V^T P^T                                        8 MFMA, transposed fragments
+// and the own block at the end joins the bucket with one rescale by 2^(R - max(R, own maximum)).
+// (The reference kernel carries a running maximum and rescales per block,
+// llama/ltriton/flash_landmark_attention.py:64-76; the result is the same sum.)
 #include <type_traits>
 
 #include "lmk_common.hpp"
@@ -33,18 +36,34 @@ struct Fwd32Cfg {
   static constexpr int ROWB = 2 * D;
   static constexpr int BLK_BYTES = 32 * ROWB;              // one block of K (or of V)
   static constexpr int BUF_BYTES = 2 * BLK_BYTES;          // K then V
-  static constexpr int NBUF = 4;
-  static constexpr int CPB = 32 * CH;                      // 16-byte chunks per block and tensor
-  static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
-  static constexpr float LAZY = 8.0f;                      // log2 headroom before Mref moves
+  static constexpr int NBUF = 4;                           // ring slots: blocks k, k+1 in use, k+2, k+3 in flight
+  static constexpr int RPD = 1024 / ROWB;                  // block rows covered by one 1 KB request
+  static constexpr int NREQ = 2 * (32 / RPD);              // requests per block (K and V)
+  static constexpr int PER_TILE = NREQ / NW;               // requests per wave and block
+  static constexpr int LM_OFF = NBUF * BUF_BYTES;          // two tiles of 32 landmark keys for the first pass
+  static constexpr int LM_TILES = 2;
+  static constexpr int LDS_BYTES = LM_OFF + LM_TILES * BLK_BYTES;
 };
+
+__device__ __forceinline__ void fw_dma16(const void* base_uniform, uint32_t voff, uint32_t lds_off) {
+  // one 1 KB request of a wave: lane i's 16 bytes land at lds_off + 16*i (lds_off travels in M0)
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(voff), "s"(base_uniform), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void fw_wait_vmcnt() {          // s_waitcnt vmcnt(N) only (gfx9 encoding)
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+
+#define LMK_INL __attribute__((always_inline))
 
 template <class T, int D>
 __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
   using C = Fwd32Cfg<T, D>;
-  extern __shared__ __align__(16) unsigned char smem[];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  extern __shared__ __align__(16) unsigned char smem[];   // used through LDS byte addresses (it starts at 0)
+  (void)smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ql = lane & 31, h = lane >> 5;
 
   const int n_qt = (p.Lq + C::QT - 1) / C::QT;
@@ -70,7 +89,9 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
   const int cblk = c0 + wave;
   const int q0 = qtile * C::QT + wave * 32;
   const int qrow = q0 + ql;
-  const int nkb = (p.Lk + 31) >> 5;                        // key blocks that exist
+  const bool rowok = qrow < p.Lq;
+  const bool waveok = q0 < p.Lq;                           // wave-uniform: the wave has at least one query row
+  const int nkb = (p.Lk + 31) >> 5;                        // key blocks that exist (the last one may be partial)
   const int nblk = min(nkb, c0 + C::NW);                   // blocks this workgroup walks
   const float c2 = p.scale_log2;
 
@@ -79,202 +100,278 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
   for (int ks = 0; ks < C::KS; ++ks) {
     u32x4_t z = {0, 0, 0, 0};
     qf[ks] = z;
-    if (qrow < p.Lq) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
+    if (rowok) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
   }
 
-  // lane-constant LDS offsets inside a 32-row tile (tile_off only looks at row & 15)
-  int koff[C::KS];
+  // row fragment ks of a tile sits at tile_off(ql, 2 ks + h) = tile_off(ql, h) ^ (32 ks): the swizzle
+  // is an XOR on the 16-byte chunk index and 2 ks only touches bits the row term leaves zero
+  const int koff0 = tile_off<D>(ql, h);
+  int kx[C::KS];
 #pragma unroll
-  for (int ks = 0; ks < C::KS; ++ks) koff[ks] = tile_off<D>(ql, 2 * ks + h);
-  int voff[C::DC][2];
+  for (int ks = 0; ks < C::KS; ++ks) kx[ks] = koff0 ^ (ks << 5);
+  // transposed fragments: lane reads 8 bytes of row 4h + i/4 (+ 8 for the second half) at column
+  // 32 dc + 16 g2 + 4 (i%4); dc and the second half are XORs on the dc = 0, first-half offset
+  int voff0;
   {
     const int i = lane & 15, g2 = (lane >> 4) & 1;
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc) {
-      const int col = 32 * dc + 16 * g2 + 4 * (i & 3);
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf)
-        voff[dc][hf] = tile_off<D>(4 * h + (i >> 2) + 8 * hf, col >> 3) + ((col >> 2) & 1) * 8;
-    }
+    const int col = 16 * g2 + 4 * (i & 3);
+    voff0 = tile_off<D>(4 * h + (i >> 2), col >> 3) + ((col >> 2) & 1) * 8;
   }
+  constexpr int VOFF_HI = (8 * C::ROWB) | 32;
+  auto fresh = [](int x) LMK_INL {                         // recompute-at-use marker for lane-only values
+    asm volatile("" : "+v"(x));
+    return x;
+  };
 
-  // ---- block loader: thread tid moves chunk tid of K and of V (threads >= CPB idle when D = 64)
-  const bool ld_on = tid < C::CPB;
-  const int ld_row = tid / C::CH, ld_ch = tid % C::CH;
-  const int ld_lds = tile_off<D>(ld_row, ld_ch);
-  u32x4_t kreg[C::NBUF], vreg[C::NBUF];
-  auto gload = [&](auto Sc, int blk) {
-    constexpr int S = decltype(Sc)::value;
-    const int key = blk * 32 + ld_row;
-    u32x4_t z = {0, 0, 0, 0};
-    kreg[S] = z;
-    vreg[S] = z;
-    if (ld_on && blk < nblk && key < p.Lk) {
-      kreg[S] = *(const u32x4_t*)(kp + 2 * ((int64_t)key * p.ks_r + 8 * ld_ch));
-      vreg[S] = *(const u32x4_t*)(vp + 2 * ((int64_t)key * p.vs_r + 8 * ld_ch));
+  // ---- requests: wave w issues request n = w*PER_TILE + d of each block (K first, then V).  In a
+  // partial last block the rows past Lk re-read the last row (they are masked, but must be readable).
+  uint32_t r_vo[C::PER_TILE], r_vo_last[C::PER_TILE];
+  int r_lds[C::PER_TILE];
+  bool r_isv[C::PER_TILE];
+  const int last_rows = p.Lk - 32 * (nkb - 1);             // rows of the last block, 1 .. 32
+#pragma unroll
+  for (int d = 0; d < C::PER_TILE; ++d) {
+    const int n = wave * C::PER_TILE + d;
+    constexpr int per = 32 / C::RPD;                       // requests per tensor
+    const int part = n % per;
+    r_isv[d] = n >= per;
+    const int row = C::RPD * part + lane / C::CH, chp = lane % C::CH;
+    const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
+    const int64_t rs = r_isv[d] ? p.vs_r : p.ks_r;
+    r_vo[d] = (uint32_t)(2 * (row * rs + 8 * (chp ^ f)));
+    r_vo_last[d] = (uint32_t)(2 * (min(row, last_rows - 1) * rs + 8 * (chp ^ f)));
+    r_lds[d] = (r_isv[d] ? C::BLK_BYTES : 0) + part * 1024;
+  }
+  auto request = [&](int slot_bytes, int blk) LMK_INL {
+    const int bb = min(blk, nkb - 1);                      // past the end: re-read the last block (never used)
+    const bool last = bb == nkb - 1;                       // wave-uniform
+#pragma unroll
+    for (int d = 0; d < C::PER_TILE; ++d) {
+      const char* base = r_isv[d] ? vp + 2 * ((int64_t)bb * 32 * p.vs_r) : kp + 2 * ((int64_t)bb * 32 * p.ks_r);
+      fw_dma16(base, last ? r_vo_last[d] : r_vo[d], slot_bytes + r_lds[d]);
     }
   };
-  auto lstore = [&](auto Sc) {                              // register set S -> LDS buffer S
-    constexpr int S = decltype(Sc)::value;
-    if (ld_on) {
-      *(u32x4_t*)(smem + S * C::BUF_BYTES + ld_lds) = kreg[S];
-      *(u32x4_t*)(smem + S * C::BUF_BYTES + C::BLK_BYTES + ld_lds) = vreg[S];
-    }
+  // first pass: tile lt holds the landmark keys (row 31) of blocks 32 lt .. 32 lt + 31, row j of the tile =
+  // block 32 lt + j, same swizzle as a K block.  Every wave issues one request per tile (with D = 64 the
+  // upper four waves repeat the lower four's, so that all waves count the same).  Only landmarks of
+  // complete earlier blocks are ever used; rows past them re-read the last complete block's landmark.
+  const int n_lm = min(c0 + C::NW - 1, p.Lk >> 5);          // landmarks any wave here can need: blocks 0 .. n_lm-1
+  const int n_lt = (n_lm + 31) >> 5;
+  auto request_lm = [&](int lt) LMK_INL {
+    constexpr int per = 32 / C::RPD;
+    const int part = wave % per;
+    const int row = C::RPD * part + lane / C::CH, chp = lane % C::CH;
+    const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
+    const int blk = min(32 * lt + row, max(n_lm - 1, 0));
+    const uint32_t vo = (uint32_t)(2 * (((int64_t)blk * 32 + 31) * p.ks_r + 8 * (chp ^ f)));
+    fw_dma16(kp, vo, C::LM_OFF + (lt & 1) * C::BLK_BYTES + part * 1024);
   };
 
-  auto qk_tile = [&](int tileoff) {
-    f32x16_t s;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) s[r] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(*(const u32x4_t*)(smem + tileoff + koff[ks]), qf[ks], s);
-    return s;
-  };
-
-  float Mref = -INFINITY, Mtrue = -INFINITY, lsum = 0.f;   // log2 domain
   f32x16_t acc[C::DC];
 #pragma unroll
   for (int dc = 0; dc < C::DC; ++dc)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dc][r] = 0.f;
+  auto zero16 = [](f32x16_t& x) LMK_INL {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) x[r] = 0.f;
+  };
 
-  auto pv_tile = [&](int vtileoff, const float* w) {
+  // ---- the stages
+  u32x4_t pf[2];                                            // packed P^T of the block: keys 0..15, 16..31
+  float Rref = -1e30f, lsum = 0.f;                          // log2 domain; -1e30 stands for "no earlier block"
+  auto stage_x = [&](int tile_bytes, f32x16_t& s) LMK_INL {
+    zero16(s);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      u32x4_t wf = {pack2<T>(w[8 * j + 0], w[8 * j + 1]), pack2<T>(w[8 * j + 2], w[8 * j + 3]),
-                    pack2<T>(w[8 * j + 4], w[8 * j + 5]), pack2<T>(w[8 * j + 6], w[8 * j + 7])};
+    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(lds_ld128(kx[ks] + tile_bytes), qf[ks], s);
+  };
+  auto zbase = [&](int slot_bytes, int* zb) LMK_INL {
+    const int b = fresh(voff0 + slot_bytes);
 #pragma unroll
-      for (int dc = 0; dc < C::DC; ++dc) {
-        const u32x2_t a0 = lds_read_tr(smem + vtileoff + 16 * j * C::ROWB + voff[dc][0]);
-        const u32x2_t a1 = lds_read_tr(smem + vtileoff + 16 * j * C::ROWB + voff[dc][1]);
-        const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
-        acc[dc] = mfma32<T>(a, wf, acc[dc]);
+    for (int dc = 0; dc < C::DC; ++dc) {
+      zb[2 * dc] = b ^ (dc << 6);
+      zb[2 * dc + 1] = b ^ ((dc << 6) | VOFF_HI);
+    }
+  };
+  auto ztr = [&](const int* zb, int n) LMK_INL {            // A operand of the n-th O^T MFMA: V^T, keys 16 j ..
+    const int j = n / C::DC, dc = n % C::DC;
+    const u32x2_t a0 = lds_ld_tr(16 * j * C::ROWB + zb[2 * dc]);
+    const u32x2_t a1 = lds_ld_tr(16 * j * C::ROWB + zb[2 * dc + 1]);
+    const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
+    return a;
+  };
+  auto stage_z = [&](int vtile_bytes) LMK_INL {            // O^T += V^T P^T
+    int zb[2 * C::DC];
+    zbase(vtile_bytes, zb);
+    constexpr int NZ = 2 * C::DC, PFZ = 2;                  // operands fetched PFZ MFMAs ahead
+    u32x4_t zf[NZ];
+#pragma unroll
+    for (int n = 0; n < PFZ; ++n) zf[n] = ztr(zb, n);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < NZ; ++n) {
+      if (n + PFZ < NZ) zf[n + PFZ] = ztr(zb, n + PFZ);
+      acc[n % C::DC] = mfma32<T>(zf[n], pf[n / C::DC], acc[n % C::DC]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // X of the next block interleaved with Y of an earlier block.  The wave issues in order, so the
+  // instruction stream is the schedule: each MFMA is followed by a slice of Y that runs while the matrix
+  // pipe is busy.  Key of register r is 8*(r/4) + 4h + r%4; the landmark is r = 15, h = 1.
+  auto stage_xy = [&](int nslot, f32x16_t& s, f32x16_t& sn) LMK_INL {
+    zero16(sn);
+    u32x4_t fk[C::KS];
+    constexpr int PFX = 2;
+#pragma unroll
+    for (int ks = 0; ks < PFX; ++ks) fk[ks] = lds_ld128(kx[ks] + nslot);
+    const float s_last = s[15];
+    float mx = 0.f, mloc = 0.f, t_lm = 0.f, den = 0.f, f = 0.f;
+    auto ywork = [&](int u) LMK_INL {
+      if (u == 0) {
+        mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+        mx = fmaxf(fmaxf(mx, s[3]), s[4]);
+        mx = fmaxf(fmaxf(mx, s[5]), s[6]);
+        mx = fmaxf(fmaxf(mx, s[7]), s[8]);
+      } else if (u == 1) {
+        mx = fmaxf(fmaxf(mx, s[9]), s[10]);
+        mx = fmaxf(fmaxf(mx, s[11]), s[12]);
+        mx = fmaxf(fmaxf(mx, s[13]), s[14]);
+        mx = fmaxf(mx, (h == 0) ? s_last : -INFINITY);
+        mx = pair_max(mx);
+        t_lm = pair_hi(s_last) * c2;
+        mloc = mx * c2;
+      } else if (u < 10) {
+#pragma unroll
+        for (int r = 2 * (u - 2); r < 2 * (u - 2) + 2; ++r) {
+          float x = fast_exp2(__builtin_fmaf(s[r], c2, -mloc));
+          if (r == 15) x = (h == 0) ? x : 0.f;             // the landmark's value row never contributes
+          s[r] = x;
+          den += x;
+        }
+      } else if (u == 10) {
+        den = pair_sum(den);
+      } else if (u == 11) {
+        const float g = fast_exp2(t_lm - Rref);             // the block's share of the global bucket
+        lsum += g;
+        f = g * fast_rcp(den);
+      } else {
+#pragma unroll
+        for (int r = 4 * (u - 12); r < 4 * (u - 12) + 4; ++r) {
+          s[r] *= f;
+          if (r & 1) {
+            uint32_t pk = pack2<T>(s[r - 1], s[r]);
+            asm volatile("" : "+v"(pk));                    // pins this slice between its two MFMAs
+            pf[r >> 3][(r >> 1) & 3] = pk;
+          }
+        }
       }
+    };
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < C::KS; ++m) {
+      if (m + PFX < C::KS) fk[m + PFX] = lds_ld128(kx[m + PFX] + nslot);
+      sn = mfma32<T>(fk[m], qf[m], sn);
+#pragma unroll
+      for (int u = (m * 16) / C::KS; u < ((m + 1) * 16) / C::KS; ++u) ywork(u);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
-  // move the reference maximum when a new score x (log2 domain) outgrows it; rare
-  auto lazy_max = [&](float x) {
-    Mtrue = fmaxf(Mtrue, x);
-    if (__any(x > Mref + C::LAZY)) {
-      const float Mnew = (x > Mref + C::LAZY) ? x : Mref;
-      const float alpha = fast_exp2(Mref - Mnew);          // 1 for lanes that keep their reference
-      Mref = Mnew;
-      lsum *= alpha;
-#pragma unroll
-      for (int dc = 0; dc < C::DC; ++dc)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[dc][r] *= alpha;
-    }
-  };
-  // earlier block: weights gate * P_local from raw scores s; t_lm = its landmark score (log2 domain)
-  auto earlier_weights = [&](const f32x16_t& s, float t_lm, float* w) {
-    float m0 = (h == 0) ? s[15] : -INFINITY;
-#pragma unroll
-    for (int r = 0; r < 15; ++r) m0 = fmaxf(m0, s[r]);
-    const float mloc = pair_max(m0) * c2;
-    float den = 0.f;
+  // the wave's own block: its visible keys join the global bucket; reference moves from R to max(R, own maximum)
+  float Mfin = 0.f;
+  auto stage_y_diag = [&](const f32x16_t& s) LMK_INL {
+    const int lim = ql - ((ql == 31) ? 1 : 0);             // the landmark query looks one to the left
+    float x[16], mt = -1e30f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      float e = fast_exp2(__builtin_fmaf(s[r], c2, -mloc));
-      if (r == 15) e = (h == 0) ? e : 0.f;
-      w[r] = e;
-      den += e;
+      const int key = 8 * (r >> 2) + 4 * h + (r & 3);
+      x[r] = (key <= lim) ? s[r] * c2 : -INFINITY;
+      mt = fmaxf(mt, x[r]);
     }
-    den = pair_sum(den);
-    const float gate = fast_exp2(t_lm - Mref);
-    lsum += gate;
-    const float f = gate * fast_rcp(den);
+    Mfin = fmaxf(Rref, pair_max(mt));
+    const float alpha = fast_exp2(Rref - Mfin);            // 0 when there was no earlier block
+    lsum *= alpha;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) w[r] *= f;
+    for (int dc = 0; dc < C::DC; ++dc)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[dc][r] *= alpha;
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      x[r] = fast_exp2(x[r] - Mfin);
+      sum += x[r];
+    }
+    lsum += pair_sum(sum);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      u32x4_t fr = {pack2<T>(x[8 * j + 0], x[8 * j + 1]), pack2<T>(x[8 * j + 2], x[8 * j + 3]),
+                    pack2<T>(x[8 * j + 4], x[8 * j + 5]), pack2<T>(x[8 * j + 6], x[8 * j + 7])};
+      pf[j] = fr;
+    }
   };
 
+  // ---- prologue: landmark tiles 0, 1 and blocks 0 .. 2 requested; all but block 2 must have landed
+  if (n_lt > 0) request_lm(0);
+  if (n_lt > 1) request_lm(1);
+#pragma unroll
+  for (int t = 0; t < C::NBUF - 1; ++t) request(t * C::BUF_BYTES, t);
+  fw_wait_vmcnt<C::PER_TILE>();
+  __syncthreads();
+
+  // ---- first pass: R = max over the earlier blocks' landmark scores (log2 domain)
+  {
+    float mx = -1e30f;
+    for (int lt = 0; lt < n_lt; ++lt) {
+      if (lt >= C::LM_TILES) {                             // requested one iteration ago, one newer request behind it
+        fw_wait_vmcnt<1>();
+        __syncthreads();
+      }
+      f32x16_t s;
+      stage_x(C::LM_OFF + (lt & 1) * C::BLK_BYTES, s);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int b = 32 * lt + 8 * (r >> 2) + 4 * h + (r & 3);
+        mx = fmaxf(mx, (b < cblk) ? s[r] : -1e30f);
+      }
+      if (n_lt > C::LM_TILES) {                            // long sequences: keep streaming tiles (wave-uniform)
+        __syncthreads();                                   // everyone has read this slot
+        request_lm(lt + C::LM_TILES);                      // past the last tile: a re-read that is never used
+      }
+    }
+    mx = pair_max(mx);
+    Rref = (cblk > 0) ? mx * c2 : -1e30f;
+  }
+
+  f32x16_t sA, sB;                                         // S^T of the even / odd blocks
+  zero16(sB);
+  stage_x(0, sA);
+
+  auto period = [&](auto Rc, int k) LMK_INL {
+    constexpr int R = decltype(Rc)::value;
+    constexpr int CUR = R * C::BUF_BYTES, NXT = ((R + 1) % C::NBUF) * C::BUF_BYTES;
+    request(((R + 3) % C::NBUF) * C::BUF_BYTES, k + 3);    // into the slot block k-1 has left
+    if (waveok && k <= cblk) {
+      f32x16_t& s = (R & 1) ? sB : sA;
+      f32x16_t& sn = (R & 1) ? sA : sB;
+      if (k < cblk) stage_xy(NXT, s, sn);
+      else stage_y_diag(s);
+      stage_z(CUR + C::BLK_BYTES);
+    }
+    fw_wait_vmcnt<C::PER_TILE>();                          // block k+2 has landed (k+3 may be in flight)
+    __syncthreads();
+  };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
-
-  // ---- prologue: blocks 0, 1 in LDS; blocks 2..5 in flight in register sets 2, 3, 0, 1
-  gload(I0{}, 0);
-  gload(I1{}, 1);
-  gload(I2{}, 2);
-  gload(I3{}, 3);
-  lstore(I0{});
-  lstore(I1{});
-  gload(I0{}, 4);
-  gload(I1{}, 5);
-  __syncthreads();
-
-  // ---- main loop: blocks 0 .. c0-1 are earlier blocks for all waves
-  f32x16_t s_cur;
-  if (c0 > 0) s_cur = qk_tile(0);
-  auto iter = [&](auto Rc, int b) {
-    constexpr int R = decltype(Rc)::value;
-    constexpr int CUR = R * C::BUF_BYTES, NXT = ((R + 1) % 4) * C::BUF_BYTES;
-    using FIL = std::integral_constant<int, (R + 2) % 4>;
-    lstore(FIL{});                                         // block b+2 (loaded four iterations ago)
-    gload(FIL{}, b + 6);
-    const float t_lm = pair_hi(s_cur[15]) * c2;
-    lazy_max(t_lm);
-    const f32x16_t s_next = qk_tile(NXT);                  // block b+1
-    float w[16];
-    earlier_weights(s_cur, t_lm, w);
-    pv_tile(CUR + C::BLK_BYTES, w);
-    s_cur = s_next;
-    __syncthreads();
-  };
-  for (int b = 0; b < c0; b += 4) {
-    iter(I0{}, b);
-    if (b + 1 < c0) iter(I1{}, b + 1);
-    if (b + 2 < c0) iter(I2{}, b + 2);
-    if (b + 3 < c0) iter(I3{}, b + 3);
+  for (int k = 0; k < nblk; k += 4) {
+    period(I0{}, k);
+    if (k + 1 < nblk) period(I1{}, k + 1);
+    if (k + 2 < nblk) period(I2{}, k + 2);
+    if (k + 3 < nblk) period(I3{}, k + 3);
   }
+  fw_wait_vmcnt<0>();                                      // nothing may still be writing LDS when the wave ends
 
-  // ---- per-wave blocks c0 .. nblk-1 (ring positions continue; register set = block % 4)
-  auto tail = [&](auto Rc, int blk) {
-    constexpr int R = decltype(Rc)::value;
-    constexpr int CUR = R * C::BUF_BYTES;
-    using FIL = std::integral_constant<int, (R + 2) % 4>;
-    lstore(FIL{});
-    gload(FIL{}, blk + 6);
-    if (blk <= cblk) {
-      const f32x16_t s = qk_tile(CUR);
-      float w[16];
-      if (blk < cblk) {
-        const float t_lm = pair_hi(s[15]) * c2;
-        lazy_max(t_lm);
-        earlier_weights(s, t_lm, w);
-      } else {
-        const int lim = ql - ((ql == 31) ? 1 : 0);         // the landmark query looks one to the left
-        float x[16], mt = -INFINITY;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = 8 * (r >> 2) + 4 * h + (r & 3);
-          x[r] = (key <= lim) ? s[r] * c2 : -INFINITY;
-          mt = fmaxf(mt, x[r]);
-        }
-        lazy_max(pair_max(mt));
-        float sum = 0.f;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          w[r] = fast_exp2(x[r] - Mref);
-          sum += w[r];
-        }
-        lsum += pair_sum(sum);
-      }
-      pv_tile(CUR + C::BLK_BYTES, w);
-    }
-    __syncthreads();
-  };
-  for (int blk = c0; blk < nblk; ++blk) {
-    switch (blk & 3) {
-      case 0: tail(I0{}, blk); break;
-      case 1: tail(I1{}, blk); break;
-      case 2: tail(I2{}, blk); break;
-      default: tail(I3{}, blk); break;
-    }
-  }
-
-  if (qrow < p.Lq) {
+  if (rowok) {
     const float inv = 1.0f / lsum;
 #pragma unroll
     for (int dc = 0; dc < C::DC; ++dc)
@@ -284,12 +381,14 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
                       pack2<T>(acc[dc][4 * g + 2] * inv, acc[dc][4 * g + 3] * inv)};
         *(u32x2_t*)(op + 2 * ((int64_t)qrow * p.os_r + 32 * dc + 8 * g + 4 * h)) = o2;
       }
-    if (h == 0) {                                          // statistics relative to the true maximum
-      p.L[(int64_t)bh * p.Lq + qrow] = lsum * fast_exp2(Mref - Mtrue);
-      p.M[(int64_t)bh * p.Lq + qrow] = Mtrue * kLn2;
+    if (h == 0) {                                          // statistics of the global bucket, relative to its maximum
+      p.L[(int64_t)bh * p.Lq + qrow] = lsum;
+      p.M[(int64_t)bh * p.Lq + qrow] = Mfin * kLn2;
     }
   }
 }
+
+#undef LMK_INL
 
 template <class T, int D>
 static int launch_fwd32_t(const FwdParams& p, hipStream_t stream) {
