@@ -2,17 +2,18 @@
 // block = 32 keys.
 //
 // Query-stationary, S^T layout (lane = query): a workgroup is 8 waves = 256 query rows, two waves
-// per SIMD; wave w owns landmark block c0 + w and keeps Q and dO fragments (B operands) and its
-// dQ^T accumulator in registers.  K/V blocks stream through a ring of six LDS slots filled by
-// direct global->LDS loads (tile k+4 is requested while tile k is computed; vmcnt is counted by
-// hand, two requests per wave and tile).  Per block a wave does three things:
+// per SIMD; wave w owns landmark block c0 + w and keeps its Q fragments (B operands) and its dQ^T
+// accumulator in registers; its 32 rows of dO sit in LDS (both in registers would pass the register
+// budget).  K/V blocks stream through a ring of four LDS slots filled by direct global->LDS loads
+// (block k+3 is requested while block k is computed; vmcnt is counted by hand, two requests per
+// wave and block).  Per block a wave does three things:
 //     X  S^T = K Q^T and dP^T = V dO^T                       16 MFMA, row fragments from LDS
 //     Y  local softmax, gate, nD, dS (and the terms a, nD, dS_landmark)      vector ALU only
 //     Z  dQ^T += K^T dS^T                                     8 MFMA, transposed fragments
-// The two waves of a SIMD would run X, Y, Z in lock-step behind the per-block barrier and fight
-// for the same pipe, so the upper four waves run half a period late: between two barriers the
-// lower waves do X(k) Y(k) Z(k) while the upper waves do Z(k-1) X(k) Y(k); one group's vector
-// phase then overlaps the other group's matrix phase.  A slot stays valid for two periods.
+// X of block k+1 is interleaved, MFMA by MFMA, with Y of block k (the wave issues in order, so the
+// instruction stream is the schedule); Z of block k follows, its operands fetched two MFMAs ahead.
+// The prologue also computes delta = rowsum(O * dO) and mhat = M log2(e) + log2(L) of the wave's
+// rows (the reference's _bwd_preprocess, llama/ltriton/flash_landmark_attention.py:125-149).
 // The per-block terms are collected in LDS and flushed to global memory every 8 blocks, so that
 // stores do not sit between the hand-counted loads.
 #include <type_traits>
