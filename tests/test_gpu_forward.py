@@ -60,6 +60,27 @@ def test_forward_matches_oracle(B, H, Lq, Lk, D, block, dtype):
     assert err <= TOL, err
 
 
+@pytest.mark.parametrize("Lq,Lk", [(4608, 4608), (256, 4352), (300, 2860)])
+def test_long_history_streams_the_landmark_tiles(Lq, Lk):
+    # more than 64 earlier blocks: the block-32 kernel's first pass (reference maximum from the landmark
+    # keys alone) runs past the two landmark tiles it fetches up front; statistics checked as well
+    from landmark_hip.attention import _launch_fwd
+    B, H, D, block = 1, 2, 128, 32
+    print(f"case long Lq{Lq} Lk{Lk}", flush=True)
+    q, k, v = make_qkv(B, H, Lq, Lk, D, seed=Lq + Lk)
+    rows = sorted({0, 1, 31, 32, 33, Lq // 2, Lq - 33, Lq - 32, Lq - 2, Lq - 1})
+    from oracle import s1
+    qf, kf, vf = (t.float()[0] for t in (q, k, v))
+    ref, L_ref, M_ref = s1.s1_attention(qf, kf, vf, block, rows=rows, return_stats=True)
+    dev = torch.device("cuda:0")
+    o, L, M = _launch_fwd(q.to(dev), k.to(dev), v.to(dev), (Lk - Lq) // block, 1 / math.sqrt(D), block)
+    torch.cuda.synchronize()
+    o, L, M = o.float().cpu()[0], L.cpu().view(H, Lq), M.cpu().view(H, Lq)
+    assert (o[:, rows] - ref).abs().max().item() <= TOL
+    assert (M[:, rows] - M_ref).abs().max() < 1e-3
+    assert ((L[:, rows] - L_ref).abs() / L_ref).max() < 1e-3
+
+
 def test_statistics_L_and_M_match_oracle():
     from landmark_hip.attention import _launch_fwd
     B, H, Lq, Lk, D, block = 1, 4, 192, 256, 128, 32
