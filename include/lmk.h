@@ -28,7 +28,7 @@ extern "C" {
 #define LMK_OK 0
 #define LMK_ERR_NULL (-1)        /* a required pointer is NULL */
 #define LMK_ERR_SHAPE (-2)       /* non-positive or inconsistent sizes */
-#define LMK_ERR_UNSUPPORTED (-3) /* head dim / block size / dtype outside the built set */
+#define LMK_ERR_UNSUPPORTED (-3) /* head dim / block size / dtype outside the built set, or rows * row stride of a slice >= 4 GiB */
 #define LMK_ERR_ALIGN (-4)       /* pointer or stride not 16-byte aligned */
 #define LMK_ERR_HISTORY (-5)     /* Lk - Lq is not n_prefix * block */
 #define LMK_ERR_PARTIAL (-6)     /* backward needs Lq and Lk to be whole blocks */

@@ -13,8 +13,12 @@ int check_tensor(const lmk_tensor4* t) {
   if (t == nullptr || t->ptr == nullptr) return LMK_ERR_NULL;
   if (!aligned16(t->ptr) || !stride_ok(t->stride_b) || !stride_ok(t->stride_h) || !stride_ok(t->stride_row))
     return LMK_ERR_ALIGN;
+  if (t->stride_row <= 0) return LMK_ERR_SHAPE;   // rows are walked forwards
   return LMK_OK;
 }
+
+// The kernels address the rows of one (batch, head) slice with 32-bit byte offsets.
+bool slice_fits_32bit(const lmk_tensor4* t, int rows) { return (int64_t)rows * t->stride_row * 2 < ((int64_t)1 << 32); }
 
 int check_common(int B, int H, int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype) {
   if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || n_prefix < 0) return LMK_ERR_SHAPE;
@@ -71,7 +75,8 @@ const char* lmk_strerror(int code) {
     case LMK_OK: return "ok";
     case LMK_ERR_NULL: return "a required pointer is NULL";
     case LMK_ERR_SHAPE: return "non-positive or inconsistent sizes";
-    case LMK_ERR_UNSUPPORTED: return "unsupported head dim (64,128), block size (32,64,128) or dtype (bf16,f16)";
+    case LMK_ERR_UNSUPPORTED:
+      return "unsupported head dim (64,128), block size (32,64,128) or dtype (bf16,f16), or a (batch, head) slice of 4 GiB or more";
     case LMK_ERR_ALIGN: return "pointer or stride not 16-byte aligned";
     case LMK_ERR_HISTORY: return "Lk - Lq must equal n_prefix * block";
     case LMK_ERR_PARTIAL: return "backward supported only for full blocks";
@@ -95,6 +100,8 @@ int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o))) return rc;
   if (L == nullptr || M == nullptr) return LMK_ERR_NULL;
   if ((rc = check_common(B, H, Lq, Lk, D, sm_scale, block, n_prefix, dtype))) return rc;
+  if (!slice_fits_32bit(q, Lq) || !slice_fits_32bit(o, Lq) || !slice_fits_32bit(k, Lk) || !slice_fits_32bit(v, Lk))
+    return LMK_ERR_UNSUPPORTED;
   lmk::FwdParams p;
   p.q = q->ptr; p.k = k->ptr; p.v = v->ptr; p.o = o->ptr;
   p.L = L; p.M = M;
@@ -137,6 +144,9 @@ int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
   if (L == nullptr || M == nullptr || workspace == nullptr) return LMK_ERR_NULL;
   if ((rc = check_common(B, H, Lq, Lk, D, sm_scale, block, n_prefix, dtype))) return rc;
   if (Lq % block != 0 || Lk % block != 0) return LMK_ERR_PARTIAL;
+  if (!slice_fits_32bit(q, Lq) || !slice_fits_32bit(o, Lq) || !slice_fits_32bit(dout, Lq) || !slice_fits_32bit(dq, Lq) ||
+      !slice_fits_32bit(k, Lk) || !slice_fits_32bit(v, Lk) || !slice_fits_32bit(dk, Lk) || !slice_fits_32bit(dv, Lk))
+    return LMK_ERR_UNSUPPORTED;
   if (!aligned16(workspace)) return LMK_ERR_ALIGN;
   if (workspace_bytes < lmk_attn_bwd_workspace_bytes(B, H, Lq, Lk, block)) return LMK_ERR_WORKSPACE;
   lmk::BwdParams p;

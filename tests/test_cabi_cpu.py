@@ -58,6 +58,8 @@ def test_forward_argument_errors(lib):
     assert _fwd(lib, q=_t4(ptr=0)) == -1                      # NULL
     assert _fwd(lib, L=0) == -1
     assert _fwd(lib, q=_t4(ptr=0x1008)) == -4                 # misaligned pointer
+    assert _fwd(lib, q=_t4(sr=-128)) == -2                    # rows are walked forwards
+    assert _fwd(lib, k=_t4(sr=1 << 26), Lq=64, Lk=64) == -3   # 64 rows x 2^26 elements x 2 bytes = 8 GiB per slice
     assert _fwd(lib, k=_t4(sr=130)) == -4                     # misaligned row stride
     assert _fwd(lib, B=0) == -2
     assert _fwd(lib, D=96) == -3
