@@ -12,7 +12,10 @@
 //          the third kernel needs:  a  with  gate*P = exp2(s*c - a),  nD,  and dS at the
 //          block's landmark key.
 //   dkdv   key-stationary, S layout (lane = key): purely elementwise between its four
-//          products S = Q K^T, dP = dO V^T, dV^T += dO^T W, dK^T += Q^T dS.
+//          products S = Q K^T, dP = dO V^T, dV^T += dO^T W, dK^T += Q^T dS
+//          (lmk_bwd_dkdv32.hip, all block sizes).
+// This file holds the pre kernel, the dQ kernel for blocks of 64 and 128 keys (block 32 has its own in
+// lmk_bwd_dq32.hip) and the dispatch.
 //
 // All probabilities are used normalised (exp2(s*c - mhat) already divides by L), so dO is
 // consumed as is; the reference's rescaled copy dO/L (:147) is not needed.
@@ -270,222 +273,6 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dq_kernel(BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// dk, dv
-// ---------------------------------------------------------------------------
-template <class T, int D, int BS>
-struct DkvCfg {
-  static constexpr int NT = BS / 32;
-  static constexpr int SQ = 64;                          // query rows per LDS stage
-  static constexpr int CH = D / 8;
-  static constexpr int TILE_BYTES = SQ * 2 * D;          // one stage of Q (or of dO)
-  static constexpr int NCH = SQ * CH / 256;
-  static constexpr int KS = D / 16;
-  static constexpr int DC = D / 32;
-  static constexpr int LDS_BYTES = 4 * TILE_BYTES;
-};
-
-template <class T, int D, int BS>
-__global__ __launch_bounds__(256, 1) void lmk_bwd_dkdv_kernel(BwdParams p) {
-  using C = DkvCfg<T, D, BS>;
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int ql = lane & 31, h = lane >> 5;
-
-  int bh, kvt;   // workgroup -> (batch*head, 128-key tile); tiles with most work (small kvt) first
-  {
-    const int bid = blockIdx.x, BH = p.B * p.H;
-    if ((BH & 7) == 0) {
-      const int xcd = bid & 7, j = bid >> 3, ngrp = BH >> 3;
-      kvt = j / ngrp;
-      bh = (j % ngrp) * 8 + xcd;
-    } else {
-      kvt = bid / BH;
-      bh = bid % BH;
-    }
-  }
-  const int b = bh / p.H, hh = bh % p.H;
-  const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h);
-  const char* kp = (const char*)p.k + 2 * (b * p.ks_b + hh * p.ks_h);
-  const char* vp = (const char*)p.v + 2 * (b * p.vs_b + hh * p.vs_h);
-  const char* gp = (const char*)p.dout + 2 * (b * p.dos_b + hh * p.dos_h);
-  char* dkp = (char*)p.dk + 2 * (b * p.dks_b + hh * p.dks_h);
-  char* dvp = (char*)p.dv + 2 * (b * p.dvs_b + hh * p.dvs_h);
-
-  const int kt = kvt * 4 + wave;                         // this wave's 32-key tile
-  const bool active = kt < (p.Lk >> 5);
-  const int krow = kt * 32 + ql;
-  const int bk = kt / C::NT, ksub = kt % C::NT;
-  const bool lm_lane = (ksub == C::NT - 1) && (ql == 31);  // this lane's key is a landmark
-  const int PT = p.n_prefix * C::NT;                     // history in 32-key tiles
-  const int nq = p.Lq >> 5;                              // 32-row query tiles
-
-  // K and V fragments stay in registers as B operands (column = key, k = head dim)
-  u32x4_t kf[C::KS], vf[C::KS];
-#pragma unroll
-  for (int ks = 0; ks < C::KS; ++ks) {
-    u32x4_t z = {0, 0, 0, 0};
-    kf[ks] = z;
-    vf[ks] = z;
-    if (active) {
-      kf[ks] = *(const u32x4_t*)(kp + 2 * ((int64_t)krow * p.ks_r + 16 * ks + 8 * h));
-      vf[ks] = *(const u32x4_t*)(vp + 2 * ((int64_t)krow * p.vs_r + 16 * ks + 8 * h));
-    }
-  }
-
-  u32x4_t qreg[C::NCH], greg[C::NCH];
-  auto load_stage = [&](int s) {
-#pragma unroll
-    for (int i = 0; i < C::NCH; ++i) {
-      const int id = tid + 256 * i, row = id / C::CH, ch = id % C::CH;
-      const int qr = s * C::SQ + row;
-      u32x4_t z = {0, 0, 0, 0};
-      qreg[i] = z;
-      greg[i] = z;
-      if (qr < p.Lq) {
-        qreg[i] = *(const u32x4_t*)(qp + 2 * ((int64_t)qr * p.qs_r + 8 * ch));
-        greg[i] = *(const u32x4_t*)(gp + 2 * ((int64_t)qr * p.dos_r + 8 * ch));
-      }
-    }
-  };
-  auto store_stage = [&](int buf) {
-    unsigned char* qb = smem + buf * 2 * C::TILE_BYTES;
-    unsigned char* gb = qb + C::TILE_BYTES;
-#pragma unroll
-    for (int i = 0; i < C::NCH; ++i) {
-      const int id = tid + 256 * i, row = id / C::CH, ch = id % C::CH;
-      *(u32x4_t*)(qb + tile_off<D>(row, ch)) = qreg[i];
-      *(u32x4_t*)(gb + tile_off<D>(row, ch)) = greg[i];
-    }
-  };
-
-  f32x16_t dkacc[C::DC], dvacc[C::DC];
-#pragma unroll
-  for (int dc = 0; dc < C::DC; ++dc)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      dkacc[dc][r] = 0.f;
-      dvacc[dc][r] = 0.f;
-    }
-  const float c2 = p.scale_log2;
-
-  // first query tile any wave of this workgroup needs: its diagonal tile index PT + j >= kvt*4
-  const int j_first = max(0, kvt * 4 - PT);
-  const int s_first = j_first / 2;
-  const int s_end = (nq + 1) / 2;
-
-  if (s_first < s_end) {
-    load_stage(s_first);
-    store_stage(s_first & 1);
-  }
-  __syncthreads();
-
-  for (int s = s_first; s < s_end; ++s) {
-    const int buf = s & 1;
-    if (s + 1 < s_end) load_stage(s + 1);
-    const unsigned char* qb = smem + buf * 2 * C::TILE_BYTES;
-    const unsigned char* gb = qb + C::TILE_BYTES;
-
-#pragma unroll
-    for (int jj = 0; jj < 2; ++jj) {
-      const int j = 2 * s + jj;                          // 32-row query tile
-      const int dtq = PT + j;                            // its diagonal key tile
-      if (active && j < nq && dtq >= kt) {
-        const int cq = dtq / C::NT, qsub = dtq % C::NT;
-        const int rb = 32 * jj;
-        f32x16_t sc, dp;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          sc[r] = 0.f;
-          dp[r] = 0.f;
-        }
-#pragma unroll
-        for (int ks = 0; ks < C::KS; ++ks) sc = mfma32<T>(load_row_frag<D>(qb, rb, ks, lane), kf[ks], sc);
-#pragma unroll
-        for (int ks = 0; ks < C::KS; ++ks) dp = mfma32<T>(load_row_frag<D>(gb, rb, ks, lane), vf[ks], dp);
-
-        // register r <-> query row 32j + 8*(r/4) + 4h + r%4 ; lane <-> key ql of the tile
-        float w[16], ds[16];
-        const int64_t rowbase = (int64_t)bh * p.Lq + 32 * j + 4 * h;
-        if (cq == bk) {
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const float4 mh = *(const float4*)(p.mhat + rowbase + 8 * g);
-            const float4 dl = *(const float4*)(p.delta + rowbase + 8 * g);
-            const float mha[4] = {mh.x, mh.y, mh.z, mh.w}, dla[4] = {dl.x, dl.y, dl.z, dl.w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int r = 4 * g + e;
-              const int qloc = 8 * g + 4 * h + e;
-              const int lim = qloc - ((qsub == C::NT - 1 && qloc == 31) ? 1 : 0);
-              const bool vis = (dtq > kt) || (ql <= lim);
-              const float pr = vis ? fast_exp2(__builtin_fmaf(sc[r], c2, -mha[e])) : 0.f;
-              w[r] = pr;
-              ds[r] = pr * (dp[r] - dla[e]);
-            }
-          }
-        } else {
-          const int64_t sbase = ((int64_t)bh * p.n_blocks + bk) * p.Lq + 32 * j + 4 * h;
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const float4 sa = *(const float4*)(p.stat_a + sbase + 8 * g);
-            const float4 sn = *(const float4*)(p.stat_n + sbase + 8 * g);
-            const float saa[4] = {sa.x, sa.y, sa.z, sa.w}, sna[4] = {sn.x, sn.y, sn.z, sn.w};
-            if (!lm_lane) {
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int r = 4 * g + e;
-                const float wt = fast_exp2(__builtin_fmaf(sc[r], c2, -saa[e]));
-                w[r] = wt;
-                ds[r] = wt * (dp[r] - sna[e]);
-              }
-            } else {
-              const float4 mh = *(const float4*)(p.mhat + rowbase + 8 * g);
-              const float4 dl = *(const float4*)(p.delta + rowbase + 8 * g);
-              const float mha[4] = {mh.x, mh.y, mh.z, mh.w}, dla[4] = {dl.x, dl.y, dl.z, dl.w};
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int r = 4 * g + e;
-                w[r] = 0.f;
-                ds[r] = fast_exp2(__builtin_fmaf(sc[r], c2, -mha[e])) * (sna[e] - dla[e]);
-              }
-            }
-          }
-        }
-#pragma unroll
-        for (int j2 = 0; j2 < 2; ++j2) {
-          u32x4_t wf = {pack2<T>(w[8 * j2 + 0], w[8 * j2 + 1]), pack2<T>(w[8 * j2 + 2], w[8 * j2 + 3]),
-                        pack2<T>(w[8 * j2 + 4], w[8 * j2 + 5]), pack2<T>(w[8 * j2 + 6], w[8 * j2 + 7])};
-          u32x4_t df = {pack2<T>(ds[8 * j2 + 0], ds[8 * j2 + 1]), pack2<T>(ds[8 * j2 + 2], ds[8 * j2 + 3]),
-                        pack2<T>(ds[8 * j2 + 4], ds[8 * j2 + 5]), pack2<T>(ds[8 * j2 + 6], ds[8 * j2 + 7])};
-#pragma unroll
-          for (int dc = 0; dc < C::DC; ++dc) {
-            dvacc[dc] = mfma32<T>(load_tr_frag<D>(gb, rb, j2, dc, lane), wf, dvacc[dc]);
-            dkacc[dc] = mfma32<T>(load_tr_frag<D>(qb, rb, j2, dc, lane), df, dkacc[dc]);
-          }
-        }
-      }
-    }
-    if (s + 1 < s_end) store_stage(buf ^ 1);
-    __syncthreads();
-  }
-
-  if (active) {
-    const float scl = p.scale;
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2_t k2 = {pack2<T>(dkacc[dc][4 * g + 0] * scl, dkacc[dc][4 * g + 1] * scl),
-                      pack2<T>(dkacc[dc][4 * g + 2] * scl, dkacc[dc][4 * g + 3] * scl)};
-        u32x2_t v2 = {pack2<T>(dvacc[dc][4 * g + 0], dvacc[dc][4 * g + 1]),
-                      pack2<T>(dvacc[dc][4 * g + 2], dvacc[dc][4 * g + 3])};
-        *(u32x2_t*)(dkp + 2 * ((int64_t)krow * p.dks_r + 32 * dc + 8 * g + 4 * h)) = k2;
-        *(u32x2_t*)(dvp + 2 * ((int64_t)krow * p.dvs_r + 32 * dc + 8 * g + 4 * h)) = v2;
-      }
-  }
-}
-
-// ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
 template <class T, int D, int BS>
@@ -508,16 +295,8 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
     hipLaunchKernelGGL(kern, dim3(p.n_qtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
   }
-  if ((phases & 4) && BS == 32) {
-    return launch_bwd_dkdv32(p, D, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream);
-  }
   if (phases & 4) {
-    using C = DkvCfg<T, D, BS>;
-    auto kern = lmk_bwd_dkdv_kernel<T, D, BS>;
-    static std::atomic<uint64_t> lds_ok{0};
-    if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
-    hipLaunchKernelGGL(kern, dim3(p.n_kvtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
-    if ((rc = (int)hipGetLastError())) return rc;
+    return launch_bwd_dkdv32(p, D, BS, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream);
   }
   return 0;
 }

@@ -1,4 +1,6 @@
-// dK/dV kernel of the backward pass, landmark block = 32 keys.
+// dK/dV kernel of the backward pass.  Written for a landmark block of 32 keys (one MFMA tile) and
+// extended to blocks of 64 and 128 keys, which are 2 or 4 key tiles: what changes is which block a key
+// tile belongs to (its terms, its landmark lane) and which query tiles share that block.
 //
 // Key-stationary.  A workgroup is 8 waves = 4 key tiles of 32 keys x 2 roles; the two waves of a
 // key tile sit on the same SIMD (waves t and t+4) and split the work so that each holds one
@@ -27,8 +29,9 @@
 
 namespace lmk {
 
-template <class T, int D>
+template <class T, int D, int BS = 32>
 struct Dkv32Cfg {
+  static constexpr int TPB = BS / 32;                      // key (and query) tiles per landmark block
   static constexpr int NKT = 4;                            // key tiles per workgroup
   static constexpr int NW = 2 * NKT;
   static constexpr int NTHR = 64 * NW;
@@ -67,9 +70,9 @@ __device__ __forceinline__ void wait_vmcnt() {             // s_waitcnt vmcnt(N)
 
 #define LMK_INL __attribute__((always_inline))
 
-template <class T, int D>
+template <class T, int D, int BS>
 __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
-  using C = Dkv32Cfg<T, D>;
+  using C = Dkv32Cfg<T, D, BS>;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -93,12 +96,13 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   const char* qp = (const char*)p.q + 2 * (b_ * p.qs_b + hh * p.qs_h);
   const char* gp = (const char*)p.dout + 2 * (b_ * p.dos_b + hh * p.dos_h);
 
-  const int nkt = p.Lk >> 5;                               // key tiles (= landmark blocks)
+  const int nkt = p.Lk >> 5;                               // key tiles (TPB per landmark block)
   const int kt = kvt * C::NKT + tile;
   const bool active = kt < nkt;
   const int krow = kt * 32 + ql;
-  const bool lm_lane = (ql == 31);                         // this lane's key is its block's landmark
-  const int PT = p.n_prefix;                               // history blocks in front of the queries
+  const bool lm_lane = (ql == 31) && (kt % C::TPB == C::TPB - 1);   // this lane's key is its block's landmark
+  const int PT = p.n_prefix * C::TPB;                      // history tiles in front of the queries
+  const int kt_end = (kt / C::TPB + 1) * C::TPB;           // first tile behind this key tile's block
   const int nq = p.Lq >> 5;
   const float c2 = p.scale_log2;
 
@@ -138,7 +142,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   const float* st_src;                                     // this lane's 16 bytes of terms for query tile 0
   {
     const int arr = min(lane / 8, 4), part = lane % 8;     // 0: a, 1: nD, 2: dS at landmark, 3: mhat, 4..: delta
-    const int bk = min(kt, p.n_blocks - 1);
+    const int bk = min(kt / C::TPB, p.n_blocks - 1);
     const int64_t plane_row = ((int64_t)bh * p.n_blocks + bk) * p.Lq, head_row = (int64_t)bh * p.Lq;
     st_src = (arr == 0) ? p.stat_a + plane_row : (arr == 1) ? p.stat_n + plane_row : (arr == 2) ? p.stat_l + plane_row
              : (arr == 3) ? p.mhat + head_row : p.delta + head_row;
@@ -216,6 +220,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     constexpr bool MASKED = decltype(Mc)::value;
     const int CST = cslot + 2 * C::TILE_BYTES + tile * 1024;   // this key tile's terms: a, nD, dslm, mhat, delta
     const int krel = 32 * (kt - (PT + i)) + ql;            // key position relative to the query tile's first row
+    const bool lmq = (PT + i) % C::TPB == C::TPB - 1;      // the tile's last row is its block's landmark query
     const int xoff = (MASKED ? CST + 384 : (lm_lane ? C::CONST_OFF : CST)) + 16 * h;
     // terms of rows 8g + 4h .. +3, fetched two MFMA slots ahead of the slice that uses them (slot m works
     // on registers r with r / 4 == grp(m)): at the top of the iteration only what the first MFMA and the
@@ -232,7 +237,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       if (MASKED) {
         // key visible to this query row?  the landmark row of a block looks one position to the left
         const int qloc = 8 * g + 4 * h + e;
-        ex = (krel <= qloc - ((qloc == 31) ? 1 : 0)) ? ex : 0.f;
+        ex = (krel <= qloc - ((qloc == 31 && lmq) ? 1 : 0)) ? ex : 0.f;
       }
       w[r] = ex;
       if (r & 1) {
@@ -274,7 +279,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 
   // ---- K role: dP of tile i (slot cslot) interleaved with dS of tile i-1 (slot pslot), then dK of tile i-1.
   auto body_k = [&](int i, int cslot, int pslot, int rslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc, auto sync) LMK_INL {
-    const bool masked = PT + (i - 1) <= kt;                // tile i-1: own block or not yet visible
+    const bool masked = PT + (i - 1) < kt_end;             // tile i-1: in the key tile's block or not yet visible
     const int CST = pslot + 2 * C::TILE_BYTES + tile * 1024;
     // y: subtrahend of dP, z: addend of dS  (byte offsets of 32-float arrays)
     const int yoff = (masked ? CST + 512 : CST + 128) + 16 * h;
@@ -398,7 +403,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     // own block and tiles that cannot see these keys yet come first, then every later tile sees all keys:
     // two loops, so that each has one code path and the accumulators stay where they are
     int i = j_first;
-    const int i_full = min(nq, max(j_first, kt - PT + 1));
+    const int i_full = min(nq, max(j_first, kt_end - PT));
     for (; i < i_full; ++i) step(std::true_type{}, i);
     for (; i < nq; ++i) step(std::false_type{}, i);
     request(wrap(sc + 4) * C::BUF_BYTES);                   // the K role finishes tile nq-1 in one more iteration
@@ -433,23 +438,31 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 
 #undef LMK_INL
 
-template <class T, int D>
+template <class T, int D, int BS>
 static int launch_dkdv32_t(const BwdParams& p, hipStream_t stream) {
-  using C = Dkv32Cfg<T, D>;
-  auto kern = lmk_bwd_dkdv32_kernel<T, D>;
+  using C = Dkv32Cfg<T, D, BS>;
+  auto kern = lmk_bwd_dkdv32_kernel<T, D, BS>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   hipLaunchKernelGGL(kern, dim3(p.n_kvtiles * p.B * p.H), dim3(C::NTHR), C::LDS_BYTES, stream, p);
   return (int)hipGetLastError();
 }
 
-int launch_bwd_dkdv32(const BwdParams& p, int D, int dtype, hipStream_t stream) {
+template <class T, int D>
+static int launch_dkdv32_b(const BwdParams& p, int BS, hipStream_t stream) {
+  if (BS == 32) return launch_dkdv32_t<T, D, 32>(p, stream);
+  if (BS == 64) return launch_dkdv32_t<T, D, 64>(p, stream);
+  if (BS == 128) return launch_dkdv32_t<T, D, 128>(p, stream);
+  return LMK_ERR_UNSUPPORTED;
+}
+
+int launch_bwd_dkdv32(const BwdParams& p, int D, int BS, int dtype, hipStream_t stream) {
   if (dtype == LMK_DTYPE_BF16) {
-    if (D == 128) return launch_dkdv32_t<bf16_t, 128>(p, stream);
-    if (D == 64) return launch_dkdv32_t<bf16_t, 64>(p, stream);
+    if (D == 128) return launch_dkdv32_b<bf16_t, 128>(p, BS, stream);
+    if (D == 64) return launch_dkdv32_b<bf16_t, 64>(p, BS, stream);
   } else if (dtype == LMK_DTYPE_F16) {
-    if (D == 128) return launch_dkdv32_t<f16_t, 128>(p, stream);
-    if (D == 64) return launch_dkdv32_t<f16_t, 64>(p, stream);
+    if (D == 128) return launch_dkdv32_b<f16_t, 128>(p, BS, stream);
+    if (D == 64) return launch_dkdv32_b<f16_t, 64>(p, BS, stream);
   }
   return LMK_ERR_UNSUPPORTED;
 }

@@ -58,7 +58,7 @@ struct BwdParams {
 // phases: bit 0 = pre, bit 1 = dq, bit 2 = dkdv
 int launch_bwd(const BwdParams& p, int D, int BS, int dtype, int phases, hipStream_t stream);
 int launch_bwd_dq32(const BwdParams& p, int D, int dtype, hipStream_t stream);     // block 32 specialisation
-int launch_bwd_dkdv32(const BwdParams& p, int D, int dtype, hipStream_t stream);   // block 32 specialisation
+int launch_bwd_dkdv32(const BwdParams& p, int D, int BS, int dtype, hipStream_t stream);   // two-role kernel, all block sizes
 
 struct RetrParams {
   const void *q, *kcache, *vcache, *cos, *sin;   // q rotated; caches un-rotated; tables (n_pos, D)

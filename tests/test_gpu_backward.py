@@ -40,6 +40,9 @@ CASES = [
     (1, 2, 128, 320, 128, 64, torch.bfloat16),
     (1, 2, 512, 512, 128, 128, torch.bfloat16),
     (1, 2, 256, 512, 128, 128, torch.bfloat16),
+    (1, 2, 576, 576, 128, 64, torch.bfloat16),     # 9 blocks of two tiles: ring wraps inside and between blocks
+    (1, 2, 384, 640, 128, 128, torch.bfloat16),    # two history blocks of four tiles
+    (2, 3, 192, 320, 128, 64, torch.float16),
     (1, 2, 256, 256, 64, 32, torch.bfloat16),
     (1, 2, 256, 256, 64, 64, torch.bfloat16),
     (1, 2, 256, 256, 64, 128, torch.bfloat16),
