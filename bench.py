@@ -211,7 +211,7 @@ def main():
     achieved = f_dom / (t_dom * 1e-3) / 1e12
     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --traffic-probe`,
     # each scaled by what the same counter reads for a 256 MiB device copy (the summary is kept under profiles/)
-    measured_traffic = {"lmk_fwd32_kernel": 204.1e6, "lmk_bwd_dq32_kernel": 346.4e6, "lmk_bwd_dkdv32_kernel": 359.7e6}
+    measured_traffic = {"lmk_fwd32_kernel": 183.6e6, "lmk_bwd_dq32_kernel": 344.0e6, "lmk_bwd_dkdv32_kernel": 357.5e6}
     roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_BF16_TFLOPS, "traffic": measured_traffic.get(dom), "avg_launch_ms": t_dom,
                 "algorithmic_gflop_per_launch": f_dom / 1e9}
