@@ -285,15 +285,17 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
     hipLaunchKernelGGL((lmk_bwd_pre_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
   }
-  if ((phases & 2) && BS == 32) {
-    if ((rc = launch_bwd_dq32(p, D, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream))) return rc;
-  } else if (phases & 2) {
-    using C = DqCfg<T, D, BS>;
-    auto kern = lmk_bwd_dq_kernel<T, D, BS>;
-    static std::atomic<uint64_t> lds_ok{0};
-    if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
-    hipLaunchKernelGGL(kern, dim3(p.n_qtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
-    if ((rc = (int)hipGetLastError())) return rc;
+  if (phases & 2) {
+    if constexpr (BS == 32) {
+      if ((rc = launch_bwd_dq32(p, D, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream))) return rc;
+    } else {
+      using C = DqCfg<T, D, BS>;
+      auto kern = lmk_bwd_dq_kernel<T, D, BS>;
+      static std::atomic<uint64_t> lds_ok{0};
+      if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
+      hipLaunchKernelGGL(kern, dim3(p.n_qtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
+      if ((rc = (int)hipGetLastError())) return rc;
+    }
   }
   if (phases & 4) {
     return launch_bwd_dkdv32(p, D, BS, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream);

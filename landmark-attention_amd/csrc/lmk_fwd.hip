@@ -263,12 +263,10 @@ static int launch_fwd_t(const FwdParams& p, hipStream_t stream) {
 
 template <class T>
 static int launch_fwd_d(const FwdParams& p, int D, int BS, hipStream_t stream) {
-  if (D == 128) {
-    if (BS == 32) return launch_fwd_t<T, 128, 32>(p, stream);
+  if (D == 128) {                                          // block 32 has its own kernel (lmk_fwd32.hip)
     if (BS == 64) return launch_fwd_t<T, 128, 64>(p, stream);
     if (BS == 128) return launch_fwd_t<T, 128, 128>(p, stream);
   } else if (D == 64) {
-    if (BS == 32) return launch_fwd_t<T, 64, 32>(p, stream);
     if (BS == 64) return launch_fwd_t<T, 64, 64>(p, stream);
     if (BS == 128) return launch_fwd_t<T, 64, 128>(p, stream);
   }
