@@ -127,14 +127,17 @@ int lmk_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kcache, const voi
 
 /* Gather of the selected K/V blocks with rotary at their slot positions and attention over
  * them (llama_mem.py:386-412), merged with the attention over the local chunk (:447-477).
- *   o_loc, L_loc, M_loc: output and statistics of lmk_attn_fwd run on the local chunk
+ *   o_loc, L_loc, M_loc: output and statistics of lmk_attn_fwd run on the local chunk;
+ *   stat_stride: floats between consecutive (batch, head) rows of L_loc and M_loc (T when they
+ *   are dense; larger when they are the last T columns of a wider window's statistics)
  *   (q against the T new keys/values); out: (B,H,T,D) final attention output.
  * Blocks are read in place from the cache; nothing of size (T, k*block, D) is materialised.
  * Built for D = 128 and block 32 or 64. */
 int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
                       const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
-                      const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, const lmk_tensor4* out, int B,
-                      int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, void* stream);
+                      const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, int64_t stat_stride,
+                      const lmk_tensor4* out, int B, int H, int T, int S, int D, float sm_scale, int block, int top_k,
+                      int dtype, void* stream);
 
 /* Local window of the attend step when the cache ends in an incomplete block of
  * inc = S % block tokens (llama_mem.py:329-342; needs inc > 0 and T + inc <= block, the

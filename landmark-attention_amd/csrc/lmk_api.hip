@@ -210,8 +210,9 @@ int lmk_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kcache, const voi
 
 int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
                       const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
-                      const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, const lmk_tensor4* out, int B,
-                      int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, void* stream) {
+                      const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, int64_t stat_stride,
+                      const lmk_tensor4* out, int B, int H, int T, int S, int D, float sm_scale, int block, int top_k,
+                      int dtype, void* stream) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(kcache)) || (rc = check_tensor(vcache)) ||
       (rc = check_tensor(o_loc)) || (rc = check_tensor(out)))
@@ -221,12 +222,13 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
   if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
   if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
   if (D != 128 || !(block == 32 || block == 64)) return LMK_ERR_UNSUPPORTED;
+  if (stat_stride < T) return LMK_ERR_SHAPE;
   if (!std::isfinite(sm_scale) || !(sm_scale > 0.f)) return LMK_ERR_SCALE;
   lmk::RetrParams p = {};
   fill_retr_common(p, B, H, T, S, D, block, top_k);
   p.q = q->ptr; p.kcache = kcache->ptr; p.vcache = vcache->ptr; p.cos = cos_table; p.sin = sin_table;
   p.idx = const_cast<int64_t*>(idx);
-  p.o_loc = o_loc->ptr; p.L_loc = L_loc; p.M_loc = M_loc; p.out = out->ptr;
+  p.o_loc = o_loc->ptr; p.L_loc = L_loc; p.M_loc = M_loc; p.stat_stride = stat_stride; p.out = out->ptr;
   p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
   p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
   p.vcs_b = vcache->stride_b; p.vcs_h = vcache->stride_h; p.vcs_r = vcache->stride_row;

@@ -64,6 +64,7 @@ struct RetrParams {
   const void *q, *kcache, *vcache, *cos, *sin;   // q rotated; caches un-rotated; tables (n_pos, D)
   const void* o_loc;                              // attention over the local chunk (gather step)
   const float *L_loc, *M_loc;
+  int64_t stat_stride;                            // floats between consecutive (batch, head) rows of L_loc, M_loc
   void* out;
   int64_t* idx;                                   // (B, H, T, k) ascending block indices
   void* lk_rot;                                   // (B*H, num_mems, D) rotated landmark keys

@@ -696,7 +696,8 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     ahi[e] += __shfl_xor(ahi[e], 32, 64);
   }
   // merge with the local chunk: out_loc (normalised), L_loc, M_loc (natural-log units)
-  const float Ml = p.M_loc[row] * kLog2e, Ll = p.L_loc[row];
+  const int64_t srow = (int64_t)bh * p.stat_stride + t;
+  const float Ml = p.M_loc[srow] * kLog2e, Ll = p.L_loc[srow];
   const float Mt = fmaxf(Mrun, Ml);
   const float wr = fast_exp2(Mrun - Mt), wl = fast_exp2(Ml - Mt) * Ll;
   const float inv = 1.0f / (lrun * wr + wl);

@@ -73,6 +73,7 @@ def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, 
     with torch.cuda.device(q.device):
         if inc == 0:
             o_loc, L_loc, M_loc = _launch_fwd(q, k_loc, v_loc, 0, sm_scale, block)
+            stat_ptrs, stat_stride = (L_loc.data_ptr(), M_loc.data_ptr()), T
         else:
             assert T + inc <= block, "new chunk and cached tail must fit one block (llama_mem.py:330)"
             q_win, k_win, v_win = (torch.empty((B, H, inc + T, D), device=q.device, dtype=q.dtype) for _ in range(3))
@@ -83,12 +84,12 @@ def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, 
                 _lib.current_stream(q.device)))
             o_win, L_win, M_win = _launch_fwd(q_win, k_win, v_win, 0, sm_scale, block)
             o_loc = o_win[:, :, inc:]                                   # a strided view: read in place
-            L_loc = L_win.view(B * H, inc + T)[:, inc:].contiguous()
-            M_loc = M_win.view(B * H, inc + T)[:, inc:].contiguous()
+            # statistics of the window's last T rows, read in place: first element and row stride
+            stat_ptrs, stat_stride = (L_win.data_ptr() + 4 * inc, M_win.data_ptr() + 4 * inc), inc + T
         out = torch.empty_like(q)
         rc = _lib.lib().lmk_gather_attend(
             _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), idx.data_ptr(), cos.data_ptr(),
-            sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(o_loc), L_loc.data_ptr(), M_loc.data_ptr(),
+            sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(o_loc), stat_ptrs[0], stat_ptrs[1], stat_stride,
             _lib.tensor4(out), B, H, T, S, D, float(sm_scale), int(block), int(top_k), _lib.DTYPE_CODES[q.dtype],
             _lib.current_stream(q.device))
     _lib.check(rc)

@@ -105,7 +105,7 @@ def test_retrieval_argument_errors(lib):
     assert topk(D=96) == -3
     assert lib.lmk_retrieve_workspace_bytes(1, 32, 256, 32768, 128, 32) >= 32 * 1024 * 128 * 2 + 2 * 32 * 256 * 1024 * 4
     # gather+attend is built for D=128 and blocks of 32/64 only
-    rc = lib.lmk_gather_attend(t, t, t, 0x7000, 0x5000, 0x6000, 128, 4096, t, 0x2000, 0x3000, t, 1, 1, 8, 64, 64, 0.1,
+    rc = lib.lmk_gather_attend(t, t, t, 0x7000, 0x5000, 0x6000, 128, 4096, t, 0x2000, 0x3000, 8, t, 1, 1, 8, 64, 64, 0.1,
                                32, 4, 0, None)
     assert rc == -3
 
