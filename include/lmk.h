@@ -155,6 +155,39 @@ int lmk_local_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_
                      int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win, const lmk_tensor4* k_win,
                      const lmk_tensor4* v_win, int B, int H, int T, int S, int D, int block, int dtype, void* stream);
 
+/* Landmark scoring + ONE selection per (batch, head), shared by all T queries: the branch
+ * `aggregate == "max_over_tokens"` of llama_mem.py:369-384, which the reference takes when the cache
+ * is offloaded to the CPU (:369-370).  Per query: scores as in lmk_retrieve_topk, fp32 softmax over
+ * the cached blocks, rounded to the model dtype (:376); per block: the maximum over the queries
+ * (:377); then the k best blocks under (value descending, index ascending).
+ *   idx_out: (B,H,k) int64 ascending (the reference's (B,H,1,k) view, :384);
+ *   block_prob_out: NULL, or (B,H,S/block) 16-bit values in the model dtype that receive the
+ *   per-head vector the selection ran on (`mem_attn_weights` after :377).
+ * torch leaves the exponential's last bit and the order of the sum to its library, so both are
+ * fixed here: 2^t by a degree-6 polynomial with separately rounded products and sums, a sum of
+ * 64 strided partial sums folded by halves, one correctly rounded division.
+ * Workspace: as for lmk_retrieve_topk (lmk_retrieve_workspace_bytes). */
+int lmk_retrieve_topk_shared(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
+                             const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                             void* block_prob_out, void* workspace, size_t workspace_bytes, int B, int H, int T, int S,
+                             int D, int block, int top_k, int dtype, void* stream);
+
+/* Keys and values every query of a head attends to after a per-head selection
+ * (llama_mem.py:386-388, 393-406): with k = min(top_k, S/block) and inc = S % block,
+ *   k_win = [selected blocks' keys rotated at their slot positions ; tail keys rotated at
+ *            S-inc .. S-1 ; k_loc]                     (B,H,k*block+inc+T,D)
+ *   v_win = [selected blocks' values ; tail values ; v_loc]
+ *   q_win = [inc zero rows ; q]                        (B,H,inc+T,D); may be NULL when inc == 0
+ * lmk_attn_fwd on (q_win or q, k_win, v_win) with Lq = inc+T, Lk = k*block+inc+T and
+ * n_prefix = k is then the reference's fused_landmark_attention call on the concatenated
+ * sequence (:441-446); its last T rows are the new tokens' output.  T + inc <= block when inc > 0
+ * (:330).  Replaces take_along_dim, apply_rotary_pos_emb and the torch.cat calls of :393-406. */
+int lmk_gather_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+                      const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
+                      int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win, const lmk_tensor4* k_win,
+                      const lmk_tensor4* v_win, int B, int H, int T, int S, int D, int block, int top_k, int dtype,
+                      void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -66,6 +66,52 @@ void fill_retr_common(lmk::RetrParams& p, int B, int H, int T, int S, int D, int
   p.sqrt_hd = (float)std::sqrt((double)D);
 }
 
+// Shared by lmk_local_window (idx == nullptr) and lmk_gather_window.
+int window_impl(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+                       const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table,
+                       const void* sin_table, int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win,
+                       const lmk_tensor4* k_win, const lmk_tensor4* v_win, int B, int H, int T, int S, int D,
+                       int block, int top_k, int dtype, void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache)) || (rc = check_tensor(vcache)) ||
+      (rc = check_tensor(k_loc)) || (rc = check_tensor(v_loc)) || (rc = check_tensor(k_win)) ||
+      (rc = check_tensor(v_win)))
+    return rc;
+  if (cos_table == nullptr || sin_table == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
+  if ((rc = check_retrieval(B, H, T, S, D, block, idx ? top_k : 1, dtype, n_pos))) return rc;
+  const int inc = S % block;
+  if (idx == nullptr && inc == 0) return LMK_ERR_CACHE;   // no tail, no selection: the new chunk alone is the window
+  if (inc > 0 && T + inc > block) return LMK_ERR_SHAPE;   // llama_mem.py:330
+  if (inc > 0 || q_win != nullptr) {                      // without a tail the queries need no padding rows
+    if ((rc = check_tensor(q_win))) return rc;
+  }
+  lmk::WindowParams p = {};
+  p.q = q->ptr; p.kcache = kcache->ptr; p.vcache = vcache->ptr; p.k_loc = k_loc->ptr; p.v_loc = v_loc->ptr;
+  p.cos = cos_table; p.sin = sin_table;
+  p.q_win = q_win ? q_win->ptr : nullptr; p.k_win = k_win->ptr; p.v_win = v_win->ptr;
+  p.B = B; p.H = H; p.T = T; p.inc = inc;
+  p.full_len = (int64_t)S - inc;
+  p.block = block;
+  p.num_mems = S / block;
+  if (idx != nullptr) {
+    p.idx = idx;
+    p.k = top_k < p.num_mems ? top_k : p.num_mems;
+    p.n_sel = p.k * block;
+    p.prefix_len = p.full_len - (int64_t)(p.k + 1) * block;        // llama_mem.py:361
+  }
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
+  p.vcs_b = vcache->stride_b; p.vcs_h = vcache->stride_h; p.vcs_r = vcache->stride_row;
+  p.kls_b = k_loc->stride_b; p.kls_h = k_loc->stride_h; p.kls_r = k_loc->stride_row;
+  p.vls_b = v_loc->stride_b; p.vls_h = v_loc->stride_h; p.vls_r = v_loc->stride_row;
+  if (q_win) { p.qws_b = q_win->stride_b; p.qws_h = q_win->stride_h; p.qws_r = q_win->stride_row; }
+  p.kws_b = k_win->stride_b; p.kws_h = k_win->stride_h; p.kws_r = k_win->stride_row;
+  p.vws_b = v_win->stride_b; p.vws_h = v_win->stride_h; p.vws_r = v_win->stride_row;
+  p.cs_r = table_stride_row;
+  return lmk::launch_local_window(p, D, dtype, (hipStream_t)stream);
+}
+
 }  // namespace
 
 extern "C" {
@@ -239,37 +285,50 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
   return lmk::launch_gather_attend(p, D, block, dtype, (hipStream_t)stream);
 }
 
+int lmk_retrieve_topk_shared(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
+                             const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                             void* block_prob_out, void* workspace, size_t workspace_bytes, int B, int H, int T, int S,
+                             int D, int block, int top_k, int dtype, void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache))) return rc;
+  if (cos_table == nullptr || sin_table == nullptr || idx_out == nullptr || workspace == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row) || !aligned16(workspace))
+    return LMK_ERR_ALIGN;
+  if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
+  const RetrLayout l = retr_layout(B, H, T, S, D, block);
+  if (workspace_bytes < l.total) return LMK_ERR_WORKSPACE;
+  lmk::RetrParams p = {};
+  fill_retr_common(p, B, H, T, S, D, block, top_k);
+  p.q = q->ptr; p.kcache = kcache->ptr; p.cos = cos_table; p.sin = sin_table; p.idx = idx_out;
+  char* w = static_cast<char*>(workspace);
+  p.lk_rot = w + l.lk_rot;
+  p.lk_norm = reinterpret_cast<float*>(w + l.lk_norm);
+  p.approx = reinterpret_cast<float*>(w + l.approx);              // every query's scores, then exponentials
+  p.agg = reinterpret_cast<uint32_t*>(w + l.exact);               // B*H*num_mems words: fits, T >= 1
+  p.agg_out = static_cast<uint16_t*>(block_prob_out);
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
+  p.cs_r = table_stride_row;
+  return lmk::launch_retrieve_topk_shared(p, D, dtype, (hipStream_t)stream);
+}
+
 int lmk_local_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,
                      const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
                      int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win, const lmk_tensor4* k_win,
                      const lmk_tensor4* v_win, int B, int H, int T, int S, int D, int block, int dtype, void* stream) {
-  int rc;
-  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache)) || (rc = check_tensor(vcache)) ||
-      (rc = check_tensor(k_loc)) || (rc = check_tensor(v_loc)) || (rc = check_tensor(q_win)) ||
-      (rc = check_tensor(k_win)) || (rc = check_tensor(v_win)))
-    return rc;
-  if (cos_table == nullptr || sin_table == nullptr) return LMK_ERR_NULL;
-  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
-  if ((rc = check_retrieval(B, H, T, S, D, block, 1, dtype, n_pos))) return rc;
-  const int inc = S % block;
-  if (inc == 0) return LMK_ERR_CACHE;             // no tail: the new chunk alone is the window
-  if (T + inc > block) return LMK_ERR_SHAPE;      // llama_mem.py:330
-  lmk::WindowParams p = {};
-  p.q = q->ptr; p.kcache = kcache->ptr; p.vcache = vcache->ptr; p.k_loc = k_loc->ptr; p.v_loc = v_loc->ptr;
-  p.cos = cos_table; p.sin = sin_table;
-  p.q_win = q_win->ptr; p.k_win = k_win->ptr; p.v_win = v_win->ptr;
-  p.B = B; p.H = H; p.T = T; p.inc = inc;
-  p.full_len = (int64_t)S - inc;
-  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
-  p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
-  p.vcs_b = vcache->stride_b; p.vcs_h = vcache->stride_h; p.vcs_r = vcache->stride_row;
-  p.kls_b = k_loc->stride_b; p.kls_h = k_loc->stride_h; p.kls_r = k_loc->stride_row;
-  p.vls_b = v_loc->stride_b; p.vls_h = v_loc->stride_h; p.vls_r = v_loc->stride_row;
-  p.qws_b = q_win->stride_b; p.qws_h = q_win->stride_h; p.qws_r = q_win->stride_row;
-  p.kws_b = k_win->stride_b; p.kws_h = k_win->stride_h; p.kws_r = k_win->stride_row;
-  p.vws_b = v_win->stride_b; p.vws_h = v_win->stride_h; p.vws_r = v_win->stride_row;
-  p.cs_r = table_stride_row;
-  return lmk::launch_local_window(p, D, dtype, (hipStream_t)stream);
+  if (q_win == nullptr) return LMK_ERR_NULL;
+  return window_impl(q, kcache, vcache, nullptr, k_loc, v_loc, cos_table, sin_table, table_stride_row, n_pos, q_win,
+                     k_win, v_win, B, H, T, S, D, block, 1, dtype, stream);
+}
+
+int lmk_gather_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+                      const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
+                      int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win, const lmk_tensor4* k_win,
+                      const lmk_tensor4* v_win, int B, int H, int T, int S, int D, int block, int top_k, int dtype,
+                      void* stream) {
+  if (idx == nullptr) return LMK_ERR_NULL;
+  return window_impl(q, kcache, vcache, idx, k_loc, v_loc, cos_table, sin_table, table_stride_row, n_pos, q_win,
+                     k_win, v_win, B, H, T, S, D, block, top_k, dtype, stream);
 }
 
 }  // extern "C"

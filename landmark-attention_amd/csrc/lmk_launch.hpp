@@ -70,6 +70,8 @@ struct RetrParams {
   void* lk_rot;                                   // (B*H, num_mems, D) rotated landmark keys
   float* lk_norm;                                 // (B*H, num_mems)
   float *approx, *exact;                          // (B*H*T, num_mems) each
+  uint32_t* agg;                                  // (B*H, num_mems) per-head maxima of the 16-bit probabilities
+  uint16_t* agg_out;                              // optional copy of agg in the model dtype
   int B, H, T, S, block, num_mems, k;
   int64_t prefix_len;                             // full_len - (k + 1) * block, may be -block
   int64_t qs_b, qs_h, qs_r, kcs_b, kcs_h, kcs_r, vcs_b, vcs_h, vcs_r, cs_r;
@@ -77,17 +79,22 @@ struct RetrParams {
   float sqrt_hd, scale_log2;
 };
 
-// local window of the attend step when the cache ends in an incomplete block of `inc` tokens
+// local window of the attend step: [n_sel rows of selected blocks | inc tail tokens | T new tokens]
 struct WindowParams {
   const void *q, *kcache, *vcache, *k_loc, *v_loc, *cos, *sin;
-  void *q_win, *k_win, *v_win;                    // (B, H, inc + T, D) each
+  void* q_win;                                    // (B, H, inc + T, D), may be null when inc == 0
+  void *k_win, *v_win;                            // (B, H, n_sel + inc + T, D) each
+  const int64_t* idx;                             // (B, H, k) ascending block indices (n_sel > 0 only)
   int B, H, T, inc;
+  int n_sel, k, block, num_mems;                  // n_sel = k * block rows of selected blocks in front, or 0
+  int64_t prefix_len;
   int64_t full_len;                               // first cached row of the tail = its rotary position
   int64_t qs_b, qs_h, qs_r, kcs_b, kcs_h, kcs_r, vcs_b, vcs_h, vcs_r, kls_b, kls_h, kls_r, vls_b, vls_h, vls_r;
   int64_t qws_b, qws_h, qws_r, kws_b, kws_h, kws_r, vws_b, vws_h, vws_r, cs_r;
 };
 
 int launch_retrieve_topk(const RetrParams& p, int D, int dtype, hipStream_t stream);
+int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream_t stream);   // one selection per head
 int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t stream);
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream);
 

@@ -42,8 +42,11 @@ __device__ __forceinline__ void rotate_chunk(const u32x4_t x, const u32x4_t othe
       r0 = -r0;
       r1 = -r1;
     }
-    const float a0 = round_to<T>(x0 * unpack_lo<T>(c[i])), a1 = round_to<T>(x1 * unpack_hi<T>(c[i]));
-    const float b0 = round_to<T>(r0 * unpack_lo<T>(s[i])), b1 = round_to<T>(r1 * unpack_hi<T>(s[i]));
+    float a0 = round_to<T>(x0 * unpack_lo<T>(c[i])), a1 = round_to<T>(x1 * unpack_hi<T>(c[i]));
+    float b0 = round_to<T>(r0 * unpack_lo<T>(s[i])), b1 = round_to<T>(r1 * unpack_hi<T>(s[i]));
+    // The rounded products are opaque to the compiler: with f16 it would otherwise turn
+    // round(round(x*c) + round(r*s)) into a half-precision fused multiply-add, which skips a rounding.
+    asm volatile("" : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
     out[2 * i] = round_to<T>(a0 + b0);
     out[2 * i + 1] = round_to<T>(a1 + b1);
   }
@@ -304,6 +307,142 @@ __global__ __launch_bounds__(256) void lmk_select_kernel(RetrParams p) {
     rank += (o < mine) ? 1 : 0;
   }
   if (lane < p.k) p.idx[row * p.k + rank] = (int64_t)mine;
+}
+
+// ---------------------------------------------------------------------------
+// one selection per head (llama_mem.py:373-384 with aggregate == "max_over_tokens"): every query's
+// scores go through an fp32 softmax over the cached blocks, are rounded to the model dtype and
+// reduced with a maximum over the queries; the head's k best blocks serve all its queries.
+// The softmax needs every score exactly as the contract defines it, so there is no bracketing
+// here: a lane evaluates the sequential dot product for its blocks.
+// ---------------------------------------------------------------------------
+
+// 2^t for t <= 0 with every rounding fixed, so that a CPU can reproduce it bit for bit:
+// n = rint(t), f = t - n (exact), degree-6 Horner polynomial with one rounding after each product
+// and each sum (the empty asm keeps the compiler from fusing them), times 2^n (exact).
+__device__ __forceinline__ float exp2_contract(float t) {
+  if (t < -126.f) return 0.f;
+  const float n = __builtin_rintf(t);
+  const float f = t - n;
+  float pl = 1.5403530393381608e-4f;
+  const float c[6] = {1.3333558146428443e-3f, 9.618129107628477e-3f, 5.550410866482158e-2f,
+                      2.402265069591007e-1f,  6.931471805599453e-1f, 1.0f};
+#pragma unroll
+  for (int i = 0; i < 6; ++i) {
+    float m = pl * f;
+    asm volatile("" : "+v"(m));
+    pl = m + c[i];
+  }
+  return __builtin_ldexpf(pl, (int)n);
+}
+
+template <class T>
+__device__ __forceinline__ uint32_t prob_bits(float x);   // non-negative fp32 -> 16-bit pattern (RNE); monotone
+template <>
+__device__ __forceinline__ uint32_t prob_bits<bf16_t>(float x) {
+  const uint32_t u = __float_as_uint(x);
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;           // integer rounding: also right for subnormal x
+}
+template <>
+__device__ __forceinline__ uint32_t prob_bits<f16_t>(float x) { return pack2<f16_t>(x, 0.f) & 0xffffu; }
+
+__global__ __launch_bounds__(256) void lmk_fill_u32_kernel(uint32_t* dst, int64_t n, uint32_t value) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = value;
+}
+
+// One wave per (batch, head, query): scores -> softmax -> 16-bit probabilities -> maximum per block
+// into agg (B*H, num_mems), which holds zeros on entry.  A lane owns the blocks m = lane, lane + 64, ...;
+// the row's sum is each lane's running sum in that order, folded across lanes by halves.
+template <class T, int D>
+__global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
+  __shared__ __align__(16) float q_lds[4][D];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;             // (bh, t)
+  if (row >= (int64_t)p.B * p.H * p.T) return;                    // whole wave leaves; no block-wide barrier below
+  const int bh = (int)(row / p.T), t = (int)(row % p.T);
+  const int b = bh / p.H, hh = bh % p.H;
+  const int NM = p.num_mems;
+  const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
+  for (int d = 2 * lane; d < D; d += 128) {
+    const uint32_t u = *(const uint32_t*)(qp + 2 * d);
+    q_lds[wave][d] = unpack_lo<T>(u);
+    q_lds[wave][d + 1] = unpack_hi<T>(u);
+  }
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_s_waitcnt(0xc07f);                             // LDS writes of this wave visible (lgkmcnt 0)
+
+  float* sc = p.approx + row * NM;                                // this row's scores, then its exponentials
+  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * NM * D);
+  float mx = -INFINITY;
+  for (int m = lane; m < NM; m += 64) {
+    const char* kr = lk + 2 * ((int64_t)m * D);
+    float acc = 0.f;
+#pragma unroll 4
+    for (int d8 = 0; d8 < D / 8; ++d8) {
+      const u32x4_t kk = *(const u32x4_t*)(kr + 16 * d8);
+      const float4 qa = *(const float4*)&q_lds[wave][8 * d8];
+      const float4 qb = *(const float4*)&q_lds[wave][8 * d8 + 4];
+      acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
+      acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
+      acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
+      acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
+      acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
+      acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
+      acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
+      acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
+    }
+    const float x = contract<T>(acc, p.sqrt_hd);
+    sc[m] = x;                                                    // read back below by the same lane only
+    mx = fmaxf(mx, x);
+  }
+#pragma unroll
+  for (int msk = 32; msk >= 1; msk >>= 1) mx = fmaxf(mx, __shfl_xor(mx, msk, 64));
+  float sum = 0.f;
+  for (int m = lane; m < NM; m += 64) {
+    float d = sc[m] - mx;
+    asm volatile("" : "+v"(d));                                   // the product below stays a product
+    const float e = exp2_contract(d * kLog2e);
+    sc[m] = e;
+    sum += e;
+  }
+#pragma unroll
+  for (int msk = 32; msk >= 1; msk >>= 1) sum = sum + __shfl_xor(sum, msk, 64);
+  uint32_t* agg = p.agg + (int64_t)bh * NM;
+  for (int m = lane; m < NM; m += 64) atomicMax(agg + m, prob_bits<T>(__fdiv_rn(sc[m], sum)));
+}
+
+// One wave per (batch, head): the k best blocks of agg under (value desc, index asc), ascending.
+__global__ __launch_bounds__(64) void lmk_block_select_kernel(RetrParams p) {
+  const int lane = threadIdx.x, bh = blockIdx.x, NM = p.num_mems;
+  const uint32_t* agg = p.agg + (int64_t)bh * NM;
+  if (p.agg_out != nullptr)                                       // the head's vector itself, in the model dtype
+    for (int m = lane; m < NM; m += 64) p.agg_out[(int64_t)bh * NM + m] = (uint16_t)agg[m];
+  int mine = -1;
+  float pv = INFINITY;
+  int pi = -1;
+  for (int j = 0; j < p.k; ++j) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int m = lane; m < NM; m += 64) {
+      const float x = (float)agg[m];                              // 16-bit patterns: exact, order-preserving
+      const bool after = (x < pv) || (x == pv && m > pi);
+      if (after && (x > bv || (x == bv && m < bi))) {
+        bv = x;
+        bi = m;
+      }
+    }
+    wave_best(bv, bi);
+    pv = bv;
+    pi = bi;
+    if (lane == j) mine = bi;
+  }
+  int rank = 0;
+  for (int j = 0; j < p.k; ++j) {
+    const int o = __shfl(mine, j, 64);
+    rank += (o < mine) ? 1 : 0;
+  }
+  if (lane < p.k) p.idx[(int64_t)bh * p.k + rank] = (int64_t)mine;
 }
 
 // ---------------------------------------------------------------------------
@@ -747,6 +886,33 @@ static int launch_topk_t(const RetrParams& p, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
+template <class T, int D>
+static int launch_topk_shared_t(const RetrParams& p, hipStream_t stream) {
+  constexpr int RPW = 256 / (D / 8);
+  const int64_t lkrows = (int64_t)p.B * p.H * p.num_mems;
+  int rc;
+  hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
+  if ((rc = (int)hipGetLastError())) return rc;
+  hipLaunchKernelGGL(lmk_fill_u32_kernel, dim3((unsigned)((lkrows + 255) / 256)), dim3(256), 0, stream, p.agg, lkrows, 0u);
+  if ((rc = (int)hipGetLastError())) return rc;
+  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  hipLaunchKernelGGL((lmk_block_prob_kernel<T, D>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+  if ((rc = (int)hipGetLastError())) return rc;
+  hipLaunchKernelGGL(lmk_block_select_kernel, dim3(p.B * p.H), dim3(64), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream_t stream) {
+  if (dtype == LMK_DTYPE_BF16) {
+    if (D == 128) return launch_topk_shared_t<bf16_t, 128>(p, stream);
+    if (D == 64) return launch_topk_shared_t<bf16_t, 64>(p, stream);
+  } else if (dtype == LMK_DTYPE_F16) {
+    if (D == 128) return launch_topk_shared_t<f16_t, 128>(p, stream);
+    if (D == 64) return launch_topk_shared_t<f16_t, 64>(p, stream);
+  }
+  return LMK_ERR_UNSUPPORTED;
+}
+
 int launch_retrieve_topk(const RetrParams& p, int D, int dtype, hipStream_t stream) {
   if (dtype == LMK_DTYPE_BF16) {
     if (D == 128) return launch_topk_t<bf16_t, 128>(p, stream);
@@ -770,26 +936,37 @@ static int launch_gather_t(const RetrParams& p, int BS, hipStream_t stream) {
 
 // ---------------------------------------------------------------------------
 // local window: [cached tail | new chunk] when the cache ends in an incomplete block
-// (llama_mem.py:321-342).  One 16-byte chunk per thread:
-//   k_win = [rot(tail keys, positions full_len ..) ; k_loc]     (:337-339)
-//   v_win = [tail values ; v_loc]                                (:340)
-//   q_win = [zero rows ; q]   -- rows in front of the queries so that the fused forward kernel,
-//           run square on the window, yields the new tokens' attention in its last T rows
+// (llama_mem.py:321-342), optionally behind the k blocks one per-head selection picked
+// (:386-388, :400-406).  One 16-byte chunk per thread:
+//   k_win = [rot(selected keys, slot positions) ; rot(tail keys, positions full_len ..) ; k_loc]
+//   v_win = [selected values ; tail values ; v_loc]
+//   q_win = [zero rows for the tail ; q]   -- rows in front of the queries so that the fused forward
+//           kernel, run with the selected blocks as history, yields the new tokens' attention in its
+//           last T rows
 // ---------------------------------------------------------------------------
 template <class T, int D>
 __global__ __launch_bounds__(256) void lmk_local_window_kernel(WindowParams p) {
   constexpr int LPR = D / 8;
   constexpr int RPW = 256 / LPR;
   const int tid = threadIdx.x, j = tid % LPR;
-  const int W = p.inc + p.T;
+  const int W = p.n_sel + p.inc + p.T;
   const int64_t row = (int64_t)blockIdx.x * RPW + tid / LPR;      // (bh, r)
   if (row >= (int64_t)p.B * p.H * W) return;
   const int bh = (int)(row / W), r = (int)(row % W);
   const int b = bh / p.H, hh = bh % p.H;
   u32x4_t qo = {0, 0, 0, 0}, ko, vo;
-  if (r < p.inc) {
-    const int64_t pos = p.full_len + r;
-    const char* src = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h + pos * p.kcs_r);
+  if (r < p.n_sel + p.inc) {
+    int64_t src_row, pos;
+    if (r < p.n_sel) {
+      const int slot = r / p.block, tok = r % p.block;
+      int64_t blk = p.idx[(int64_t)bh * p.k + slot];
+      blk = blk < 0 ? 0 : (blk >= p.num_mems ? p.num_mems - 1 : blk);   // never read outside the cache
+      src_row = blk * p.block + tok;
+      pos = (int64_t)r + (blk >= p.num_mems - p.k ? p.block : 0) + p.prefix_len;   // llama_mem.py:386-388
+    } else {
+      src_row = pos = p.full_len + (r - p.n_sel);
+    }
+    const char* src = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h + src_row * p.kcs_r);
     const u32x4_t x = *(const u32x4_t*)(src + 16 * j);
     const u32x4_t other = *(const u32x4_t*)(src + 16 * (j ^ (LPR / 2)));
     const u32x4_t c = *(const u32x4_t*)((const char*)p.cos + 2 * (pos * p.cs_r) + 16 * j);
@@ -797,22 +974,23 @@ __global__ __launch_bounds__(256) void lmk_local_window_kernel(WindowParams p) {
     float o[8];
     rotate_chunk<T>(x, other, c, s, j >= LPR / 2, o);
     ko = u32x4_t{pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
-    vo = *(const u32x4_t*)((const char*)p.vcache + 2 * (b * p.vcs_b + hh * p.vcs_h + pos * p.vcs_r) + 16 * j);
+    vo = *(const u32x4_t*)((const char*)p.vcache + 2 * (b * p.vcs_b + hh * p.vcs_h + src_row * p.vcs_r) + 16 * j);
   } else {
-    const int t = r - p.inc;
+    const int t = r - p.n_sel - p.inc;
     qo = *(const u32x4_t*)((const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + t * p.qs_r) + 16 * j);
     ko = *(const u32x4_t*)((const char*)p.k_loc + 2 * (b * p.kls_b + hh * p.kls_h + t * p.kls_r) + 16 * j);
     vo = *(const u32x4_t*)((const char*)p.v_loc + 2 * (b * p.vls_b + hh * p.vls_h + t * p.vls_r) + 16 * j);
   }
-  *(u32x4_t*)((char*)p.q_win + 2 * (b * p.qws_b + hh * p.qws_h + r * p.qws_r) + 16 * j) = qo;
-  *(u32x4_t*)((char*)p.k_win + 2 * (b * p.kws_b + hh * p.kws_h + r * p.kws_r) + 16 * j) = ko;
-  *(u32x4_t*)((char*)p.v_win + 2 * (b * p.vws_b + hh * p.vws_h + r * p.vws_r) + 16 * j) = vo;
+  if (r >= p.n_sel && p.q_win != nullptr)
+    *(u32x4_t*)((char*)p.q_win + 2 * (b * p.qws_b + hh * p.qws_h + (int64_t)(r - p.n_sel) * p.qws_r) + 16 * j) = qo;
+  *(u32x4_t*)((char*)p.k_win + 2 * (b * p.kws_b + hh * p.kws_h + (int64_t)r * p.kws_r) + 16 * j) = ko;
+  *(u32x4_t*)((char*)p.v_win + 2 * (b * p.vws_b + hh * p.vws_h + (int64_t)r * p.vws_r) + 16 * j) = vo;
 }
 
 template <class T, int D>
 static int launch_window_t(const WindowParams& p, hipStream_t stream) {
   constexpr int RPW = 256 / (D / 8);
-  const int64_t rows = (int64_t)p.B * p.H * (p.inc + p.T);
+  const int64_t rows = (int64_t)p.B * p.H * (p.n_sel + p.inc + p.T);
   hipLaunchKernelGGL((lmk_local_window_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
   return (int)hipGetLastError();
 }

@@ -1,8 +1,9 @@
 """Mem-cache retrieval at inference: landmark scoring, top-k block selection and
 attention over the gathered blocks, on the HIP kernels.
 
-Mirrors the per-head, per-token branch of ``LlamaAttention.forward``
-(``llama/llama_mem.py:318-430`` retrieval, ``:447-477`` attend) with the reference's own
+Mirrors ``LlamaAttention.forward`` (``llama/llama_mem.py:318-430`` retrieval, ``:447-477``
+attend): the per-head, per-token selection (``aggregate is None``) and the selection shared by
+all queries of a head (``aggregate == "max_over_tokens"``, ``:373-377``), with the reference's own
 conventions: ``past_key_value = (K_without_rotary, V)`` each ``(B, nh, S, hd)`` (``:424-430``),
 ``block = mem_freq + 1`` with the landmark as the last token of a block, queries and local
 keys already rotated (``:298``), ``cos/sin`` the model-dtype tables of
@@ -33,12 +34,20 @@ def _tables(cos, sin, dtype):
     return cos, sin
 
 
-def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int):
+def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, return_block_probs=False):
     """Indices ``(B, nh, T, k)`` int64, ascending, of the ``k = min(top_k, S // block)`` cached
     blocks whose landmark keys score highest against each query (``llama_mem.py:344-384``).
 
     Equivalent to ``(q @ rot(landmark_keys)^T / sqrt(hd)).topk(k).indices.sort()`` with the
-    product accumulated sequentially in fp32 and ties broken towards the lower index."""
+    product accumulated sequentially in fp32 and ties broken towards the lower index.
+
+    ``aggregate="max_over_tokens"`` (``:373-377``): one set per head, ``(B, nh, 1, k)`` -- the
+    scores go through an fp32 softmax over the blocks, are rounded to the model dtype and reduced
+    with a maximum over the queries before the top-k; ``return_block_probs`` also returns that
+    per-head vector ``(B, nh, 1, S // block)`` (``mem_attn_weights`` after ``:377``)."""
+    if aggregate not in (None, "max_over_tokens"):
+        raise NotImplementedError(aggregate)                            # llama_mem.py:381-382
+    assert aggregate or not return_block_probs, "the per-head vector exists only with aggregate='max_over_tokens'"
     B, H, T, D = q.shape
     S = k_cache.shape[2]
     assert k_cache.shape == (B, H, S, D) and q.dtype == k_cache.dtype and q.is_cuda and k_cache.is_cuda
@@ -46,16 +55,23 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int):
     cos, sin = _tables(cos, sin, q.dtype)
     lib = _lib.lib()
     k = min(top_k, S // block)                      # complete blocks only (llama_mem.py:321-324,358-359)
-    idx = torch.empty((B, H, T, k), device=q.device, dtype=torch.int64)
+    idx = torch.empty((B, H, 1 if aggregate else T, k), device=q.device, dtype=torch.int64)
     nbytes = lib.lmk_retrieve_workspace_bytes(B, H, T, S, D, int(block))
+    probs = None
     with torch.cuda.device(q.device):
         ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
-        rc = lib.lmk_retrieve_topk(_lib.tensor4(q), _lib.tensor4(k_cache), cos.data_ptr(), sin.data_ptr(),
-                                   cos.stride(0), cos.shape[0], idx.data_ptr(), ws.data_ptr(), nbytes,
-                                   B, H, T, S, D, int(block), int(top_k), _lib.DTYPE_CODES[q.dtype],
-                                   _lib.current_stream(q.device))
+        tail = (ws.data_ptr(), nbytes, B, H, T, S, D, int(block), int(top_k), _lib.DTYPE_CODES[q.dtype],
+                _lib.current_stream(q.device))
+        head = (_lib.tensor4(q), _lib.tensor4(k_cache), cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0],
+                idx.data_ptr())
+        if aggregate:
+            if return_block_probs:
+                probs = torch.empty((B, H, 1, S // block), device=q.device, dtype=q.dtype)
+            rc = lib.lmk_retrieve_topk_shared(*head, probs.data_ptr() if return_block_probs else None, *tail)
+        else:
+            rc = lib.lmk_retrieve_topk(*head, *tail)
     _lib.check(rc)
-    return idx
+    return (idx, probs) if return_block_probs else idx
 
 
 def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
@@ -96,13 +112,45 @@ def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, 
     return out
 
 
-def retrieve_and_attend(q, past_key_value, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
+def attend_shared(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
+    """Attention output ``(B, nh, T, hd)`` when all queries of a head share the blocks
+    ``idx (B, nh, 1, k)`` (``llama_mem.py:400-406``): the selected blocks, rotated at their slot
+    positions, and the local window form one key/value sequence, and the fused forward kernel
+    runs on it with the selected blocks as history (``:441-446``)."""
+    B, H, T, D = q.shape
+    S = k_cache.shape[2]
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    q, k_cache, v_cache, k_loc, v_loc = (_lib.kernel_ready(t) for t in (q, k_cache, v_cache, k_loc, v_loc))
+    cos, sin = _tables(cos, sin, q.dtype)
+    inc = S % block
+    k = min(top_k, S // block)
+    assert idx.shape == (B, H, 1, k) and idx.dtype == torch.int64 and idx.is_contiguous()
+    assert inc == 0 or T + inc <= block, "new chunk and cached tail must fit one block (llama_mem.py:330)"
+    with torch.cuda.device(q.device):
+        k_win, v_win = (torch.empty((B, H, k * block + inc + T, D), device=q.device, dtype=q.dtype) for _ in range(2))
+        q_win = torch.empty((B, H, inc + T, D), device=q.device, dtype=q.dtype) if inc else None
+        _lib.check(_lib.lib().lmk_gather_window(
+            _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), idx.data_ptr(), _lib.tensor4(k_loc),
+            _lib.tensor4(v_loc), cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0],
+            _lib.tensor4(q_win) if inc else None, _lib.tensor4(k_win), _lib.tensor4(v_win), B, H, T, S, D, int(block),
+            int(top_k), _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device)))
+        o, _, _ = _launch_fwd(q_win if inc else q, k_win, v_win, k, sm_scale, block)
+    return o[:, :, inc:] if inc else o
+
+
+def retrieve_and_attend(q, past_key_value, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None,
+                        aggregate=None):
     """One inference step of the mem-cache path: returns ``(out, idx)``.
 
     ``past_key_value = (K_without_rotary, V)``; ``k_loc`` rotated, ``v_loc``: the new chunk.
-    The caller appends the un-rotated new keys and values to the cache afterwards
-    (``llama_mem.py:424-430``)."""
+    ``aggregate`` as in ``llama_mem.py:369-382``: ``None`` selects per (head, query),
+    ``"max_over_tokens"`` once per head.  The caller appends the un-rotated new keys and values to
+    the cache afterwards (``:424-430``)."""
     k_cache, v_cache = past_key_value[0], past_key_value[1]
-    idx = retrieve_topk(q, k_cache, cos, sin, block, top_k)
-    out = gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
+    idx = retrieve_topk(q, k_cache, cos, sin, block, top_k, aggregate)
+    if aggregate:
+        out = attend_shared(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
+    else:
+        out = gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
     return out, idx

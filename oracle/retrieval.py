@@ -27,6 +27,19 @@ way; on rows without a tie at the k-th place both agree, which
 ``tests/test_oracle_retrieval.py`` checks, together with a brute-force loop,
 the integer position formulas on hand-worked cases, and agreement of the
 bf16-faithful attend with the fp32 closed form of ``oracle/s1.py``.
+
+One selection per head (``aggregate == "max_over_tokens"``, ``:373-377``, the branch the
+reference takes when the cache is offloaded to the CPU): the scores of every query go
+through an fp32 softmax over the cached blocks, are rounded to the model dtype and reduced
+with ``amax`` over the queries; the top-k of that per-head vector is shared by all queries,
+the selected blocks become ordinary history blocks in front of the local window
+(``:400-406``) and the attention is the fused forward's (``:441-446``).  ``torch.softmax``
+leaves the exponential's last bit and the order of the sum to the library, so both are fixed
+here (``exp2_contract``, ``softmax_contract``) with operations numpy and the GPU round
+identically: no fused multiply-add, a polynomial evaluated by Horner's rule with separate
+products and sums, a per-lane sequential sum followed by a halving tree.  Pinned in
+``tests/test_oracle_retrieval.py`` against ``numpy.exp2`` / ``torch.softmax`` (to a few ulp),
+against a literal Python loop, and against ``torch.topk`` on heads without a boundary tie.
 """
 from __future__ import annotations
 
@@ -110,6 +123,119 @@ def boundary_tie_rows(scores, k: int):
     if top.shape[-1] <= k:
         return torch.zeros(top.shape[:-1], dtype=torch.bool)
     return top[..., k - 1] == top[..., k]
+
+
+# --------------------------------------------------- one selection per head
+_LOG2E = np.float32(1.4426950408889634)
+# Taylor coefficients of 2**f = exp(f ln 2) up to degree 6 (|f| <= 1/2: truncation < 1.3e-7)
+_EXP2_COEF = [np.float32(c) for c in (1.0, 0.6931471805599453, 0.2402265069591007, 0.05550410866482158,
+                                      0.009618129107628477, 0.0013333558146428443, 0.00015403530393381608)]
+
+
+def exp2_contract(t):
+    """``2**t`` for fp32 ``t <= 0`` with every rounding fixed: ``n = rint(t)`` (ties to even),
+    ``f = t - n`` (exact), degree-6 Horner polynomial in ``f`` with one fp32 rounding after each
+    product and each sum, scaled by ``2**n`` (exact).  ``t < -126`` gives 0, so no fp32
+    subnormal is ever produced here."""
+    t = np.asarray(t, dtype=np.float32)
+    n = np.rint(t)
+    f = (t - n).astype(np.float32)
+    p = np.full_like(f, _EXP2_COEF[6])
+    for c in _EXP2_COEF[5::-1]:
+        p = (p * f).astype(np.float32)
+        p = (p + c).astype(np.float32)
+    out = np.ldexp(p, np.maximum(n, -126).astype(np.int32)).astype(np.float32)
+    return np.where(t < np.float32(-126.0), np.float32(0.0), out)
+
+
+def softmax_contract(scores, dtype):
+    """Softmax over the last dim of fp32 ``scores`` (…, M), rounded to ``dtype`` (``:376``).
+
+    ``e_m = exp2_contract((x_m - max) * log2(e))``; the sum runs the way one 64-lane wave adds
+    it: lane ``l`` adds ``e_l, e_{l+64}, …`` in that order, then the 64 partial sums are folded
+    by halves (32, 16, … 1); ``p_m = e_m / sum`` is one correctly rounded fp32 division."""
+    x = scores.float().numpy()
+    mx = x.max(axis=-1, keepdims=True)
+    e = exp2_contract(((x - mx).astype(np.float32) * _LOG2E).astype(np.float32))
+    M = e.shape[-1]
+    pad = (-M) % 64
+    ep = np.concatenate((e, np.zeros(e.shape[:-1] + (pad,), np.float32)), axis=-1)
+    ep = ep.reshape(e.shape[:-1] + (-1, 64))
+    part = np.zeros(e.shape[:-1] + (64,), np.float32)
+    for r in range(ep.shape[-2]):
+        part = (part + ep[..., r, :]).astype(np.float32)
+    w = 32
+    while w >= 1:
+        part = (part[..., :w] + part[..., w:2 * w]).astype(np.float32)
+        w //= 2
+    prob = (e / part).astype(np.float32)
+    return torch.from_numpy(prob).to(dtype)
+
+
+def aggregate_max_over_tokens(scores):
+    """(B, nh, 1, M) in the scores' dtype: softmax over blocks per query, then the largest
+    probability any query gives a block (``llama_mem.py:376-377``)."""
+    return softmax_contract(scores, scores.dtype).amax(dim=2, keepdim=True)
+
+
+def shared_window(k_cache, v_cache, k_loc, v_loc, idx, cos, sin, block: int, top_k: int):
+    """Keys and values every query of a head attends to in the ``max_over_tokens`` branch
+    (``llama_mem.py:400-406``): the ``k`` selected blocks, keys rotated at their slot positions
+    (``:386-388,403``), then the local window (tail of an incomplete cached block, new chunk).
+    idx: (B, nh, 1, k).  Returns (B, nh, k*bs + inc + T, hd) each."""
+    S = k_cache.shape[2]
+    g = retrieval_geometry(S, block, top_k)
+    k = g["k"]
+    if g["incomplete_len"]:
+        k_loc, v_loc = local_window(k_cache, v_cache, k_loc, v_loc, cos, sin, block)
+    pos = gather_positions(idx, g["num_mems"], k, block, g["prefix_len"])           # (B,nh,1,k,bs)
+    ksel = apply_rotary(gather_blocks(k_cache, idx, block), cos, sin, pos)[:, :, 0].flatten(2, 3)
+    vsel = gather_blocks(v_cache, idx, block)[:, :, 0].flatten(2, 3)
+    return torch.cat((ksel, k_loc), dim=2), torch.cat((vsel, v_loc), dim=2)
+
+
+def retrieve_and_attend_shared(q, k_cache, v_cache, k_loc, v_loc, is_mem_loc, cos, sin, block: int, top_k: int,
+                               idx=None, n_buckets: int = 64):
+    """The ``max_over_tokens`` step in the model dtype through the reference's high-level attend
+    (``llama_mem.py:447-477``).  Returns ``(out (B,nh,T,hd), idx (B,nh,1,k) int64)``."""
+    B, nh, T, hd = q.shape
+    S = k_cache.shape[2]
+    g = retrieval_geometry(S, block, top_k)
+    inc, k = g["incomplete_len"], g["k"]
+    if inc:
+        assert T + inc <= block                                                     # :330
+    if idx is None:
+        idx = select_topk(aggregate_max_over_tokens(landmark_scores(q, k_cache, cos, sin, block, top_k)), k)
+    keys, values = shared_window(k_cache, v_cache, k_loc, v_loc, idx, cos, sin, block, top_k)
+    add, im_loc, ls_loc = local_masks(is_mem_loc, T, q.dtype)
+    n_front = k * block + inc
+    add = torch.cat((torch.zeros(add.shape[0], 1, T, n_front, dtype=add.dtype), add), dim=-1)
+    im_front = torch.zeros(n_front, dtype=torch.bool)
+    im_front[block - 1 : k * block : block] = True                                   # :415
+    ls_front = torch.zeros(n_front, dtype=torch.bool)
+    ls_front[k * block :] = True                                                     # :335 (tail), :420 (selected)
+    im = torch.cat((im_front.expand(im_loc.shape[0], 1, T, -1), im_loc), dim=-1).expand(B, nh, T, -1)
+    ls = torch.cat((ls_front.expand(ls_loc.shape[0], 1, T, -1), ls_loc), dim=-1).expand(B, nh, T, -1)
+    x = (q @ keys.transpose(2, 3)) / math.sqrt(hd) + add                            # :448,460
+    x = torch.max(x, torch.tensor(torch.finfo(q.dtype).min, dtype=q.dtype))         # :461
+    w = grouped_softmax(x, im, ls, n_buckets).to(q.dtype)                           # :469
+    return w @ values, idx                                                          # :477
+
+
+def retrieve_and_attend_shared_s1(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block: int, top_k: int, idx):
+    """Same step as the fp32 closed form: the selected blocks are history blocks of the fused
+    forward (``fused_landmark_attention`` with ``n_history_blocks = k``, ``llama_mem.py:441-446``).
+    Returns (B, nh, T, hd) fp32."""
+    B, nh, T, hd = q.shape
+    inc = k_cache.shape[2] % block
+    keys, values = shared_window(k_cache, v_cache, k_loc, v_loc, idx, cos, sin, block, top_k)
+    if inc:                       # the tail opens the current block; zero rows stand in for its queries
+        q = torch.cat((torch.zeros(B, nh, inc, hd, dtype=q.dtype), q), dim=2)
+    out = torch.empty(B, nh, T, hd)
+    for b in range(B):
+        for h in range(nh):
+            out[b, h] = s1_attention(q[b, h].float(), keys[b, h].float(), values[b, h].float(), block)[inc:]
+    return out
 
 
 # --------------------------------------------------------------------- gather

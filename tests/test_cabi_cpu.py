@@ -30,7 +30,7 @@ def _declared():
 def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
-            "lmk_strerror"} <= set(names)
+            "lmk_retrieve_topk_shared", "lmk_gather_window", "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
 
@@ -116,6 +116,24 @@ def test_retrieval_argument_errors(lib):
     assert window(64, 4) == -9
     assert window(70, 27) == -2
     assert window(20, 4) == -9
+
+    # one selection per head: same argument contract as the per-token entry point
+    def shared(S=64, top_k=4, n_pos=4096, wsb=1 << 30, idx=0x7000):
+        return lib.lmk_retrieve_topk_shared(t, t, 0x5000, 0x6000, 128, n_pos, idx, None, 0x4000, wsb, 1, 1, 8, S, 128, 32, top_k,
+                                            0, None)
+
+    assert shared(idx=0) == -1 and shared(S=16) == -9 and shared(top_k=0) == -10 and shared(n_pos=32) == -11
+    assert shared(wsb=64) == -8
+
+    # selected blocks + local window: padded queries are required only when there is a tail
+    def gwin(S, T, idx=0x7000, q_win=t):
+        return lib.lmk_gather_window(t, t, t, idx, t, t, 0x5000, 0x6000, 128, 4096, q_win, t, t, 1, 1, T, S, 128, 32, 4, 0,
+                                     None)
+
+    assert gwin(64, 4, idx=0) == -1
+    assert gwin(70, 27) == -2                                  # llama_mem.py:330
+    assert gwin(70, 4, q_win=None) == -1
+    assert gwin(20, 4) == -9
 
 
 def test_python_shim_rejects_what_the_reference_rejects():

@@ -136,20 +136,101 @@ def test_incomplete_cached_block(n_mems, inc, T, block, top_k):
         assert (out[b, h, t] - o).abs().max().item() <= 2e-2, (b, h, t)
 
 
-def test_local_window_rows_bit_exact():
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_local_window_rows_bit_exact(dtype):
     # the window builder alone: rotated tail keys bit for bit, values and new rows copied, zero query rows
     from landmark_hip import _lib
     B, H, T, D, block, inc = 1, 2, 3, 128, 32, 6
     S = 4 * block + inc
-    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=77)
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=77, dtype=dtype)
     k_ref, v_ref = oret.local_window(kc, vc, kl, vl, cos, sin, block)
     dev = lambda t: t.cuda()
     qd, kcd, vcd, kld, vld, cd, sd = map(dev, (q, kc, vc, kl, vl, cos, sin))
     qw, kw, vw = (torch.full((B, H, inc + T, D), 3.0, device="cuda:0", dtype=q.dtype) for _ in range(3))
     T4 = _lib.tensor4
     _lib.check(_lib.lib().lmk_local_window(T4(qd), T4(kcd), T4(vcd), T4(kld), T4(vld), cd.data_ptr(), sd.data_ptr(),
-                                           cd.stride(0), cd.shape[0], T4(qw), T4(kw), T4(vw), B, H, T, S, D, block, 0,
-                                           _lib.current_stream(qd.device)))
+                                           cd.stride(0), cd.shape[0], T4(qw), T4(kw), T4(vw), B, H, T, S, D, block,
+                                           _lib.DTYPE_CODES[dtype], _lib.current_stream(qd.device)))
+    torch.cuda.synchronize()
+    assert torch.equal(kw.cpu(), k_ref) and torch.equal(vw.cpu(), v_ref)
+    assert torch.equal(qw.cpu()[:, :, inc:], q) and (qw.cpu()[:, :, :inc] == 0).all()
+
+
+SHARED_CASES = [
+    # B, H, T, n_mems, inc, D, block, top_k, dtype, scale
+    (1, 2, 8, 64, 0, 128, 32, 4, torch.bfloat16, 0.5),
+    (2, 3, 40, 20, 0, 128, 32, 5, torch.bfloat16, 0.5),
+    (1, 2, 16, 3, 0, 128, 32, 5, torch.bfloat16, 0.5),       # fewer cached blocks than top_k
+    (1, 2, 100, 1500, 0, 128, 32, 4, torch.bfloat16, 0.5),   # more blocks than one sweep of 1024, ragged lanes
+    (1, 2, 64, 40, 0, 128, 64, 3, torch.bfloat16, 0.5),
+    (1, 2, 32, 50, 0, 64, 32, 4, torch.bfloat16, 0.5),
+    (1, 2, 24, 70, 0, 128, 32, 4, torch.float16, 0.5),       # fp16 probabilities reach the subnormal range
+    (1, 2, 24, 300, 0, 128, 32, 8, torch.bfloat16, 6.0),     # peaked softmax: probabilities down to subnormals and zero
+    (1, 2, 1, 300, 0, 128, 32, 8, torch.bfloat16, 6.0),      # one query: the head's vector is that query's probabilities
+    (1, 2, 5, 17, 9, 128, 32, 4, torch.bfloat16, 0.5),       # cache ends in an incomplete block
+    (1, 3, 1, 33, 31, 128, 32, 2, torch.bfloat16, 0.5),      # decode step that lands on the landmark
+    (1, 2, 20, 12, 40, 128, 64, 3, torch.float16, 0.5),
+]
+
+
+@pytest.mark.parametrize("B,H,T,n_mems,inc,D,block,top_k,dtype,scale", SHARED_CASES)
+def test_selection_shared_by_the_queries_of_a_head(B, H, T, n_mems, inc, D, block, top_k, dtype, scale):
+    # aggregate == "max_over_tokens" (llama_mem.py:373-377): indices bit for bit, attention within 2e-2 of the
+    # fp32 closed form with the selected blocks as history and of the model-dtype high-level restatement
+    from landmark_hip.retrieval import retrieve_and_attend
+    S = n_mems * block + inc
+    print(f"case B{B} H{H} T{T} n_mems{n_mems} inc{inc} D{D} bs{block} k{top_k} {dtype} x{scale}", flush=True)
+    g = torch.Generator().manual_seed(S + T)
+    mk = lambda *s, a=0.5: (torch.randn(*s, generator=g) * a).to(dtype)
+    q, kc, vc, kl, vl = mk(B, H, T, D, a=scale), mk(B, H, S, D, a=scale), mk(B, H, S, D), mk(B, H, T, D), mk(B, H, T, D)
+    cos, sin = orot.rotary_tables(S + T, D, dtype)
+    k = min(top_k, n_mems)
+    sc = oret.landmark_scores(q, kc, cos, sin, block, top_k)
+    agg = oret.aggregate_max_over_tokens(sc)
+    want = oret.select_topk(agg, k)
+    dev = lambda t: t.cuda()
+    out, idx = retrieve_and_attend(dev(q), (dev(kc), dev(vc)), dev(kl), dev(vl), dev(cos), dev(sin), block, top_k,
+                                   aggregate="max_over_tokens")
+    torch.cuda.synchronize()
+    assert idx.shape == (B, H, 1, k) and idx.dtype == torch.int64
+    assert torch.equal(idx.cpu(), want)
+    # the vector the selection ran on, bit for bit (exponential, order of the sum, division, rounding, maximum)
+    from landmark_hip.retrieval import retrieve_topk
+    idx2, probs = retrieve_topk(dev(q), dev(kc), dev(cos), dev(sin), block, top_k, aggregate="max_over_tokens",
+                                return_block_probs=True)
+    assert torch.equal(idx2, idx) and torch.equal(probs.cpu().view(torch.int16), agg.view(torch.int16))
+    # the library expression agrees on heads where its values equal the contract's and the k-th place is not tied
+    lib = torch.softmax(sc, dim=-1, dtype=torch.float32).to(dtype).amax(dim=2, keepdim=True)
+    ok = ~oret.boundary_tie_rows(lib, k) & (lib == agg).all(-1)
+    assert torch.equal(idx.cpu()[ok], lib.topk(k, dim=-1).indices.sort(-1).values[ok])
+    ref32 = oret.retrieve_and_attend_shared_s1(q, kc, vc, kl, vl, cos, sin, block, top_k, want)
+    assert (out.float().cpu() - ref32).abs().max().item() <= 2e-2
+    if scale > 1:            # scores of magnitude 100: their 16-bit rounding alone moves the high-level path's weights
+        return
+    is_mem = ((torch.arange(T) + inc) % block == block - 1)[None].expand(B, T)
+    ref16, _ = oret.retrieve_and_attend_shared(q, kc, vc, kl, vl, is_mem, cos, sin, block, top_k, idx=want,
+                                               n_buckets=max(64, k + T // block + 2))
+    assert (out.float().cpu() - ref16.float()).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gather_window_rows_bit_exact(dtype):
+    # the builder alone: selected keys rotated at their slot positions bit for bit, values copied, then tail and chunk
+    from landmark_hip import _lib
+    B, H, T, D, block, inc, top_k, n_mems = 1, 2, 3, 128, 32, 6, 3, 9
+    S = n_mems * block + inc
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=78, dtype=dtype)
+    idx = torch.tensor([[0, 6, 8], [2, 3, 7]]).view(B, H, 1, top_k)      # 6.. are among the newest three: bumped
+    k_ref, v_ref = oret.shared_window(kc, vc, kl, vl, idx, cos, sin, block, top_k)
+    dev = lambda t: t.cuda()
+    qd, kcd, vcd, kld, vld, cd, sd, idxd = map(dev, (q, kc, vc, kl, vl, cos, sin, idx))
+    W = top_k * block + inc + T
+    qw = torch.full((B, H, inc + T, D), 3.0, device="cuda:0", dtype=q.dtype)
+    kw, vw = (torch.full((B, H, W, D), 3.0, device="cuda:0", dtype=q.dtype) for _ in range(2))
+    T4 = _lib.tensor4
+    _lib.check(_lib.lib().lmk_gather_window(T4(qd), T4(kcd), T4(vcd), idxd.data_ptr(), T4(kld), T4(vld), cd.data_ptr(),
+                                            sd.data_ptr(), cd.stride(0), cd.shape[0], T4(qw), T4(kw), T4(vw), B, H, T, S,
+                                            D, block, top_k, _lib.DTYPE_CODES[dtype], _lib.current_stream(qd.device)))
     torch.cuda.synchronize()
     assert torch.equal(kw.cpu(), k_ref) and torch.equal(vw.cpu(), v_ref)
     assert torch.equal(qw.cpu()[:, :, inc:], q) and (qw.cpu()[:, :, :inc] == 0).all()

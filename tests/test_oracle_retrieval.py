@@ -200,3 +200,100 @@ def test_incomplete_cached_block_literal_row():
                 loc = torch.softmax((kb[: bs - 1] @ qq) / math.sqrt(hd), 0)
                 o = o + w[j] * (loc @ vb[: bs - 1])
             assert (out[0, h, t].double() - o).abs().max() < 2e-5, (h, t)
+
+
+# ------------------------------------------------- one selection per head (max_over_tokens, llama_mem.py:373-377)
+def test_exp2_contract_against_numpy_and_exact_at_integers():
+    import numpy as np
+    t = -np.abs(np.random.default_rng(0).normal(size=50000)).astype(np.float32) * np.float32(25.0)
+    got = retrieval.exp2_contract(t)
+    want = np.exp2(t.astype(np.float64))
+    assert got.dtype == np.float32
+    assert (np.abs(got - want) <= 5e-7 * want).all()
+    n = -np.arange(0, 127, dtype=np.float32)
+    assert np.array_equal(retrieval.exp2_contract(n), np.exp2(n))           # powers of two come out exactly
+    assert retrieval.exp2_contract(np.float32(-126.5)) == 0 and retrieval.exp2_contract(np.float32(-1e30)) == 0
+    # monotone over a fine grid (a flipped coefficient sign or a dropped term breaks this)
+    grid = -np.linspace(0, 40, 200001).astype(np.float32)
+    assert (np.diff(retrieval.exp2_contract(grid)) <= 0).all()
+
+
+def test_softmax_contract_literal_loop_and_torch_softmax():
+    import numpy as np
+    x = _rand(2, 3, 4, 200, seed=30, dtype=torch.bfloat16, scale=3.0).float()
+    got = retrieval.softmax_contract(x, torch.bfloat16)
+    # literal wave order on one row: 64 lanes add their strided elements in turn, then fold by halves
+    row = x[1, 2, 3].numpy()
+    e = retrieval.exp2_contract(((row - row.max()).astype(np.float32) * np.float32(1.4426950408889634)).astype(np.float32))
+    lanes = [np.float32(0.0)] * 64
+    for m in range(len(e)):
+        lanes[m % 64] = np.float32(lanes[m % 64] + e[m])
+    w = 32
+    while w:
+        lanes = [np.float32(lanes[i] + lanes[i + w]) for i in range(w)]
+        w //= 2
+    want = torch.tensor([np.float32(v / lanes[0]) for v in e]).to(torch.bfloat16)
+    assert torch.equal(got[1, 2, 3], want)
+    # library softmax: same values up to the last bit of the 16-bit result, and on nearly every element
+    lib = torch.softmax(x, dim=-1, dtype=torch.float32)
+    assert (got.float() - lib).abs().max() <= lib.max() * 2 ** -8
+    assert (got != lib.to(torch.bfloat16)).float().mean() < 1e-3
+    assert (got.float().sum(-1) - 1).abs().max() < 2e-2
+
+
+def test_shared_selection_equals_torch_expression_on_untied_heads():
+    B, nh, T, hd, bs, nm, k = 2, 4, 12, 16, 8, 40, 3
+    S = nm * bs
+    q = _rand(B, nh, T, hd, seed=31, dtype=torch.bfloat16, scale=1.5)
+    kc = _rand(B, nh, S, hd, seed=32, dtype=torch.bfloat16, scale=1.5)
+    cos, sin = rotary.rotary_tables(S + T, hd, torch.bfloat16)
+    sc = retrieval.landmark_scores(q, kc, cos, sin, bs, k)
+    agg = retrieval.aggregate_max_over_tokens(sc)
+    assert agg.shape == (B, nh, 1, nm) and agg.dtype == torch.bfloat16
+    idx = retrieval.select_topk(agg, k)
+    assert idx.shape == (B, nh, 1, k)
+    lib = torch.softmax(sc, dim=-1, dtype=torch.float32).to(sc.dtype).amax(dim=2, keepdim=True)      # :376-377
+    lib_idx = lib.topk(k, dim=-1).indices.sort(dim=-1).values                                         # :384
+    ok = ~retrieval.boundary_tie_rows(lib, k) & (lib == agg).all(-1)
+    assert ok.float().mean() > 0.7
+    assert torch.equal(idx[ok], lib_idx[ok])
+
+
+@pytest.mark.parametrize("inc,T", [(0, 16), (0, 5), (3, 4), (5, 3)])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+def test_shared_attend_equals_closed_form_with_history_blocks(dtype, tol, inc, T):
+    B, nh, hd, bs, nm, k = 1, 2, 16, 8, 6, 3
+    S = nm * bs + inc
+    q = _rand(B, nh, T, hd, seed=40, dtype=dtype, scale=0.5)
+    kc = _rand(B, nh, S, hd, seed=41, dtype=dtype, scale=0.5)
+    vc = _rand(B, nh, S, hd, seed=42, dtype=dtype, scale=0.5)
+    kl = _rand(B, nh, T, hd, seed=43, dtype=dtype, scale=0.5)
+    vl = _rand(B, nh, T, hd, seed=44, dtype=dtype, scale=0.5)
+    is_mem = ((torch.arange(T) + inc) % bs == bs - 1)[None]
+    cos, sin = rotary.rotary_tables(S + T, hd, dtype)
+    out, idx = retrieval.retrieve_and_attend_shared(q, kc, vc, kl, vl, is_mem, cos, sin, bs, k)
+    assert idx.shape == (B, nh, 1, k) and (idx[..., 1:] > idx[..., :-1]).all()
+    ref = retrieval.retrieve_and_attend_shared_s1(q, kc, vc, kl, vl, cos, sin, bs, k, idx)
+    assert (out.float() - ref).abs().max() < tol
+    # every query of a head uses the head's one set: the per-token step with that set forced gives the same
+    per_tok, _ = retrieval.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, bs, k, idx=idx.expand(B, nh, T, k))
+    assert (out.float() - per_tok.float()).abs().max() < tol
+
+
+def test_shared_window_rows_hand_worked():
+    # 5 blocks of 4 + tail of 2, top-2, head picks blocks {1, 4}: block 4 is among the newest two -> bumped one block
+    bs, nm, inc, T, hd = 4, 5, 2, 1, 8
+    S = nm * bs + inc
+    kc = _rand(1, 1, S, hd, seed=50)
+    vc = _rand(1, 1, S, hd, seed=51)
+    kl, vl = _rand(1, 1, T, hd, seed=52), _rand(1, 1, T, hd, seed=53)
+    cos, sin = rotary.rotary_tables(S + T, hd)
+    idx = torch.tensor([1, 4]).view(1, 1, 1, 2)
+    keys, values = retrieval.shared_window(kc, vc, kl, vl, idx, cos, sin, bs, 2)
+    assert keys.shape == (1, 1, 2 * bs + inc + T, hd)
+    prefix_len = 20 - 3 * 4
+    want_pos = [prefix_len + r for r in range(4)] + [prefix_len + 4 + 4 + r for r in range(4)] + [20, 21]
+    src = list(range(4, 8)) + list(range(16, 20)) + [20, 21]
+    want = rotary.apply_rotary(kc[0, 0, src], cos, sin, torch.tensor(want_pos))
+    assert torch.equal(keys[0, 0, : 2 * bs + inc], want) and torch.equal(keys[0, 0, -1], kl[0, 0, 0])
+    assert torch.equal(values[0, 0, : 2 * bs + inc], vc[0, 0, src]) and torch.equal(values[0, 0, -1], vl[0, 0, 0])
