@@ -116,6 +116,35 @@ def decode_bench(n=50, warm=5):
             "topk_ms": t_topk, "gather_attend_ms": t_att}
 
 
+def side_legs(n=30, warm=5):
+    """Two callers' steps either side of the attention kernels: the per-head selection of the offloaded-cache
+    branch on config 4's shapes, and the rotary embedding of q and k at config 2's shapes."""
+    import torch
+    from landmark_hip.retrieval import attend_shared, retrieve_topk
+    from landmark_hip.rotary import apply_rotary_pos_emb
+    dev = torch.device("cuda:0")
+    B, H, T, S, D, block, top_k = 1, 32, 256, 32768, 128, 32, 4
+    g = torch.Generator().manual_seed(2)
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.5).bfloat16().to(dev)
+    q, kc, vc, kl, vl = mk(B, H, T, D), mk(B, H, S, D), mk(B, H, S, D), mk(B, H, T, D), mk(B, H, T, D)
+    inv = 1.0 / (10000 ** (torch.arange(0, D, 2).float() / D))
+    ang = torch.outer(torch.arange(S + T).float(), inv)
+    ang = torch.cat((ang, ang), -1)
+    cos, sin = ang.cos().bfloat16().to(dev), ang.sin().bfloat16().to(dev)
+    idx = retrieve_topk(q, kc, cos, sin, block, top_k, aggregate="max_over_tokens")
+    t_sel = _time_launches(lambda: retrieve_topk(q, kc, cos, sin, block, top_k, aggregate="max_over_tokens"), n, warm)
+    t_att = _time_launches(lambda: attend_shared(q, kc, vc, idx, kl, vl, cos, sin, block, top_k), n, warm)
+    Bq, Lq = 2, 2048
+    xq, xk = mk(Bq, H, Lq, D), mk(Bq, H, Lq, D)
+    pos = torch.arange(Lq, device=dev)[None]
+    t_rot = _time_launches(lambda: apply_rotary_pos_emb(xq, xk, cos, sin, pos), n, warm)
+    rot_bytes = 2 * 2 * xq.numel() * 2 + 2 * Lq * D * 2
+    return {"per_head_selection": {"workload": "config 4 shapes, aggregate=max_over_tokens", "topk_ms": t_sel,
+                                   "attend_ms": t_att},
+            "rotary": {"workload": "q and k of config 2, (2,32,2048,128) bf16 each", "ms": t_rot,
+                       "GBps": rot_bytes / 1e6 / t_rot, "frac_hbm": rot_bytes / 1e6 / t_rot / PEAK_HBM_GBS}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -235,6 +264,7 @@ def main():
     if not a.no_retrieval:
         line["retrieval"] = retrieval_bench()
         line["retrieval_decode"] = decode_bench()
+        line.update(side_legs())
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

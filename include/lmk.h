@@ -188,6 +188,16 @@ int lmk_gather_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
                       const lmk_tensor4* v_win, int B, int H, int T, int S, int D, int block, int top_k, int dtype,
                       void* stream);
 
+/* Rotary position embedding of one (B,H,L,D) tensor: out = x*cos[pos] + rotate_half(x)*sin[pos] with
+ * pos = position_ids[b*pos_stride_b + l], rounded to the model dtype after each of the three elementwise
+ * operations, i.e. bit for bit what apply_rotary_pos_emb (llama/llama_mem.py:127-149) yields for q or
+ * for k in a 16-bit model (its call sites: :298 on the projections, :340, :366, :403 on cached keys).
+ * position_ids: device int64, (B,L) with pos_stride_b = L, or one row shared by the batch with
+ * pos_stride_b = 0; positions outside [0, n_pos) are clamped to the tables' ends.  out may alias x. */
+int lmk_apply_rotary(const lmk_tensor4* x, const lmk_tensor4* out, const void* cos_table, const void* sin_table,
+                     int64_t table_stride_row, int64_t n_pos, const int64_t* position_ids, int64_t pos_stride_b, int B,
+                     int H, int L, int D, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

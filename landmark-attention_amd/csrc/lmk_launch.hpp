@@ -93,6 +93,17 @@ struct WindowParams {
   int64_t qws_b, qws_h, qws_r, kws_b, kws_h, kws_r, vws_b, vws_h, vws_r, cs_r;
 };
 
+// rotary embedding of a (B, H, L, D) tensor at positions pos[b * pos_stride_b + l]
+struct RotaryParams {
+  const void *x, *cos, *sin;
+  void* out;
+  const int64_t* pos;
+  int64_t pos_stride_b, n_pos;
+  int B, H, L;
+  int64_t xs_b, xs_h, xs_r, os_b, os_h, os_r, cs_r;
+};
+
+int launch_rotary(const RotaryParams& p, int D, int dtype, hipStream_t stream);
 int launch_retrieve_topk(const RetrParams& p, int D, int dtype, hipStream_t stream);
 int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream_t stream);   // one selection per head
 int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t stream);

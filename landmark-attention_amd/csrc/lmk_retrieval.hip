@@ -995,6 +995,54 @@ static int launch_window_t(const WindowParams& p, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// rotary embedding of a whole (B, H, L, D) tensor at per-(batch, token) positions
+// (apply_rotary_pos_emb, llama_mem.py:134-149): x*cos + rotate_half(x)*sin with the model dtype's
+// rounding after each of the three elementwise operations.  One 16-byte chunk per thread; a row's
+// chunks sit in one wave and every lane loads before any lane stores, so out may be x itself.
+// ---------------------------------------------------------------------------
+template <class T, int D>
+__global__ __launch_bounds__(256) void lmk_rotary_kernel(RotaryParams p) {
+  constexpr int LPR = D / 8;
+  constexpr int RPW = 256 / LPR;
+  const int tid = threadIdx.x, j = tid % LPR;
+  const int64_t row = (int64_t)blockIdx.x * RPW + tid / LPR;      // (b, h, l)
+  if (row >= (int64_t)p.B * p.H * p.L) return;
+  const int l = (int)(row % p.L);
+  const int bh = (int)(row / p.L);
+  const int b = bh / p.H, hh = bh % p.H;
+  int64_t pos = p.pos[(int64_t)b * p.pos_stride_b + l];
+  pos = pos < 0 ? 0 : (pos >= p.n_pos ? p.n_pos - 1 : pos);      // never read outside the tables
+  const char* src = (const char*)p.x + 2 * (b * p.xs_b + hh * p.xs_h + (int64_t)l * p.xs_r);
+  const u32x4_t x = *(const u32x4_t*)(src + 16 * j);
+  const u32x4_t other = *(const u32x4_t*)(src + 16 * (j ^ (LPR / 2)));
+  const u32x4_t c = *(const u32x4_t*)((const char*)p.cos + 2 * (pos * p.cs_r) + 16 * j);
+  const u32x4_t s = *(const u32x4_t*)((const char*)p.sin + 2 * (pos * p.cs_r) + 16 * j);
+  float o[8];
+  rotate_chunk<T>(x, other, c, s, j >= LPR / 2, o);
+  const u32x4_t r = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
+  *(u32x4_t*)((char*)p.out + 2 * (b * p.os_b + hh * p.os_h + (int64_t)l * p.os_r) + 16 * j) = r;
+}
+
+template <class T, int D>
+static int launch_rotary_t(const RotaryParams& p, hipStream_t stream) {
+  constexpr int RPW = 256 / (D / 8);
+  const int64_t rows = (int64_t)p.B * p.H * p.L;
+  hipLaunchKernelGGL((lmk_rotary_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+int launch_rotary(const RotaryParams& p, int D, int dtype, hipStream_t stream) {
+  if (dtype == LMK_DTYPE_BF16) {
+    if (D == 128) return launch_rotary_t<bf16_t, 128>(p, stream);
+    if (D == 64) return launch_rotary_t<bf16_t, 64>(p, stream);
+  } else if (dtype == LMK_DTYPE_F16) {
+    if (D == 128) return launch_rotary_t<f16_t, 128>(p, stream);
+    if (D == 64) return launch_rotary_t<f16_t, 64>(p, stream);
+  }
+  return LMK_ERR_UNSUPPORTED;
+}
+
 int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t stream) {
   if (dtype == LMK_DTYPE_BF16) {
     if (D == 128) return launch_window_t<bf16_t, 128>(p, stream);

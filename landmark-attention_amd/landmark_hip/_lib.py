@@ -70,6 +70,8 @@ def lib() -> ctypes.CDLL:
         L.lmk_gather_window.restype = i
         L.lmk_gather_window.argtypes = [T4, T4, T4, vp, T4, T4, vp, vp, i64, i64, T4, T4, T4,
                                         i, i, i, i, i, i, i, i, vp]
+        L.lmk_apply_rotary.restype = i
+        L.lmk_apply_rotary.argtypes = [T4, T4, vp, vp, i64, i64, vp, i64, i, i, i, i, i, vp]
         _lib = L
     return _lib
 

@@ -1,0 +1,41 @@
+"""Rotary position embedding on the HIP kernel, with the reference's call surface.
+
+``apply_rotary_pos_emb(q, k, cos, sin, position_ids)`` mirrors ``llama/llama_mem.py:134-149``:
+``cos``/``sin`` are the ``(1, 1, n_pos, hd)`` (or ``(n_pos, hd)``) model-dtype tables of
+``LlamaRotaryEmbedding`` (``:95-124``), ``position_ids`` is ``(bs, seq)`` or ``(1, seq)`` int64, ``q`` may
+be ``None`` (``:143-144``).  One launch per tensor replaces the reference's gather of the table rows,
+two products, ``rotate_half``'s concatenation and the sum, and gives the same bits: every one of the
+three elementwise operations rounds to the model dtype, as torch's 16-bit arithmetic does.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .retrieval import _tables
+
+
+def _rotate(x, cos, sin, position_ids, out=None):
+    B, H, L, D = x.shape
+    assert position_ids.dim() == 2 and position_ids.shape[1] == L and position_ids.shape[0] in (1, B)
+    assert position_ids.dtype == torch.int64 and position_ids.device == x.device
+    x = _lib.kernel_ready(x)
+    position_ids = position_ids.contiguous()
+    if out is None:
+        out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().lmk_apply_rotary(_lib.tensor4(x), _lib.tensor4(out), cos.data_ptr(), sin.data_ptr(),
+                                         cos.stride(0), cos.shape[0], position_ids.data_ptr(),
+                                         L if position_ids.shape[0] == B and B > 1 else 0, B, H, L, D,
+                                         _lib.DTYPE_CODES[x.dtype], _lib.current_stream(x.device))
+    _lib.check(rc)
+    return out
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, position_ids):
+    """``(q_embed, k_embed)`` as ``llama_mem.py:134-149`` returns them; ``q_embed`` is ``None`` when
+    ``q`` is.  q, k: ``(B, nh, L, hd)`` bf16/fp16 on the GPU with hd 64 or 128."""
+    assert k.is_cuda and k.dtype in _lib.DTYPE_CODES
+    cos, sin = _tables(cos, sin, k.dtype)
+    q_embed = None if q is None else _rotate(q, cos, sin, position_ids)
+    return q_embed, _rotate(k, cos, sin, position_ids)

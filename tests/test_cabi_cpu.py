@@ -30,7 +30,7 @@ def _declared():
 def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
-            "lmk_retrieve_topk_shared", "lmk_gather_window", "lmk_strerror"} <= set(names)
+            "lmk_retrieve_topk_shared", "lmk_gather_window", "lmk_apply_rotary", "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
 
@@ -134,6 +134,13 @@ def test_retrieval_argument_errors(lib):
     assert gwin(70, 27) == -2                                  # llama_mem.py:330
     assert gwin(70, 4, q_win=None) == -1
     assert gwin(20, 4) == -9
+
+    # rotary of a whole tensor
+    def rot(pos=0x7000, D=128, n_pos=64, stride=8, L=8, dtype=0):
+        return lib.lmk_apply_rotary(t, t, 0x5000, 0x6000, 128, n_pos, pos, stride, 1, 1, L, D, dtype, None)
+
+    assert rot(pos=0) == -1 and rot(D=96) == -3 and rot(n_pos=0) == -11 and rot(stride=-1) == -2 and rot(L=0) == -2
+    assert rot(dtype=5) == -3
 
 
 def test_python_shim_rejects_what_the_reference_rejects():

@@ -1,0 +1,79 @@
+"""Rotary embedding kernel against the oracle and against torch's own 16-bit elementwise arithmetic:
+bit for bit (llama/llama_mem.py:127-149)."""
+import pytest
+import torch
+
+from oracle import rotary as orot
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(B, H, L, D, dtype, seed, n_pos=None):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, L, D, generator=g).to(dtype)
+    k = torch.randn(B, H, L, D, generator=g).to(dtype)
+    n_pos = n_pos or 4 * L + 7
+    cos, sin = orot.rotary_tables(n_pos, D, dtype)
+    return q, k, cos, sin, n_pos, g
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,L,D", [(2, 3, 70, 128), (1, 2, 33, 64), (3, 1, 1, 128)])
+def test_rotary_bit_exact_against_oracle_and_torch_arithmetic(B, H, L, D, dtype):
+    from landmark_hip.rotary import apply_rotary_pos_emb
+    print(f"case B{B} H{H} L{L} D{D} {dtype}", flush=True)
+    q, k, cos, sin, n_pos, g = _case(B, H, L, D, dtype, seed=B * 100 + L)
+    pos = torch.randint(0, n_pos, (B, L), generator=g)
+    want_q = orot.apply_rotary(q, cos, sin, pos[:, None, :])
+    want_k = orot.apply_rotary(k, cos, sin, pos[:, None, :])
+    # the reference's expression evaluated by torch in the model dtype (one rounding per elementwise op)
+    c, s = cos[pos].unsqueeze(1), sin[pos].unsqueeze(1)
+    assert torch.equal(want_k, (k * c) + (orot.rotate_half(k) * s))
+    dev = lambda t: t.cuda()
+    gq, gk = apply_rotary_pos_emb(dev(q), dev(k), dev(cos)[None, None], dev(sin)[None, None], dev(pos))
+    torch.cuda.synchronize()
+    assert torch.equal(gq.cpu(), want_q) and torch.equal(gk.cpu(), want_k)
+    # q is optional (llama_mem.py:143-144); one row of positions serves the whole batch
+    row = pos[:1]
+    none_q, gk1 = apply_rotary_pos_emb(None, dev(k), dev(cos), dev(sin), dev(row))
+    assert none_q is None and torch.equal(gk1.cpu(), orot.apply_rotary(k, cos, sin, row[:, None, :]))
+
+
+def test_rotary_on_projection_layout_and_in_place():
+    # (B, L, H, D) memory viewed as (B, H, L, D), as the projections leave it (llama_mem.py:287-289)
+    from landmark_hip import _lib
+    from landmark_hip.rotary import apply_rotary_pos_emb
+    B, H, L, D = 2, 4, 50, 128
+    q, k, cos, sin, n_pos, g = _case(B, H, L, D, torch.bfloat16, seed=5)
+    pos = torch.arange(13, 13 + L)[None].expand(B, L).contiguous()
+    kd = k.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3)
+    assert not kd.is_contiguous()
+    _, gk = apply_rotary_pos_emb(None, kd, cos.cuda(), sin.cuda(), pos.cuda())
+    want = orot.apply_rotary(k, cos, sin, pos[:, None, :])
+    assert gk.stride() == kd.stride() and torch.equal(gk.cpu(), want)
+    # out aliasing x through the C ABI
+    x = k.cuda()
+    cd, sd, pd = cos.cuda(), sin.cuda(), pos.cuda()
+    _lib.check(_lib.lib().lmk_apply_rotary(_lib.tensor4(x), _lib.tensor4(x), cd.data_ptr(), sd.data_ptr(), cd.stride(0),
+                                           cd.shape[0], pd.data_ptr(), L, B, H, L, D, 0, _lib.current_stream(x.device)))
+    torch.cuda.synchronize()
+    assert torch.equal(x.cpu(), want)
+
+
+def test_rotary_feeds_the_fused_attention_like_the_reference_layer():
+    # the layer's order of operations (llama_mem.py:287-298, 441-446): rotate q and k, then fused attention
+    from landmark_hip.rotary import apply_rotary_pos_emb
+    from ltriton.flash_landmark_attention import fused_landmark_attention
+    from oracle import s1
+    B, H, L, D, block = 1, 2, 96, 128, 32
+    q, k, cos, sin, n_pos, g = _case(B, H, L, D, torch.bfloat16, seed=9, n_pos=L)
+    q, k = q * 0.5, k * 0.5
+    v = (torch.randn(B, H, L, D, generator=g) * 0.5).bfloat16()
+    pos = torch.arange(L)[None]
+    qr, kr = apply_rotary_pos_emb(q.cuda(), k.cuda(), cos.cuda(), sin.cuda(), pos.cuda())
+    is_mem = (torch.arange(L) % block == block - 1)[None].cuda()
+    out = fused_landmark_attention(qr, kr, v.cuda(), is_mem, block_size=block)
+    pq, pk = orot.apply_rotary(q, cos, sin, pos[:, None, :]), orot.apply_rotary(k, cos, sin, pos[:, None, :])
+    for h in range(H):
+        ref = s1.s1_attention(pq[0, h].float(), pk[0, h].float(), v[0, h].float(), block)
+        assert (out[0, h].float().cpu() - ref).abs().max().item() <= 2e-2
