@@ -1,0 +1,62 @@
+"""Growing KV cache for the mem-cache inference path.
+
+The reference keeps ``past_key_value = (K_without_rotary, V)`` and appends every new chunk with
+``torch.cat`` (``llama/llama_mem.py:424-430``), which copies the whole cache once per layer and
+step.  ``LandmarkKVCache`` holds the same two tensors in buffers with spare room along the
+sequence axis, so an append writes only the new rows; ``past_key_value`` hands out
+``(B, nh, S, hd)`` views of the filled part, which the retrieval kernels read in place through
+their strides.  Blocks stay contiguous per (batch, head): block ``m`` of a head is the
+``block * hd`` elements at row ``m * block``, the landmark key its last row.
+"""
+from __future__ import annotations
+
+import torch
+
+from .retrieval import retrieve_and_attend
+
+
+class LandmarkKVCache:
+    """``(K_without_rotary, V)`` of one attention layer with amortised O(new rows) appends."""
+
+    def __init__(self, batch: int, heads: int, head_dim: int, dtype, device, capacity: int = 4096):
+        self._k = torch.empty((batch, heads, capacity, head_dim), dtype=dtype, device=device)
+        self._v = torch.empty_like(self._k)
+        self.length = 0
+
+    @property
+    def capacity(self) -> int:
+        return self._k.shape[2]
+
+    @property
+    def past_key_value(self):
+        """The reference's cache tuple (``llama_mem.py:430``): views, no copy."""
+        return self._k[:, :, : self.length], self._v[:, :, : self.length]
+
+    def _reserve(self, rows: int) -> None:
+        if rows <= self.capacity:
+            return
+        cap = max(rows, 2 * self.capacity)
+        for name in ("_k", "_v"):
+            old = getattr(self, name)
+            new = torch.empty(old.shape[:2] + (cap, old.shape[3]), dtype=old.dtype, device=old.device)
+            new[:, :, : self.length] = old[:, :, : self.length]
+            setattr(self, name, new)
+
+    def append(self, key_states_before_pos, value_states) -> None:
+        """``torch.cat([past, new], dim=2)`` of ``llama_mem.py:424-425`` without re-copying ``past``."""
+        t = key_states_before_pos.shape[2]
+        assert key_states_before_pos.shape == value_states.shape == self._k.shape[:2] + (t, self._k.shape[3])
+        self._reserve(self.length + t)
+        self._k[:, :, self.length : self.length + t] = key_states_before_pos
+        self._v[:, :, self.length : self.length + t] = value_states
+        self.length += t
+
+    def step(self, query_states, key_states, key_states_before_pos, value_states, cos, sin, block: int, top_k: int,
+             sm_scale=None, aggregate=None):
+        """Attention of a new chunk against the cache, then the append (``llama_mem.py:318-430,447-477``):
+        ``query_states`` and ``key_states`` rotated at the chunk's positions, ``key_states_before_pos`` the
+        same keys without rotary.  Needs at least one complete cached block; returns ``(out, idx)``."""
+        out, idx = retrieve_and_attend(query_states, self.past_key_value, key_states, value_states, cos, sin,
+                                       block, top_k, sm_scale, aggregate)
+        self.append(key_states_before_pos, value_states)
+        return out, idx
