@@ -354,48 +354,83 @@ __global__ __launch_bounds__(256) void lmk_fill_u32_kernel(uint32_t* dst, int64_
 // One wave per (batch, head, query): scores -> softmax -> 16-bit probabilities -> maximum per block
 // into agg (B*H, num_mems), which holds zeros on entry.  A lane owns the blocks m = lane, lane + 64, ...;
 // the row's sum is each lane's running sum in that order, folded across lanes by halves.
+// A workgroup is four queries of one (batch, head): tiles of 128 rotated landmark keys are staged
+// through LDS with coalesced loads and shared by the four waves (a lane reading its own key row
+// straight from memory is one 64-byte request per lane and instruction); the query sits in registers.
 template <class T, int D>
 __global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
-  __shared__ __align__(16) float q_lds[4][D];
+  constexpr int ROWB = 2 * D + 16;                                // padded key row: a 16-lane group reads 16 B each, all banks
+  constexpr int CPR = D / 8;                                      // 16-byte chunks per key row
+  constexpr int TM = 128;                                         // landmark keys per tile: two per lane
+  constexpr int NCH = TM * CPR / 256;                             // chunks per thread and tile
+  __shared__ __align__(16) unsigned char tile[TM * ROWB];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t row = (int64_t)blockIdx.x * 4 + wave;             // (bh, t)
-  if (row >= (int64_t)p.B * p.H * p.T) return;                    // whole wave leaves; no block-wide barrier below
-  const int bh = (int)(row / p.T), t = (int)(row % p.T);
+  const int n_rg = (p.T + 3) / 4;
+  const int bh = blockIdx.x / n_rg, t = (blockIdx.x % n_rg) * 4 + wave;
+  const bool active = t < p.T;                                    // idle waves still help with the tiles
   const int b = bh / p.H, hh = bh % p.H;
   const int NM = p.num_mems;
-  const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
-  for (int d = 2 * lane; d < D; d += 128) {
-    const uint32_t u = *(const uint32_t*)(qp + 2 * d);
-    q_lds[wave][d] = unpack_lo<T>(u);
-    q_lds[wave][d + 1] = unpack_hi<T>(u);
+  float qf[D];
+  {
+    const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)(active ? t : 0) * p.qs_r);
+#pragma unroll
+    for (int c = 0; c < CPR; ++c) {
+      const u32x4_t u = *(const u32x4_t*)(qp + 16 * c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        qf[8 * c + 2 * i] = unpack_lo<T>(u[i]);
+        qf[8 * c + 2 * i + 1] = unpack_hi<T>(u[i]);
+      }
+    }
   }
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_s_waitcnt(0xc07f);                             // LDS writes of this wave visible (lgkmcnt 0)
-
+  const int64_t row = (int64_t)bh * p.T + (active ? t : 0);
   float* sc = p.approx + row * NM;                                // this row's scores, then its exponentials
   const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * NM * D);
-  float mx = -INFINITY;
-  for (int m = lane; m < NM; m += 64) {
-    const char* kr = lk + 2 * ((int64_t)m * D);
-    float acc = 0.f;
-#pragma unroll 4
-    for (int d8 = 0; d8 < D / 8; ++d8) {
-      const u32x4_t kk = *(const u32x4_t*)(kr + 16 * d8);
-      const float4 qa = *(const float4*)&q_lds[wave][8 * d8];
-      const float4 qb = *(const float4*)&q_lds[wave][8 * d8 + 4];
-      acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
-      acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
-      acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
-      acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
-      acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
-      acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
-      acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
-      acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
+
+  auto fetch = [&](int m0, u32x4_t* r) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = i * 256 + tid, kr = c / CPR, col = c % CPR;
+      u32x4_t z = {0, 0, 0, 0};
+      r[i] = (m0 + kr < NM) ? *(const u32x4_t*)(lk + 2 * ((int64_t)(m0 + kr) * D) + 16 * col) : z;
     }
-    const float x = contract<T>(acc, p.sqrt_hd);
-    sc[m] = x;                                                    // read back below by the same lane only
-    mx = fmaxf(mx, x);
+  };
+  u32x4_t nxt[NCH];
+  fetch(0, nxt);
+  float mx = -INFINITY;
+  for (int m0 = 0; m0 < NM; m0 += TM) {
+    __syncthreads();                                              // the previous tile has been read by every wave
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = i * 256 + tid;
+      *(u32x4_t*)(tile + (c / CPR) * ROWB + 16 * (c % CPR)) = nxt[i];
+    }
+    __syncthreads();
+    if (m0 + TM < NM) fetch(m0 + TM, nxt);                        // in flight during the arithmetic below
+#pragma unroll 1
+    for (int half = 0; half < TM / 64; ++half) {
+      const int m = m0 + 64 * half + lane;
+      if (!(active && m < NM)) continue;
+      const unsigned char* kr = tile + (64 * half + lane) * ROWB;
+      float acc = 0.f;
+#pragma unroll
+      for (int d8 = 0; d8 < CPR; ++d8) {
+        const u32x4_t kk = *(const u32x4_t*)(kr + 16 * d8);
+        acc = __builtin_fmaf(qf[8 * d8 + 0], unpack_lo<T>(kk[0]), acc);
+        acc = __builtin_fmaf(qf[8 * d8 + 1], unpack_hi<T>(kk[0]), acc);
+        acc = __builtin_fmaf(qf[8 * d8 + 2], unpack_lo<T>(kk[1]), acc);
+        acc = __builtin_fmaf(qf[8 * d8 + 3], unpack_hi<T>(kk[1]), acc);
+        acc = __builtin_fmaf(qf[8 * d8 + 4], unpack_lo<T>(kk[2]), acc);
+        acc = __builtin_fmaf(qf[8 * d8 + 5], unpack_hi<T>(kk[2]), acc);
+        acc = __builtin_fmaf(qf[8 * d8 + 6], unpack_lo<T>(kk[3]), acc);
+        acc = __builtin_fmaf(qf[8 * d8 + 7], unpack_hi<T>(kk[3]), acc);
+      }
+      const float x = contract<T>(acc, p.sqrt_hd);
+      sc[m] = x;                                                  // read back below by the same lane only
+      mx = fmaxf(mx, x);
+    }
   }
+  if (!active) return;                                            // no block-wide barrier below
 #pragma unroll
   for (int msk = 32; msk >= 1; msk >>= 1) mx = fmaxf(mx, __shfl_xor(mx, msk, 64));
   float sum = 0.f;
@@ -895,8 +930,7 @@ static int launch_topk_shared_t(const RetrParams& p, hipStream_t stream) {
   if ((rc = (int)hipGetLastError())) return rc;
   hipLaunchKernelGGL(lmk_fill_u32_kernel, dim3((unsigned)((lkrows + 255) / 256)), dim3(256), 0, stream, p.agg, lkrows, 0u);
   if ((rc = (int)hipGetLastError())) return rc;
-  const int64_t rows = (int64_t)p.B * p.H * p.T;
-  hipLaunchKernelGGL((lmk_block_prob_kernel<T, D>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL((lmk_block_prob_kernel<T, D>), dim3((unsigned)(p.B * p.H * ((p.T + 3) / 4))), dim3(256), 0, stream, p);
   if ((rc = (int)hipGetLastError())) return rc;
   hipLaunchKernelGGL(lmk_block_select_kernel, dim3(p.B * p.H), dim3(64), 0, stream, p);
   return (int)hipGetLastError();
