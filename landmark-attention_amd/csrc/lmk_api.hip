@@ -267,7 +267,7 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
     return LMK_ERR_NULL;
   if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
   if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
-  if (D != 128 || !(block == 32 || block == 64)) return LMK_ERR_UNSUPPORTED;
+  if (D != 128 || !(block == 32 || block == 64 || block == 128)) return LMK_ERR_UNSUPPORTED;
   if (stat_stride < T) return LMK_ERR_SHAPE;
   if (!std::isfinite(sm_scale) || !(sm_scale > 0.f)) return LMK_ERR_SCALE;
   lmk::RetrParams p = {};

@@ -85,7 +85,8 @@ def test_fp16_indices_bit_exact():
 @pytest.mark.parametrize("B,H,T,S,block,top_k", [(1, 2, 64, 24 * 32, 32, 4), (1, 2, 128, 12 * 64, 64, 3),
                                                   (2, 2, 96, 3 * 32, 32, 5),
                                                   (1, 2, 1, 24 * 32, 32, 4),      # decode: first token of a new block
-                                                  (1, 2, 5, 12 * 64, 64, 3)])
+                                                  (1, 2, 5, 12 * 64, 64, 3),
+                                                  (1, 2, 160, 9 * 128, 128, 3), (2, 2, 7, 2 * 128, 128, 4)])
 def test_gather_attend_matches_oracle(B, H, T, S, block, top_k):
     from landmark_hip.retrieval import retrieve_and_attend
     D = 128
@@ -115,6 +116,8 @@ def test_gather_attend_matches_oracle(B, H, T, S, block, top_k):
     (3, 5, 2, 32, 5),           # fewer complete blocks than top_k
     (12, 40, 24, 64, 3),        # block 64, ends on the landmark
     (12, 17, 1, 64, 3),
+    (7, 100, 28, 128, 2),       # block 128, ends on the landmark
+    (7, 5, 1, 128, 4),
 ])
 def test_incomplete_cached_block(n_mems, inc, T, block, top_k):
     from landmark_hip.retrieval import retrieve_and_attend
