@@ -144,3 +144,24 @@ def test_baseline_config1_full_size():
     err = (out - ref).abs().max().item()
     print("config1 max abs err", err, flush=True)
     assert err <= TOL
+
+
+def test_baseline_config3_full_size():
+    # benchmark config 3: B1 H32 L16384 D128 block 32, is_mem omitted (landmarks at fixed stride): 512 blocks,
+    # the landmark softmax of the last rows runs over 511 earlier blocks
+    from oracle import s1
+    B, H, L, D, block = 1, 32, 16384, 128, 32
+    q, k, v = make_qkv(B, H, L, L, D, seed=0)
+    print("config3 inputs ready", flush=True)
+    out = _run(q, k, v, block, is_mem=None).float().cpu()
+    rows = [0, 30, 31, 32, 1023, 1024, 8191, 8192, 12345, 16351, 16352, 16382, 16383]
+    worst = 0.0
+    for h in (0, 13, 31):
+        ref = s1.s1_attention(q[0, h].float(), k[0, h].float(), v[0, h].float(), block, rows=rows)
+        worst = max(worst, (out[0, h, rows] - ref).abs().max().item())
+    print("config3 max abs err on sampled rows", worst, flush=True)
+    assert worst <= TOL
+    # every row of every head: the weights sum to one (values all ones -> output all ones)
+    ones = torch.ones_like(v)
+    out1 = _run(q, k, ones, block, is_mem=None).float()
+    assert (out1 - 1).abs().max().item() <= 1e-2
