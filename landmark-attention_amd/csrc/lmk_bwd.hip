@@ -57,37 +57,58 @@ __global__ __launch_bounds__(256) void lmk_bwd_pre_kernel(BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// dq (+ per-block statistics)
+// dq (+ per-block statistics), landmark blocks of 64 and 128 keys
 // ---------------------------------------------------------------------------
+// A workgroup is 8 waves = 256 query rows, two waves per SIMD; a wave keeps the fragments of its 32
+// rows of Q and dO and its dQ^T accumulator in registers.  One stage is one landmark block: its K and
+// V rows come into one of two LDS buffers by direct global->LDS loads (no staging registers: the kernel
+// has to stay inside 256 registers for two waves to share a SIMD), requested one stage ahead, each wave
+// fetching its share; one barrier per stage.  The block's local softmax needs all its scores before any
+// weight is final, so the S^T tiles of the whole block stay in registers; with four tiles per block the
+// dP^T tiles do not fit beside them and are computed twice (once for nD, once for dS).
 template <class T, int D, int BS>
 struct DqCfg {
-  static constexpr int NT = BS / 32;
-  static constexpr int NB = (BS >= 64) ? 1 : 64 / BS;
-  static constexpr int SK = NB * BS;
+  static constexpr int NT = BS / 32;                       // MFMA tiles per landmark block
+  static constexpr int NW = 8;
   static constexpr int CH = D / 8;
-  static constexpr int TILE_BYTES = SK * 2 * D;
-  static constexpr int NCH = SK * CH / 256;
   static constexpr int KS = D / 16;
   static constexpr int DC = D / 32;
-  static constexpr int LDS_BYTES = 4 * TILE_BYTES;
+  static constexpr int ROWB = 2 * D;
+  static constexpr int TILE_BYTES = BS * ROWB;             // K (or V) of one block
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES;       // K, then V
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static constexpr int RPD = 1024 / ROWB;                  // rows covered by one 1 KB request
+  static constexpr int NREQ = 2 * BS / RPD;                // requests per stage
+  static constexpr int PER_WAVE = NREQ / NW;
+  static constexpr bool KEEP_DP = NT <= 2;                 // dP^T tiles kept beside the S^T tiles
+  static_assert(NREQ % NW == 0, "every wave issues the same number of requests");
 };
 
+// One 1 KB direct global->LDS request of a wave: lane i's 16 bytes land at lds_off + 16*i.
+// lds_off must be wave-uniform (it travels in M0).
+__device__ __forceinline__ void dq_dma16(const void* base_uniform, uint32_t voff, uint32_t lds_off) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(voff), "s"(base_uniform), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory");
+}
+
 template <class T, int D, int BS>
-__global__ __launch_bounds__(256, 1) void lmk_bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<T, D, BS>;
   extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ql = lane & 31, h = lane >> 5;
 
-  int bh, qtile;
+  const int nq256 = (p.Lq + 255) >> 8;
+  int bh, qt;                                              // (batch*head, 256-row query tile); most work first
   {
     const int bid = blockIdx.x, BH = p.B * p.H;
     if ((BH & 7) == 0) {
       const int xcd = bid & 7, j = bid >> 3, ngrp = BH >> 3;
-      qtile = p.n_qtiles - 1 - j / ngrp;
+      qt = nq256 - 1 - j / ngrp;
       bh = (j % ngrp) * 8 + xcd;
     } else {
-      qtile = p.n_qtiles - 1 - bid / BH;
+      qt = nq256 - 1 - bid / BH;
       bh = bid % BH;
     }
   }
@@ -98,12 +119,11 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dq_kernel(BwdParams p) {
   const char* gp = (const char*)p.dout + 2 * (b * p.dos_b + hh * p.dos_h);
   char* dqp = (char*)p.dq + 2 * (b * p.dqs_b + hh * p.dqs_h);
 
-  const int q0 = qtile * 128 + wave * 32;
+  const int q0 = qt * 256 + wave * 32;
   const int dt = p.n_prefix * C::NT + (q0 >> 5);
-  const int cblk = dt / C::NT, tsub = dt % C::NT;
-  const bool active = q0 < p.Lq;
+  const int cblk = dt / C::NT, tsub = dt % C::NT;          // the wave's own block and its tile inside it
+  const bool active = q0 < p.Lq;                           // Lq is a multiple of the block: whole tiles only
   const int qrow = q0 + ql;
-  const bool rowok = qrow < p.Lq;
 
   u32x4_t qf[C::KS], gf[C::KS];
 #pragma unroll
@@ -111,39 +131,40 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dq_kernel(BwdParams p) {
     u32x4_t z = {0, 0, 0, 0};
     qf[ks] = z;
     gf[ks] = z;
-    if (rowok) {
+    if (active) {
       qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
       gf[ks] = *(const u32x4_t*)(gp + 2 * ((int64_t)qrow * p.dos_r + 16 * ks + 8 * h));
     }
   }
-  const float mhat = rowok ? p.mhat[(int64_t)bh * p.Lq + qrow] : 0.f;
-  const float delta = rowok ? p.delta[(int64_t)bh * p.Lq + qrow] : 0.f;
+  const float mhat = active ? p.mhat[(int64_t)bh * p.Lq + qrow] : 0.f;
+  const float delta = active ? p.delta[(int64_t)bh * p.Lq + qrow] : 0.f;
 
-  const int tiles_needed = min(p.Lk >> 5, p.n_prefix * C::NT + qtile * 4 + 4);
-  const int n_stages = (tiles_needed * 32 + C::SK - 1) / C::SK;
-  u32x4_t kreg[C::NCH], vreg[C::NCH];
-  auto load_stage = [&](int s) {
+  // stages = blocks up to the own block of the workgroup's last query tile
+  const int last_q0 = min(qt * 256 + 224, p.Lq - 32);
+  const int n_stages = min(p.n_blocks, (p.n_prefix * C::NT + (last_q0 >> 5)) / C::NT + 1);
+
+  // this wave's requests of a stage: request r covers rows RPD*(r % (BS/RPD)) .. of K (r < BS/RPD) or V.
+  // The LDS swizzle is applied on the source side: lane i lands at +16*i, i.e. row i/CH, chunk position
+  // i%CH, so it fetches the chunk tile_off() stores there.
+  uint32_t src[C::PER_WAVE];                               // per-lane byte offset inside the (batch, head) slice of K or V
+  const int n_k = BS / C::RPD;                             // requests that fetch K rows; the rest fetch V rows
 #pragma unroll
-    for (int i = 0; i < C::NCH; ++i) {
-      const int id = tid + 256 * i, row = id / C::CH, ch = id % C::CH;
-      const int key = s * C::SK + row;
-      u32x4_t z = {0, 0, 0, 0};
-      kreg[i] = z;
-      vreg[i] = z;
-      if (key < p.Lk) {
-        kreg[i] = *(const u32x4_t*)(kp + 2 * ((int64_t)key * p.ks_r + 8 * ch));
-        vreg[i] = *(const u32x4_t*)(vp + 2 * ((int64_t)key * p.vs_r + 8 * ch));
-      }
-    }
-  };
-  auto store_stage = [&](int buf) {
-    unsigned char* kb = smem + buf * 2 * C::TILE_BYTES;
-    unsigned char* vb = kb + C::TILE_BYTES;
+  for (int i = 0; i < C::PER_WAVE; ++i) {
+    const int r = wave * C::PER_WAVE + i;
+    const bool is_v = r >= n_k;
+    const int row = C::RPD * (r % n_k) + lane / C::CH, cp = lane % C::CH;
+    const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
+    src[i] = (uint32_t)(2 * ((int64_t)row * (is_v ? p.vs_r : p.ks_r) + 8 * (cp ^ f)));
+  }
+  const uint32_t step_k = (uint32_t)(2 * (int64_t)BS * p.ks_r), step_v = (uint32_t)(2 * (int64_t)BS * p.vs_r);
+  auto request = [&](int buf) {                            // next block in key order -> buffer buf
 #pragma unroll
-    for (int i = 0; i < C::NCH; ++i) {
-      const int id = tid + 256 * i, row = id / C::CH, ch = id % C::CH;
-      *(u32x4_t*)(kb + tile_off<D>(row, ch)) = kreg[i];
-      *(u32x4_t*)(vb + tile_off<D>(row, ch)) = vreg[i];
+    for (int i = 0; i < C::PER_WAVE; ++i) {
+      const int r = wave * C::PER_WAVE + i;
+      const bool is_v = r >= n_k;                          // wave-uniform
+      const int dst = buf * C::STAGE_BYTES + (is_v ? C::TILE_BYTES : 0) + C::RPD * (r % n_k) * C::ROWB;
+      dq_dma16(is_v ? vp : kp, src[i], dst);
+      src[i] += is_v ? step_v : step_k;
     }
   };
 
@@ -154,112 +175,125 @@ __global__ __launch_bounds__(256, 1) void lmk_bwd_dq_kernel(BwdParams p) {
     for (int r = 0; r < 16; ++r) acc[dc][r] = 0.f;
   const float c2 = p.scale_log2;
 
-  auto row_tile = [&](const unsigned char* buf, int rb, const u32x4_t* bf) {
+  // LDS byte offsets of this lane's operand fragments inside a 32-row tile: the swizzle repeats every 16
+  // rows, so a tile at row 32u is the same offsets plus 32u rows -- an immediate of the LDS instruction
+  int koff[C::KS];
+#pragma unroll
+  for (int ks = 0; ks < C::KS; ++ks) koff[ks] = tile_off<D>(ql, 2 * ks + h);
+  int voff[C::DC][2];
+  {
+    const int i = lane & 15, g2 = (lane >> 4) & 1;
+#pragma unroll
+    for (int dc = 0; dc < C::DC; ++dc) {
+      const int col = 32 * dc + 16 * g2 + 4 * (i & 3);
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+        voff[dc][hf] = tile_off<D>(4 * h + (i >> 2) + 8 * hf, col >> 3) + ((col >> 2) & 1) * 8;
+    }
+  }
+  auto row_tile = [&](int tile_bytes, const u32x4_t* bf) {   // (32 rows of the LDS tile) x (this wave's 32 queries)
     f32x16_t s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(load_row_frag<D>(buf, rb, ks, lane), bf[ks], s);
+    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(lds_ld128(tile_bytes + koff[ks]), bf[ks], s);
     return s;
   };
-  auto dq_tile = [&](const unsigned char* kb, int rb, const float* ds) {
+  auto dq_tile = [&](int tile_bytes, const float* ds) {      // dQ^T += (K tile)^T dS^T
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       u32x4_t wf = {pack2<T>(ds[8 * j + 0], ds[8 * j + 1]), pack2<T>(ds[8 * j + 2], ds[8 * j + 3]),
                     pack2<T>(ds[8 * j + 4], ds[8 * j + 5]), pack2<T>(ds[8 * j + 6], ds[8 * j + 7])};
 #pragma unroll
-      for (int dc = 0; dc < C::DC; ++dc) acc[dc] = mfma32<T>(load_tr_frag<D>(kb, rb, j, dc, lane), wf, acc[dc]);
+      for (int dc = 0; dc < C::DC; ++dc) {
+        const int base = tile_bytes + 16 * j * C::ROWB;
+        const u32x2_t a0 = lds_ld_tr(base + voff[dc][0]), a1 = lds_ld_tr(base + voff[dc][1]);
+        const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
+        acc[dc] = mfma32<T>(a, wf, acc[dc]);
+      }
     }
   };
 
-  load_stage(0);
-  store_stage(0);
-  __syncthreads();
-
+  request(0);
   for (int s = 0; s < n_stages; ++s) {
     const int buf = s & 1;
-    if (s + 1 < n_stages) load_stage(s + 1);
-    const unsigned char* kb = smem + buf * 2 * C::TILE_BYTES;
-    const unsigned char* vb = kb + C::TILE_BYTES;
-
-    if (active) {
+    __builtin_amdgcn_s_waitcnt(0x0f70);                    // vmcnt(0): this wave's share of stage s has landed
+    __syncthreads();                                       // ... and everyone's; stage s-1 has been consumed
+    if (s + 1 < n_stages) request(buf ^ 1);
+    const int kb = buf * C::STAGE_BYTES, vb = kb + C::TILE_BYTES;   // LDS byte addresses (the dynamic array starts at 0)
+    if (!active) continue;
+    if (s < cblk) {
+      f32x16_t sc[C::NT], dp[C::KEEP_DP ? C::NT : 1];
 #pragma unroll
-      for (int jb = 0; jb < C::NB; ++jb) {
-        const int blk = s * C::NB + jb;
-        const int rb0 = jb * BS;
-        if (blk < cblk) {
-          f32x16_t sc[C::NT], dp[C::NT];
+      for (int u = 0; u < C::NT; ++u) sc[u] = row_tile(kb + 32 * u * C::ROWB, qf);
+      const float s_last = sc[C::NT - 1][15];
+      float mx = (h == 0) ? s_last : -INFINITY;
 #pragma unroll
-          for (int u = 0; u < C::NT; ++u) sc[u] = row_tile(kb, rb0 + 32 * u, qf);
+      for (int u = 0; u < C::NT; ++u)
 #pragma unroll
-          for (int u = 0; u < C::NT; ++u) dp[u] = row_tile(vb, rb0 + 32 * u, gf);
-          const float s_last = sc[C::NT - 1][15];
-          float mx = (h == 0) ? s_last : -INFINITY;
+        for (int r = 0; r < 16; ++r)
+          if (!(u == C::NT - 1 && r == 15)) mx = fmaxf(mx, sc[u][r]);
+      mx = pair_max(mx);
+      const float t_lm = pair_hi(s_last) * c2;
+      const float mloc = mx * c2;
+      float den = 0.f, spd = 0.f;
 #pragma unroll
-          for (int u = 0; u < C::NT; ++u)
+      for (int u = 0; u < C::NT; ++u) {
+        f32x16_t& d = dp[C::KEEP_DP ? u : 0];
+        d = row_tile(vb + 32 * u * C::ROWB, gf);
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-              if (!(u == C::NT - 1 && r == 15)) mx = fmaxf(mx, sc[u][r]);
-          mx = pair_max(mx);
-          const float t_lm = pair_hi(s_last) * c2;
-          const float mloc = mx * c2;
-          float den = 0.f, spd = 0.f;
+        for (int r = 0; r < 16; ++r) {
+          float e = fast_exp2(__builtin_fmaf(sc[u][r], c2, -mloc));
+          if (u == C::NT - 1 && r == 15) e = (h == 0) ? e : 0.f;
+          sc[u][r] = e;
+          den += e;
+          spd = __builtin_fmaf(e, d[r], spd);
+        }
+      }
+      den = pair_sum(den);
+      spd = pair_sum(spd);
+      const float invden = fast_rcp(den);
+      const float nD = spd * invden;
+      const float glog = t_lm - mhat;                      // log2 of the normalised gate
+      const float g = fast_exp2(glog);
+      const float f = g * invden;
+      if (h == 0) {
+        const int64_t si = ((int64_t)bh * p.n_blocks + s) * p.Lq + qrow;
+        p.stat_a[si] = mloc + fast_log2(den) - glog;
+        p.stat_n[si] = nD;
+        p.stat_l[si] = g * (nD - delta);                   // dS at the block's landmark key
+      }
 #pragma unroll
-          for (int u = 0; u < C::NT; ++u)
+      for (int u = 0; u < C::NT; ++u) {
+        if (!C::KEEP_DP) dp[0] = row_tile(vb + 32 * u * C::ROWB, gf);
+        const f32x16_t& d = dp[C::KEEP_DP ? u : 0];
+        float ds[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              float e = fast_exp2(__builtin_fmaf(sc[u][r], c2, -mloc));
-              if (u == C::NT - 1 && r == 15) e = (h == 0) ? e : 0.f;
-              sc[u][r] = e;
-              den += e;
-              spd = __builtin_fmaf(e, dp[u][r], spd);
-            }
-          den = pair_sum(den);
-          spd = pair_sum(spd);
-          const float invden = fast_rcp(den);
-          const float nD = spd * invden;
-          const float glog = t_lm - mhat;               // log2 of the normalised gate
-          const float g = fast_exp2(glog);
-          const float f = g * invden;
-          if (h == 0 && rowok) {
-            const int64_t si = ((int64_t)bh * p.n_blocks + blk) * p.Lq + qrow;
-            p.stat_a[si] = mloc + fast_log2(den) - glog;
-            p.stat_n[si] = nD;
-            p.stat_l[si] = g * (nD - delta);              // dS at the block's landmark key
+        for (int r = 0; r < 16; ++r) ds[r] = sc[u][r] * f * (d[r] - nD);
+        if (u == C::NT - 1 && h == 1) ds[15] = g * (nD - delta);
+        dq_tile(kb + 32 * u * C::ROWB, ds);
+      }
+    } else if (s == cblk) {
+      const int lim = ql - ((tsub == C::NT - 1 && ql == 31) ? 1 : 0);
+#pragma unroll
+      for (int u = 0; u < C::NT; ++u) {
+        if (u <= tsub) {
+          f32x16_t sc = row_tile(kb + 32 * u * C::ROWB, qf);
+          f32x16_t d = row_tile(vb + 32 * u * C::ROWB, gf);
+          float ds[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = 8 * (r >> 2) + 4 * h + (r & 3);
+            const float pr = (u < tsub || key <= lim) ? fast_exp2(__builtin_fmaf(sc[r], c2, -mhat)) : 0.f;
+            ds[r] = pr * (d[r] - delta);
           }
-#pragma unroll
-          for (int u = 0; u < C::NT; ++u) {
-            float ds[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) ds[r] = sc[u][r] * f * (dp[u][r] - nD);
-            if (u == C::NT - 1 && h == 1) ds[15] = g * (nD - delta);
-            dq_tile(kb, rb0 + 32 * u, ds);
-          }
-        } else if (blk == cblk) {
-          const int lim = ql - ((tsub == C::NT - 1 && ql == 31) ? 1 : 0);
-#pragma unroll
-          for (int u = 0; u < C::NT; ++u) {
-            if (u <= tsub) {
-              f32x16_t sc = row_tile(kb, rb0 + 32 * u, qf);
-              f32x16_t dp = row_tile(vb, rb0 + 32 * u, gf);
-              float ds[16];
-#pragma unroll
-              for (int r = 0; r < 16; ++r) {
-                const int key = 8 * (r >> 2) + 4 * h + (r & 3);
-                const float pr = (u < tsub || key <= lim) ? fast_exp2(__builtin_fmaf(sc[r], c2, -mhat)) : 0.f;
-                ds[r] = pr * (dp[r] - delta);
-              }
-              dq_tile(kb, rb0 + 32 * u, ds);
-            }
-          }
+          dq_tile(kb + 32 * u * C::ROWB, ds);
         }
       }
     }
-    if (s + 1 < n_stages) store_stage(buf ^ 1);
-    __syncthreads();
   }
 
-  if (active && rowok) {
+  if (active) {
     const float sc = p.scale;
 #pragma unroll
     for (int dc = 0; dc < C::DC; ++dc)
@@ -293,7 +327,7 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
       auto kern = lmk_bwd_dq_kernel<T, D, BS>;
       static std::atomic<uint64_t> lds_ok{0};
       if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
-      hipLaunchKernelGGL(kern, dim3(p.n_qtiles * p.B * p.H), dim3(256), C::LDS_BYTES, stream, p);
+      hipLaunchKernelGGL(kern, dim3(((p.Lq + 255) / 256) * p.B * p.H), dim3(64 * C::NW), C::LDS_BYTES, stream, p);
       if ((rc = (int)hipGetLastError())) return rc;
     }
   }
