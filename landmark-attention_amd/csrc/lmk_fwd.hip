@@ -1,13 +1,15 @@
 // Forward kernel of fused landmark attention for gfx950.
 //
 // Replaces `_fwd_kernel` of the reference (llama/ltriton/flash_landmark_attention.py:6-122).
-// One workgroup = 4 waves = 128 consecutive query rows; every wave owns 32 queries and
+// This file: landmark blocks of 64 and 128 keys (block 32 has its own kernel in lmk_fwd32.hip).
+// One workgroup = 8 waves = 256 consecutive query rows; every wave owns 32 queries and
 // keeps S^T = K Q^T tiles in the MFMA C layout (lane = query, registers = keys), so the
 // landmark grouped softmax never leaves a lane pair:
 //   earlier block b:  local softmax over its BS-1 normal keys, gate = online softmax over
 //                     the landmark scores, acc = acc*alpha + (gate * P_local) V
 //   own block:        plain causal online softmax joined to the same running (M, l)
-// K and V stream through LDS in stages of SK = max(BS, 64) keys, double buffered;
+// K and V stream through LDS one landmark block per stage, double buffered, by direct global->LDS
+// loads (no staging registers: two waves share a SIMD, so a wave has 256 registers);
 // V is kept row-major and transposed on the way out of LDS by ds_read_b64_tr_b16.
 #include <cstdlib>
 
@@ -19,36 +21,50 @@ namespace lmk {
 template <class T, int D, int BS>
 struct FwdCfg {
   static constexpr int NT = BS / 32;                    // 32-key tiles per landmark block
-  static constexpr int NB = (BS >= 64) ? 1 : 64 / BS;   // landmark blocks per LDS stage
-  static constexpr int SK = NB * BS;                    // keys per stage
+  static constexpr int NW = 8;
   static constexpr int ROWB = 2 * D;
   static constexpr int CH = D / 8;                      // 16-byte chunks per row
-  static constexpr int TILE_BYTES = SK * ROWB;          // one stage of K (or of V)
-  static constexpr int NCH = SK * CH / 256;             // chunks per thread per tensor per stage
+  static constexpr int NB = (BS >= 128) ? 1 : 128 / BS;  // landmark blocks per stage
+  static constexpr int SK = NB * BS;                    // keys per stage
+  static constexpr int TILE_BYTES = SK * ROWB;          // K (or V) of one stage
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES;    // K, then V
   static constexpr int KS = D / 16;                     // MFMA k-steps over the head dim
   static constexpr int DC = D / 32;                     // 32-wide output chunks of the head dim
-  static constexpr int LDS_BYTES = 4 * TILE_BYTES;      // 2 buffers x (K, V)
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;     // two stages
+  static constexpr int RPD = 1024 / ROWB;               // rows covered by one 1 KB request
+  static constexpr int NREQ = 2 * SK / RPD;             // requests per stage
+  static constexpr int PER_WAVE = NREQ / NW;
+  static_assert(NREQ % NW == 0, "every wave issues the same number of requests");
 };
 
+// One 1 KB direct global->LDS request of a wave: lane i's 16 bytes land at lds_off + 16*i.
+// lds_off must be wave-uniform (it travels in M0).
+__device__ __forceinline__ void fwd_dma16(const void* base_uniform, uint32_t voff, uint32_t lds_off) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(voff), "s"(base_uniform), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory");
+}
+
 template <class T, int D, int BS>
-__global__ __launch_bounds__(256, (BS >= 128 ? 1 : 2)) void lmk_fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   using C = FwdCfg<T, D, BS>;
   extern __shared__ __align__(16) unsigned char smem[];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ql = lane & 31, h = lane >> 5;
 
-  // ---- workgroup -> (batch*head, 128-row query tile); heavy tiles first, one head per XCD slot
-  int bh, qtile;
+  // ---- workgroup -> (batch*head, 256-row query tile); heavy tiles first, one head per XCD slot
+  const int nq256 = (p.Lq + 255) >> 8;
+  int bh, qt;
   {
     const int bid = blockIdx.x;
     const int BH = p.B * p.H;
     if ((BH & 7) == 0) {
       const int xcd = bid & 7, j = bid >> 3, ngrp = BH >> 3;
-      qtile = p.n_qtiles - 1 - j / ngrp;
+      qt = nq256 - 1 - j / ngrp;
       bh = (j % ngrp) * 8 + xcd;
     } else {
-      qtile = p.n_qtiles - 1 - bid / BH;
+      qt = nq256 - 1 - bid / BH;
       bh = bid % BH;
     }
   }
@@ -58,7 +74,7 @@ __global__ __launch_bounds__(256, (BS >= 128 ? 1 : 2)) void lmk_fwd_kernel(FwdPa
   const char* vp = (const char*)p.v + 2 * (b * p.vs_b + hh * p.vs_h);
   char* op = (char*)p.o + 2 * (b * p.os_b + hh * p.os_h);
 
-  const int q0 = qtile * 128 + wave * 32;               // first query row of this wave
+  const int q0 = qt * 256 + wave * 32;                  // first query row of this wave
   const int dt = p.n_prefix * C::NT + (q0 >> 5);        // its diagonal 32-key tile (absolute)
   const int cblk = dt / C::NT, tsub = dt % C::NT;       // its landmark block and sub-tile
   const bool active = q0 < p.Lq;
@@ -73,33 +89,41 @@ __global__ __launch_bounds__(256, (BS >= 128 ? 1 : 2)) void lmk_fwd_kernel(FwdPa
     if (qrow < p.Lq) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
   }
 
-  // ---- stage loader: thread handles chunks id = tid + 256*i -> (row = id / CH, chunk = id % CH)
-  const int tiles_needed = min((p.Lk + 31) >> 5, p.n_prefix * C::NT + qtile * 4 + 4);
-  const int n_stages = (tiles_needed * 32 + C::SK - 1) / C::SK;
-  u32x4_t kreg[C::NCH], vreg[C::NCH];
-  auto load_stage = [&](int s) {
+  // ---- stages of SK keys (one or two landmark blocks), up to the own block of the workgroup's last
+  // query tile.  K and V rows come by direct global->LDS loads, requested one stage ahead, each wave its
+  // share: request r covers rows RPD*(r % (SK/RPD)) .. of K (r < SK/RPD) or of V.  The LDS swizzle is applied
+  // on the source side: lane i lands at +16*i, i.e. row i/CH, chunk position i%CH, so it fetches the
+  // chunk tile_off() stores there.  Rows past Lk (a partial last stage) are clamped to the last row;
+  // they are keys no query can see.
+  const int last_q0 = min(qt * 256 + 224, ((p.Lq - 1) >> 5) << 5);
+  const int n_kstages = (p.Lk + C::SK - 1) / C::SK;
+  const int n_stages = min(n_kstages, ((p.n_prefix * C::NT + (last_q0 >> 5)) / C::NT) / C::NB + 1);
+  constexpr int n_k = C::SK / C::RPD;                   // requests that fetch K rows; the rest fetch V rows
+  uint32_t src[C::PER_WAVE], src_last[C::PER_WAVE];     // per-lane byte offsets inside the (batch, head) slice
 #pragma unroll
-    for (int i = 0; i < C::NCH; ++i) {
-      const int id = tid + 256 * i, row = id / C::CH, ch = id % C::CH;
-      const int key = s * C::SK + row;
-      u32x4_t z = {0, 0, 0, 0};
-      kreg[i] = z;
-      vreg[i] = z;
-      if (key < p.Lk) {
-        kreg[i] = *(const u32x4_t*)(kp + 2 * ((int64_t)key * p.ks_r + 8 * ch));
-        vreg[i] = *(const u32x4_t*)(vp + 2 * ((int64_t)key * p.vs_r + 8 * ch));
-      }
-    }
-  };
-  auto store_stage = [&](int buf) {
-    unsigned char* kb = smem + buf * 2 * C::TILE_BYTES;
-    unsigned char* vb = kb + C::TILE_BYTES;
+  for (int i = 0; i < C::PER_WAVE; ++i) {
+    const int r = wave * C::PER_WAVE + i;
+    const bool is_v = r >= n_k;
+    const int row = C::RPD * (r % n_k) + lane / C::CH, cp = lane % C::CH;
+    const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
+    const int64_t rs = is_v ? p.vs_r : p.ks_r;
+    src[i] = (uint32_t)(2 * ((int64_t)row * rs + 8 * (cp ^ f)));
+    const int row_last = min((n_kstages - 1) * C::SK + row, p.Lk - 1);
+    src_last[i] = (uint32_t)(2 * ((int64_t)row_last * rs + 8 * (cp ^ f)));
+  }
+  const uint32_t step_k = (uint32_t)(2 * (int64_t)C::SK * p.ks_r), step_v = (uint32_t)(2 * (int64_t)C::SK * p.vs_r);
+  int blk_req = 0;                                      // stage the next request fetches
+  auto request = [&](int buf) {
+    const bool last = blk_req == n_kstages - 1;         // wave-uniform
 #pragma unroll
-    for (int i = 0; i < C::NCH; ++i) {
-      const int id = tid + 256 * i, row = id / C::CH, ch = id % C::CH;
-      *(u32x4_t*)(kb + tile_off<D>(row, ch)) = kreg[i];
-      *(u32x4_t*)(vb + tile_off<D>(row, ch)) = vreg[i];
+    for (int i = 0; i < C::PER_WAVE; ++i) {
+      const int r = wave * C::PER_WAVE + i;
+      const bool is_v = r >= n_k;                       // wave-uniform
+      const int dst = buf * C::STAGE_BYTES + (is_v ? C::TILE_BYTES : 0) + C::RPD * (r % n_k) * C::ROWB;
+      fwd_dma16(is_v ? vp : kp, last ? src_last[i] : src[i], dst);
+      src[i] += is_v ? step_v : step_k;
     }
+    ++blk_req;
   };
 
   // ---- running state (log2 domain): M = max of the global bucket, l = its sum
@@ -112,21 +136,42 @@ __global__ __launch_bounds__(256, (BS >= 128 ? 1 : 2)) void lmk_fwd_kernel(FwdPa
 
   const float c2 = p.scale_log2;
 
-  auto qk_tile = [&](const unsigned char* kb, int rb) {
+  // LDS byte offsets of this lane's operand fragments inside a 32-row tile: the swizzle repeats every 16
+  // rows, so a tile at row 32u is the same offsets plus 32u rows -- an immediate of the LDS instruction
+  int koff[C::KS];
+#pragma unroll
+  for (int ks = 0; ks < C::KS; ++ks) koff[ks] = tile_off<D>(ql, 2 * ks + h);
+  int voff[C::DC][2];
+  {
+    const int i = lane & 15, g2 = (lane >> 4) & 1;
+#pragma unroll
+    for (int dc = 0; dc < C::DC; ++dc) {
+      const int col = 32 * dc + 16 * g2 + 4 * (i & 3);
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+        voff[dc][hf] = tile_off<D>(4 * h + (i >> 2) + 8 * hf, col >> 3) + ((col >> 2) & 1) * 8;
+    }
+  }
+  auto qk_tile = [&](int tile_bytes) {                  // S^T of the 32 keys at LDS byte address tile_bytes
     f32x16_t s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(load_row_frag<D>(kb, rb, ks, lane), qf[ks], s);
+    for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(lds_ld128(tile_bytes + koff[ks]), qf[ks], s);
     return s;
   };
-  auto pv_tile = [&](const unsigned char* vb, int rb, const float* w) {
+  auto pv_tile = [&](int tile_bytes, const float* w) {  // O^T += (V tile)^T W
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       u32x4_t wf = {pack2<T>(w[8 * j + 0], w[8 * j + 1]), pack2<T>(w[8 * j + 2], w[8 * j + 3]),
                     pack2<T>(w[8 * j + 4], w[8 * j + 5]), pack2<T>(w[8 * j + 6], w[8 * j + 7])};
 #pragma unroll
-      for (int dc = 0; dc < C::DC; ++dc) acc[dc] = mfma32<T>(load_tr_frag<D>(vb, rb, j, dc, lane), wf, acc[dc]);
+      for (int dc = 0; dc < C::DC; ++dc) {
+        const int base = tile_bytes + 16 * j * C::ROWB;
+        const u32x2_t a0 = lds_ld_tr(base + voff[dc][0]), a1 = lds_ld_tr(base + voff[dc][1]);
+        const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
+        acc[dc] = mfma32<T>(a, wf, acc[dc]);
+      }
     }
   };
   auto rescale = [&](float alpha) {
@@ -138,98 +183,92 @@ __global__ __launch_bounds__(256, (BS >= 128 ? 1 : 2)) void lmk_fwd_kernel(FwdPa
     }
   };
 
-  load_stage(0);
-  store_stage(0);
-  __syncthreads();
-
+  request(0);
   for (int s = 0; s < n_stages; ++s) {
     const int buf = s & 1;
-    if (s + 1 < n_stages) load_stage(s + 1);
-    const unsigned char* kb = smem + buf * 2 * C::TILE_BYTES;
-    const unsigned char* vb = kb + C::TILE_BYTES;
-
-    if (active) {
+    __builtin_amdgcn_s_waitcnt(0x0f70);                 // vmcnt(0): this wave's share of stage s has landed
+    __syncthreads();                                    // ... and everyone's; stage s-1 has been consumed
+    if (s + 1 < n_stages) request(buf ^ 1);
+    if (!active) continue;
 #pragma unroll
-      for (int jb = 0; jb < C::NB; ++jb) {
-        const int blk = s * C::NB + jb;                 // absolute landmark block
-        const int rb0 = jb * BS;                        // its first LDS row
-        if (blk < cblk) {
-          // ---------------- earlier block: local softmax gated by its landmark
-          f32x16_t sc[C::NT];
+    for (int jb = 0; jb < C::NB; ++jb) {
+      const int blk = s * C::NB + jb;                     // absolute landmark block
+      // LDS byte addresses of the block's K and V rows (the dynamic array starts at 0)
+      const int kb = buf * C::STAGE_BYTES + jb * BS * C::ROWB, vb = kb + C::TILE_BYTES;
+      if (blk < cblk) {
+        // ---------------- earlier block: local softmax gated by its landmark
+        f32x16_t sc[C::NT];
 #pragma unroll
-          for (int u = 0; u < C::NT; ++u) sc[u] = qk_tile(kb, rb0 + 32 * u);
-          // key of register r in tile u: 32u + 8*(r/4) + 4h + r%4; the landmark is (NT-1, r=15, h=1)
-          const float s_last = sc[C::NT - 1][15];
-          float mx = (h == 0) ? s_last : -INFINITY;
+        for (int u = 0; u < C::NT; ++u) sc[u] = qk_tile(kb + 32 * u * C::ROWB);
+        // key of register r in tile u: 32u + 8*(r/4) + 4h + r%4; the landmark is (NT-1, r=15, h=1)
+        const float s_last = sc[C::NT - 1][15];
+        float mx = (h == 0) ? s_last : -INFINITY;
 #pragma unroll
-          for (int u = 0; u < C::NT; ++u)
+        for (int u = 0; u < C::NT; ++u)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-              if (!(u == C::NT - 1 && r == 15)) mx = fmaxf(mx, sc[u][r]);
-          mx = pair_max(mx);
-          const float t_lm = pair_hi(s_last) * c2;      // landmark score, log2 domain
-          const float mloc = mx * c2;
-          float den = 0.f;
+          for (int r = 0; r < 16; ++r)
+            if (!(u == C::NT - 1 && r == 15)) mx = fmaxf(mx, sc[u][r]);
+        mx = pair_max(mx);
+        const float t_lm = pair_hi(s_last) * c2;          // landmark score, log2 domain
+        const float mloc = mx * c2;
+        float den = 0.f;
 #pragma unroll
-          for (int u = 0; u < C::NT; ++u)
+        for (int u = 0; u < C::NT; ++u)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float e = fast_exp2(__builtin_fmaf(sc[u][r], c2, -mloc));
+            if (u == C::NT - 1 && r == 15) e = (h == 0) ? e : 0.f;
+            sc[u][r] = e;
+            den += e;
+          }
+        den = pair_sum(den);
+        const float Mnew = fmaxf(Mrun, t_lm);
+        const float alpha = fast_exp2(Mrun - Mnew);
+        const float gate = fast_exp2(t_lm - Mnew);
+        lrun = lrun * alpha + gate;
+        Mrun = Mnew;
+        rescale(alpha);
+        const float f = gate * fast_rcp(den);
+#pragma unroll
+        for (int u = 0; u < C::NT; ++u) {
+          float w[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) w[r] = sc[u][r] * f;
+          pv_tile(vb + 32 * u * C::ROWB, w);
+        }
+      } else if (blk == cblk) {
+        // ---------------- own block: causal tiles 0..tsub join the global bucket
+        const int lim = ql - ((tsub == C::NT - 1 && ql == 31) ? 1 : 0);  // landmark query looks one left
+#pragma unroll
+        for (int u = 0; u < C::NT; ++u) {
+          if (u <= tsub) {
+            f32x16_t sc = qk_tile(kb + 32 * u * C::ROWB);
+            float x[16];
+            float mt = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              float e = fast_exp2(__builtin_fmaf(sc[u][r], c2, -mloc));
-              if (u == C::NT - 1 && r == 15) e = (h == 0) ? e : 0.f;
-              sc[u][r] = e;
-              den += e;
+              const int key = 8 * (r >> 2) + 4 * h + (r & 3);
+              x[r] = (u < tsub || key <= lim) ? sc[r] * c2 : -INFINITY;
+              mt = fmaxf(mt, x[r]);
             }
-          den = pair_sum(den);
-          const float Mnew = fmaxf(Mrun, t_lm);
-          const float alpha = fast_exp2(Mrun - Mnew);
-          const float gate = fast_exp2(t_lm - Mnew);
-          lrun = lrun * alpha + gate;
-          Mrun = Mnew;
-          rescale(alpha);
-          const float f = gate * fast_rcp(den);
+            mt = pair_max(mt);
+            const float Mnew = fmaxf(Mrun, mt);
+            const float alpha = fast_exp2(Mrun - Mnew);
+            float sum = 0.f;
 #pragma unroll
-          for (int u = 0; u < C::NT; ++u) {
-            float w[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) w[r] = sc[u][r] * f;
-            pv_tile(vb, rb0 + 32 * u, w);
-          }
-        } else if (blk == cblk) {
-          // ---------------- own block: causal tiles 0..tsub join the global bucket
-          const int lim = ql - ((tsub == C::NT - 1 && ql == 31) ? 1 : 0);  // landmark query looks one left
-#pragma unroll
-          for (int u = 0; u < C::NT; ++u) {
-            if (u <= tsub) {
-              f32x16_t sc = qk_tile(kb, rb0 + 32 * u);
-              float x[16];
-              float mt = -INFINITY;
-#pragma unroll
-              for (int r = 0; r < 16; ++r) {
-                const int key = 8 * (r >> 2) + 4 * h + (r & 3);
-                x[r] = (u < tsub || key <= lim) ? sc[r] * c2 : -INFINITY;
-                mt = fmaxf(mt, x[r]);
-              }
-              mt = pair_max(mt);
-              const float Mnew = fmaxf(Mrun, mt);
-              const float alpha = fast_exp2(Mrun - Mnew);
-              float sum = 0.f;
-#pragma unroll
-              for (int r = 0; r < 16; ++r) {
-                x[r] = fast_exp2(x[r] - Mnew);
-                sum += x[r];
-              }
-              sum = pair_sum(sum);
-              lrun = lrun * alpha + sum;
-              Mrun = Mnew;
-              rescale(alpha);
-              pv_tile(vb, rb0 + 32 * u, x);
+            for (int r = 0; r < 16; ++r) {
+              x[r] = fast_exp2(x[r] - Mnew);
+              sum += x[r];
             }
+            sum = pair_sum(sum);
+            lrun = lrun * alpha + sum;
+            Mrun = Mnew;
+            rescale(alpha);
+            pv_tile(vb + 32 * u * C::ROWB, x);
           }
         }
       }
     }
-    if (s + 1 < n_stages) store_stage(buf ^ 1);
-    __syncthreads();
   }
 
   // ---- epilogue: out = acc / l, statistics in natural-log units like the reference
@@ -256,8 +295,8 @@ static int launch_fwd_t(const FwdParams& p, hipStream_t stream) {
   auto kern = lmk_fwd_kernel<T, D, BS>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
-  const int grid = p.n_qtiles * p.B * p.H;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), C::LDS_BYTES, stream, p);
+  const int grid = ((p.Lq + 255) / 256) * p.B * p.H;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * C::NW), C::LDS_BYTES, stream, p);
   return (int)hipGetLastError();
 }
 
