@@ -86,8 +86,8 @@ int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
  * LMK_BWD_DQ: dQ and the per-block terms, LMK_BWD_DKDV: dK and dV), in that order.  Each phase
  * consumes what the earlier ones left in `workspace`, so a subset is only meaningful after a
  * full run on the same arguments; it exists to time and profile the kernels one by one.
- * With block 32 the dQ kernel computes the row terms itself: LMK_BWD_PRE launches the separate
- * row-term kernel only when LMK_BWD_DQ is not selected.
+ * The dQ kernel computes the row terms itself: LMK_BWD_PRE launches the separate row-term kernel
+ * only when LMK_BWD_DQ is not selected.
  * No counterpart in the reference (its backward is a single launch, :373-388). */
 #define LMK_BWD_PRE 1
 #define LMK_BWD_DQ 2

@@ -5,7 +5,8 @@
 // program per (batch, head) and read-modify-writes dQ in global memory; here the work is
 // split so that every accumulator stays in registers and no atomics are needed:
 //
-//   pre    delta = rowsum(O * dO),  mhat = M*log2(e) + log2(L)          (per query row)
+//   pre    delta = rowsum(O * dO),  mhat = M*log2(e) + log2(L)          (per query row; the dQ kernels do
+//          this in their prologue, the separate kernel exists for timing the phases one by one)
 //   dq     query-stationary, S^T layout (lane = query): recomputes the local softmax of
 //          every earlier block, the gate, nD = rowsum(P * dP), forms dS and accumulates
 //          dQ^T = K^T dS^T.  It also writes, per (query, earlier block), the three numbers
@@ -136,8 +137,28 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
       gf[ks] = *(const u32x4_t*)(gp + 2 * ((int64_t)qrow * p.dos_r + 16 * ks + 8 * h));
     }
   }
-  const float mhat = active ? p.mhat[(int64_t)bh * p.Lq + qrow] : 0.f;
-  const float delta = active ? p.delta[(int64_t)bh * p.Lq + qrow] : 0.f;
+  // row terms (the reference's _bwd_preprocess, flash_landmark_attention.py:125-149): delta = rowsum(O * dO)
+  // from the dO fragments already in registers, mhat = M*log2(e) + log2(L); left in the workspace for the
+  // dK/dV kernel as well
+  float mhat = 0.f, delta = 0.f;
+  if (active) {
+    const char* orow = (const char*)p.o + 2 * (b * p.os_b + hh * p.os_h + (int64_t)qrow * p.os_r);
+    float sum = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < C::KS; ++ks) {
+      const u32x4_t o4 = *(const u32x4_t*)(orow + 2 * (16 * ks + 8 * h));
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        sum += unpack_lo<T>(o4[i]) * unpack_lo<T>(gf[ks][i]) + unpack_hi<T>(o4[i]) * unpack_hi<T>(gf[ks][i]);
+    }
+    delta = pair_sum(sum);
+    const int64_t ri = (int64_t)bh * p.Lq + qrow;
+    mhat = p.M[ri] * kLog2e + fast_log2(p.L[ri]);
+    if (h == 0) {
+      p.delta[ri] = delta;
+      p.mhat[ri] = mhat;
+    }
+  }
 
   // stages = blocks up to the own block of the workgroup's last query tile
   const int last_q0 = min(qt * 256 + 224, p.Lq - 32);
@@ -312,8 +333,8 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
 template <class T, int D, int BS>
 static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
   int rc;
-  // block 32: the dQ kernel computes delta and mhat itself, so the separate pass only runs when asked for alone
-  if ((phases & 1) && !(BS == 32 && (phases & 2))) {
+  // the dQ kernels compute delta and mhat themselves, so the separate pass only runs when asked for alone
+  if ((phases & 1) && !(phases & 2)) {
     constexpr int RPW = 256 / (D / 8);
     const int64_t rows = (int64_t)p.B * p.H * p.Lq;
     hipLaunchKernelGGL((lmk_bwd_pre_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
