@@ -88,9 +88,9 @@ def tensor4(t: torch.Tensor) -> Tensor4:
 
 
 def kernel_ready(t: torch.Tensor) -> torch.Tensor:
-    """Return ``t`` itself when the kernels can read it in place (unit stride along D,
-    16-byte aligned base and strides), otherwise a contiguous copy."""
-    if (t.stride(3) == 1 and t.data_ptr() % 16 == 0 and all(t.stride(i) % 8 == 0 for i in range(3))):
+    """Return ``t`` itself when the kernels can read it in place (unit stride along D, rows walked
+    forwards, 16-byte aligned base and strides), otherwise a contiguous copy."""
+    if (t.stride(3) == 1 and t.stride(2) > 0 and t.data_ptr() % 16 == 0 and all(t.stride(i) % 8 == 0 for i in range(3))):
         return t
     return t.contiguous()
 

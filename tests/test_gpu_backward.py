@@ -94,6 +94,27 @@ def test_reference_script_loss_and_blhd_layout(block):
         assert a.transpose(1, 2).is_contiguous()             # gradients come back in their input's layout
 
 
+def test_broadcast_upstream_gradient_and_activation_checkpointing():
+    # out.sum().backward() hands the backward an expanded scalar (all strides 0); the reference's layers call the
+    # op under torch.utils.checkpoint (llama_mem.py:847-859), which re-runs the forward inside the backward
+    from torch.utils.checkpoint import checkpoint
+    from ltriton.flash_landmark_attention import fused_landmark_attention
+    from oracle import s1
+    B, H, L, D, block = 1, 2, 128, 128, 32
+    q, k, v = make_qkv(B, H, L, L, D, seed=21)
+    dev = torch.device("cuda:0")
+    is_mem = torch.arange(L, device=dev) % block == block - 1
+    qc, kc, vc = (t.float().clone().requires_grad_(True) for t in (q, k, v))
+    r = torch.autograd.grad(s1.s1_attention(qc, kc, vc, block).sum(), [qc, kc, vc])
+    for use_checkpoint in (False, True):
+        qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+        fn = lambda a, b_, c: fused_landmark_attention(a, b_, c, is_mem, block_size=block)
+        out = checkpoint(fn, qd, kd, vd, use_reentrant=False) if use_checkpoint else fn(qd, kd, vd)
+        out.sum().backward()
+        for a, b_ in zip((qd.grad, kd.grad, vd.grad), r):
+            assert (a.float().cpu() - b_).abs().max().item() <= TOL, use_checkpoint
+
+
 def test_partial_block_backward_is_rejected():
     from ltriton.flash_landmark_attention import fused_landmark_attention
     q, k, v = make_qkv(1, 2, 100, 100, 128, seed=12)
