@@ -165,3 +165,25 @@ def test_baseline_config3_full_size():
     ones = torch.ones_like(v)
     out1 = _run(q, k, ones, block, is_mem=None).float()
     assert (out1 - 1).abs().max().item() <= 1e-2
+
+
+def test_runs_on_the_callers_stream():
+    # the library launches on the stream it is given: work queued on a side stream behind a long-running
+    # producer must see the producer's result, with no synchronisation by the library
+    from ltriton.flash_landmark_attention import fused_landmark_attention
+    B, H, L, D, block = 1, 2, 256, 128, 32
+    q, k, v = make_qkv(B, H, L, L, D, seed=31)
+    dev = torch.device("cuda:0")
+    ref = _run(q, k, v, block)
+    side = torch.cuda.Stream(device=dev)
+    qd, kd = q.to(dev), k.to(dev)
+    vd = torch.zeros_like(qd)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        big = torch.randn(4096, 4096, device=dev)
+        for _ in range(20):
+            big = big @ big * 1e-4                              # keeps the side stream busy
+        vd.copy_(v.to(dev, non_blocking=True))                  # v arrives late, on the side stream
+        out = fused_landmark_attention(qd, kd, vd, None, block_size=block)
+    side.synchronize()
+    assert torch.equal(out, ref)
