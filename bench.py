@@ -112,8 +112,22 @@ def decode_bench(n=50, warm=5):
     idx = retrieve_topk(q, kc, cos, sin, block, top_k)
     t_topk = _time_launches(lambda: retrieve_topk(q, kc, cos, sin, block, top_k), n, warm)
     t_att = _time_launches(lambda: gather_attend(q, kc, vc, idx, kl, vl, cos, sin, block, top_k), n, warm)
+    # the same step (selection + attend, six launches) recorded once into a HIP graph and replayed
+    def step():
+        i = retrieve_topk(q, kc, cos, sin, block, top_k)
+        return gather_attend(q, kc, vc, i, kl, vl, cos, sin, block, top_k)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    t_graph = _time_launches(graph.replay, n, warm)
     return {"workload": "decode: 1 new token, H32 D128, cache 32775 tok (1024 blocks of 32 + tail of 7), top-4",
-            "topk_ms": t_topk, "gather_attend_ms": t_att}
+            "topk_ms": t_topk, "gather_attend_ms": t_att, "step_from_hip_graph_ms": t_graph}
 
 
 def side_legs(n=30, warm=5):
