@@ -187,3 +187,17 @@ def test_runs_on_the_callers_stream():
         out = fused_landmark_attention(qd, kd, vd, None, block_size=block)
     side.synchronize()
     assert torch.equal(out, ref)
+
+
+@pytest.mark.parametrize("block", [32, 64, 128])
+@pytest.mark.parametrize("D", [64, 128])
+def test_ragged_and_tiny_shapes(block, D):
+    # query counts around every tile and block boundary, with and without history blocks; forward only
+    # (the reference masks partial tiles in the forward, flash_landmark_attention.py:44,118-122)
+    for n_prefix, Lq in [(0, 1), (0, 31), (0, 33), (1, 5), (0, 65), (3, 40), (0, 127), (1, 129), (0, 257), (3, 300)]:
+        Lk = Lq + n_prefix * block
+        q, k, v = make_qkv(1, 2, Lq, Lk, D, seed=Lq * 7 + n_prefix)
+        print(f"case bs{block} D{D} prefix{n_prefix} Lq{Lq}", flush=True)
+        out = _run(q, k, v, block, is_mem=None).float().cpu()
+        ref, _, _ = oracle_forward(q, k, v, block)
+        assert (out - ref).abs().max().item() <= TOL, (n_prefix, Lq)
