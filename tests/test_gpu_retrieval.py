@@ -239,11 +239,13 @@ def test_gather_window_rows_bit_exact(dtype):
     assert torch.equal(qw.cpu()[:, :, inc:], q) and (qw.cpu()[:, :, :inc] == 0).all()
 
 
-def test_baseline_config4_full_size():
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_baseline_config4_full_size(seed):
     # benchmark config 4: H32 D128, 32768 cached tokens = 1024 blocks of 32, 256 queries, top-4
+    # (seed 0 is the benchmark's, 1 and 2 for robustness)
     from landmark_hip.retrieval import retrieve_and_attend
     B, H, T, S, D, block, top_k = 1, 32, 256, 32768, 128, 32, 4
-    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=0)
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=seed)
     sc = oret.landmark_scores(q, kc, cos, sin, block, top_k)
     want = oret.select_topk(sc, top_k)
     ties = oret.boundary_tie_rows(sc, top_k)
