@@ -159,6 +159,50 @@ def side_legs(n=30, warm=5):
                        "GBps": rot_bytes / 1e6 / t_rot, "frac_hbm": rot_bytes / 1e6 / t_rot / PEAK_HBM_GBS}}
 
 
+def other_shape(spec, n=30, warm=5):
+    """Per-kernel and whole-step times of fwd+bwd at another shape: spec = "B,H,L,D,block[,f16]".
+    Prints one JSON line of its own; the headline line is not produced."""
+    import torch
+    from landmark_hip import _lib
+    from landmark_hip.attention import _launch_bwd, _launch_fwd
+    parts = spec.split(",")
+    B, H, L, D, block = (int(x) for x in parts[:5])
+    dtype = torch.float16 if parts[5:] == ["f16"] else torch.bfloat16
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    q, k, v, do = ((torch.randn(B, H, L, D, generator=g) * 0.5).to(dtype).to(dev) for _ in range(4))
+    scale = 1.0 / math.sqrt(D)
+    o, Ls, M = _launch_fwd(q, k, v, 0, scale, block)
+    lib, T4 = _lib.lib(), _lib.tensor4
+    dq, dk, dv = (torch.empty_like(q) for _ in range(3))
+    nbytes = lib.lmk_attn_bwd_workspace_bytes(B, H, L, L, block)
+    ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+    stream = _lib.current_stream(dev)
+
+    def phase(mask):
+        _lib.check(lib.lmk_attn_bwd_phases(T4(q), T4(k), T4(v), T4(o), T4(do), Ls.data_ptr(), M.data_ptr(), T4(dq),
+                                           T4(dk), T4(dv), ws.data_ptr(), nbytes, B, H, L, L, D, scale, block, 0,
+                                           _lib.DTYPE_CODES[dtype], mask, stream))
+
+    def step():
+        _launch_fwd(q, k, v, 0, scale, block)
+        phase(7)
+
+    t_spin = time.perf_counter()
+    while time.perf_counter() - t_spin < 0.3:              # leave the idle power state
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+    t = {"fwd_ms": _time_launches(lambda: _launch_fwd(q, k, v, 0, scale, block), n, warm),
+         "dq_ms": _time_launches(lambda: phase(2), n, warm), "dkdv_ms": _time_launches(lambda: phase(4), n, warm),
+         "step_ms": _time_launches(step, n, warm)}
+    flops = 3.5 * 4 * B * H * L * L * D / 2
+    t.update({"shape": {"B": B, "H": H, "L": L, "D": D, "block": block, "dtype": str(dtype).split(".")[-1]},
+              "TFLOPs": flops / (t["step_ms"] * 1e-3) / 1e12,
+              "frac_of_mfma_peak": flops / (t["step_ms"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS})
+    print(json.dumps(t))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -169,6 +213,9 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="run a few steps plus a 256 MiB device copy and exit (for rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE runs: the copy's counters calibrate the kernels')")
+    ap.add_argument("--shape", action="append", default=[], metavar="B,H,L,D,block[,f16]",
+                    help="time fwd+bwd and its three kernels at another shape instead of the headline run "
+                         "(may be given several times)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; every (batch, head) slice is independent, so more GPUs "
@@ -178,6 +225,10 @@ def main():
     from landmark_hip.attention import FusedLandmarkAttention, _launch_bwd, _launch_fwd
     _lib.lib()
     assert torch.cuda.is_available(), "bench.py needs the GPU; there is no CPU path"
+    if a.shape:
+        for spec in a.shape:
+            other_shape(spec)
+        return
     dev = torch.device("cuda:0")
     B, H, L, D, block = 2, 32, 2048, 128, 32
     scale = 1.0 / math.sqrt(D)
