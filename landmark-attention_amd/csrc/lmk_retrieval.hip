@@ -725,181 +725,16 @@ __device__ __forceinline__ float sum8(float d) {                  // sum over th
 // evaluated in fp32 from the 16-bit cache and table values (the reference rounds the rotated key to
 // the model dtype first; the difference is far inside the 2e-2 bound of this step, and selection --
 // where bits matter -- does not go through here).
+// A block passes through the registers in chunks of at most 64 keys -- first the keys of every chunk
+// (scores of the whole block, which the block's softmax needs before any weight is final), then the
+// values, so keys and values are never live together and the kernel keeps several waves per SIMD.  The
+// loads of the next chunk are issued before the arithmetic on the current one.
 template <class T, int D, int BS>
 __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
-  static_assert(D == 128, "lane mapping below assumes 16 chunks of 8 head dims per row");
-  constexpr int KPG = BS / 8;                                     // keys per 8-lane group per block
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int j = lane & 7, g = lane >> 3;                           // head-dim chunk pair, key group
-  const int64_t row = (int64_t)blockIdx.x * 4 + wave;             // (bh, t)
-  const int64_t total = (int64_t)p.B * p.H * p.T;
-  if (row >= total) return;
-  const int bh = (int)(row / p.T), t = (int)(row % p.T);
-  const int b = bh / p.H, hh = bh % p.H;
-
-  auto unpack8 = [](const u32x4_t u, float* o) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      o[2 * i] = unpack_lo<T>(u[i]);
-      o[2 * i + 1] = unpack_hi<T>(u[i]);
-    }
-  };
-  float qlo[8], qhi[8];
-  {
-    const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
-    unpack8(*(const u32x4_t*)(qp + 16 * j), qlo);
-    unpack8(*(const u32x4_t*)(qp + 128 + 16 * j), qhi);
-  }
-  const char* kc = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h);
-  const char* vc = (const char*)p.vcache + 2 * (b * p.vcs_b + hh * p.vcs_h);
-  const float c2 = p.scale_log2;
-
-  float Mrun = -INFINITY, lrun = 0.f;
-  float alo[8], ahi[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    alo[i] = 0.f;
-    ahi[i] = 0.f;
-  }
-
-  // K/V of block js+1 are requested before block js is worked on: a wave keeps two blocks in flight
-  u32x4_t klo[KPG], khi[KPG], vlo[KPG], vhi[KPG], nklo[KPG], nkhi[KPG], nvlo[KPG], nvhi[KPG];
-  auto fetch = [&](int blk, u32x4_t* a, u32x4_t* bq, u32x4_t* c, u32x4_t* dq) {
-    const int64_t key0 = (int64_t)blk * BS;
-#pragma unroll
-    for (int i = 0; i < KPG; ++i) {
-      const int kk = g + 8 * i;                                   // this group's keys
-      const char* kr = kc + 2 * ((key0 + kk) * p.kcs_r) + 16 * j;
-      const char* vr = vc + 2 * ((key0 + kk) * p.vcs_r) + 16 * j;
-      a[i] = *(const u32x4_t*)(kr);
-      bq[i] = *(const u32x4_t*)(kr + 128);
-      c[i] = *(const u32x4_t*)(vr);
-      dq[i] = *(const u32x4_t*)(vr + 128);
-    }
-  };
-  int blk_next = (int)p.idx[row * p.k];
-  fetch(blk_next, nklo, nkhi, nvlo, nvhi);
-  for (int js = 0; js < p.k; ++js) {
-    const int blk = blk_next;
-    const int64_t pos0 = (int64_t)js * BS + ((blk >= p.num_mems - p.k) ? BS : 0) + p.prefix_len;
-#pragma unroll
-    for (int i = 0; i < KPG; ++i) {
-      klo[i] = nklo[i];
-      khi[i] = nkhi[i];
-      vlo[i] = nvlo[i];
-      vhi[i] = nvhi[i];
-    }
-    if (js + 1 < p.k) {
-      blk_next = (int)p.idx[row * p.k + js + 1];
-      fetch(blk_next, nklo, nkhi, nvlo, nvhi);
-    }
-    float sc[KPG];
-#pragma unroll
-    for (int i = 0; i < KPG; ++i) {
-      const int kk = g + 8 * i;
-      const char* cr = (const char*)p.cos + 2 * ((pos0 + kk) * p.cs_r) + 16 * j;
-      const char* sr = (const char*)p.sin + 2 * ((pos0 + kk) * p.cs_r) + 16 * j;
-      float kl[8], kh[8], cl[8], ch[8], sl[8], sh[8];
-      unpack8(klo[i], kl);
-      unpack8(khi[i], kh);
-      unpack8(*(const u32x4_t*)(cr), cl);
-      unpack8(*(const u32x4_t*)(cr + 128), ch);
-      unpack8(*(const u32x4_t*)(sr), sl);
-      unpack8(*(const u32x4_t*)(sr + 128), sh);
-      float d = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        // rotate_half: the first half pairs with -x[d + D/2], the second with x[d - D/2]
-        const float rl = __builtin_fmaf(kl[e], cl[e], -kh[e] * sl[e]);
-        const float rh = __builtin_fmaf(kh[e], ch[e], kl[e] * sh[e]);
-        d = __builtin_fmaf(qlo[e], rl, d);
-        d = __builtin_fmaf(qhi[e], rh, d);
-      }
-      sc[i] = sum8(d) * c2;                                       // log2 domain
-    }
-    // landmark = key BS-1 = group 7, i = KPG-1
-    const float t_lm = __shfl(sc[KPG - 1], 56, 64);
-    float mx = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < KPG; ++i)
-      if (!(i == KPG - 1 && g == 7)) mx = fmaxf(mx, sc[i]);
-    mx = fmaxf(mx, dpp_f<0x128>(mx));                             // row_ror 8: the other key group of the row
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    float den = 0.f;
-#pragma unroll
-    for (int i = 0; i < KPG; ++i) {
-      float e = fast_exp2(sc[i] - mx);
-      if (i == KPG - 1 && g == 7) e = 0.f;
-      sc[i] = e;
-      den += e;
-    }
-    den += dpp_f<0x128>(den);
-    den += __shfl_xor(den, 16, 64);
-    den += __shfl_xor(den, 32, 64);
-    const float Mnew = fmaxf(Mrun, t_lm);
-    const float alpha = fast_exp2(Mrun - Mnew);
-    const float gate = fast_exp2(t_lm - Mnew);
-    lrun = lrun * alpha + gate;
-    Mrun = Mnew;
-    const float f = gate / den;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      alo[e] *= alpha;
-      ahi[e] *= alpha;
-    }
-#pragma unroll
-    for (int i = 0; i < KPG; ++i) {
-      const float w = round_to<T>(sc[i] * f);                     // weights enter PV in the model dtype
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        alo[2 * e] = __builtin_fmaf(w, unpack_lo<T>(vlo[i][e]), alo[2 * e]);
-        alo[2 * e + 1] = __builtin_fmaf(w, unpack_hi<T>(vlo[i][e]), alo[2 * e + 1]);
-        ahi[2 * e] = __builtin_fmaf(w, unpack_lo<T>(vhi[i][e]), ahi[2 * e]);
-        ahi[2 * e + 1] = __builtin_fmaf(w, unpack_hi<T>(vhi[i][e]), ahi[2 * e + 1]);
-      }
-    }
-  }
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {                                   // sum over the eight key groups
-    alo[e] += dpp_f<0x128>(alo[e]);
-    ahi[e] += dpp_f<0x128>(ahi[e]);
-    alo[e] += __shfl_xor(alo[e], 16, 64);
-    ahi[e] += __shfl_xor(ahi[e], 16, 64);
-    alo[e] += __shfl_xor(alo[e], 32, 64);
-    ahi[e] += __shfl_xor(ahi[e], 32, 64);
-  }
-  // merge with the local chunk: out_loc (normalised), L_loc, M_loc (natural-log units)
-  const int64_t srow = (int64_t)bh * p.stat_stride + t;
-  const float Ml = p.M_loc[srow] * kLog2e, Ll = p.L_loc[srow];
-  const float Mt = fmaxf(Mrun, Ml);
-  const float wr = fast_exp2(Mrun - Mt), wl = fast_exp2(Ml - Mt) * Ll;
-  const float inv = 1.0f / (lrun * wr + wl);
-  if (g == 0) {
-    const char* olp = (const char*)p.o_loc + 2 * (b * p.ols_b + hh * p.ols_h + (int64_t)t * p.ols_r) + 16 * j;
-    char* outp = (char*)p.out + 2 * (b * p.outs_b + hh * p.outs_h + (int64_t)t * p.outs_r) + 16 * j;
-    float ol[8], o[8];
-    unpack8(*(const u32x4_t*)(olp), ol);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = (alo[i] * wr + ol[i] * wl) * inv;
-    u32x4_t ov = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
-    *(u32x4_t*)(outp) = ov;
-    unpack8(*(const u32x4_t*)(olp + 128), ol);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = (ahi[i] * wr + ol[i] * wl) * inv;
-    u32x4_t ov2 = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
-    *(u32x4_t*)(outp + 128) = ov2;
-  }
-}
-
-// Blocks of more than 64 keys: same lane mapping and arithmetic as lmk_gather_attend_kernel, but a
-// block passes through the registers in chunks of 64 keys -- first the keys of every chunk (scores
-// of the whole block, which the block's softmax needs before any weight is final), then the values.
-// The loads of the next chunk are issued before the arithmetic on the current one.
-template <class T, int D, int BS>
-__global__ __launch_bounds__(256) void lmk_gather_attend_chunked_kernel(RetrParams p) {
-  static_assert(D == 128 && BS % 64 == 0, "16 chunks of 8 head dims per row; whole chunks of 64 keys");
-  constexpr int NC = BS / 64;                                     // chunks per block
+  static_assert(D == 128 && (BS == 32 || BS % 64 == 0), "16 chunks of 8 head dims per row; whole chunks of keys");
+  constexpr int CK = BS < 64 ? BS : 64;                           // keys per chunk
+  constexpr int KPG = CK / 8;                                     // keys per 8-lane group and chunk
+  constexpr int NC = BS / CK;                                     // chunks per block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int j = lane & 7, g = lane >> 3;                           // head-dim chunk pair, key group
   const int64_t row = (int64_t)blockIdx.x * 4 + wave;             // (bh, t)
@@ -932,11 +767,11 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_chunked_kernel(RetrPara
     ahi[i] = 0.f;
   }
 
-  // one chunk = 64 rows of K or of V: this lane's 8 rows (g, g+8, ..) x its two 16-byte pieces
-  u32x4_t clo[8], chi[8], nlo[8], nhi[8];
+  // one chunk = CK rows of K or of V: this lane's KPG rows (g, g+8, ..) x its two 16-byte pieces
+  u32x4_t clo[KPG], chi[KPG], nlo[KPG], nhi[KPG];
   auto fetch = [&](const char* base, int64_t row_stride, int64_t key0) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < KPG; ++i) {
       const char* r = base + 2 * ((key0 + g + 8 * i) * row_stride) + 16 * j;
       nlo[i] = *(const u32x4_t*)(r);
       nhi[i] = *(const u32x4_t*)(r + 128);
@@ -944,7 +779,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_chunked_kernel(RetrPara
   };
   auto take = [&]() {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < KPG; ++i) {
       clo[i] = nlo[i];
       chi[i] = nhi[i];
     }
@@ -954,15 +789,15 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_chunked_kernel(RetrPara
   for (int js = 0; js < p.k; ++js) {
     const int64_t key0 = (int64_t)blk * BS;
     const int64_t pos0 = (int64_t)js * BS + ((blk >= p.num_mems - p.k) ? BS : 0) + p.prefix_len;
-    float sc[8 * NC];
+    float sc[KPG * NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       take();
-      if (c + 1 < NC) fetch(kc, p.kcs_r, key0 + 64 * (c + 1));
+      if (c + 1 < NC) fetch(kc, p.kcs_r, key0 + CK * (c + 1));
       else fetch(vc, p.vcs_r, key0);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int kk = 64 * c + g + 8 * i;
+      for (int i = 0; i < KPG; ++i) {
+        const int kk = CK * c + g + 8 * i;
         const char* cr = (const char*)p.cos + 2 * ((pos0 + kk) * p.cs_r) + 16 * j;
         const char* sr = (const char*)p.sin + 2 * ((pos0 + kk) * p.cs_r) + 16 * j;
         float kl[8], kh[8], cl[8], ch[8], sl[8], sh[8];
@@ -980,23 +815,23 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_chunked_kernel(RetrPara
           d = __builtin_fmaf(qlo[e], rl, d);
           d = __builtin_fmaf(qhi[e], rh, d);
         }
-        sc[8 * c + i] = sum8(d) * c2;                             // log2 domain
+        sc[KPG * c + i] = sum8(d) * c2;                           // log2 domain
       }
     }
-    // landmark = key BS-1 = last chunk, group 7, i = 7
-    const float t_lm = __shfl(sc[8 * NC - 1], 56, 64);
+    // landmark = key BS-1 = last chunk, group 7, last of the group's keys
+    const float t_lm = __shfl(sc[KPG * NC - 1], 56, 64);
     float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 8 * NC; ++i)
-      if (!(i == 8 * NC - 1 && g == 7)) mx = fmaxf(mx, sc[i]);
+    for (int i = 0; i < KPG * NC; ++i)
+      if (!(i == KPG * NC - 1 && g == 7)) mx = fmaxf(mx, sc[i]);
     mx = fmaxf(mx, dpp_f<0x128>(mx));                             // row_ror 8: the other key group of the row
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     float den = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8 * NC; ++i) {
+    for (int i = 0; i < KPG * NC; ++i) {
       float e = fast_exp2(sc[i] - mx);
-      if (i == 8 * NC - 1 && g == 7) e = 0.f;
+      if (i == KPG * NC - 1 && g == 7) e = 0.f;
       sc[i] = e;
       den += e;
     }
@@ -1019,11 +854,11 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_chunked_kernel(RetrPara
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       take();
-      if (c + 1 < NC) fetch(vc, p.vcs_r, key0 + 64 * (c + 1));
+      if (c + 1 < NC) fetch(vc, p.vcs_r, key0 + CK * (c + 1));
       else if (js + 1 < p.k) fetch(kc, p.kcs_r, (int64_t)blk_next * BS);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float w = round_to<T>(sc[8 * c + i] * f);           // weights enter PV in the model dtype
+      for (int i = 0; i < KPG; ++i) {
+        const float w = round_to<T>(sc[KPG * c + i] * f);         // weights enter PV in the model dtype
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           alo[2 * e] = __builtin_fmaf(w, unpack_lo<T>(clo[i][e]), alo[2 * e]);
@@ -1139,7 +974,7 @@ static int launch_gather_t(const RetrParams& p, int BS, hipStream_t stream) {
   const dim3 grid((unsigned)((rows + 3) / 4));
   if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 32>), grid, dim3(256), 0, stream, p);
   else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 64>), grid, dim3(256), 0, stream, p);
-  else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_chunked_kernel<T, 128, 128>), grid, dim3(256), 0, stream, p);
+  else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 128>), grid, dim3(256), 0, stream, p);
   else return LMK_ERR_UNSUPPORTED;
   return (int)hipGetLastError();
 }
