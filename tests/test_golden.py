@@ -45,3 +45,20 @@ def test_retrieval_fixture_matches_restated_reference_path():
     out32, _ = retrieval.retrieve_and_attend(q.float(), kc.float(), vc.float(), kl.float(), vl.float(), is_mem,
                                              cos.float(), sin.float(), block, top_k, idx=f["idx"])
     assert (out32 - f["out"]).abs().max() < 2e-2                 # fp32 tables differ from the bf16 ones the fixture used
+
+
+def test_shared_selection_fixture_matches_vectorised_contract():
+    f = load("shared_selection_h1_t4_s2115_d64_b32_k3.npz")
+    block, top_k = int(f["block"]), int(f["top_k"])
+    q, kc, vc, kl, vl = (f[n + "_bf16bits"].view(torch.bfloat16) for n in ("q", "k_cache", "v_cache", "k_loc", "v_loc"))
+    S, T, D = kc.shape[2], q.shape[2], q.shape[3]
+    cos, sin = rotary.rotary_tables(S + T, D, torch.bfloat16)
+    agg = retrieval.aggregate_max_over_tokens(retrieval.landmark_scores(q, kc, cos, sin, block, top_k))
+    assert torch.equal(agg[:, :, 0].float(), f["block_probs"])    # the head's vector, bit for bit
+    inc = S % block
+    is_mem = ((torch.arange(T) + inc) % block == block - 1)[None]
+    out, idx = retrieval.retrieve_and_attend_shared(q, kc, vc, kl, vl, is_mem, cos, sin, block, top_k)
+    assert torch.equal(idx, f["idx"])
+    assert (out.float() - f["out"]).abs().max() < 2e-2
+    ref32 = retrieval.retrieve_and_attend_shared_s1(q, kc, vc, kl, vl, cos, sin, block, top_k, f["idx"])
+    assert (ref32 - f["out"]).abs().max() < 2e-3

@@ -40,3 +40,20 @@ def test_retrieval_fixture_indices_and_output():
     torch.cuda.synchronize()
     assert torch.equal(idx.cpu(), f["idx"])
     assert (out.float().cpu() - f["out"]).abs().max().item() <= TOL
+
+
+def test_shared_selection_fixture_probabilities_indices_and_output():
+    from landmark_hip.retrieval import attend_shared, retrieve_topk
+    from oracle import rotary
+    f = load("shared_selection_h1_t4_s2115_d64_b32_k3.npz")
+    block, top_k = int(f["block"]), int(f["top_k"])
+    dev = torch.device("cuda:0")
+    q, kc, vc, kl, vl = (f[n + "_bf16bits"].view(torch.bfloat16).to(dev)
+                         for n in ("q", "k_cache", "v_cache", "k_loc", "v_loc"))
+    cos, sin = (t.to(dev) for t in rotary.rotary_tables(kc.shape[2] + q.shape[2], q.shape[3], torch.bfloat16))
+    idx, probs = retrieve_topk(q, kc, cos, sin, block, top_k, aggregate="max_over_tokens", return_block_probs=True)
+    torch.cuda.synchronize()
+    assert torch.equal(probs.float().cpu()[:, :, 0], f["block_probs"])
+    assert torch.equal(idx.cpu(), f["idx"])
+    out = attend_shared(q, kc, vc, idx, kl, vl, cos, sin, block, top_k)
+    assert (out.float().cpu() - f["out"]).abs().max().item() <= TOL
