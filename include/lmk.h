@@ -112,7 +112,7 @@ int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
  * attend step (:329-342; see lmk_local_window). */
 
 /* Bytes of device workspace lmk_retrieve_topk needs: rotated landmark keys and their norms,
- * plus two fp32 score planes of B*H*T*(S/block). */
+ * plus two fp32 planes of B*H*T*(S/block) that only lmk_retrieve_topk_shared writes. */
 size_t lmk_retrieve_workspace_bytes(int B, int H, int T, int S, int D, int block);
 
 /* Landmark scoring + top-k selection (llama_mem.py:344-384, aggregate=None branch).

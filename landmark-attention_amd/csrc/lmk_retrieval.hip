@@ -93,52 +93,7 @@ __global__ __launch_bounds__(256) void lmk_landmark_keys_kernel(RetrParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// score: approximate fp32 scores with MFMA, S^T layout (lane = query, registers = landmarks)
-// ---------------------------------------------------------------------------
-template <class T, int D>
-__global__ __launch_bounds__(256) void lmk_score_kernel(RetrParams p) {
-  constexpr int KS = D / 16;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int ql = lane & 31, h = lane >> 5;
-  const int n_qt = (p.T + 127) / 128;
-  const int bh = blockIdx.x / n_qt, qt = blockIdx.x % n_qt;
-  const int b = bh / p.H, hh = bh % p.H;
-  const int q0 = qt * 128 + wave * 32;
-  if (q0 >= p.T) return;
-  const int qrow = q0 + ql;
-  const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h);
-  u32x4_t qf[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    u32x4_t z = {0, 0, 0, 0};
-    qf[ks] = z;
-    if (qrow < p.T) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
-  }
-  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * p.num_mems * D);
-  float* out = p.approx + ((int64_t)bh * p.T + qrow) * p.num_mems;
-  for (int m0 = 0; m0 < p.num_mems; m0 += 32) {
-    const int m = m0 + ql;
-    f32x16_t s;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) s[r] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      u32x4_t a = {0, 0, 0, 0};
-      if (m < p.num_mems) a = *(const u32x4_t*)(lk + 2 * ((int64_t)m * D + 16 * ks + 8 * h));
-      s = mfma32<T>(a, qf[ks], s);
-    }
-    if (qrow < p.T) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int mm = m0 + 8 * (r >> 2) + 4 * h + (r & 3);
-        if (mm < p.num_mems) out[mm] = s[r];
-      }
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------
-// select: exact top-k per query row, one wave per row
+// helpers of the selection: the rounding contract and a wave-wide arg-best
 // ---------------------------------------------------------------------------
 template <class T>
 __device__ __forceinline__ float contract(float dot, float sqrt_hd) {
@@ -175,138 +130,6 @@ __device__ __forceinline__ void wave_best(float& v, int& i) {
   }
   v = bv;
   i = bi;
-}
-
-constexpr int kSelSeg = 1024;   // landmarks handled per sweep of the contender list
-
-template <class T, int D>
-__global__ __launch_bounds__(256) void lmk_select_kernel(RetrParams p) {
-  __shared__ __align__(16) float q_lds[4][D];
-  __shared__ int cand[4][kSelSeg];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t row = (int64_t)blockIdx.x * 4 + wave;             // (bh, t)
-  const int64_t total = (int64_t)p.B * p.H * p.T;
-  if (row >= total) return;                                       // whole wave leaves; no block-wide barrier below
-  const int bh = (int)(row / p.T), t = (int)(row % p.T);
-  const int b = bh / p.H, hh = bh % p.H;
-  const int NM = p.num_mems;
-
-  // q row -> fp32 in LDS (read back as a broadcast), and its norm
-  const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
-  float qn = 0.f;
-  for (int d = 2 * lane; d < D; d += 128) {
-    const uint32_t u = *(const uint32_t*)(qp + 2 * d);
-    const float x0 = unpack_lo<T>(u), x1 = unpack_hi<T>(u);
-    q_lds[wave][d] = x0;
-    q_lds[wave][d + 1] = x1;
-    qn += x0 * x0 + x1 * x1;
-  }
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) qn += __shfl_xor(qn, m, 64);
-  const float eps_q = sqrtf(qn) * 1.000001f * (1.0f / 16384.0f);
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_s_waitcnt(0xc07f);                             // LDS writes of this wave visible (lgkmcnt 0)
-
-  const float* approx = p.approx + row * NM;
-  float* exact = p.exact + row * NM;
-  const float* lkn = p.lk_norm + (int64_t)bh * NM;
-  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * NM * D);
-  const float sq = p.sqrt_hd;
-
-  // ---- tau = k-th best lower end
-  float tau = INFINITY;
-  {
-    float pv = INFINITY;
-    int pi = -1;
-    for (int j = 0; j < p.k; ++j) {
-      float bv = -INFINITY;
-      int bi = 0x7fffffff;
-      for (int m = lane; m < NM; m += 64) {
-        const float lo = contract<T>(approx[m] - eps_q * lkn[m], sq);
-        const bool after = (lo < pv) || (lo == pv && m > pi);     // strictly after the previous pick
-        if (after && (lo > bv || (lo == bv && m < bi))) {
-          bv = lo;
-          bi = m;
-        }
-      }
-      wave_best(bv, bi);
-      pv = bv;
-      pi = bi;
-    }
-    tau = pv;
-  }
-
-  // ---- contenders: upper end reaches tau -> exact score in the defined order; others -inf
-  for (int seg = 0; seg < NM; seg += kSelSeg) {
-    int count = 0;
-    for (int m0 = seg; m0 < min(NM, seg + kSelSeg); m0 += 64) {
-      const int m = m0 + lane;
-      bool is_c = false;
-      if (m < NM) {
-        const float hi = contract<T>(approx[m] + eps_q * lkn[m], sq);
-        is_c = hi >= tau;
-        if (!is_c) exact[m] = -INFINITY;
-      }
-      const uint64_t bal = __ballot(is_c);
-      if (is_c) cand[wave][count + __popcll(bal & ((1ull << lane) - 1))] = m;
-      count += __popcll(bal);
-    }
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    for (int c0 = 0; c0 < count; c0 += 64) {
-      if (c0 + lane < count) {
-        const int m = cand[wave][c0 + lane];
-        const char* kr = lk + 2 * ((int64_t)m * D);
-        float acc = 0.f;
-#pragma unroll 4
-        for (int d8 = 0; d8 < D / 8; ++d8) {
-          const u32x4_t kk = *(const u32x4_t*)(kr + 16 * d8);
-          const float4 qa = *(const float4*)&q_lds[wave][8 * d8];
-          const float4 qb = *(const float4*)&q_lds[wave][8 * d8 + 4];
-          acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
-          acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
-          acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
-          acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
-          acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
-          acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
-          acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
-          acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
-        }
-        exact[m] = contract<T>(acc, sq);
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
-  }
-  __threadfence_block();
-
-  // ---- k best exact scores, then ascending order
-  int mine = -1;                                                 // lane j keeps the j-th pick
-  {
-    float pv = INFINITY;
-    int pi = -1;
-    for (int j = 0; j < p.k; ++j) {
-      float bv = -INFINITY;
-      int bi = 0x7fffffff;
-      for (int m = lane; m < NM; m += 64) {
-        const float x = exact[m];
-        const bool after = (x < pv) || (x == pv && m > pi);
-        if (after && (x > bv || (x == bv && m < bi))) {
-          bv = x;
-          bi = m;
-        }
-      }
-      wave_best(bv, bi);
-      pv = bv;
-      pi = bi;
-      if (lane == j) mine = bi;
-    }
-  }
-  int rank = 0;
-  for (int j = 0; j < p.k; ++j) {
-    const int o = __shfl(mine, j, 64);
-    rank += (o < mine) ? 1 : 0;
-  }
-  if (lane < p.k) p.idx[row * p.k + rank] = (int64_t)mine;
 }
 
 // ---------------------------------------------------------------------------
@@ -481,15 +304,18 @@ __global__ __launch_bounds__(64) void lmk_block_select_kernel(RetrParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// fused score + select for caches of at most kFusedMaxMems landmark blocks: the approximate scores
-// of 32 query rows never leave the CU
+// fused score + select: the approximate scores of 32 query rows never leave the CU
 // ---------------------------------------------------------------------------
-// A workgroup (4 waves) owns 32 consecutive query rows of one (batch, head).
-//   score   the waves split the landmarks; S = Q LK^T by MFMA with the landmark in the lane, so a
-//           register (= one query row) lands in 32 consecutive LDS words
-//   select  each wave takes 8 of the rows in turn; a lane holds the 16 scores m = 64 j + lane of the
+// A workgroup (16 waves) owns 32 consecutive query rows of one (batch, head) and walks the cached blocks
+// in segments of at most kFusedMaxMems:
+//   score   the waves split the segment's landmarks; S = Q LK^T by MFMA with the landmark in the lane,
+//           so a register (= one query row) lands in 32 consecutive LDS words
+//   select  each wave takes 2 of the rows in turn; a lane holds the 16 scores m = 64 j + lane of the
 //           row in registers: bracket, k-th best lower end, exact re-evaluation of the contenders
-//           (written back over their approximate score), k best, ascending order
+//           (written back over their approximate score), k best
+//   merge   (more than one segment) a row's k best are the k best of the segments' k best: lane j of the
+//           row's wave keeps the j-th best (score, index) so far and every segment's picks are inserted
+//           in order; ascending index order at the end
 // The bracket uses a cheap monotone over-/under-estimate of the rounding contract: round_T(x) / sqrt(hd)
 // is replaced by a multiplication by the rounded reciprocal, pushed outwards by 2^-21 relative (the
 // product is within 2^-22 of the correctly rounded quotient) before the final rounding.  That only
@@ -499,14 +325,14 @@ constexpr int kFusedRows = 32;
 constexpr int kFusedWaves = 16;
 constexpr int kFusedList = 128;                                   // contender list per wave: flushed at 64, a ballot adds <= 64
 
-template <class T, int D>
+template <class T, int D, bool SEGMENTS>
 __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrParams p) {
   constexpr int KS = D / 16;
   constexpr int NJ = kFusedMaxMems / 64;                          // scores per lane and row
   extern __shared__ __align__(16) unsigned char smem[];
-  const int NM = p.num_mems;
-  const int NMr = (NM + 63) & ~63;                                // columns read by the select phase
-  const int NMp = NMr + 32;                                       // row stride (words): the two half-waves of a store
+  const int NMall = p.num_mems;
+  const int seg_cap = NMall < kFusedMaxMems ? NMall : kFusedMaxMems;
+  const int NMp = ((seg_cap + 63) & ~63) + 32;                    // row stride (words): the two half-waves of a store
                                                                   // then hit different banks
   float* sc = (float*)smem;                                       // [32][NMp]
   float* q_lds = sc + kFusedRows * NMp;                           // [waves][D]
@@ -518,8 +344,8 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
   const int bh = blockIdx.x / n_qt, t0 = (blockIdx.x % n_qt) * kFusedRows;
   const int b = bh / p.H, hh = bh % p.H;
   const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h);
-  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * NM * D);
-  const float* lkn = p.lk_norm + (int64_t)bh * NM;
+  const char* lk_all = (const char*)p.lk_rot + 2 * ((int64_t)bh * NMall * D);
+  const float* lkn_all = p.lk_norm + (int64_t)bh * NMall;
 
   // ---- the 32 query rows -> LDS (the select phase reads them from there)
   for (int c = tid; c < kFusedRows * (D / 8); c += 64 * kFusedWaves) {
@@ -528,180 +354,251 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
     if (t0 + r < p.T) v = *(const u32x4_t*)(qp + 2 * ((int64_t)(t0 + r) * p.qs_r + 8 * ch));
     *(u32x4_t*)(q_raw + r * 2 * D + 16 * ch) = v;
   }
-  // ---- score: A = query rows (lane -> row), B = landmark keys (lane -> landmark)
-  {
-    u32x4_t qf[KS];
-    const int qrow = t0 + ql;
+  // running k best of every row this wave owns (rows wave, wave + 16): lane j holds the j-th best so far
+  float run_v[kFusedRows / kFusedWaves];
+  int run_i[kFusedRows / kFusedWaves];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      u32x4_t z = {0, 0, 0, 0};
-      qf[ks] = z;
-      if (qrow < p.T) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
-    }
-    for (int m0 = 32 * wave; m0 < NMr; m0 += 32 * kFusedWaves) {
-      const int m = m0 + ql;
-      u32x4_t kf[KS];
+  for (int i = 0; i < kFusedRows / kFusedWaves; ++i) {
+    run_v[i] = -INFINITY;
+    run_i[i] = 0x7fffffff;
+  }
+  // ---- the cached blocks in segments of at most kFusedMaxMems: a row's k best are the k best of the
+  // segments' k best, merged under the same order
+  for (int seg = 0; seg < NMall; seg += kFusedMaxMems) {
+    const int NM = min(NMall - seg, kFusedMaxMems);                 // landmarks of this segment
+    const int NMr = (NM + 63) & ~63;                                // columns read by the select phase
+    const char* lk = lk_all + 2 * ((int64_t)seg * D);
+    const float* lkn = lkn_all + seg;
+    // ---- score: A = query rows (lane -> row), B = landmark keys (lane -> landmark)
+    {
+      u32x4_t qf[KS];
+      const int qrow = t0 + ql;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         u32x4_t z = {0, 0, 0, 0};
-        kf[ks] = z;
-        if (m < NM) kf[ks] = *(const u32x4_t*)(lk + 2 * ((int64_t)m * D + 16 * ks + 8 * h));
+        qf[ks] = z;
+        if (qrow < p.T) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
       }
-      f32x16_t s;
+      for (int m0 = 32 * wave; m0 < NMr; m0 += 32 * kFusedWaves) {
+        const int m = m0 + ql;
+        u32x4_t kf[KS];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[r] = 0.f;
+        for (int ks = 0; ks < KS; ++ks) {
+          u32x4_t z = {0, 0, 0, 0};
+          kf[ks] = z;
+          if (m < NM) kf[ks] = *(const u32x4_t*)(lk + 2 * ((int64_t)m * D + 16 * ks + 8 * h));
+        }
+        f32x16_t s;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) s = mfma32<T>(qf[ks], kf[ks], s);
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) sc[(8 * (r >> 2) + 4 * h + (r & 3)) * NMp + m] = (m < NM) ? s[r] : -INFINITY;
-    }
-  }
-  __syncthreads();
-
-  // ---- select
-  float nrm[NJ];                                                  // |k_m| of this lane's landmarks
+        for (int ks = 0; ks < KS; ++ks) s = mfma32<T>(qf[ks], kf[ks], s);
 #pragma unroll
-  for (int j = 0; j < NJ; ++j) {
-    const int m = 64 * j + lane;
-    nrm[j] = (m < NM) ? lkn[m] : 0.f;
-  }
-  const float sq = p.sqrt_hd, inv_sq = 1.0f / sq;
-  float* qrow_lds = q_lds + wave * D;
-  int* cnd = cand + wave * kFusedList;
-  const int nj = NMr >> 6;                                        // slices in use (wave-uniform)
-
-  // wave-wide arg-best of v[] under (value desc, index asc); the winner's slot is set to -inf
-  auto take_best = [&](float* v, float& bv_out, int& bi_out) {
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-#pragma unroll
-    for (int j = 0; j < NJ; ++j)
-      if (j < nj && v[j] > bv) {                                  // ascending j = ascending index: strict > keeps the first
-        bv = v[j];
-        bi = 64 * j + lane;
+        for (int r = 0; r < 16; ++r) sc[(8 * (r >> 2) + 4 * h + (r & 3)) * NMp + m] = (m < NM) ? s[r] : -INFINITY;
       }
-    wave_best(bv, bi);
-    const int win = __builtin_amdgcn_readfirstlane(bi);
-    const bool owner = lane == (win & 63);
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) v[j] = (owner && j == (win >> 6)) ? -INFINITY : v[j];
-    bv_out = bv;
-    bi_out = win;
-  };
-
-  for (int qi = wave; qi < kFusedRows; qi += kFusedWaves) {
-    const int t = t0 + qi;
-    if (t >= p.T) break;                                          // wave-uniform
-    const int64_t row = (int64_t)bh * p.T + t;
-    // q row -> fp32 in LDS (read back as a broadcast), and its norm
-    const unsigned char* qr = q_raw + qi * 2 * D;
-    float qn = 0.f;
-    for (int d = 2 * lane; d < D; d += 128) {
-      const uint32_t u = *(const uint32_t*)(qr + 2 * d);
-      const float x0 = unpack_lo<T>(u), x1 = unpack_hi<T>(u);
-      qrow_lds[d] = x0;
-      qrow_lds[d + 1] = x1;
-      qn += x0 * x0 + x1 * x1;
     }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) qn += __shfl_xor(qn, m, 64);
-    const float eps_q = sqrtf(qn) * 1.000001f * (1.0f / 16384.0f);
+    __syncthreads();
 
-    float* srow = sc + qi * NMp;
-    float lo[NJ], hi[NJ];
+    // ---- select
+    float nrm[NJ];                                                  // |k_m| of this lane's landmarks
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      lo[j] = -INFINITY;
-      hi[j] = -INFINITY;
-      if (j < nj) {
-        const float a = srow[64 * j + lane];
-        if (a > -INFINITY) {
-          const float e = eps_q * nrm[j];
-          const float cl = round_to<T>(a - e) * inv_sq, ch = round_to<T>(a + e) * inv_sq;
-          lo[j] = round_to<T>(cl - fabsf(cl) * 4.76837158203125e-7f);
-          hi[j] = round_to<T>(ch + fabsf(ch) * 4.76837158203125e-7f);
-        }
-      }
+      const int m = 64 * j + lane;
+      nrm[j] = (m < NM) ? lkn[m] : 0.f;
     }
-    // tau = k-th best lower end
-    float tau = -INFINITY;
-    for (int j = 0; j < p.k; ++j) {
-      int bi;
-      take_best(lo, tau, bi);
-    }
-    // contenders: upper end reaches tau.  They are collected in a short list and evaluated exactly,
-    // one lane per contender, whenever the list holds a wave's worth (and at the end).
-    auto evaluate = [&](int count) {
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_s_waitcnt(0xc07f);                         // this wave's LDS writes (q row, list) are visible
-      for (int c0 = 0; c0 < count; c0 += 64) {
-        if (c0 + lane < count) {
-          const int m = cnd[c0 + lane];
-          const char* kr = lk + 2 * ((int64_t)m * D);
-          float acc = 0.f;
+    const float sq = p.sqrt_hd, inv_sq = 1.0f / sq;
+    float* qrow_lds = q_lds + wave * D;
+    int* cnd = cand + wave * kFusedList;
+    const int nj = NMr >> 6;                                        // slices in use (wave-uniform)
+
+    // wave-wide arg-best of v[] under (value desc, index asc); the winner's slot is set to -inf
+    auto take_best = [&](float* v, float& bv_out, int& bi_out) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
 #pragma unroll
-          for (int g = 0; g < D / 64; ++g) {                      // 8 loads in flight, then their 64 dependent fmas
-            u32x4_t kv[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) kv[i] = *(const u32x4_t*)(kr + 16 * (8 * g + i));
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-              const u32x4_t kk = kv[i];
-              const float4 qa = *(const float4*)&qrow_lds[8 * (8 * g + i)];
-              const float4 qb = *(const float4*)&qrow_lds[8 * (8 * g + i) + 4];
-              acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
-              acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
-              acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
-              acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
-              acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
-              acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
-              acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
-              acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
-            }
-          }
-          srow[m] = contract<T>(acc, sq);
+      for (int j = 0; j < NJ; ++j)
+        if (j < nj && v[j] > bv) {                                  // ascending j = ascending index: strict > keeps the first
+          bv = v[j];
+          bi = 64 * j + lane;
         }
-      }
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_s_waitcnt(0xc07f);
+      wave_best(bv, bi);
+      const int win = __builtin_amdgcn_readfirstlane(bi);
+      const bool owner = lane == (win & 63);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) v[j] = (owner && j == (win >> 6)) ? -INFINITY : v[j];
+      bv_out = bv;
+      bi_out = win;
     };
-    uint32_t is_c = 0;
-    int count = 0;
+
+    for (int qi = wave, ri = 0; qi < kFusedRows; qi += kFusedWaves, ++ri) {
+      const int t = t0 + qi;
+      if (t >= p.T) break;                                          // wave-uniform
+      // q row -> fp32 in LDS (read back as a broadcast), and its norm
+      const unsigned char* qr = q_raw + qi * 2 * D;
+      float qn = 0.f;
+      for (int d = 2 * lane; d < D; d += 128) {
+        const uint32_t u = *(const uint32_t*)(qr + 2 * d);
+        const float x0 = unpack_lo<T>(u), x1 = unpack_hi<T>(u);
+        qrow_lds[d] = x0;
+        qrow_lds[d + 1] = x1;
+        qn += x0 * x0 + x1 * x1;
+      }
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      if (j < nj) {
-        const bool c = hi[j] >= tau && hi[j] > -INFINITY;
-        const uint64_t bal = __ballot(c);
-        if (c) {
-          cnd[count + __popcll(bal & ((1ull << lane) - 1))] = 64 * j + lane;
-          is_c |= 1u << j;
-        }
-        count += __popcll(bal);
-        if (count >= 64) {                                        // wave-uniform
-          evaluate(count);
-          count = 0;
+      for (int m = 32; m >= 1; m >>= 1) qn += __shfl_xor(qn, m, 64);
+      const float eps_q = sqrtf(qn) * 1.000001f * (1.0f / 16384.0f);
+
+      float* srow = sc + qi * NMp;
+      float lo[NJ], hi[NJ];
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        lo[j] = -INFINITY;
+        hi[j] = -INFINITY;
+        if (j < nj) {
+          const float a = srow[64 * j + lane];
+          if (a > -INFINITY) {
+            const float e = eps_q * nrm[j];
+            const float cl = round_to<T>(a - e) * inv_sq, ch = round_to<T>(a + e) * inv_sq;
+            lo[j] = round_to<T>(cl - fabsf(cl) * 4.76837158203125e-7f);
+            hi[j] = round_to<T>(ch + fabsf(ch) * 4.76837158203125e-7f);
+          }
         }
       }
-    }
-    if (count > 0) evaluate(count);
-    // k best exact scores, then ascending order
-    float x[NJ];
+      // tau = k-th best lower end
+      float tau = -INFINITY;
+      for (int j = 0; j < p.k; ++j) {
+        int bi;
+        take_best(lo, tau, bi);
+      }
+      // contenders: upper end reaches tau.  They are collected in a short list and evaluated exactly,
+      // one lane per contender, whenever the list holds a wave's worth (and at the end).
+      auto evaluate = [&](int count) {
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f);                         // this wave's LDS writes (q row, list) are visible
+        for (int c0 = 0; c0 < count; c0 += 64) {
+          if (c0 + lane < count) {
+            const int m = cnd[c0 + lane];
+            const char* kr = lk + 2 * ((int64_t)m * D);
+            float acc = 0.f;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) x[j] = (j < nj && ((is_c >> j) & 1)) ? srow[64 * j + lane] : -INFINITY;
-    int mine = -1;                                               // lane j keeps the j-th pick
-    for (int j = 0; j < p.k; ++j) {
-      float bv;
-      int bi;
-      take_best(x, bv, bi);
-      if (lane == j) mine = bi;
+            for (int g = 0; g < D / 64; ++g) {                      // 8 loads in flight, then their 64 dependent fmas
+              u32x4_t kv[8];
+#pragma unroll
+              for (int i = 0; i < 8; ++i) kv[i] = *(const u32x4_t*)(kr + 16 * (8 * g + i));
+#pragma unroll
+              for (int i = 0; i < 8; ++i) {
+                const u32x4_t kk = kv[i];
+                const float4 qa = *(const float4*)&qrow_lds[8 * (8 * g + i)];
+                const float4 qb = *(const float4*)&qrow_lds[8 * (8 * g + i) + 4];
+                acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
+                acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
+                acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
+                acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
+                acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
+                acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
+                acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
+                acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
+              }
+            }
+            srow[m] = contract<T>(acc, sq);
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+      };
+      uint32_t is_c = 0;
+      int count = 0;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        if (j < nj) {
+          const bool c = hi[j] >= tau && hi[j] > -INFINITY;
+          const uint64_t bal = __ballot(c);
+          if (c) {
+            cnd[count + __popcll(bal & ((1ull << lane) - 1))] = 64 * j + lane;
+            is_c |= 1u << j;
+          }
+          count += __popcll(bal);
+          if (count >= 64) {                                        // wave-uniform
+            evaluate(count);
+            count = 0;
+          }
+        }
+      }
+      if (count > 0) evaluate(count);
+      // k best exact scores, then ascending order
+      float x[NJ];
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) x[j] = (j < nj && ((is_c >> j) & 1)) ? srow[64 * j + lane] : -INFINITY;
+      if constexpr (!SEGMENTS) {                                  // one segment: its k best are the row's
+        int mine = -1;                                           // lane j keeps the j-th pick
+        for (int j = 0; j < p.k; ++j) {
+          float bv;
+          int bi;
+          take_best(x, bv, bi);
+          if (lane == j) mine = bi;
+        }
+        int rank = 0;
+        for (int j = 0; j < p.k; ++j) {
+          const int o = __shfl(mine, j, 64);
+          rank += (o < mine) ? 1 : 0;
+        }
+        if (lane < p.k) p.idx[((int64_t)bh * p.T + t) * p.k + rank] = (int64_t)mine;
+        __builtin_amdgcn_wave_barrier();                          // the next row reuses the q row and the list
+        continue;
+      }
+      // the segment's k best exact scores, best first, each inserted into the row's running list
+      float rv = -INFINITY;
+      int rx = 0x7fffffff;
+#pragma unroll
+      for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
+        if (i == ri) {
+          rv = run_v[i];
+          rx = run_i[i];
+        }
+      for (int j = 0; j < p.k; ++j) {
+        float bv;
+        int bi;
+        take_best(x, bv, bi);
+        if (!(bv > -INFINITY)) break;                               // fewer than k landmarks in this segment (wave-uniform)
+        bi += seg;
+        const bool better = lane < p.k && (rv > bv || (rv == bv && rx < bi));   // a prefix of the sorted list
+        const int pos = __popcll(__ballot(better));
+        if (pos >= p.k) break;                                      // worse than the k kept: so are the rest
+        const float up_v = __shfl_up(rv, 1, 64);
+        const int up_i = __shfl_up(rx, 1, 64);
+        if (lane > pos) {
+          rv = up_v;
+          rx = up_i;
+        } else if (lane == pos) {
+          rv = bv;
+          rx = bi;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
+        if (i == ri) {
+          run_v[i] = rv;
+          run_i[i] = rx;
+        }
+      __builtin_amdgcn_wave_barrier();                              // the next row reuses the q row and the list
     }
+    __syncthreads();                                                // the next segment overwrites the score tile
+  }
+
+  // ---- ascending order of the k kept blocks
+  if constexpr (!SEGMENTS) return;
+  for (int qi = wave, ri = 0; qi < kFusedRows; qi += kFusedWaves, ++ri) {
+    const int t = t0 + qi;
+    if (t >= p.T) break;
+    int mine = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
+      if (i == ri) mine = run_i[i];
     int rank = 0;
     for (int j = 0; j < p.k; ++j) {
       const int o = __shfl(mine, j, 64);
       rank += (o < mine) ? 1 : 0;
     }
-    if (lane < p.k) p.idx[row * p.k + rank] = (int64_t)mine;
-    __builtin_amdgcn_wave_barrier();                              // the next row reuses the q row and the list
+    if (lane < p.k) p.idx[((int64_t)bh * p.T + t) * p.k + rank] = (int64_t)mine;
   }
 }
 
@@ -912,22 +809,23 @@ static int launch_topk_t(const RetrParams& p, hipStream_t stream) {
   hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
   int rc;
   if ((rc = (int)hipGetLastError())) return rc;
+  const int seg_cap = p.num_mems < kFusedMaxMems ? p.num_mems : kFusedMaxMems;
+  const int NMr = (seg_cap + 63) & ~63;
+  const int lds = (kFusedRows * (NMr + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
+  constexpr int lds_max = (kFusedRows * (kFusedMaxMems + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
+  const int n_rt = (p.T + kFusedRows - 1) / kFusedRows;
+  const dim3 grid(p.B * p.H * n_rt), block(64 * kFusedWaves);
   if (p.num_mems <= kFusedMaxMems) {
-    const int NMr = (p.num_mems + 63) & ~63;
-    const int lds = (kFusedRows * (NMr + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
-    auto kern = lmk_topk_fused_kernel<T, D>;
+    auto kern = lmk_topk_fused_kernel<T, D, false>;
     static std::atomic<uint64_t> lds_ok{0};
-    constexpr int lds_max = (kFusedRows * (kFusedMaxMems + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
-    if (int rc = allow_dynamic_lds(kern, lds_max, lds_ok)) return rc;
-    const int n_rt = (p.T + kFusedRows - 1) / kFusedRows;
-    hipLaunchKernelGGL(kern, dim3(p.B * p.H * n_rt), dim3(64 * kFusedWaves), lds, stream, p);
-    return (int)hipGetLastError();
+    if ((rc = allow_dynamic_lds(kern, lds_max, lds_ok))) return rc;
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, p);
+  } else {
+    auto kern = lmk_topk_fused_kernel<T, D, true>;
+    static std::atomic<uint64_t> lds_ok{0};
+    if ((rc = allow_dynamic_lds(kern, lds_max, lds_ok))) return rc;
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, p);
   }
-  const int n_qt = (p.T + 127) / 128;
-  hipLaunchKernelGGL((lmk_score_kernel<T, D>), dim3(p.B * p.H * n_qt), dim3(256), 0, stream, p);
-  if ((rc = (int)hipGetLastError())) return rc;
-  const int64_t rows = (int64_t)p.B * p.H * p.T;
-  hipLaunchKernelGGL((lmk_select_kernel<T, D>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
   return (int)hipGetLastError();
 }
 

@@ -27,6 +27,9 @@ CASES = [
     (1, 2, 64, 40 * 64, 128, 64, 4),
     (1, 2, 32, 50 * 32, 64, 32, 4),
     (1, 2, 16, 70 * 16, 128, 16, 3),       # selection does not depend on the block size set of the attend kernels
+    (1, 2, 40, 2500 * 32, 128, 32, 5),     # more than 1024 cached blocks: three segments, the last one ragged
+    (1, 1, 3, 2048 * 16, 128, 16, 64),     # two full segments, the longest list to merge
+    (1, 2, 1, 3000 * 32, 64, 32, 4),       # one query against a long cache
 ]
 
 
