@@ -430,6 +430,16 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
       bi_out = win;
     };
 
+    // the same with one candidate (value v, index id, unique in the wave) per lane
+    auto take_one = [&](float& v, int id, float& bv_out, int& bi_out) {
+      float bv = v;
+      int bi = id;
+      wave_best(bv, bi);
+      if (bi == id) v = -INFINITY;
+      bv_out = bv;
+      bi_out = bi;
+    };
+
     for (int qi = wave, ri = 0; qi < kFusedRows; qi += kFusedWaves, ++ri) {
       const int t = t0 + qi;
       if (t >= p.T) break;                                          // wave-uniform
@@ -463,11 +473,17 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
           }
         }
       }
-      // tau = k-th best lower end
+      // tau = the k-th best of the lanes' best lower ends: k different blocks reach it, so the k-th best
+      // exact score does too (a little below the k-th best lower end itself, and k times cheaper to find)
       float tau = -INFINITY;
-      for (int j = 0; j < p.k; ++j) {
-        int bi;
-        take_best(lo, tau, bi);
+      {
+        float lm = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) lm = fmaxf(lm, lo[j]);
+        for (int j = 0; j < p.k; ++j) {
+          int bi;
+          take_one(lm, lane, tau, bi);
+        }
       }
       // contenders: upper end reaches tau.  They are collected in a short list and evaluated exactly,
       // one lane per contender, whenever the list holds a wave's worth (and at the end).
@@ -507,6 +523,7 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
       };
       uint32_t is_c = 0;
       int count = 0;
+      bool flushed = false;                                         // wave-uniform: the list was emptied on the way
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         if (j < nj) {
@@ -520,65 +537,78 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
           if (count >= 64) {                                        // wave-uniform
             evaluate(count);
             count = 0;
+            flushed = true;
           }
         }
       }
       if (count > 0) evaluate(count);
-      // k best exact scores, then ascending order
-      float x[NJ];
+      // k best exact scores, best first, handed to `use`: in a single segment they are the row's (written
+      // in ascending index order), otherwise each is inserted into the row's running list
+      auto consume = [&](auto&& pick) {
+        if constexpr (!SEGMENTS) {
+          int mine = -1;                                           // lane j keeps the j-th pick
+          for (int j = 0; j < p.k; ++j) {
+            float bv;
+            int bi;
+            pick(bv, bi);
+            if (lane == j) mine = bi;
+          }
+          int rank = 0;
+          for (int j = 0; j < p.k; ++j) {
+            const int o = __shfl(mine, j, 64);
+            rank += (o < mine) ? 1 : 0;
+          }
+          if (lane < p.k) p.idx[((int64_t)bh * p.T + t) * p.k + rank] = (int64_t)mine;
+        } else {
+          float rv = -INFINITY;
+          int rx = 0x7fffffff;
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) x[j] = (j < nj && ((is_c >> j) & 1)) ? srow[64 * j + lane] : -INFINITY;
-      if constexpr (!SEGMENTS) {                                  // one segment: its k best are the row's
-        int mine = -1;                                           // lane j keeps the j-th pick
-        for (int j = 0; j < p.k; ++j) {
-          float bv;
-          int bi;
-          take_best(x, bv, bi);
-          if (lane == j) mine = bi;
+          for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
+            if (i == ri) {
+              rv = run_v[i];
+              rx = run_i[i];
+            }
+          for (int j = 0; j < p.k; ++j) {
+            float bv;
+            int bi;
+            pick(bv, bi);
+            if (!(bv > -INFINITY)) break;                           // fewer than k landmarks in this segment (wave-uniform)
+            bi += seg;
+            const bool better = lane < p.k && (rv > bv || (rv == bv && rx < bi));   // a prefix of the sorted list
+            const int pos = __popcll(__ballot(better));
+            if (pos >= p.k) break;                                  // worse than the k kept: so are the rest
+            const float up_v = __shfl_up(rv, 1, 64);
+            const int up_i = __shfl_up(rx, 1, 64);
+            if (lane > pos) {
+              rv = up_v;
+              rx = up_i;
+            } else if (lane == pos) {
+              rv = bv;
+              rx = bi;
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
+            if (i == ri) {
+              run_v[i] = rv;
+              run_i[i] = rx;
+            }
         }
-        int rank = 0;
-        for (int j = 0; j < p.k; ++j) {
-          const int o = __shfl(mine, j, 64);
-          rank += (o < mine) ? 1 : 0;
+      };
+      if (!flushed) {                                               // the usual case: few contenders, still in the list
+        float cv = -INFINITY;
+        int ci = 0x7fffffff;
+        if (lane < count) {
+          ci = cnd[lane];
+          cv = srow[ci];
         }
-        if (lane < p.k) p.idx[((int64_t)bh * p.T + t) * p.k + rank] = (int64_t)mine;
-        __builtin_amdgcn_wave_barrier();                          // the next row reuses the q row and the list
-        continue;
+        consume([&](float& bv, int& bi) { take_one(cv, ci, bv, bi); });
+      } else {                                                      // exact scores picked up from the row, 16 per lane
+        float x[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) x[j] = (j < nj && ((is_c >> j) & 1)) ? srow[64 * j + lane] : -INFINITY;
+        consume([&](float& bv, int& bi) { take_best(x, bv, bi); });
       }
-      // the segment's k best exact scores, best first, each inserted into the row's running list
-      float rv = -INFINITY;
-      int rx = 0x7fffffff;
-#pragma unroll
-      for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
-        if (i == ri) {
-          rv = run_v[i];
-          rx = run_i[i];
-        }
-      for (int j = 0; j < p.k; ++j) {
-        float bv;
-        int bi;
-        take_best(x, bv, bi);
-        if (!(bv > -INFINITY)) break;                               // fewer than k landmarks in this segment (wave-uniform)
-        bi += seg;
-        const bool better = lane < p.k && (rv > bv || (rv == bv && rx < bi));   // a prefix of the sorted list
-        const int pos = __popcll(__ballot(better));
-        if (pos >= p.k) break;                                      // worse than the k kept: so are the rest
-        const float up_v = __shfl_up(rv, 1, 64);
-        const int up_i = __shfl_up(rx, 1, 64);
-        if (lane > pos) {
-          rv = up_v;
-          rx = up_i;
-        } else if (lane == pos) {
-          rv = bv;
-          rx = bi;
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
-        if (i == ri) {
-          run_v[i] = rv;
-          run_i[i] = rx;
-        }
       __builtin_amdgcn_wave_barrier();                              // the next row reuses the q row and the list
     }
     __syncthreads();                                                // the next segment overwrites the score tile
