@@ -332,8 +332,8 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
   extern __shared__ __align__(16) unsigned char smem[];
   const int NMall = p.num_mems;
   const int seg_cap = NMall < kFusedMaxMems ? NMall : kFusedMaxMems;
-  const int NMp = ((seg_cap + 63) & ~63) + 32;                    // row stride (words): the two half-waves of a store
-                                                                  // then hit different banks
+  const int NMp = ((seg_cap + 63) & ~63) + 8;                     // row stride (words): the two half-waves of a store
+                                                                  // (rows 4 apart) then hit different banks
   float* sc = (float*)smem;                                       // [32][NMp]
   float* q_lds = sc + kFusedRows * NMp;                           // [waves][D]
   int* cand = (int*)(q_lds + kFusedWaves * D);                    // [waves][kFusedList]
@@ -841,8 +841,8 @@ static int launch_topk_t(const RetrParams& p, hipStream_t stream) {
   if ((rc = (int)hipGetLastError())) return rc;
   const int seg_cap = p.num_mems < kFusedMaxMems ? p.num_mems : kFusedMaxMems;
   const int NMr = (seg_cap + 63) & ~63;
-  const int lds = (kFusedRows * (NMr + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
-  constexpr int lds_max = (kFusedRows * (kFusedMaxMems + 32) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
+  const int lds = (kFusedRows * (NMr + 8) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
+  constexpr int lds_max = (kFusedRows * (kFusedMaxMems + 8) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
   const int n_rt = (p.T + kFusedRows - 1) / kFusedRows;
   const dim3 grid(p.B * p.H * n_rt), block(64 * kFusedWaves);
   if (p.num_mems <= kFusedMaxMems) {
