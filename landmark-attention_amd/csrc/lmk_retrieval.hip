@@ -270,12 +270,23 @@ __global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
   for (int m = lane; m < NM; m += 64) atomicMax(agg + m, prob_bits<T>(__fdiv_rn(sc[m], sum)));
 }
 
-// One wave per (batch, head): the k best blocks of agg under (value desc, index asc), ascending.
-__global__ __launch_bounds__(64) void lmk_block_select_kernel(RetrParams p) {
-  const int lane = threadIdx.x, bh = blockIdx.x, NM = p.num_mems;
+// One workgroup per (batch, head): the k best blocks of agg under (value desc, index asc), ascending.
+// Four waves bring the head's vector into LDS (and write the copy the caller may have asked for); the
+// first wave then picks k times over it.  Vectors too long for the LDS buffer are read in place.
+constexpr int kSelectLds = 8192;                                  // words of the LDS copy
+
+__global__ __launch_bounds__(256) void lmk_block_select_kernel(RetrParams p) {
+  __shared__ uint32_t cached[kSelectLds];
+  const int tid = threadIdx.x, lane = tid & 63, bh = blockIdx.x, NM = p.num_mems;
   const uint32_t* agg = p.agg + (int64_t)bh * NM;
-  if (p.agg_out != nullptr)                                       // the head's vector itself, in the model dtype
-    for (int m = lane; m < NM; m += 64) p.agg_out[(int64_t)bh * NM + m] = (uint16_t)agg[m];
+  const bool in_lds = NM <= kSelectLds;                           // uniform
+  for (int m = tid; m < NM; m += 256) {
+    const uint32_t v = agg[m];
+    if (in_lds) cached[m] = v;
+    if (p.agg_out != nullptr) p.agg_out[(int64_t)bh * NM + m] = (uint16_t)v;   // the head's vector itself, in the model dtype
+  }
+  __syncthreads();
+  if (tid >= 64) return;
   int mine = -1;
   float pv = INFINITY;
   int pi = -1;
@@ -283,7 +294,7 @@ __global__ __launch_bounds__(64) void lmk_block_select_kernel(RetrParams p) {
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     for (int m = lane; m < NM; m += 64) {
-      const float x = (float)agg[m];                              // 16-bit patterns: exact, order-preserving
+      const float x = (float)(in_lds ? cached[m] : agg[m]);       // 16-bit patterns: exact, order-preserving
       const bool after = (x < pv) || (x == pv && m > pi);
       if (after && (x > bv || (x == bv && m < bi))) {
         bv = x;
@@ -870,7 +881,7 @@ static int launch_topk_shared_t(const RetrParams& p, hipStream_t stream) {
   if ((rc = (int)hipGetLastError())) return rc;
   hipLaunchKernelGGL((lmk_block_prob_kernel<T, D>), dim3((unsigned)(p.B * p.H * ((p.T + 3) / 4))), dim3(256), 0, stream, p);
   if ((rc = (int)hipGetLastError())) return rc;
-  hipLaunchKernelGGL(lmk_block_select_kernel, dim3(p.B * p.H), dim3(64), 0, stream, p);
+  hipLaunchKernelGGL(lmk_block_select_kernel, dim3(p.B * p.H), dim3(256), 0, stream, p);
   return (int)hipGetLastError();
 }
 
