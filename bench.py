@@ -164,7 +164,7 @@ def other_shape(spec, n=30, warm=5):
     Prints one JSON line of its own; the headline line is not produced."""
     import torch
     from landmark_hip import _lib
-    from landmark_hip.attention import _launch_bwd, _launch_fwd
+    from landmark_hip.attention import _launch_fwd
     parts = spec.split(",")
     B, H, L, D, block = (int(x) for x in parts[:5])
     dtype = torch.float16 if parts[5:] == ["f16"] else torch.bfloat16
@@ -222,7 +222,7 @@ def main():
                  "would only shard heads with no exchange step. Run with --gpus 1.")
     import torch
     from landmark_hip import _lib
-    from landmark_hip.attention import FusedLandmarkAttention, _launch_bwd, _launch_fwd
+    from landmark_hip.attention import FusedLandmarkAttention, _launch_fwd
     _lib.lib()
     assert torch.cuda.is_available(), "bench.py needs the GPU; there is no CPU path"
     if a.shape:

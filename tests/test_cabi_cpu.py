@@ -1,6 +1,5 @@
 """CPU-side checks of the C ABI: the shared library loads without a GPU, exports every
 symbol include/lmk.h declares, and rejects bad arguments on the host before any launch."""
-import ctypes
 import os
 import re
 
