@@ -132,11 +132,11 @@ __device__ __forceinline__ u32x2_t lds_read_tr(const unsigned char* p) {
 // every address with a vector instruction.
 typedef __attribute__((address_space(3))) u32x4_t* lds_u32x4_ptr;
 typedef __attribute__((address_space(3))) float* lds_f32_ptr;
-__device__ __forceinline__ u32x4_t lds_ld128(int addr) { return *(lds_u32x4_ptr)(uint32_t)addr; }
-__device__ __forceinline__ void lds_st128(int addr, u32x4_t v) { *(lds_u32x4_ptr)(uint32_t)addr = v; }
-__device__ __forceinline__ void lds_st32(int addr, float v) { *(lds_f32_ptr)(uint32_t)addr = v; }
+__device__ __forceinline__ u32x4_t lds_ld128(int addr) { return *(lds_u32x4_ptr)(uintptr_t)(uint32_t)addr; }
+__device__ __forceinline__ void lds_st128(int addr, u32x4_t v) { *(lds_u32x4_ptr)(uintptr_t)(uint32_t)addr = v; }
+__device__ __forceinline__ void lds_st32(int addr, float v) { *(lds_f32_ptr)(uintptr_t)(uint32_t)addr = v; }
 __device__ __forceinline__ u32x2_t lds_ld_tr(int addr) {
-  s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(uint32_t)addr);
+  s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(uintptr_t)(uint32_t)addr);
   return __builtin_bit_cast(u32x2_t, v);
 }
 
