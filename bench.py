@@ -112,9 +112,16 @@ def decode_bench(n=50, warm=5):
     idx = retrieve_topk(q, kc, cos, sin, block, top_k)
     t_topk = _time_launches(lambda: retrieve_topk(q, kc, cos, sin, block, top_k), n, warm)
     t_att = _time_launches(lambda: gather_attend(q, kc, vc, idx, kl, vl, cos, sin, block, top_k), n, warm)
-    # the same step (selection + attend, six launches) recorded once into a HIP graph and replayed
+    # between two landmarks the rotated landmark keys of the previous step are still valid (what
+    # LandmarkKVCache.step does): the selection without that launch
+    from landmark_hip import _lib
+    ws = torch.empty(_lib.lib().lmk_retrieve_workspace_bytes(B, H, T, S, D, block), device=dev, dtype=torch.uint8)
+    retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws)
+    t_reuse = _time_launches(lambda: retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws,
+                                                   reuse_landmark_keys=True), n, warm)
+    # the same step (selection with reused keys + attend, five launches) recorded once into a HIP graph and replayed
     def step():
-        i = retrieve_topk(q, kc, cos, sin, block, top_k)
+        i = retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws, reuse_landmark_keys=True)
         return gather_attend(q, kc, vc, i, kl, vl, cos, sin, block, top_k)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -127,7 +134,8 @@ def decode_bench(n=50, warm=5):
         step()
     t_graph = _time_launches(graph.replay, n, warm)
     return {"workload": "decode: 1 new token, H32 D128, cache 32775 tok (1024 blocks of 32 + tail of 7), top-4",
-            "topk_ms": t_topk, "gather_attend_ms": t_att, "step_from_hip_graph_ms": t_graph}
+            "topk_ms": t_topk, "topk_reusing_landmark_keys_ms": t_reuse, "gather_attend_ms": t_att,
+            "step_from_hip_graph_ms": t_graph}
 
 
 def side_legs(n=30, warm=5):

@@ -125,6 +125,18 @@ int lmk_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kcache, const voi
                       size_t workspace_bytes, int B, int H, int T, int S, int D, int block, int top_k, int dtype,
                       void* stream);
 
+/* Same as lmk_retrieve_topk when `workspace` still holds the rotated landmark keys a previous
+ * lmk_retrieve_topk or lmk_retrieve_topk_reuse call left there for the same B, H, D, block, top_k, tables and
+ * S/block, and the complete blocks of the cache have not changed since: the rotation of the landmark keys
+ * (llama_mem.py:357-366) is skipped.  That is every decode step between two landmarks -- the positions
+ * of :359-365 move only when a block completes -- when the cache is appended to in place.  T may differ from
+ * call to call (the keys sit at the front of the workspace); workspace_bytes is checked for this call's T.
+ * No counterpart in the reference, which rotates every cached landmark key on every call. */
+int lmk_retrieve_topk_reuse(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
+                            const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                            void* workspace, size_t workspace_bytes, int B, int H, int T, int S, int D, int block,
+                            int top_k, int dtype, void* stream);
+
 /* Gather of the selected K/V blocks with rotary at their slot positions and attention over
  * them (llama_mem.py:386-412), merged with the attention over the local chunk (:447-477).
  *   o_loc, L_loc, M_loc: output and statistics of lmk_attn_fwd run on the local chunk;

@@ -228,10 +228,10 @@ size_t lmk_retrieve_workspace_bytes(int B, int H, int T, int S, int D, int block
   return retr_layout(B, H, T, S, D, block).total;
 }
 
-int lmk_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table, const void* sin_table,
-                      int64_t table_stride_row, int64_t n_pos, int64_t* idx_out, void* workspace,
-                      size_t workspace_bytes, int B, int H, int T, int S, int D, int block, int top_k, int dtype,
-                      void* stream) {
+static int retrieve_topk_impl(bool reuse_landmark_keys, const lmk_tensor4* q, const lmk_tensor4* kcache,
+                              const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
+                              int64_t* idx_out, void* workspace, size_t workspace_bytes, int B, int H, int T, int S,
+                              int D, int block, int top_k, int dtype, void* stream) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(kcache))) return rc;
   if (cos_table == nullptr || sin_table == nullptr || idx_out == nullptr || workspace == nullptr) return LMK_ERR_NULL;
@@ -251,7 +251,23 @@ int lmk_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kcache, const voi
   p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
   p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
   p.cs_r = table_stride_row;
-  return lmk::launch_retrieve_topk(p, D, dtype, (hipStream_t)stream);
+  return lmk::launch_retrieve_topk(p, D, dtype, reuse_landmark_keys, (hipStream_t)stream);
+}
+
+int lmk_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table, const void* sin_table,
+                      int64_t table_stride_row, int64_t n_pos, int64_t* idx_out, void* workspace,
+                      size_t workspace_bytes, int B, int H, int T, int S, int D, int block, int top_k, int dtype,
+                      void* stream) {
+  return retrieve_topk_impl(false, q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, workspace,
+                            workspace_bytes, B, H, T, S, D, block, top_k, dtype, stream);
+}
+
+int lmk_retrieve_topk_reuse(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
+                            const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                            void* workspace, size_t workspace_bytes, int B, int H, int T, int S, int D, int block,
+                            int top_k, int dtype, void* stream) {
+  return retrieve_topk_impl(true, q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, workspace,
+                            workspace_bytes, B, H, T, S, D, block, top_k, dtype, stream);
 }
 
 int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,

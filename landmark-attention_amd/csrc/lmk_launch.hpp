@@ -104,7 +104,7 @@ struct RotaryParams {
 };
 
 int launch_rotary(const RotaryParams& p, int D, int dtype, hipStream_t stream);
-int launch_retrieve_topk(const RetrParams& p, int D, int dtype, hipStream_t stream);
+int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landmark_keys, hipStream_t stream);
 int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream_t stream);   // one selection per head
 int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t stream);
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream);

@@ -844,12 +844,14 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
 // launchers
 // ---------------------------------------------------------------------------
 template <class T, int D>
-static int launch_topk_t(const RetrParams& p, hipStream_t stream) {
+static int launch_topk_t(const RetrParams& p, bool reuse_landmark_keys, hipStream_t stream) {
   constexpr int RPW = 256 / (D / 8);
   const int64_t lkrows = (int64_t)p.B * p.H * p.num_mems;
-  hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
   int rc;
-  if ((rc = (int)hipGetLastError())) return rc;
+  if (!reuse_landmark_keys) {
+    hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
+    if ((rc = (int)hipGetLastError())) return rc;
+  }
   const int seg_cap = p.num_mems < kFusedMaxMems ? p.num_mems : kFusedMaxMems;
   const int NMr = (seg_cap + 63) & ~63;
   const int lds = (kFusedRows * (NMr + 8) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
@@ -896,13 +898,13 @@ int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream
   return LMK_ERR_UNSUPPORTED;
 }
 
-int launch_retrieve_topk(const RetrParams& p, int D, int dtype, hipStream_t stream) {
+int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landmark_keys, hipStream_t stream) {
   if (dtype == LMK_DTYPE_BF16) {
-    if (D == 128) return launch_topk_t<bf16_t, 128>(p, stream);
-    if (D == 64) return launch_topk_t<bf16_t, 64>(p, stream);
+    if (D == 128) return launch_topk_t<bf16_t, 128>(p, reuse_landmark_keys, stream);
+    if (D == 64) return launch_topk_t<bf16_t, 64>(p, reuse_landmark_keys, stream);
   } else if (dtype == LMK_DTYPE_F16) {
-    if (D == 128) return launch_topk_t<f16_t, 128>(p, stream);
-    if (D == 64) return launch_topk_t<f16_t, 64>(p, stream);
+    if (D == 128) return launch_topk_t<f16_t, 128>(p, reuse_landmark_keys, stream);
+    if (D == 64) return launch_topk_t<f16_t, 64>(p, reuse_landmark_keys, stream);
   }
   return LMK_ERR_UNSUPPORTED;
 }

@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import torch
 
+from . import _lib
 from .retrieval import retrieve_and_attend
 
 
@@ -22,6 +23,8 @@ class LandmarkKVCache:
         self._k = torch.empty((batch, heads, capacity, head_dim), dtype=dtype, device=device)
         self._v = torch.empty_like(self._k)
         self.length = 0
+        self._ws = None                     # retrieval workspace, kept between steps
+        self._ws_key = None                 # what the rotated landmark keys in it were made for
 
     @property
     def capacity(self) -> int:
@@ -55,8 +58,22 @@ class LandmarkKVCache:
              sm_scale=None, aggregate=None):
         """Attention of a new chunk against the cache, then the append (``llama_mem.py:318-430,447-477``):
         ``query_states`` and ``key_states`` rotated at the chunk's positions, ``key_states_before_pos`` the
-        same keys without rotary.  Needs at least one complete cached block; returns ``(out, idx)``."""
+        same keys without rotary.  Needs at least one complete cached block; returns ``(out, idx)``.
+
+        The landmark keys are rotated at positions that move only when a cached block completes
+        (``:359-365``), and appends never touch complete blocks, so between two landmarks the rotated keys of
+        the previous step are reused (per-token selection; same tables, block and top_k)."""
+        B, H, T, D = query_states.shape
+        nbytes = _lib.lib().lmk_retrieve_workspace_bytes(B, H, T, self.length, D, int(block))
+        if self._ws is None or self._ws.numel() < nbytes or self._ws.device != query_states.device:
+            self._ws = torch.empty(max(nbytes, 2 * (self._ws.numel() if self._ws is not None else 0)),
+                                   device=query_states.device, dtype=torch.uint8)
+            self._ws_key = None
+        key = (self.length // block, int(block), int(top_k), cos.data_ptr(), sin.data_ptr(), self._k.data_ptr())
+        reuse = aggregate is None and key == self._ws_key
         out, idx = retrieve_and_attend(query_states, self.past_key_value, key_states, value_states, cos, sin,
-                                       block, top_k, sm_scale, aggregate)
+                                       block, top_k, sm_scale, aggregate, workspace=self._ws,
+                                       reuse_landmark_keys=reuse)
+        self._ws_key = key if aggregate is None else None
         self.append(key_states_before_pos, value_states)
         return out, idx

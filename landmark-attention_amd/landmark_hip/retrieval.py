@@ -34,7 +34,8 @@ def _tables(cos, sin, dtype):
     return cos, sin
 
 
-def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, return_block_probs=False):
+def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, return_block_probs=False,
+                  workspace=None, reuse_landmark_keys=False):
     """Indices ``(B, nh, T, k)`` int64, ascending, of the ``k = min(top_k, S // block)`` cached
     blocks whose landmark keys score highest against each query (``llama_mem.py:344-384``).
 
@@ -44,7 +45,13 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, 
     ``aggregate="max_over_tokens"`` (``:373-377``): one set per head, ``(B, nh, 1, k)`` -- the
     scores go through an fp32 softmax over the blocks, are rounded to the model dtype and reduced
     with a maximum over the queries before the top-k; ``return_block_probs`` also returns that
-    per-head vector ``(B, nh, 1, S // block)`` (``mem_attn_weights`` after ``:377``)."""
+    per-head vector ``(B, nh, 1, S // block)`` (``mem_attn_weights`` after ``:377``).
+
+    ``workspace``: a uint8 device tensor to use instead of a fresh allocation (at least
+    ``lmk_retrieve_workspace_bytes`` long).  ``reuse_landmark_keys``: the workspace still holds the
+    rotated landmark keys of the previous call and neither the complete cached blocks nor their
+    number have changed -- the case of every decode step between two landmarks -- so they are not
+    rotated again (per-token selection only)."""
     if aggregate not in (None, "max_over_tokens"):
         raise NotImplementedError(aggregate)                            # llama_mem.py:381-382
     assert aggregate or not return_block_probs, "the per-head vector exists only with aggregate='max_over_tokens'"
@@ -58,8 +65,13 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, 
     idx = torch.empty((B, H, 1 if aggregate else T, k), device=q.device, dtype=torch.int64)
     nbytes = lib.lmk_retrieve_workspace_bytes(B, H, T, S, D, int(block))
     probs = None
+    assert not (reuse_landmark_keys and (aggregate or workspace is None))
     with torch.cuda.device(q.device):
-        ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+        if workspace is None:
+            ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+        else:
+            ws = workspace
+            assert ws.dtype == torch.uint8 and ws.is_contiguous() and ws.numel() >= nbytes and ws.device == q.device
         tail = (ws.data_ptr(), nbytes, B, H, T, S, D, int(block), int(top_k), _lib.DTYPE_CODES[q.dtype],
                 _lib.current_stream(q.device))
         head = (_lib.tensor4(q), _lib.tensor4(k_cache), cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0],
@@ -68,6 +80,8 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, 
             if return_block_probs:
                 probs = torch.empty((B, H, 1, S // block), device=q.device, dtype=q.dtype)
             rc = lib.lmk_retrieve_topk_shared(*head, probs.data_ptr() if return_block_probs else None, *tail)
+        elif reuse_landmark_keys:
+            rc = lib.lmk_retrieve_topk_reuse(*head, *tail)
         else:
             rc = lib.lmk_retrieve_topk(*head, *tail)
     _lib.check(rc)
@@ -140,7 +154,7 @@ def attend_shared(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, 
 
 
 def retrieve_and_attend(q, past_key_value, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None,
-                        aggregate=None):
+                        aggregate=None, workspace=None, reuse_landmark_keys=False):
     """One inference step of the mem-cache path: returns ``(out, idx)``.
 
     ``past_key_value = (K_without_rotary, V)``; ``k_loc`` rotated, ``v_loc``: the new chunk.
@@ -148,7 +162,8 @@ def retrieve_and_attend(q, past_key_value, k_loc, v_loc, cos, sin, block: int, t
     ``"max_over_tokens"`` once per head.  The caller appends the un-rotated new keys and values to
     the cache afterwards (``:424-430``)."""
     k_cache, v_cache = past_key_value[0], past_key_value[1]
-    idx = retrieve_topk(q, k_cache, cos, sin, block, top_k, aggregate)
+    idx = retrieve_topk(q, k_cache, cos, sin, block, top_k, aggregate, workspace=workspace,
+                        reuse_landmark_keys=reuse_landmark_keys)
     if aggregate:
         out = attend_shared(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
     else:

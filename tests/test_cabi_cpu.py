@@ -29,7 +29,8 @@ def _declared():
 def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
-            "lmk_retrieve_topk_shared", "lmk_gather_window", "lmk_apply_rotary", "lmk_strerror"} <= set(names)
+            "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary",
+            "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
 
@@ -97,6 +98,8 @@ def test_retrieval_argument_errors(lib):
         return lib.lmk_retrieve_topk(t, t, cos, 0x6000, 128, n_pos, 0x7000, ws, wsb, 1, 1, 8, S, D, block, top_k, 0, None)
 
     assert topk(cos=0) == -1
+    assert lib.lmk_retrieve_topk_reuse(t, t, 0x5000, 0x6000, 128, 4096, 0x7000, 0x4000, 64, 1, 1, 8, 64, 128, 32, 4, 0,
+                                       None) == -8      # the workspace is still checked for this call's size
     assert topk(S=16) == -9                                   # less than one complete block
     assert topk(top_k=0) == -10 and topk(top_k=65) == -10
     assert topk(n_pos=32) == -11

@@ -242,6 +242,25 @@ def test_gather_window_rows_bit_exact(dtype):
     assert torch.equal(qw.cpu()[:, :, inc:], q) and (qw.cpu()[:, :, :inc] == 0).all()
 
 
+def test_reusing_rotated_landmark_keys_between_landmarks():
+    # decode steps between two landmarks: the number of complete blocks, hence every landmark position, stays
+    # put, and the second call may skip the rotation (other queries, another T, a longer tail)
+    from landmark_hip import _lib
+    from landmark_hip.retrieval import retrieve_topk
+    B, H, D, block, top_k = 1, 3, 128, 32, 4
+    S = 50 * block + 3
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, 5, S + 8, D, seed=91)
+    dev = lambda t: t.cuda()
+    kcd, cd, sd = dev(kc), dev(cos), dev(sin)
+    ws = torch.empty(_lib.lib().lmk_retrieve_workspace_bytes(B, H, 5, S + 8, D, block), device="cuda:0", dtype=torch.uint8)
+    first = retrieve_topk(dev(q), kcd[:, :, :S], cd, sd, block, top_k, workspace=ws)
+    assert torch.equal(first.cpu(), oret.select_topk(oret.landmark_scores(q, kc[:, :, :S], cos, sin, block, top_k), top_k))
+    q2 = q[:, :, :2] * 1.5
+    again = retrieve_topk(dev(q2), kcd[:, :, : S + 8], cd, sd, block, top_k, workspace=ws, reuse_landmark_keys=True)
+    want = oret.select_topk(oret.landmark_scores(q2, kc[:, :, : S + 8], cos, sin, block, top_k), top_k)
+    assert torch.equal(again.cpu(), want)
+
+
 @pytest.mark.parametrize("seed", [0, 1, 2])
 def test_baseline_config4_full_size(seed):
     # benchmark config 4: H32 D128, 32768 cached tokens = 1024 blocks of 32, 256 queries, top-4
