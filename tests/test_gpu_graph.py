@@ -22,7 +22,8 @@ def _capture(fn):
     return g, res
 
 
-def test_decode_step_replays_from_a_graph():
+@pytest.mark.parametrize("aggregate", [None, "max_over_tokens"])
+def test_decode_step_replays_from_a_graph(aggregate):
     from landmark_hip.retrieval import retrieve_and_attend
     B, H, D, block, top_k, T = 1, 4, 128, 32, 4, 1
     S = 40 * block + 9                                           # cache with an incomplete block
@@ -30,7 +31,7 @@ def test_decode_step_replays_from_a_graph():
     mk = lambda *s: (torch.randn(*s, generator=gen) * 0.5).bfloat16().cuda()
     q, kc, vc, kl, vl = mk(B, H, T, D), mk(B, H, S, D), mk(B, H, S, D), mk(B, H, T, D), mk(B, H, T, D)
     cos, sin = (t.cuda() for t in orot.rotary_tables(S + T, D, torch.bfloat16))
-    step = lambda: retrieve_and_attend(q, (kc, vc), kl, vl, cos, sin, block, top_k)
+    step = lambda: retrieve_and_attend(q, (kc, vc), kl, vl, cos, sin, block, top_k, aggregate=aggregate)
     out_e, idx_e = step()
     torch.cuda.synchronize()
     out_e, idx_e = out_e.clone(), idx_e.clone()
@@ -44,7 +45,7 @@ def test_decode_step_replays_from_a_graph():
         step()                                                   # eager work between the replays
     # new inputs in the captured buffers: the replay follows them
     q2 = mk(B, H, T, D)
-    out2, idx2 = retrieve_and_attend(q2, (kc, vc), kl, vl, cos, sin, block, top_k)
+    out2, idx2 = retrieve_and_attend(q2, (kc, vc), kl, vl, cos, sin, block, top_k, aggregate=aggregate)
     torch.cuda.synchronize()
     out2, idx2 = out2.clone(), idx2.clone()
     q.copy_(q2)
