@@ -667,7 +667,7 @@ __device__ __forceinline__ float sum8(float d) {                  // sum over th
 // (scores of the whole block, which the block's softmax needs before any weight is final), then the
 // values, so keys and values are never live together and the kernel keeps several waves per SIMD.  The
 // loads of the next chunk are issued before the arithmetic on the current one.
-template <class T, int D, int BS>
+template <class T, int D, int BS, bool SPLIT>
 __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   static_assert(D == 128 && (BS == 32 || BS % 64 == 0), "16 chunks of 8 head dims per row; whole chunks of keys");
   constexpr int CK = BS < 64 ? BS : 64;                           // keys per chunk
@@ -675,8 +675,11 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   constexpr int NC = BS / CK;                                     // chunks per block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int j = lane & 7, g = lane >> 3;                           // head-dim chunk pair, key group
-  const int64_t row = (int64_t)blockIdx.x * 4 + wave;             // (bh, t)
-  if (row >= (int64_t)p.B * p.H * p.T) return;
+  // (bh, t): a wave's own row, or -- SPLIT, for launches with few rows -- the workgroup's row, whose
+  // selected blocks the four waves share out (block js goes to wave js % 4) and merge at the end
+  const int64_t row = SPLIT ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
+  if (row >= (int64_t)p.B * p.H * p.T) return;                    // SPLIT: the whole workgroup leaves
+  const int js0 = SPLIT ? wave : 0, jstep = SPLIT ? 4 : 1;
   const int bh = (int)(row / p.T), t = (int)(row % p.T);
   const int b = bh / p.H, hh = bh % p.H;
 
@@ -722,9 +725,12 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       chi[i] = nhi[i];
     }
   };
-  int blk = (int)p.idx[row * p.k];
-  fetch(kc, p.kcs_r, (int64_t)blk * BS);
-  for (int js = 0; js < p.k; ++js) {
+  int blk = 0;
+  if (js0 < p.k) {
+    blk = (int)p.idx[row * p.k + js0];
+    fetch(kc, p.kcs_r, (int64_t)blk * BS);
+  }
+  for (int js = js0; js < p.k; js += jstep) {
     const int64_t key0 = (int64_t)blk * BS;
     const int64_t pos0 = (int64_t)js * BS + ((blk >= p.num_mems - p.k) ? BS : 0) + p.prefix_len;
     float sc[KPG * NC];
@@ -788,12 +794,12 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       ahi[e] *= alpha;
     }
     int blk_next = blk;
-    if (js + 1 < p.k) blk_next = (int)p.idx[row * p.k + js + 1];
+    if (js + jstep < p.k) blk_next = (int)p.idx[row * p.k + js + jstep];
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       take();
       if (c + 1 < NC) fetch(vc, p.vcs_r, key0 + CK * (c + 1));
-      else if (js + 1 < p.k) fetch(kc, p.kcs_r, (int64_t)blk_next * BS);
+      else if (js + jstep < p.k) fetch(kc, p.kcs_r, (int64_t)blk_next * BS);
 #pragma unroll
       for (int i = 0; i < KPG; ++i) {
         const float w = round_to<T>(sc[KPG * c + i] * f);         // weights enter PV in the model dtype
@@ -816,6 +822,43 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     ahi[e] += __shfl_xor(ahi[e], 16, 64);
     alo[e] += __shfl_xor(alo[e], 32, 64);
     ahi[e] += __shfl_xor(ahi[e], 32, 64);
+  }
+  if constexpr (SPLIT) {                                          // the four waves' partial (M, l, acc) -> wave 0
+    __shared__ float part_acc[4][128];
+    __shared__ float part_ml[4][2];
+    if (g == 0) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        part_acc[wave][8 * j + e] = alo[e];
+        part_acc[wave][64 + 8 * j + e] = ahi[e];
+      }
+      if (j == 0) {
+        part_ml[wave][0] = Mrun;
+        part_ml[wave][1] = lrun;
+      }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float Mall = part_ml[0][0];                                   // wave 0 always has a block (k >= 1)
+#pragma unroll
+    for (int w = 1; w < 4; ++w) Mall = fmaxf(Mall, part_ml[w][0]);
+    lrun = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      alo[e] = 0.f;
+      ahi[e] = 0.f;
+    }
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float sw = fast_exp2(part_ml[w][0] - Mall);           // 0 for a wave without blocks (M = -inf)
+      lrun = __builtin_fmaf(part_ml[w][1], sw, lrun);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        alo[e] = __builtin_fmaf(part_acc[w][8 * j + e], sw, alo[e]);
+        ahi[e] = __builtin_fmaf(part_acc[w][64 + 8 * j + e], sw, ahi[e]);
+      }
+    }
+    Mrun = Mall;
   }
   // merge with the local chunk: out_loc (normalised), L_loc, M_loc (natural-log units)
   const int64_t srow = (int64_t)bh * p.stat_stride + t;
@@ -912,10 +955,18 @@ int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landm
 template <class T>
 static int launch_gather_t(const RetrParams& p, int BS, hipStream_t stream) {
   const int64_t rows = (int64_t)p.B * p.H * p.T;
+  if (rows <= 1024 && p.k > 1) {          // fewer rows than SIMDs: one workgroup per row, its waves share the blocks out
+    const dim3 grid((unsigned)rows);
+    if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 32, true>), grid, dim3(256), 0, stream, p);
+    else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 64, true>), grid, dim3(256), 0, stream, p);
+    else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 128, true>), grid, dim3(256), 0, stream, p);
+    else return LMK_ERR_UNSUPPORTED;
+    return (int)hipGetLastError();
+  }
   const dim3 grid((unsigned)((rows + 3) / 4));
-  if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 32>), grid, dim3(256), 0, stream, p);
-  else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 64>), grid, dim3(256), 0, stream, p);
-  else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 128>), grid, dim3(256), 0, stream, p);
+  if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 32, false>), grid, dim3(256), 0, stream, p);
+  else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 64, false>), grid, dim3(256), 0, stream, p);
+  else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 128, false>), grid, dim3(256), 0, stream, p);
   else return LMK_ERR_UNSUPPORTED;
   return (int)hipGetLastError();
 }
