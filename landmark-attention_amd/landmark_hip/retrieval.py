@@ -88,42 +88,54 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, 
     return (idx, probs) if return_block_probs else idx
 
 
+def _local_window_attention(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block, sm_scale):
+    """Attention of the new tokens over the local window alone (the new chunk, behind the tail of an
+    incomplete cached block if there is one, ``llama_mem.py:329-342``) with the fused forward kernel.
+    Returns ``(o_loc, (L_ptr, M_ptr), stat_stride, tensors)``: output view, addresses and row stride of
+    its statistics, and every tensor that must stay alive until the gather kernel has read them."""
+    B, H, T, D = q.shape
+    S = k_cache.shape[2]
+    inc = S % block
+    if inc == 0:
+        o_loc, L_loc, M_loc = _launch_fwd(q, k_loc, v_loc, 0, sm_scale, block)
+        return o_loc, (L_loc.data_ptr(), M_loc.data_ptr()), T, (o_loc, L_loc, M_loc)
+    assert T + inc <= block, "new chunk and cached tail must fit one block (llama_mem.py:330)"
+    q_win, k_win, v_win = (torch.empty((B, H, inc + T, D), device=q.device, dtype=q.dtype) for _ in range(3))
+    _lib.check(_lib.lib().lmk_local_window(
+        _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), _lib.tensor4(k_loc), _lib.tensor4(v_loc),
+        cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(q_win), _lib.tensor4(k_win),
+        _lib.tensor4(v_win), B, H, T, S, D, int(block), _lib.DTYPE_CODES[q.dtype],
+        _lib.current_stream(q.device)))
+    o_win, L_win, M_win = _launch_fwd(q_win, k_win, v_win, 0, sm_scale, block)
+    # the window's last T rows, read in place: a strided view, and first element + row stride of the statistics
+    return (o_win[:, :, inc:], (L_win.data_ptr() + 4 * inc, M_win.data_ptr() + 4 * inc), inc + T,
+            (q_win, k_win, v_win, o_win, L_win, M_win))
+
+
+def _gather(q, k_cache, v_cache, idx, cos, sin, block, top_k, sm_scale, local):
+    B, H, T, D = q.shape
+    o_loc, stat_ptrs, stat_stride, _ = local
+    out = torch.empty_like(q)
+    _lib.check(_lib.lib().lmk_gather_attend(
+        _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), idx.data_ptr(), cos.data_ptr(),
+        sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(o_loc), stat_ptrs[0], stat_ptrs[1], stat_stride,
+        _lib.tensor4(out), B, H, T, k_cache.shape[2], D, float(sm_scale), int(block), int(top_k),
+        _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device)))
+    return out
+
+
 def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
     """Attention output ``(B, nh, T, hd)`` over the blocks ``idx`` selects plus the local window
     (``llama_mem.py:386-412,447-477``).  The local window -- the new chunk, behind the tail of
     an incomplete cached block if there is one (``:329-342``) -- is attended with the fused
     forward kernel; the gather kernel reads the selected blocks in place and merges both parts."""
-    B, H, T, D = q.shape
-    S = k_cache.shape[2]
     if sm_scale is None:
-        sm_scale = 1.0 / math.sqrt(D)
+        sm_scale = 1.0 / math.sqrt(q.shape[-1])
     q, k_cache, v_cache, k_loc, v_loc = (_lib.kernel_ready(t) for t in (q, k_cache, v_cache, k_loc, v_loc))
     cos, sin = _tables(cos, sin, q.dtype)
-    inc = S % block
     with torch.cuda.device(q.device):
-        if inc == 0:
-            o_loc, L_loc, M_loc = _launch_fwd(q, k_loc, v_loc, 0, sm_scale, block)
-            stat_ptrs, stat_stride = (L_loc.data_ptr(), M_loc.data_ptr()), T
-        else:
-            assert T + inc <= block, "new chunk and cached tail must fit one block (llama_mem.py:330)"
-            q_win, k_win, v_win = (torch.empty((B, H, inc + T, D), device=q.device, dtype=q.dtype) for _ in range(3))
-            _lib.check(_lib.lib().lmk_local_window(
-                _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), _lib.tensor4(k_loc), _lib.tensor4(v_loc),
-                cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(q_win), _lib.tensor4(k_win),
-                _lib.tensor4(v_win), B, H, T, S, D, int(block), _lib.DTYPE_CODES[q.dtype],
-                _lib.current_stream(q.device)))
-            o_win, L_win, M_win = _launch_fwd(q_win, k_win, v_win, 0, sm_scale, block)
-            o_loc = o_win[:, :, inc:]                                   # a strided view: read in place
-            # statistics of the window's last T rows, read in place: first element and row stride
-            stat_ptrs, stat_stride = (L_win.data_ptr() + 4 * inc, M_win.data_ptr() + 4 * inc), inc + T
-        out = torch.empty_like(q)
-        rc = _lib.lib().lmk_gather_attend(
-            _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), idx.data_ptr(), cos.data_ptr(),
-            sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(o_loc), stat_ptrs[0], stat_ptrs[1], stat_stride,
-            _lib.tensor4(out), B, H, T, S, D, float(sm_scale), int(block), int(top_k), _lib.DTYPE_CODES[q.dtype],
-            _lib.current_stream(q.device))
-    _lib.check(rc)
-    return out
+        local = _local_window_attention(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block, sm_scale)
+        return _gather(q, k_cache, v_cache, idx, cos, sin, block, top_k, sm_scale, local)
 
 
 def attend_shared(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
@@ -162,10 +174,18 @@ def retrieve_and_attend(q, past_key_value, k_loc, v_loc, cos, sin, block: int, t
     ``"max_over_tokens"`` once per head.  The caller appends the un-rotated new keys and values to
     the cache afterwards (``:424-430``)."""
     k_cache, v_cache = past_key_value[0], past_key_value[1]
-    idx = retrieve_topk(q, k_cache, cos, sin, block, top_k, aggregate, workspace=workspace,
-                        reuse_landmark_keys=reuse_landmark_keys)
     if aggregate:
-        out = attend_shared(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
-    else:
-        out = gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
+        idx = retrieve_topk(q, k_cache, cos, sin, block, top_k, aggregate)
+        return attend_shared(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale), idx
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(q.shape[-1])
+    q, k_cache, v_cache, k_loc, v_loc = (_lib.kernel_ready(t) for t in (q, k_cache, v_cache, k_loc, v_loc))
+    cos, sin = _tables(cos, sin, q.dtype)
+    with torch.cuda.device(q.device):
+        # (Running the local-window attention on a second stream beside the selection was tried: the
+        # fork and join cost more than the 20 us it hides.)
+        idx = retrieve_topk(q, k_cache, cos, sin, block, top_k, workspace=workspace,
+                            reuse_landmark_keys=reuse_landmark_keys)
+        local = _local_window_attention(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block, sm_scale)
+        out = _gather(q, k_cache, v_cache, idx, cos, sin, block, top_k, sm_scale, local)
     return out, idx
