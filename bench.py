@@ -258,6 +258,17 @@ def main():
             step()
             dst.copy_(src)                  # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
+        # the config 4 retrieval step, three times as well
+        from landmark_hip.retrieval import retrieve_and_attend
+        Br, Hr, Tr, Sr, top_k = 1, 32, 256, 32768, 4
+        mk = lambda *s: (torch.randn(*s, generator=g) * 0.5).bfloat16().to(dev)
+        qr, kc, vc, kl, vl = mk(Br, Hr, Tr, D), mk(Br, Hr, Sr, D), mk(Br, Hr, Sr, D), mk(Br, Hr, Tr, D), mk(Br, Hr, Tr, D)
+        ang = torch.outer(torch.arange(Sr + Tr).float(), 1.0 / (10000 ** (torch.arange(0, D, 2).float() / D)))
+        ang = torch.cat((ang, ang), -1)
+        cos, sin = ang.cos().bfloat16().to(dev), ang.sin().bfloat16().to(dev)
+        for _ in range(3):
+            retrieve_and_attend(qr, (kc, vc), kl, vl, cos, sin, block, top_k)
+        torch.cuda.synchronize()
         return
 
     # The GPU leaves its idle power state only after some tens of milliseconds of work (a 25-step run reads

@@ -352,7 +352,10 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ql = lane & 31, h = lane >> 5;
   const int n_qt = (p.T + kFusedRows - 1) / kFusedRows;
-  const int bh = blockIdx.x / n_qt, t0 = (blockIdx.x % n_qt) * kFusedRows;
+  // Workgroups go to the eight XCDs in turn; the ones that read the same head's landmark keys are put on
+  // one XCD, so the keys come out of HBM once rather than once per L2.
+  const int wg = (gridDim.x & 7) ? (int)blockIdx.x : (int)((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3));
+  const int bh = wg / n_qt, t0 = (wg % n_qt) * kFusedRows;
   const int b = bh / p.H, hh = bh % p.H;
   const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h);
   const char* lk_all = (const char*)p.lk_rot + 2 * ((int64_t)bh * NMall * D);
