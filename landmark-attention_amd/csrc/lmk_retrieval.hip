@@ -647,6 +647,185 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
 }
 
 // ---------------------------------------------------------------------------
+// select without the bracket, for a handful of query rows (decoding).  The fused kernel gives a
+// workgroup 32 rows and a row one wave: with one row per head fifteen of its sixteen waves idle and
+// the row's steps run one behind the other on 32 CUs.  Here a row's cached blocks are split into
+// slices of 256 over as many workgroups (one wave per SIMD, one block per thread): every score is
+// evaluated as the contract defines it (the sequential dot product of `evaluate` above), a workgroup
+// leaves its slice's k best (score, index) in the workspace, and a second small kernel merges a row's
+// slices.  Costs a launch, spreads the work over the chip.
+// ---------------------------------------------------------------------------
+constexpr int kSliceWaves = 4;
+constexpr int kSliceMems = 64 * kSliceWaves;                      // cached blocks per workgroup
+constexpr int kSliceMaxRows = 1024;                               // rows (batch x head x query) up to which this path is used
+constexpr int kSliceMaxCand = 1024;                               // candidates (slices x k) the merge holds, 16 per lane
+constexpr int kSliceRowB = 80;                                    // bytes per staged quarter row: 64 + 16, conflict-free b128 reads
+
+template <class T, int D>
+__global__ __launch_bounds__(64 * kSliceWaves) void lmk_topk_slice_kernel(RetrParams p, int n_slices) {
+  constexpr int NQ = D / 32;                                      // a key row passes through LDS in quarters of 32 dims
+  __shared__ __align__(16) float q_lds[D];
+  __shared__ __align__(16) unsigned char stage_all[kSliceWaves * 64 * kSliceRowB];
+  __shared__ float list_v[kSliceWaves][64];
+  __shared__ int list_i[kSliceWaves][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int NM = p.num_mems;
+  const int64_t row = blockIdx.x / n_slices;                      // (batch, head, query)
+  const int slice = blockIdx.x % n_slices;
+  const int bh = (int)(row / p.T), t = (int)(row % p.T);
+  const int b = bh / p.H, hh = bh % p.H;
+  const char* qr = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
+  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * NM * D);
+  unsigned char* stage = stage_all + wave * 64 * kSliceRowB;
+  // The wave's 64 blocks (lane l scores block mw + l): the key rows come in with four lanes per row and
+  // quarter (64 contiguous bytes) and go through LDS to the lane that owns the row -- a lane reading its
+  // own 256-byte row would touch 64 cache lines per load instruction.
+  const int mw = slice * kSliceMems + 64 * wave;
+  u32x4_t ld[NQ][4];
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int mr = min(mw + 16 * i + (lane >> 2), NM - 1);        // rows past the end re-read the last one; their score is dropped
+      ld[qt][i] = *(const u32x4_t*)(lk + 2 * ((int64_t)mr * D) + 64 * qt + 16 * (lane & 3));
+    }
+  if (tid < D / 2) {
+    const uint32_t u = *(const uint32_t*)(qr + 4 * tid);
+    q_lds[2 * tid] = unpack_lo<T>(u);
+    q_lds[2 * tid + 1] = unpack_hi<T>(u);
+  }
+  __syncthreads();
+
+  float acc = 0.f;
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *(u32x4_t*)(stage + (16 * i + (lane >> 2)) * kSliceRowB + 16 * (lane & 3)) = ld[qt][i];
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    int q0 = 0;
+    asm volatile("" : "+v"(q0) : : "memory");                       // q is read from LDS quarter by quarter ...
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {                                   // the sequential dot product of the contract, d ascending
+      const u32x4_t kk = *(const u32x4_t*)(stage + lane * kSliceRowB + 16 * c);
+      const float4 qa = *(const float4*)&q_lds[q0 + 32 * qt + 8 * c];
+      const float4 qb = *(const float4*)&q_lds[q0 + 32 * qt + 8 * c + 4];
+      acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
+      acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
+      acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
+      acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
+      acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
+      acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
+      acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
+      acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
+    }
+    asm volatile("" : "+v"(acc));                                   // ... and its 32 fmas are done before the next one is read:
+                                                                    // left alone the compiler reads all of q and the keys first and spills
+    __builtin_amdgcn_wave_barrier();                                // the next quarter overwrites the rows
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+  }
+  const int m = mw + lane;
+  float cv = (m < NM) ? contract<T>(acc, p.sqrt_hd) : -INFINITY;
+  int ci = (m < NM) ? m : 0x7fffffff;
+  // lane j <- the j-th best of the wave's 64 scores
+  float rv = -INFINITY;
+  int rx = 0x7fffffff;
+  for (int j = 0; j < p.k; ++j) {
+    float bv = cv;
+    int bi = ci;
+    wave_best(bv, bi);
+    if (bi == ci) cv = -INFINITY;
+    if (lane == j) {
+      rv = bv;
+      rx = bi;
+    }
+  }
+  list_v[wave][lane] = rv;
+  list_i[wave][lane] = rx;
+  __syncthreads();
+  if (wave != 0) return;
+
+  // lane j holds the j-th entry of every wave's list; k picks over the lists, pick j -> candidate j of the slice
+  float x[kSliceWaves];
+  int xi[kSliceWaves];
+#pragma unroll
+  for (int w = 0; w < kSliceWaves; ++w) {
+    x[w] = list_v[w][lane];
+    xi[w] = list_i[w][lane];
+  }
+  float out_v = -INFINITY;
+  int out_i = 0x7fffffff;
+  for (int j = 0; j < p.k; ++j) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int w = 0; w < kSliceWaves; ++w)
+      if (x[w] > bv || (x[w] == bv && xi[w] < bi)) {
+        bv = x[w];
+        bi = xi[w];
+      }
+    const int own = bi;                                             // block indices are unique over the lists
+    wave_best(bv, bi);
+#pragma unroll
+    for (int w = 0; w < kSliceWaves; ++w)
+      if (own == bi && xi[w] == bi) x[w] = -INFINITY;
+    if (lane == j) {
+      out_v = bv;
+      out_i = bi;
+    }
+  }
+  if (lane < p.k) {
+    const int64_t at = row * NM + (int64_t)slice * p.k + lane;      // n_slices * k <= num_mems: a row of the score planes holds them
+    p.approx[at] = out_v;
+    ((int*)p.exact)[at] = out_i;
+  }
+}
+
+// One wave per query row: the k best of the row's n_slices * k candidates, written in ascending index order.
+__global__ __launch_bounds__(256) void lmk_topk_slice_merge_kernel(RetrParams p, int n_slices) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= (int64_t)p.B * p.H * p.T) return;                      // wave-uniform
+  const int n_cand = n_slices * p.k;
+  constexpr int NJ = kSliceMaxCand / 64;
+  float x[NJ];
+  int xi[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const int c = 64 * j + lane;
+    x[j] = -INFINITY;
+    xi[j] = 0x7fffffff;
+    if (c < n_cand) {
+      x[j] = p.approx[row * p.num_mems + c];
+      xi[j] = ((const int*)p.exact)[row * p.num_mems + c];
+    }
+  }
+  int mine = 0x7fffffff;
+  for (int j = 0; j < p.k; ++j) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int w = 0; w < NJ; ++w)
+      if (x[w] > bv || (x[w] == bv && xi[w] < bi)) {
+        bv = x[w];
+        bi = xi[w];
+      }
+    const int own = bi;
+    wave_best(bv, bi);
+#pragma unroll
+    for (int w = 0; w < NJ; ++w)
+      if (own == bi && xi[w] == bi) x[w] = -INFINITY;
+    if (lane == j) mine = bi;
+  }
+  int rank = 0;
+  for (int j = 0; j < p.k; ++j) {
+    const int o = __shfl(mine, j, 64);
+    rank += (o < mine) ? 1 : 0;
+  }
+  if (lane < p.k) p.idx[row * p.k + rank] = (int64_t)mine;
+}
+
+// ---------------------------------------------------------------------------
 // gather + attend over the selected blocks, merged with the local-chunk attention
 // ---------------------------------------------------------------------------
 template <int CTRL>
@@ -897,6 +1076,14 @@ static int launch_topk_t(const RetrParams& p, bool reuse_landmark_keys, hipStrea
   if (!reuse_landmark_keys) {
     hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
     if ((rc = (int)hipGetLastError())) return rc;
+  }
+  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  const int n_slices = (p.num_mems + kSliceMems - 1) / kSliceMems;
+  if (rows <= kSliceMaxRows && (int64_t)n_slices * p.k <= kSliceMaxCand) {   // a handful of rows: every score exact, slices over the chip
+    hipLaunchKernelGGL((lmk_topk_slice_kernel<T, D>), dim3((unsigned)(rows * n_slices)), dim3(64 * kSliceWaves), 0, stream, p, n_slices);
+    if ((rc = (int)hipGetLastError())) return rc;
+    hipLaunchKernelGGL(lmk_topk_slice_merge_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p, n_slices);
+    return (int)hipGetLastError();
   }
   const int seg_cap = p.num_mems < kFusedMaxMems ? p.num_mems : kFusedMaxMems;
   const int NMr = (seg_cap + 63) & ~63;

@@ -30,6 +30,14 @@ CASES = [
     (1, 2, 40, 2500 * 32, 128, 32, 5),     # more than 1024 cached blocks: three segments, the last one ragged
     (1, 1, 3, 2048 * 16, 128, 16, 64),     # two full segments, the longest list to merge
     (1, 2, 1, 3000 * 32, 64, 32, 4),       # one query against a long cache
+    (1, 2, 3, 1024 * 32, 128, 32, 64),     # few rows: four slices of 256 blocks, 256 candidates to merge
+    (1, 1, 5, 4100 * 16, 128, 16, 60),     # few rows, 17 slices x 60 > 1024 candidates: back on the fused kernel
+    # more than 1024 query rows (B * H * T): the fused score + select kernel
+    (1, 2, 530, 33 * 32, 128, 32, 1),
+    (2, 3, 200, 20 * 32, 128, 32, 5),
+    (1, 2, 520, 50 * 32, 64, 32, 4),
+    (1, 2, 520, 2500 * 32, 128, 32, 5),
+    (1, 1, 1030, 2048 * 16, 128, 16, 64),
 ]
 
 
@@ -46,10 +54,11 @@ def test_topk_indices_bit_exact(B, H, T, S, D, block, top_k):
     assert torch.equal(got.cpu(), want)
 
 
-def test_topk_with_massive_ties():
+@pytest.mark.parametrize("T", [8, 520])                             # few rows: sliced kernel; many: fused kernel
+def test_topk_with_massive_ties(T):
     # identical landmark keys in many blocks: every score ties, the lowest indices must win
     from landmark_hip.retrieval import retrieve_topk
-    B, H, T, S, D, block, top_k = 1, 2, 8, 2100 * 32, 128, 32, 4    # > 1024 landmarks: two list sweeps
+    B, H, S, D, block, top_k = 1, 2, 2100 * 32, 128, 32, 4          # > 1024 landmarks: two list sweeps / nine slices
     q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=3)
     kc[:, :, block - 1::block] = kc[:, :, block - 1:block]
     sc = oret.landmark_scores(q, kc, cos, sin, block, top_k)
@@ -58,12 +67,13 @@ def test_topk_with_massive_ties():
     assert torch.equal(got.cpu(), want)
 
 
+@pytest.mark.parametrize("T", [40, 520])                            # few rows: sliced kernel; many: fused kernel
 @pytest.mark.parametrize("n_mems,top_k", [(700, 4), (1024, 64), (130, 7)])
-def test_topk_ties_inside_one_workgroup(n_mems, top_k):
+def test_topk_ties_inside_one_workgroup(n_mems, top_k, T):
     # at most 1024 landmarks: scores stay on the CU; identical landmark keys make every block a
     # contender, so the contender list is flushed several times, and a large top_k runs many rounds
     from landmark_hip.retrieval import retrieve_topk
-    B, H, T, D, block = 1, 2, 40, 128, 32
+    B, H, D, block = 1, 2, 128, 32
     S = n_mems * block
     print(f"case ties n_mems{n_mems} k{top_k}", flush=True)
     q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=n_mems)
@@ -76,9 +86,10 @@ def test_topk_ties_inside_one_workgroup(n_mems, top_k):
     assert torch.equal(got.cpu(), want)
 
 
-def test_fp16_indices_bit_exact():
+@pytest.mark.parametrize("T", [24, 520])
+def test_fp16_indices_bit_exact(T):
     from landmark_hip.retrieval import retrieve_topk
-    B, H, T, S, D, block, top_k = 1, 2, 24, 48 * 32, 128, 32, 4
+    B, H, S, D, block, top_k = 1, 2, 48 * 32, 128, 32, 4
     q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=4, dtype=torch.float16)
     want = oret.select_topk(oret.landmark_scores(q, kc, cos, sin, block, top_k), top_k)
     got = retrieve_topk(q.cuda(), kc.cuda(), cos.cuda(), sin.cuda(), block, top_k)
