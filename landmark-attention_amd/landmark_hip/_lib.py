@@ -5,6 +5,7 @@ caller gets an exception, never a fallback.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 
@@ -85,17 +86,36 @@ def check(code: int) -> None:
 
 def tensor4(t: torch.Tensor) -> Tensor4:
     """Describe a (B, H, L, D) tensor with unit stride along D."""
-    assert t.dim() == 4 and t.stride(3) == 1
-    return Tensor4(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+    s = t.stride()
+    assert len(s) == 4 and s[3] == 1
+    return Tensor4(t.data_ptr(), s[0], s[1], s[2])
 
 
 def kernel_ready(t: torch.Tensor) -> torch.Tensor:
     """Return ``t`` itself when the kernels can read it in place (unit stride along D, rows walked
     forwards, 16-byte aligned base and strides), otherwise a contiguous copy."""
-    if (t.stride(3) == 1 and t.stride(2) > 0 and t.data_ptr() % 16 == 0 and all(t.stride(i) % 8 == 0 for i in range(3))):
+    s = t.stride()
+    if s[3] == 1 and s[2] > 0 and s[0] % 8 == 0 and s[1] % 8 == 0 and s[2] % 8 == 0 and t.data_ptr() % 16 == 0:
         return t
     return t.contiguous()
 
 
+_SAME_DEVICE = contextlib.nullcontext()
+
+
+def on_device(device):
+    """Context that makes ``device`` current for the launches inside; free when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device(device)
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # the handle without a Stream object around it
+
+
 def current_stream(device) -> int:
+    """hipStream_t of torch's current stream on ``device`` (a decode step asks several times per token)."""
+    if _raw_stream is not None:
+        index = device.index
+        return _raw_stream(torch.cuda.current_device() if index is None else index)
     return torch.cuda.current_stream(device).cuda_stream

@@ -66,7 +66,7 @@ class FusedLandmarkAttention(torch.autograd.Function):
         assert d in SUPPORTED_HEAD_DIMS, f"HIP kernels are built for head dims {SUPPORTED_HEAD_DIMS}"
         assert block_size in SUPPORTED_BLOCKS, f"HIP kernels are built for block sizes {SUPPORTED_BLOCKS}"
         q, k, v = _lib.kernel_ready(q), _lib.kernel_ready(k), _lib.kernel_ready(v)
-        with torch.cuda.device(q.device):
+        with _lib.on_device(q.device):
             o, L, m = _launch_fwd(q, k, v, n_prefix_q, sm_scale, block_size)
         ctx.save_for_backward(q, k, v, o, L, m)
         ctx.sm_scale = sm_scale
@@ -81,7 +81,7 @@ class FusedLandmarkAttention(torch.autograd.Function):
         assert q.shape[2] % BLOCK == 0, "Backward supported only for full blocks"
         assert k.shape[2] % BLOCK == 0, "Backward supported only for full blocks"
         do = _lib.kernel_ready(do)
-        with torch.cuda.device(q.device):
+        with _lib.on_device(q.device):
             dq, dk, dv = _launch_bwd(q, k, v, o, do, l, m, ctx.N_PREFIX_Q, ctx.sm_scale, BLOCK)
         return dq, dk, dv, None, None, None
 

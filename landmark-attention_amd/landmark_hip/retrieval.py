@@ -66,7 +66,7 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, 
     nbytes = lib.lmk_retrieve_workspace_bytes(B, H, T, S, D, int(block))
     probs = None
     assert not (reuse_landmark_keys and (aggregate or workspace is None))
-    with torch.cuda.device(q.device):
+    with _lib.on_device(q.device):
         if workspace is None:
             ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
         else:
@@ -133,7 +133,7 @@ def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, 
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
     q, k_cache, v_cache, k_loc, v_loc = (_lib.kernel_ready(t) for t in (q, k_cache, v_cache, k_loc, v_loc))
     cos, sin = _tables(cos, sin, q.dtype)
-    with torch.cuda.device(q.device):
+    with _lib.on_device(q.device):
         local = _local_window_attention(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block, sm_scale)
         return _gather(q, k_cache, v_cache, idx, cos, sin, block, top_k, sm_scale, local)
 
@@ -153,7 +153,7 @@ def attend_shared(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, 
     k = min(top_k, S // block)
     assert idx.shape == (B, H, 1, k) and idx.dtype == torch.int64 and idx.is_contiguous()
     assert inc == 0 or T + inc <= block, "new chunk and cached tail must fit one block (llama_mem.py:330)"
-    with torch.cuda.device(q.device):
+    with _lib.on_device(q.device):
         k_win, v_win = (torch.empty((B, H, k * block + inc + T, D), device=q.device, dtype=q.dtype) for _ in range(2))
         q_win = torch.empty((B, H, inc + T, D), device=q.device, dtype=q.dtype) if inc else None
         _lib.check(_lib.lib().lmk_gather_window(
@@ -181,7 +181,7 @@ def retrieve_and_attend(q, past_key_value, k_loc, v_loc, cos, sin, block: int, t
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
     q, k_cache, v_cache, k_loc, v_loc = (_lib.kernel_ready(t) for t in (q, k_cache, v_cache, k_loc, v_loc))
     cos, sin = _tables(cos, sin, q.dtype)
-    with torch.cuda.device(q.device):
+    with _lib.on_device(q.device):
         # (Running the local-window attention on a second stream beside the selection was tried: the
         # fork and join cost more than the 20 us it hides.)
         idx = retrieve_topk(q, k_cache, cos, sin, block, top_k, workspace=workspace,

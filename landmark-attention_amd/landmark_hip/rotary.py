@@ -23,7 +23,7 @@ def _rotate(x, cos, sin, position_ids, out=None):
     position_ids = position_ids.contiguous()
     if out is None:
         out = torch.empty_like(x)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         rc = _lib.lib().lmk_apply_rotary(_lib.tensor4(x), _lib.tensor4(out), cos.data_ptr(), sin.data_ptr(),
                                          cos.stride(0), cos.shape[0], position_ids.data_ptr(),
                                          L if position_ids.shape[0] == B and B > 1 else 0, B, H, L, D,
