@@ -151,6 +151,19 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
                       const lmk_tensor4* out, int B, int H, int T, int S, int D, float sm_scale, int block, int top_k,
                       int dtype, void* stream);
 
+/* The attend step in one call: lmk_local_window (when S % block > 0), lmk_attn_fwd on the local
+ * window and lmk_gather_attend, enqueued back to back with the window, its output and its statistics
+ * in `workspace` (at least lmk_attend_workspace_bytes(...) bytes, 16-byte aligned).  Same result as
+ * the three calls -- llama_mem.py:321-342 (window), :386-412 and :447-477 (gather, scores, grouped
+ * softmax, output) -- for callers whose per-call host cost matters: a decode step spends more time
+ * in the binding than on the GPU.  k_loc, v_loc: the new chunk (B,H,T,D), keys rotated. */
+size_t lmk_attend_workspace_bytes(int B, int H, int T, int S, int D, int block);
+int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+               const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
+               int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* out, void* workspace,
+               size_t workspace_bytes, int B, int H, int T, int S, int D, float sm_scale, int block, int top_k,
+               int dtype, void* stream);
+
 /* Local window of the attend step when the cache ends in an incomplete block of
  * inc = S % block tokens (llama_mem.py:329-342; needs inc > 0 and T + inc <= block, the
  * reference's assert at :330).  Writes, each (B,H,inc+T,D):

@@ -368,4 +368,65 @@ int lmk_apply_rotary(const lmk_tensor4* x, const lmk_tensor4* out, const void* c
   return lmk::launch_rotary(p, D, dtype, (hipStream_t)stream);
 }
 
+// ---- the attend step as one call: local window, fused forward on it, gather + attend ----
+namespace {
+struct AttendLayout {
+  size_t q_win, k_win, v_win, o_win, L, M, total;
+  int W;   // rows of the local window: inc + T
+};
+AttendLayout attend_layout(int B, int H, int T, int S, int D, int block) {
+  AttendLayout l;
+  const int inc = S % block;
+  l.W = inc + T;
+  const size_t rows = (size_t)B * H * l.W, tile = align256(rows * D * 2), stat = align256(rows * 4);
+  l.q_win = 0;
+  l.k_win = inc ? tile : 0;                  // without a tail the new chunk is the window: only o, L, M are needed
+  l.v_win = inc ? 2 * tile : 0;
+  l.o_win = inc ? 3 * tile : 0;
+  l.L = l.o_win + tile;
+  l.M = l.L + stat;
+  l.total = l.M + stat;
+  return l;
+}
+}  // namespace
+
+size_t lmk_attend_workspace_bytes(int B, int H, int T, int S, int D, int block) {
+  if (B <= 0 || H <= 0 || T <= 0 || S <= 0 || D <= 0 || block <= 0) return 0;
+  return attend_layout(B, H, T, S, D, block).total;
+}
+
+int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+               const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
+               int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* out, void* workspace,
+               size_t workspace_bytes, int B, int H, int T, int S, int D, float sm_scale, int block, int top_k,
+               int dtype, void* stream) {
+  if (workspace == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(workspace)) return LMK_ERR_ALIGN;
+  if (B <= 0 || H <= 0 || T <= 0 || S <= 0 || D <= 0 || block <= 0) return LMK_ERR_SHAPE;
+  const int inc = S % block;
+  if (inc && T + inc > block) return LMK_ERR_SHAPE;             // llama_mem.py:330
+  const AttendLayout l = attend_layout(B, H, T, S, D, block);
+  if (workspace_bytes < l.total) return LMK_ERR_WORKSPACE;
+  char* w = static_cast<char*>(workspace);
+  const int64_t W = l.W;
+  auto win = [&](size_t off) { return lmk_tensor4{w + off, (int64_t)H * W * D, W * D, (int64_t)D}; };
+  const lmk_tensor4 q_win = win(l.q_win), k_win = win(l.k_win), v_win = win(l.v_win), o_win = win(l.o_win);
+  float* L = reinterpret_cast<float*>(w + l.L);
+  float* M = reinterpret_cast<float*>(w + l.M);
+  int rc;
+  if (inc) {
+    if ((rc = lmk_local_window(q, kcache, vcache, k_loc, v_loc, cos_table, sin_table, table_stride_row, n_pos, &q_win,
+                               &k_win, &v_win, B, H, T, S, D, block, dtype, stream)))
+      return rc;
+    if ((rc = lmk_attn_fwd(&q_win, &k_win, &v_win, &o_win, L, M, B, H, (int)W, (int)W, D, sm_scale, block, 0, dtype, stream)))
+      return rc;
+  } else if ((rc = lmk_attn_fwd(q, k_loc, v_loc, &o_win, L, M, B, H, T, T, D, sm_scale, block, 0, dtype, stream))) {
+    return rc;
+  }
+  // the window's last T rows, read in place
+  const lmk_tensor4 o_loc = {w + l.o_win + (size_t)inc * D * 2, o_win.stride_b, o_win.stride_h, o_win.stride_row};
+  return lmk_gather_attend(q, kcache, vcache, idx, cos_table, sin_table, table_stride_row, n_pos, &o_loc, L + inc,
+                           M + inc, W, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream);
+}
+
 }  // extern "C"

@@ -66,6 +66,11 @@ def lib() -> ctypes.CDLL:
         L.lmk_gather_attend.restype = i
         L.lmk_gather_attend.argtypes = [T4, T4, T4, vp, vp, vp, i64, i64, T4, vp, vp, i64, T4,
                                         i, i, i, i, i, f, i, i, i, vp]
+        L.lmk_attend_workspace_bytes.restype = sz
+        L.lmk_attend_workspace_bytes.argtypes = [i, i, i, i, i, i]
+        L.lmk_attend.restype = i
+        L.lmk_attend.argtypes = [T4, T4, T4, vp, T4, T4, vp, vp, i64, i64, T4, vp, sz,
+                                 i, i, i, i, i, f, i, i, i, vp]
         L.lmk_local_window.restype = i
         L.lmk_local_window.argtypes = [T4, T4, T4, T4, T4, vp, vp, i64, i64, T4, T4, T4, i, i, i, i, i, i, i, vp]
         L.lmk_retrieve_topk_shared.restype = i

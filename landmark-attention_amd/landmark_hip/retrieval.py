@@ -88,42 +88,6 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, 
     return (idx, probs) if return_block_probs else idx
 
 
-def _local_window_attention(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block, sm_scale):
-    """Attention of the new tokens over the local window alone (the new chunk, behind the tail of an
-    incomplete cached block if there is one, ``llama_mem.py:329-342``) with the fused forward kernel.
-    Returns ``(o_loc, (L_ptr, M_ptr), stat_stride, tensors)``: output view, addresses and row stride of
-    its statistics, and every tensor that must stay alive until the gather kernel has read them."""
-    B, H, T, D = q.shape
-    S = k_cache.shape[2]
-    inc = S % block
-    if inc == 0:
-        o_loc, L_loc, M_loc = _launch_fwd(q, k_loc, v_loc, 0, sm_scale, block)
-        return o_loc, (L_loc.data_ptr(), M_loc.data_ptr()), T, (o_loc, L_loc, M_loc)
-    assert T + inc <= block, "new chunk and cached tail must fit one block (llama_mem.py:330)"
-    q_win, k_win, v_win = (torch.empty((B, H, inc + T, D), device=q.device, dtype=q.dtype) for _ in range(3))
-    _lib.check(_lib.lib().lmk_local_window(
-        _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), _lib.tensor4(k_loc), _lib.tensor4(v_loc),
-        cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(q_win), _lib.tensor4(k_win),
-        _lib.tensor4(v_win), B, H, T, S, D, int(block), _lib.DTYPE_CODES[q.dtype],
-        _lib.current_stream(q.device)))
-    o_win, L_win, M_win = _launch_fwd(q_win, k_win, v_win, 0, sm_scale, block)
-    # the window's last T rows, read in place: a strided view, and first element + row stride of the statistics
-    return (o_win[:, :, inc:], (L_win.data_ptr() + 4 * inc, M_win.data_ptr() + 4 * inc), inc + T,
-            (q_win, k_win, v_win, o_win, L_win, M_win))
-
-
-def _gather(q, k_cache, v_cache, idx, cos, sin, block, top_k, sm_scale, local):
-    B, H, T, D = q.shape
-    o_loc, stat_ptrs, stat_stride, _ = local
-    out = torch.empty_like(q)
-    _lib.check(_lib.lib().lmk_gather_attend(
-        _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), idx.data_ptr(), cos.data_ptr(),
-        sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(o_loc), stat_ptrs[0], stat_ptrs[1], stat_stride,
-        _lib.tensor4(out), B, H, T, k_cache.shape[2], D, float(sm_scale), int(block), int(top_k),
-        _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device)))
-    return out
-
-
 def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
     """Attention output ``(B, nh, T, hd)`` over the blocks ``idx`` selects plus the local window
     (``llama_mem.py:386-412,447-477``).  The local window -- the new chunk, behind the tail of
@@ -133,9 +97,28 @@ def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, 
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
     q, k_cache, v_cache, k_loc, v_loc = (_lib.kernel_ready(t) for t in (q, k_cache, v_cache, k_loc, v_loc))
     cos, sin = _tables(cos, sin, q.dtype)
+    return _attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
+
+
+def _attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale):
+    """Local window, fused forward on it and gather + attend through the one-call entry point (inputs
+    already in kernel layout): one trip through the binding instead of three, one scratch allocation
+    instead of six -- a decode step spends more time on the host than on the GPU."""
+    B, H, T, D = q.shape
+    S = k_cache.shape[2]
+    assert idx.dtype == torch.int64 and idx.is_contiguous() and idx.shape[:3] == (B, H, T)
+    assert S % block == 0 or T + S % block <= block, "new chunk and cached tail must fit one block (llama_mem.py:330)"
+    lib = _lib.lib()
+    nbytes = lib.lmk_attend_workspace_bytes(B, H, T, S, D, int(block))
     with _lib.on_device(q.device):
-        local = _local_window_attention(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block, sm_scale)
-        return _gather(q, k_cache, v_cache, idx, cos, sin, block, top_k, sm_scale, local)
+        ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+        out = torch.empty_like(q)
+        _lib.check(lib.lmk_attend(
+            _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), idx.data_ptr(), _lib.tensor4(k_loc),
+            _lib.tensor4(v_loc), cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(out),
+            ws.data_ptr(), nbytes, B, H, T, S, D, float(sm_scale), int(block), int(top_k),
+            _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device)))
+    return out
 
 
 def attend_shared(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
@@ -186,6 +169,5 @@ def retrieve_and_attend(q, past_key_value, k_loc, v_loc, cos, sin, block: int, t
         # fork and join cost more than the 20 us it hides.)
         idx = retrieve_topk(q, k_cache, cos, sin, block, top_k, workspace=workspace,
                             reuse_landmark_keys=reuse_landmark_keys)
-        local = _local_window_attention(q, k_cache, v_cache, k_loc, v_loc, cos, sin, block, sm_scale)
-        out = _gather(q, k_cache, v_cache, idx, cos, sin, block, top_k, sm_scale, local)
+        out = _attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
     return out, idx
