@@ -136,9 +136,13 @@ def decode_bench(n=50, warm=5):
     with torch.cuda.graph(graph):
         step()
     t_graph = _time_launches(graph.replay, n, warm)
+    # and called eagerly as the one host call a decode loop makes (selection with reused keys + attend)
+    from landmark_hip.retrieval import retrieve_and_attend
+    t_eager = _time_launches(lambda: retrieve_and_attend(q, (kc, vc), kl, vl, cos, sin, block, top_k, workspace=ws,
+                                                         reuse_landmark_keys=True), n, warm)
     return {"workload": "decode: 1 new token, H32 D128, cache 32775 tok (1024 blocks of 32 + tail of 7), top-4",
             "topk_ms": t_topk, "topk_reusing_landmark_keys_ms": t_reuse, "gather_attend_ms": t_att,
-            "step_from_hip_graph_ms": t_graph}
+            "step_from_hip_graph_ms": t_graph, "step_eager_one_call_ms": t_eager}
 
 
 def side_legs(n=30, warm=5):

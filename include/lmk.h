@@ -164,6 +164,16 @@ int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor
                size_t workspace_bytes, int B, int H, int T, int S, int D, float sm_scale, int block, int top_k,
                int dtype, void* stream);
 
+/* One inference step of the mem-cache path in one call: lmk_retrieve_topk (or lmk_retrieve_topk_reuse
+ * when reuse_landmark_keys != 0) followed by lmk_attend on the indices it wrote -- llama_mem.py:321-412
+ * and :447-477.  Same results as the two calls; idx_out (B,H,T,k) int64 is an output. */
+int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,
+                            const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table,
+                            const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                            const lmk_tensor4* out, void* retrieve_workspace, size_t retrieve_workspace_bytes,
+                            int reuse_landmark_keys, void* attend_workspace, size_t attend_workspace_bytes, int B,
+                            int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, void* stream);
+
 /* Local window of the attend step when the cache ends in an incomplete block of
  * inc = S % block tokens (llama_mem.py:329-342; needs inc > 0 and T + inc <= block, the
  * reference's assert at :330).  Writes, each (B,H,inc+T,D):

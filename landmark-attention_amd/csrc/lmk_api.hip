@@ -429,4 +429,23 @@ int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor
                            M + inc, W, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream);
 }
 
+int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,
+                            const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table,
+                            const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                            const lmk_tensor4* out, void* retrieve_workspace, size_t retrieve_workspace_bytes,
+                            int reuse_landmark_keys, void* attend_workspace, size_t attend_workspace_bytes, int B,
+                            int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, void* stream) {
+  if (attend_workspace == nullptr) return LMK_ERR_NULL;                 // before the selection is enqueued
+  if (S > 0 && block > 0 && S % block && T + S % block > block) return LMK_ERR_SHAPE;
+  if (B > 0 && H > 0 && T > 0 && S > 0 && D > 0 && block > 0 &&
+      attend_workspace_bytes < attend_layout(B, H, T, S, D, block).total)
+    return LMK_ERR_WORKSPACE;
+  if (int rc = retrieve_topk_impl(reuse_landmark_keys != 0, q, kcache, cos_table, sin_table, table_stride_row, n_pos,
+                                  idx_out, retrieve_workspace, retrieve_workspace_bytes, B, H, T, S, D, block, top_k,
+                                  dtype, stream))
+    return rc;
+  return lmk_attend(q, kcache, vcache, idx_out, k_loc, v_loc, cos_table, sin_table, table_stride_row, n_pos, out,
+                    attend_workspace, attend_workspace_bytes, B, H, T, S, D, sm_scale, block, top_k, dtype, stream);
+}
+
 }  // extern "C"

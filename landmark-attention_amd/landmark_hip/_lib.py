@@ -71,6 +71,9 @@ def lib() -> ctypes.CDLL:
         L.lmk_attend.restype = i
         L.lmk_attend.argtypes = [T4, T4, T4, vp, T4, T4, vp, vp, i64, i64, T4, vp, sz,
                                  i, i, i, i, i, f, i, i, i, vp]
+        L.lmk_retrieve_and_attend.restype = i
+        L.lmk_retrieve_and_attend.argtypes = [T4, T4, T4, T4, T4, vp, vp, i64, i64, vp, T4, vp, sz, i, vp, sz,
+                                              i, i, i, i, i, f, i, i, i, vp]
         L.lmk_local_window.restype = i
         L.lmk_local_window.argtypes = [T4, T4, T4, T4, T4, vp, vp, i64, i64, T4, T4, T4, i, i, i, i, i, i, i, vp]
         L.lmk_retrieve_topk_shared.restype = i

@@ -164,10 +164,28 @@ def retrieve_and_attend(q, past_key_value, k_loc, v_loc, cos, sin, block: int, t
         sm_scale = 1.0 / math.sqrt(q.shape[-1])
     q, k_cache, v_cache, k_loc, v_loc = (_lib.kernel_ready(t) for t in (q, k_cache, v_cache, k_loc, v_loc))
     cos, sin = _tables(cos, sin, q.dtype)
+    # Selection and attend step through the one-call entry point.  (Running the local-window attention on a
+    # second stream beside the selection was tried: the fork and join cost more than the 20 us it hides.)
+    B, H, T, D = q.shape
+    S = k_cache.shape[2]
+    assert k_cache.shape == (B, H, S, D) and q.dtype == k_cache.dtype and q.is_cuda and k_cache.is_cuda
+    assert S % block == 0 or T + S % block <= block, "new chunk and cached tail must fit one block (llama_mem.py:330)"
+    assert not (reuse_landmark_keys and workspace is None)
+    lib = _lib.lib()
+    rbytes = lib.lmk_retrieve_workspace_bytes(B, H, T, S, D, int(block))
+    abytes = lib.lmk_attend_workspace_bytes(B, H, T, S, D, int(block))
     with _lib.on_device(q.device):
-        # (Running the local-window attention on a second stream beside the selection was tried: the
-        # fork and join cost more than the 20 us it hides.)
-        idx = retrieve_topk(q, k_cache, cos, sin, block, top_k, workspace=workspace,
-                            reuse_landmark_keys=reuse_landmark_keys)
-        out = _attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block, top_k, sm_scale)
+        if workspace is None:
+            workspace = torch.empty(rbytes, device=q.device, dtype=torch.uint8)
+        else:
+            assert (workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.numel() >= rbytes
+                    and workspace.device == q.device)
+        idx = torch.empty((B, H, T, min(top_k, S // block)), device=q.device, dtype=torch.int64)
+        aws = torch.empty(abytes, device=q.device, dtype=torch.uint8)
+        out = torch.empty_like(q)
+        _lib.check(lib.lmk_retrieve_and_attend(
+            _lib.tensor4(q), _lib.tensor4(k_cache), _lib.tensor4(v_cache), _lib.tensor4(k_loc), _lib.tensor4(v_loc),
+            cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0], idx.data_ptr(), _lib.tensor4(out),
+            workspace.data_ptr(), rbytes, int(bool(reuse_landmark_keys)), aws.data_ptr(), abytes, B, H, T, S, D,
+            float(sm_scale), int(block), int(top_k), _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device)))
     return out, idx

@@ -29,7 +29,7 @@ def _declared():
 def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
-            "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend",
+            "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend",
             "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
@@ -130,6 +130,17 @@ def test_retrieval_argument_errors(lib):
     a256 = lambda x: (x + 255) & ~255
     assert lib.lmk_attend_workspace_bytes(1, 32, 256, 32768, 128, 32) == a256(32 * 256 * 128 * 2) + 2 * a256(32 * 256 * 4)
     assert lib.lmk_attend_workspace_bytes(1, 32, 1, 32768 + 7, 128, 32) == 4 * a256(32 * 8 * 128 * 2) + 2 * a256(32 * 8 * 4)
+
+    # selection + attend in one call: the attend workspace and the tail are checked before the selection is enqueued
+    def both(S=64, T=8, aws=0x4000, awsb=1 << 30, wsb=1 << 30):
+        return lib.lmk_retrieve_and_attend(t, t, t, t, t, 0x5000, 0x6000, 128, 4096, 0x7000, t, 0x8000, wsb, 0, aws, awsb,
+                                           1, 1, T, S, 128, 0.1, 32, 4, 0, None)
+
+    assert both(aws=None) == -1
+    assert both(awsb=64) == -8
+    assert both(wsb=64) == -8
+    assert both(S=70, T=27) == -2
+    assert both(S=20, T=4) == -9
 
     # one selection per head: same argument contract as the per-token entry point
     def shared(S=64, top_k=4, n_pos=4096, wsb=1 << 30, idx=0x7000):
