@@ -46,11 +46,38 @@ def _time_launches(fn, n, warm):
     return e0.elapsed_time(e1) / n
 
 
-def cpu_baseline(sample_heads=8):
-    """Oracle (closed form, fp32, torch on the host cores) on a bounded sample of the same
-    workload: forward+backward of `sample_heads` of the 64 (batch, head) slices of config 2."""
+def config0_inputs(seed=0):
+    """Benchmark config 0 exactly as specified: q, k, v ~ N(0,1) fp32 (2,8,510,128), a landmark at every
+    51st position (50 regular tokens + 1 landmark per block)."""
     import torch
-    from oracle import s1
+    B, H, L, D, block = 2, 8, 510, 128, 51
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(B, H, L, D, generator=g) for _ in range(3))
+    is_mem = (torch.arange(L) % block == block - 1)[None].expand(B, L)
+    return q, k, v, is_mem, block
+
+
+def cpu_baseline(sample_heads=8, budget_s=10.0):
+    """The reference's high-level PyTorch path on the host cores, as restated in oracle/highlevel.py
+    (lm_benchmark/models/landmark.py:196-236: scores, causal and landmark masks, bucketed softmax by
+    scatter/gather with 16 buckets, weights @ v), forward at benchmark config 0 exactly as specified
+    (B2 H8 L510 D128, block 51, fp32, seed 0): median of at least 10 runs.  A second, labelled entry times the
+    closed form (oracle/s1.py) forward+backward on a sample of config 2's slices."""
+    import statistics
+
+    import torch
+    from oracle import highlevel, s1
+    q0, k0, v0, is_mem0, _ = config0_inputs(0)
+    with torch.no_grad():
+        highlevel.attention_lm_benchmark(q0, k0, v0, is_mem0, n_buckets=16)     # untimed first pass
+        times = []
+        t_all = time.perf_counter()
+        while len(times) < 10 or (time.perf_counter() - t_all < 5.0 and len(times) < 40):
+            t0 = time.perf_counter()
+            highlevel.attention_lm_benchmark(q0, k0, v0, is_mem0, n_buckets=16)
+            times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    flops0 = 4 * 2 * 8 * 510 * 510 * 128 / 2
     L, D, block = 2048, 128, 32
     g = torch.Generator().manual_seed(0)
     q, k, v = ((torch.randn(sample_heads, L, D, generator=g) * 0.5).bfloat16().float().requires_grad_(True) for _ in range(3))
@@ -58,17 +85,24 @@ def cpu_baseline(sample_heads=8):
     torch.autograd.grad(s1.s1_attention(q, k, v, block), [q, k, v], do)      # untimed first pass (allocator, threads)
     t0 = time.perf_counter()
     reps = 0
-    while True:                                                              # about 10-15 s of CPU work
+    while True:
         out = s1.s1_attention(q, k, v, block)
         torch.autograd.grad(out, [q, k, v], do)
         reps += 1
-        if time.perf_counter() - t0 > 12.0 or reps >= 20:
+        if time.perf_counter() - t0 > budget_s or reps >= 20:
             break
     dt = (time.perf_counter() - t0) / reps
     flops = 3.5 * 4 * sample_heads * L * L * D / 2
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"fwd+bwd of {sample_heads} of the 64 (batch,head) slices of config 2 through oracle/s1.py "
-                      f"(fp32, torch CPU, autograd), {reps} reps, {dt:.2f} s each; host has {os.cpu_count()} logical cpus"}
+    threads, cpus = torch.get_num_threads(), os.cpu_count()
+    return {"value": flops0 / med / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"benchmark config 0 as specified (B2 H8 L510 D128, block 51, fp32, seed 0), forward through "
+                      f"oracle/highlevel.attention_lm_benchmark (scatter/gather grouped softmax, 16 buckets), median of "
+                      f"{len(times)} runs = {med * 1e3:.1f} ms (min {min(times) * 1e3:.1f}); torch.get_num_threads() = {threads}, "
+                      f"os.cpu_count() = {cpus}; 1.065 GFLOP on the conventional causal count",
+            "config0_forward_ms": med * 1e3,
+            "config2_sample": {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                               "sample": f"fwd+bwd of {sample_heads} of the 64 (batch,head) slices of config 2 through "
+                                         f"oracle/s1.py (closed form, fp32, torch CPU, autograd), {reps} reps, {dt:.2f} s each"}}
 
 
 def retrieval_bench(n=20, warm=3):

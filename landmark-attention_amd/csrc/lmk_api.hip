@@ -388,6 +388,29 @@ AttendLayout attend_layout(int B, int H, int T, int S, int D, int block) {
   l.total = l.M + stat;
   return l;
 }
+
+// Every argument check of the attend step's three stages (local window, fused forward on it, gather +
+// attend), run before the first of them is enqueued: a rejected call has launched nothing.
+int attend_precheck(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+                    const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
+                    int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* out, const void* workspace, int B,
+                    int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, bool need_idx) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache)) || (rc = check_tensor(vcache)) ||
+      (rc = check_tensor(k_loc)) || (rc = check_tensor(v_loc)) || (rc = check_tensor(out)))
+    return rc;
+  if (cos_table == nullptr || sin_table == nullptr || workspace == nullptr || (need_idx && idx == nullptr))
+    return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row) || !aligned16(workspace))
+    return LMK_ERR_ALIGN;
+  if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
+  if (D != 128 || !(block == 32 || block == 64 || block == 128)) return LMK_ERR_UNSUPPORTED;   // gather + attend, fused forward
+  if (!std::isfinite(sm_scale) || !(sm_scale > 0.f)) return LMK_ERR_SCALE;
+  const int inc = S % block;
+  if (inc && T + inc > block) return LMK_ERR_SHAPE;             // llama_mem.py:330
+  if (!slice_fits_32bit(q, T) || !slice_fits_32bit(k_loc, T) || !slice_fits_32bit(v_loc, T)) return LMK_ERR_UNSUPPORTED;
+  return LMK_OK;
+}
 }  // namespace
 
 size_t lmk_attend_workspace_bytes(int B, int H, int T, int S, int D, int block) {
@@ -400,11 +423,10 @@ int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor
                int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* out, void* workspace,
                size_t workspace_bytes, int B, int H, int T, int S, int D, float sm_scale, int block, int top_k,
                int dtype, void* stream) {
-  if (workspace == nullptr) return LMK_ERR_NULL;
-  if (!aligned16(workspace)) return LMK_ERR_ALIGN;
-  if (B <= 0 || H <= 0 || T <= 0 || S <= 0 || D <= 0 || block <= 0) return LMK_ERR_SHAPE;
+  if (int rc = attend_precheck(q, kcache, vcache, idx, k_loc, v_loc, cos_table, sin_table, table_stride_row, n_pos, out,
+                               workspace, B, H, T, S, D, sm_scale, block, top_k, dtype, true))
+    return rc;
   const int inc = S % block;
-  if (inc && T + inc > block) return LMK_ERR_SHAPE;             // llama_mem.py:330
   const AttendLayout l = attend_layout(B, H, T, S, D, block);
   if (workspace_bytes < l.total) return LMK_ERR_WORKSPACE;
   char* w = static_cast<char*>(workspace);
@@ -435,11 +457,14 @@ int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, con
                             const lmk_tensor4* out, void* retrieve_workspace, size_t retrieve_workspace_bytes,
                             int reuse_landmark_keys, void* attend_workspace, size_t attend_workspace_bytes, int B,
                             int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, void* stream) {
-  if (attend_workspace == nullptr) return LMK_ERR_NULL;                 // before the selection is enqueued
-  if (S > 0 && block > 0 && S % block && T + S % block > block) return LMK_ERR_SHAPE;
-  if (B > 0 && H > 0 && T > 0 && S > 0 && D > 0 && block > 0 &&
-      attend_workspace_bytes < attend_layout(B, H, T, S, D, block).total)
-    return LMK_ERR_WORKSPACE;
+  // everything the attend step would reject is rejected here, before the selection is enqueued
+  if (int rc = attend_precheck(q, kcache, vcache, idx_out, k_loc, v_loc, cos_table, sin_table, table_stride_row, n_pos,
+                               out, attend_workspace, B, H, T, S, D, sm_scale, block, top_k, dtype, true))
+    return rc;
+  if (attend_workspace_bytes < attend_layout(B, H, T, S, D, block).total) return LMK_ERR_WORKSPACE;
+  if (retrieve_workspace == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(retrieve_workspace)) return LMK_ERR_ALIGN;
+  if (retrieve_workspace_bytes < retr_layout(B, H, T, S, D, block).total) return LMK_ERR_WORKSPACE;
   if (int rc = retrieve_topk_impl(reuse_landmark_keys != 0, q, kcache, cos_table, sin_table, table_stride_row, n_pos,
                                   idx_out, retrieve_workspace, retrieve_workspace_bytes, B, H, T, S, D, block, top_k,
                                   dtype, stream))

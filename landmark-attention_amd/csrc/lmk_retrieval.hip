@@ -132,6 +132,20 @@ __device__ __forceinline__ void wave_best(float& v, int& i) {
   i = bi;
 }
 
+// Lane j < k holds the j-th pick of a row; the k picks are written in ascending order as int64.
+// Every value is first clamped into the cache (a row whose scores are all NaN picks nothing, and a
+// pick left at its initial value must not become a block index), and equal values are ranked by
+// lane, so that all k slots of the row are always written with indices the gather may follow.
+__device__ __forceinline__ void write_ascending(int64_t* row_out, int mine, int lane, int k, int num_mems) {
+  mine = min(max(mine, 0), num_mems - 1);
+  int rank = 0;
+  for (int j = 0; j < k; ++j) {
+    const int o = __shfl(mine, j, 64);
+    rank += (o < mine || (o == mine && j < lane)) ? 1 : 0;
+  }
+  if (lane < k) row_out[rank] = (int64_t)mine;
+}
+
 // ---------------------------------------------------------------------------
 // one selection per head (llama_mem.py:373-384 with aggregate == "max_over_tokens"): every query's
 // scores go through an fp32 softmax over the cached blocks, are rounded to the model dtype and
@@ -306,12 +320,7 @@ __global__ __launch_bounds__(256) void lmk_block_select_kernel(RetrParams p) {
     pi = bi;
     if (lane == j) mine = bi;
   }
-  int rank = 0;
-  for (int j = 0; j < p.k; ++j) {
-    const int o = __shfl(mine, j, 64);
-    rank += (o < mine) ? 1 : 0;
-  }
-  if (lane < p.k) p.idx[(int64_t)bh * p.k + rank] = (int64_t)mine;
+  write_ascending(p.idx + (int64_t)bh * p.k, mine, lane, p.k, p.num_mems);
 }
 
 // ---------------------------------------------------------------------------
@@ -567,12 +576,7 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
             pick(bv, bi);
             if (lane == j) mine = bi;
           }
-          int rank = 0;
-          for (int j = 0; j < p.k; ++j) {
-            const int o = __shfl(mine, j, 64);
-            rank += (o < mine) ? 1 : 0;
-          }
-          if (lane < p.k) p.idx[((int64_t)bh * p.T + t) * p.k + rank] = (int64_t)mine;
+          write_ascending(p.idx + ((int64_t)bh * p.T + t) * p.k, mine, lane, p.k, p.num_mems);
         } else {
           float rv = -INFINITY;
           int rx = 0x7fffffff;
@@ -637,12 +641,7 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
 #pragma unroll
     for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
       if (i == ri) mine = run_i[i];
-    int rank = 0;
-    for (int j = 0; j < p.k; ++j) {
-      const int o = __shfl(mine, j, 64);
-      rank += (o < mine) ? 1 : 0;
-    }
-    if (lane < p.k) p.idx[((int64_t)bh * p.T + t) * p.k + rank] = (int64_t)mine;
+    write_ascending(p.idx + ((int64_t)bh * p.T + t) * p.k, mine, lane, p.k, p.num_mems);
   }
 }
 
@@ -817,12 +816,7 @@ __global__ __launch_bounds__(256) void lmk_topk_slice_merge_kernel(RetrParams p,
       if (own == bi && xi[w] == bi) x[w] = -INFINITY;
     if (lane == j) mine = bi;
   }
-  int rank = 0;
-  for (int j = 0; j < p.k; ++j) {
-    const int o = __shfl(mine, j, 64);
-    rank += (o < mine) ? 1 : 0;
-  }
-  if (lane < p.k) p.idx[row * p.k + rank] = (int64_t)mine;
+  write_ascending(p.idx + row * p.k, mine, lane, p.k, p.num_mems);
 }
 
 // ---------------------------------------------------------------------------
@@ -909,7 +903,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   };
   int blk = 0;
   if (js0 < p.k) {
-    blk = (int)p.idx[row * p.k + js0];
+    blk = min(max((int)p.idx[row * p.k + js0], 0), p.num_mems - 1);      // idx is a caller's array: never read outside the cache
     fetch(kc, p.kcs_r, (int64_t)blk * BS);
   }
   for (int js = js0; js < p.k; js += jstep) {
@@ -976,7 +970,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       ahi[e] *= alpha;
     }
     int blk_next = blk;
-    if (js + jstep < p.k) blk_next = (int)p.idx[row * p.k + js + jstep];
+    if (js + jstep < p.k) blk_next = min(max((int)p.idx[row * p.k + js + jstep], 0), p.num_mems - 1);
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       take();

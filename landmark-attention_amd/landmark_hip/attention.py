@@ -86,17 +86,38 @@ class FusedLandmarkAttention(torch.autograd.Function):
         return dq, dk, dv, None, None, None
 
 
+# Masks that have already passed the check of ``flash_landmark_attention.py:393-394``, keyed by what
+# identifies a tensor's content without reading it: storage address, in-place version counter, layout.
+# A layer stack hands the same mask to every layer and every step, so the device->host sync of the
+# comparison is paid once per mask instead of once per call.
+_VALIDATED_MASKS: dict = {}
+_VALIDATED_MASKS_MAX = 64
+
+
+def _check_is_mem(is_mem, block_size):
+    key = (is_mem.device, is_mem.data_ptr(), is_mem._version, tuple(is_mem.shape), tuple(is_mem.stride()),
+           is_mem.dtype, int(block_size))
+    if key in _VALIDATED_MASKS:
+        return
+    expected_is_mem = torch.arange(0, is_mem.shape[-1], device=is_mem.device) % block_size == (block_size - 1)
+    assert (is_mem == expected_is_mem).all()
+    if len(_VALIDATED_MASKS) >= _VALIDATED_MASKS_MAX:
+        _VALIDATED_MASKS.clear()
+    # the entry keeps the tensor alive, so its address cannot be handed to another mask meanwhile
+    _VALIDATED_MASKS[key] = is_mem
+
+
 def fused_landmark_attention(q, k, v, is_mem, sm_scale=None, block_size=64):
     """Landmark grouped-softmax causal attention, landmarks at every ``block_size``-th key.
 
     q: (B, H, Lq, D); k, v: (B, H, Lk, D) with ``Lk - Lq`` a whole number of blocks of
     history.  ``is_mem`` (bool, last dim Lk) must mark exactly the positions
-    ``j % block_size == block_size - 1`` (checked as in the reference, ``:393-394``, which
-    costs one device->host sync); pass ``None`` to skip the check.
+    ``j % block_size == block_size - 1`` (checked as in the reference, ``:393-394``; the check
+    costs one device->host sync, paid once per distinct mask tensor state, not per call); pass
+    ``None`` to skip the check.
     """
     if is_mem is not None:
-        expected_is_mem = torch.arange(0, is_mem.shape[-1], device=is_mem.device) % block_size == (block_size - 1)
-        assert (is_mem == expected_is_mem).all()
+        _check_is_mem(is_mem, block_size)
 
     n_history_kv = k.shape[-2] - q.shape[-2]
     assert n_history_kv % block_size == 0

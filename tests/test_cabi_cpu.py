@@ -142,6 +142,22 @@ def test_retrieval_argument_errors(lib):
     assert both(S=70, T=27) == -2
     assert both(S=20, T=4) == -9
 
+    # what a later stage of the fused entry points would reject is rejected before the first launch
+    def both_x(D=128, block=32, out=t, idx=0x7000, scale=0.1):
+        return lib.lmk_retrieve_and_attend(t, t, t, t, t, 0x5000, 0x6000, 128, 4096, idx, out, 0x8000, 1 << 30, 0, 0x4000,
+                                           1 << 30, 1, 1, 8, 64, D, scale, block, 4, 0, None)
+
+    def attend_x(D=128, block=32, out=t, idx=0x7000, scale=0.1):
+        return lib.lmk_attend(t, t, t, idx, t, t, 0x5000, 0x6000, 128, 4096, out, 0x4000, 1 << 30, 1, 1, 8, 64, D, scale,
+                              block, 4, 0, None)
+
+    for f in (both_x, attend_x):
+        assert f(D=64) == -3                                    # the gather kernel is built for D = 128
+        assert f(block=16) == -3                                # the fused forward for blocks of 32, 64, 128
+        assert f(out=None) == -1
+        assert f(idx=0) == -1
+        assert f(scale=0.0) == -7
+
     # one selection per head: same argument contract as the per-token entry point
     def shared(S=64, top_k=4, n_pos=4096, wsb=1 << 30, idx=0x7000):
         return lib.lmk_retrieve_topk_shared(t, t, 0x5000, 0x6000, 128, n_pos, idx, None, 0x4000, wsb, 1, 1, 8, S, 128, 32, top_k,
@@ -177,3 +193,23 @@ def test_python_shim_rejects_what_the_reference_rejects():
     with pytest.raises(AssertionError):                       # history not whole blocks (:397)
         fused_landmark_attention(q, torch.zeros(1, 1, 40, 128, dtype=torch.bfloat16), q, None, block_size=32)
     assert issubclass(FusedLandmarkAttention, torch.autograd.Function)
+
+
+def test_is_mem_is_validated_once_per_mask_state():
+    # the reference compares the mask with the expected pattern on every call (one device->host sync each,
+    # flash_landmark_attention.py:393-394); the shim remembers masks that passed and re-checks a tensor only
+    # after an in-place write to it
+    import torch
+    from landmark_hip import attention
+    attention._VALIDATED_MASKS.clear()
+    mask = torch.arange(128) % 32 == 31
+    attention._check_is_mem(mask, 32)
+    attention._check_is_mem(mask, 32)
+    assert len(attention._VALIDATED_MASKS) == 1
+    with pytest.raises(AssertionError):
+        attention._check_is_mem(mask, 64)                      # same tensor, other block size: checked again
+    mask[5] = True                                             # bumps the version counter
+    with pytest.raises(AssertionError):
+        attention._check_is_mem(mask, 32)
+    with pytest.raises(AssertionError):
+        attention._check_is_mem(torch.zeros(128, dtype=torch.bool), 32)

@@ -146,3 +146,80 @@ def test_baseline_config2_full_size(seed):
         err = (g.float().cpu() - r).abs().max().item()
         print("config2", name, "max abs err", err, flush=True)
         assert err <= TOL, (name, err)
+
+
+@pytest.mark.parametrize("scale", [0.05, 0.3])
+@pytest.mark.parametrize("block,Lq,Lk", [(32, 256, 384), (64, 256, 384), (128, 256, 512)])
+def test_gradients_with_a_custom_softmax_scale(scale, block, Lq, Lk):
+    # sm_scale enters the backward twice: through the exponent (scale * log2 e) and as the factor of dQ and dK
+    B, H, D = 1, 2, 128
+    print(f"case scale{scale} bs{block} Lq{Lq} Lk{Lk}", flush=True)
+    q, k, v = make_qkv(B, H, Lq, Lk, D, seed=int(1000 * scale) + block)
+    do = torch.randn(B, H, Lq, D, generator=torch.Generator().manual_seed(7)).bfloat16()
+    rq, rk, rv = oracle_grads(q, k, v, do, block, scale=scale)
+    gq, gk, gv = _grads(q, k, v, do, block, scale=scale)
+    for name, g, r in (("dq", gq, rq), ("dk", gk, rk), ("dv", gv, rv)):
+        err = (g.float().cpu() - r).abs().max().item()
+        assert err <= TOL, (name, err)
+
+
+@pytest.mark.parametrize("Lq,Lk", [(256, 4352), (4608, 4608)])
+def test_gradients_beyond_64_blocks(Lq, Lk):
+    # 136 and 144 landmark blocks of 32: long history in front of few queries, and a long square problem
+    B, H, D, block = 1, 2, 128, 32
+    print(f"case long Lq{Lq} Lk{Lk}", flush=True)
+    q, k, v = make_qkv(B, H, Lq, Lk, D, seed=Lq + Lk)
+    do = torch.randn(B, H, Lq, D, generator=torch.Generator().manual_seed(8)).bfloat16()
+    rq, rk, rv = oracle_grads(q, k, v, do, block, chunk=1)
+    gq, gk, gv = _grads(q, k, v, do, block)
+    for name, g, r in (("dq", gq, rq), ("dk", gk, rk), ("dv", gv, rv)):
+        err = (g.float().cpu() - r).abs().max().item()
+        print("long", name, "max abs err", err, flush=True)
+        assert err <= TOL, (name, err)
+
+
+@pytest.mark.parametrize("block", [32, 64])
+def test_large_magnitude_inputs_forward_and_backward(block):
+    # inputs four times the benchmark's spread: scores reach +-25, far from the fixed reference maximum the
+    # block-32 forward takes from the landmark scores alone.  Tolerance: 2e-2 of the largest reference value
+    # (16-bit outputs carry a relative rounding error, so the absolute bound scales with the magnitude).
+    from tests.util import oracle_forward
+    from ltriton.flash_landmark_attention import fused_landmark_attention
+    B, H, Lq, Lk, D = 1, 4, 512, 640, 128
+    q, k, v = make_qkv(B, H, Lq, Lk, D, seed=40 + block, scale=2.0)
+    do = torch.randn(B, H, Lq, D, generator=torch.Generator().manual_seed(9)).bfloat16()
+    ref, _, _ = oracle_forward(q, k, v, block)
+    out = fused_landmark_attention(q.cuda(), k.cuda(), v.cuda(), None, block_size=block)
+    err = (out.float().cpu() - ref).abs().max().item()
+    assert torch.isfinite(out.float()).all()
+    assert err <= TOL * max(1.0, ref.abs().max().item()), ("out", err)
+    rq, rk, rv = oracle_grads(q, k, v, do, block)
+    gq, gk, gv = _grads(q, k, v, do, block)
+    for name, g, r in (("dq", gq, rq), ("dk", gk, rk), ("dv", gv, rv)):
+        err = (g.float().cpu() - r).abs().max().item()
+        bound = TOL * max(1.0, r.abs().max().item())
+        print("large magnitude", name, "max abs err", err, "bound", bound, flush=True)
+        assert torch.isfinite(g.float()).all()
+        assert err <= bound, (name, err, bound)
+
+
+def test_reference_script_case():
+    # the reference's own parity script: B2 H8 L1024 D128, mem_freq 63 -> block 64, bf16, torch.rand inputs on
+    # (B,L,H,D)-backed views (test_flash_landmark_attention.py:84-102); forward asserted at rtol=atol=1e-2 (:147),
+    # gradients of (out**2).sum() compared at rtol=atol=4e-2 (:156-165; printed there, asserted here)
+    from ltriton.flash_landmark_attention import fused_landmark_attention
+    from oracle import s1
+    B, H, L, D, block = 2, 8, 1024, 128, 64
+    g = torch.Generator().manual_seed(1234)
+    q, k, v = (torch.rand(B, L, H, D, generator=g).bfloat16().transpose(1, 2) for _ in range(3))
+    dev = torch.device("cuda:0")
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    is_mem = torch.arange(L, device=dev) % block == block - 1
+    out = fused_landmark_attention(qd, kd, vd, is_mem, block_size=block)
+    grads = torch.autograd.grad((out ** 2).sum(), [qd, kd, vd])
+    qc, kc, vc = (t.float().clone().requires_grad_(True) for t in (q, k, v))
+    exact = s1.s1_attention(qc, kc, vc, block)
+    exact_grads = torch.autograd.grad((exact ** 2).sum(), [qc, kc, vc])
+    assert torch.allclose(out.float().cpu(), exact.detach(), rtol=1e-2, atol=1e-2)
+    for name, a, b_ in zip("qkv", grads, exact_grads):
+        assert torch.allclose(a.float().cpu(), b_, rtol=4e-2, atol=4e-2), f"d{name}"

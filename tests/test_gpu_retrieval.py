@@ -296,3 +296,40 @@ def test_baseline_config4_full_size(seed):
     out = out.float().cpu()
     for (b, h, t), o in ref32.items():
         assert (out[b, h, t] - o).abs().max().item() <= 2e-2, (b, h, t)
+
+
+@pytest.mark.parametrize("T,n_mems", [(8, 64), (520, 64), (40, 2500)])   # sliced, fused, segmented selection
+def test_nan_queries_keep_indices_inside_the_cache(T, n_mems):
+    # a NaN score wins no comparison, so a row of NaN scores picks nothing: the indices written must still
+    # be block numbers of the cache (the gather follows them), and the output is NaN rather than a fault
+    from landmark_hip.retrieval import retrieve_and_attend
+    B, H, D, block, top_k = 1, 2, 128, 32, 4
+    S = n_mems * block
+    print(f"case nan T{T} n_mems{n_mems}", flush=True)
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=11)
+    q[:, 0] = float("nan")                                           # head 0: every score NaN; head 1 untouched
+    out, idx = retrieve_and_attend(q.cuda(), (kc.cuda(), vc.cuda()), kl.cuda(), vl.cuda(), cos.cuda(), sin.cuda(),
+                                   block, top_k)
+    torch.cuda.synchronize()
+    idx = idx.cpu()
+    assert int(idx.min()) >= 0 and int(idx.max()) < n_mems
+    assert torch.isnan(out[:, 0].float()).all()
+    sc = oret.landmark_scores(q[:, 1:], kc[:, 1:], cos, sin, block, top_k)
+    assert torch.equal(idx[:, 1:], oret.select_topk(sc, top_k))
+    assert torch.isfinite(out[:, 1].float()).all()
+
+
+def test_gather_clamps_indices_outside_the_cache():
+    # idx is a caller's array at the C ABI: values outside 0 .. num_mems-1 are read as the nearest block
+    from landmark_hip.retrieval import gather_attend
+    B, H, T, n_mems, D, block, top_k = 1, 2, 16, 40, 128, 32, 4
+    S = n_mems * block
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=12)
+    dev = [t.cuda() for t in (q, kc, vc)]
+    bad = torch.tensor([-7, 3, n_mems + 5, 2 ** 31 - 1]).expand(B, H, T, top_k).contiguous()
+    clamped = bad.clamp(0, n_mems - 1)
+    got = gather_attend(*dev, bad.cuda(), kl.cuda(), vl.cuda(), cos.cuda(), sin.cuda(), block, top_k)
+    want = gather_attend(*dev, clamped.cuda(), kl.cuda(), vl.cuda(), cos.cuda(), sin.cuda(), block, top_k)
+    torch.cuda.synchronize()
+    assert torch.isfinite(got.float()).all()
+    assert torch.equal(got, want)

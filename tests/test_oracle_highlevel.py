@@ -65,3 +65,21 @@ def test_irregular_landmarks_row_sums_and_block_structure():
     s = (q[0, 0, 1] @ k[0, 0, :2].T) / math.sqrt(d)
     assert torch.allclose(w[0, 0, 1, :2], torch.softmax(s, 0), atol=1e-12)
     assert (w[0, 0][:, is_mem[0]] == 0).all()         # landmark columns never carry weight
+
+
+def test_benchmark_config0_full_size_restatement_equals_closed_form():
+    # benchmark config 0 as specified: B2 H8 L510 D128, a landmark at every 51st position, fp32, seed 0,
+    # scale 1/sqrt(128); the lm_benchmark flavour with its default 16 buckets (10 blocks need 11) against the
+    # closed form.  This is the workload bench.py's CPU baseline times.
+    from bench import config0_inputs
+    q, k, v, is_mem, block = config0_inputs(0)
+    assert q.shape == (2, 8, 510, 128) and q.dtype == torch.float32 and block == 51
+    assert is_mem.sum().item() == 2 * 10 and bool(is_mem[0, 50]) and not bool(is_mem[0, 49])
+    a = highlevel.attention_lm_benchmark(q, k, v, is_mem, n_buckets=16)
+    b = s1.s1_attention(q, k, v, block)
+    assert torch.isfinite(a).all()
+    assert (a - b).abs().max().item() <= 2e-5
+    # and in float64, where both are exact to rounding
+    a64 = highlevel.attention_lm_benchmark(q.double(), k.double(), v.double(), is_mem, n_buckets=16)
+    assert (a64 - s1.s1_attention(q.double(), k.double(), v.double(), block)).abs().max().item() <= 1e-12
+    assert (a64 - a).abs().max().item() <= 2e-5

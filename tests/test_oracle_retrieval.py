@@ -297,3 +297,64 @@ def test_shared_window_rows_hand_worked():
     want = rotary.apply_rotary(kc[0, 0, src], cos, sin, torch.tensor(want_pos))
     assert torch.equal(keys[0, 0, : 2 * bs + inc], want) and torch.equal(keys[0, 0, -1], kl[0, 0, 0])
     assert torch.equal(values[0, 0, : 2 * bs + inc], vc[0, 0, src]) and torch.equal(values[0, 0, -1], vl[0, 0, 0])
+
+
+# ---------------------------------------- the score contract against the reference's literal expression
+@pytest.mark.parametrize("seed", [0, 1])
+def test_score_contract_against_the_literal_torch_expression(seed):
+    """The reference scores with ``torch.matmul(q, mem_key.transpose(2, 3)) / math.sqrt(hd)`` in the model
+    dtype and selects with ``topk(k).indices.sort()`` (``llama/llama_mem.py:367,384``).  torch's bf16 matmul
+    accumulates in fp32 in an order of its own; the contract fixes the sequential order.  On inputs of
+    benchmark config 4's shape and distribution (8 of its 32 heads) this evaluates the literal expression
+    with torch on the CPU and bounds how far the two are apart:
+
+    * the division step is identical, element for element, given the same product;
+    * the products differ in fewer than 2 in 10^4 elements, and every difference is either one bf16 ulp
+      (an fp32 sum that sat next to a rounding boundary) or belongs to a product so close to zero
+      (|dot| < 2^-12) that fp32 accumulation error (< 2^-19 absolute) spans several of its tiny ulps;
+    * under the same total order the two score sets select the same blocks in every row but those holding
+      a differing score, and ``torch.topk`` itself disagrees with the contract only in rows with a tie at
+      the k-th place or a differing score.
+    The measured rates are printed (run with -s) and recorded in the design notes."""
+    H, T, S, D, block, k = 8, 256, 32768, 128, 32, 4
+    q = _rand(1, H, T, D, seed=100 + seed, dtype=torch.bfloat16, scale=0.5)
+    kc = _rand(1, H, S, D, seed=200 + seed, dtype=torch.bfloat16, scale=0.5)
+    cos, sin = rotary.rotary_tables(S + T, D, torch.bfloat16)
+    geo = retrieval.retrieval_geometry(S, block, k)
+    lk = kc[..., : geo["full_len"], :].unflatten(-2, (geo["num_mems"], block))[..., block - 1, :]
+    mem_key = rotary.apply_rotary(lk, cos, sin, geo["mem_pos"])                  # llama_mem.py:366
+    product = torch.matmul(q, mem_key.transpose(2, 3))                           # the literal expression, :367
+    literal = product / math.sqrt(D)
+    assert literal.dtype == torch.bfloat16
+    contract = retrieval.landmark_scores(q, kc, cos, sin, block, k)
+    dot = retrieval.sequential_dot_fp32(q, mem_key)
+
+    # the division: fp32 quotient by float32(sqrt(hd)), rounded once
+    assert torch.equal(literal, (product.float() / torch.tensor(math.sqrt(D), dtype=torch.float32)).bfloat16())
+
+    def ordinal(x):                                                               # bf16 values on an integer line
+        i = x.view(torch.int16).to(torch.int32)
+        return torch.where(i < 0, -(i & 0x7FFF), i)
+
+    first = dot.bfloat16()
+    ulps = (ordinal(product) - ordinal(first)).abs()
+    n_diff = int((ulps > 0).sum())
+    assert n_diff <= 2e-4 * ulps.numel()
+    several = ulps > 1
+    assert (dot[several].abs() < 2.0 ** -12).all()
+    assert ((product.float() - first.float())[several].abs() < 2.0 ** -19).all()
+
+    score_diff_rows = (literal != contract).any(-1)
+    want = retrieval.select_topk(contract, k)
+    same_order = retrieval.select_topk(literal, k)
+    rows_same_order = (want != same_order).any(-1)
+    assert not (rows_same_order & ~score_diff_rows).any()
+    torch_topk = literal.float().topk(k, dim=-1).indices.sort(-1).values          # :384
+    rows_topk = (want != torch_topk).any(-1)
+    ties = retrieval.boundary_tie_rows(contract, k) | retrieval.boundary_tie_rows(literal, k)
+    assert not (rows_topk & ~ties & ~score_diff_rows).any()
+    print(f"seed {seed}: products differing {n_diff} of {ulps.numel()} ({n_diff / ulps.numel():.1e}), "
+          f"{int(several.sum())} of them near zero by more than one ulp; scores differing "
+          f"{int((literal != contract).sum())}; rows selecting other blocks under the same order "
+          f"{int(rows_same_order.sum())} of {rows_topk.numel()}; rows where torch.topk differs {int(rows_topk.sum())} "
+          f"(tie rows: {int(ties.sum())})")
