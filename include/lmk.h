@@ -137,6 +137,20 @@ int lmk_retrieve_topk_reuse(const lmk_tensor4* q, const lmk_tensor4* kcache, con
                             void* workspace, size_t workspace_bytes, int B, int H, int T, int S, int D, int block,
                             int top_k, int dtype, void* stream);
 
+/* lmk_retrieve_topk for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): same arguments without the workspace, same kernels, same
+ * indices.  It has no counterpart in the reference.  The workspace is a fixed array of
+ * lmk_retrieve_static_max_bytes() = 16 MiB of device memory inside the library (one copy per GPU the library
+ * runs on, held until the process ends); the call allocates and frees nothing.  Sizes whose workspace
+ * (lmk_retrieve_workspace_bytes) exceeds that limit are rejected with LMK_ERR_WORKSPACE -- a decode step of
+ * 32 heads against 32768 cached tokens needs 8.7 MB, a chunk of 256 queries does not fit.  Every call on a
+ * GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls on one
+ * stream are ordered.  Nothing in the array needs to start at zero (every kernel writes what it later reads). */
+size_t lmk_retrieve_static_max_bytes(void);
+int lmk_retrieve_topk_static(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
+                             const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out, int B,
+                             int H, int T, int S, int D, int block, int top_k, int dtype, void* stream);
+
 /* Gather of the selected K/V blocks with rotary at their slot positions and attention over
  * them (llama_mem.py:386-412), merged with the attention over the local chunk (:447-477).
  *   o_loc, L_loc, M_loc: output and statistics of lmk_attn_fwd run on the local chunk;

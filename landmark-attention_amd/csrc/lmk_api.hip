@@ -2,9 +2,44 @@
 // to the kernel launchers.  Declarations and the contract live in include/lmk.h.
 #include <cmath>
 
+#include <mutex>
+
 #include "lmk_launch.hpp"
 
+// Scratch memory of lmk_retrieve_topk_static: the selection's workspace (rotated landmark keys, their norms
+// and the two score planes) for callers that may not allocate.  Every GPU the library runs on holds its own
+// copy of this array, at its own address, until the process ends.  In host code the array's name is only a
+// handle for hipGetSymbolAddress: kernels and copies get the device address that call returns.
+#define LMK_STATIC_SCRATCH_BYTES (16u << 20)
+static __device__ __align__(256) unsigned char scratch[LMK_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};          // device address of `scratch` on each device, looked up once
+
+// Address of the current device's copy of `scratch`; *rc is 0 or a hipError_t.
+void* static_scratch(int* rc) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    *rc = e != hipSuccess ? (int)e : (int)hipErrorInvalidDevice;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));           // with device `dev` current
+    if (e != hipSuccess || ptr == nullptr) {
+      *rc = e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *rc = 0;
+  return g_scratch_ptr[dev];
+}
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 bool stride_ok(int64_t s) { return (s & 7) == 0; }  // 8 elements x 2 bytes = 16 bytes
@@ -228,16 +263,26 @@ size_t lmk_retrieve_workspace_bytes(int B, int H, int T, int S, int D, int block
   return retr_layout(B, H, T, S, D, block).total;
 }
 
+// The host-side checks of the selection, everything but the workspace.
+static int retrieve_topk_check(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
+                               const void* sin_table, int64_t table_stride_row, int64_t n_pos, const int64_t* idx_out,
+                               int B, int H, int T, int S, int D, int block, int top_k, int dtype) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache))) return rc;
+  if (cos_table == nullptr || sin_table == nullptr || idx_out == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
+  return check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos);
+}
+
 static int retrieve_topk_impl(bool reuse_landmark_keys, const lmk_tensor4* q, const lmk_tensor4* kcache,
                               const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
                               int64_t* idx_out, void* workspace, size_t workspace_bytes, int B, int H, int T, int S,
                               int D, int block, int top_k, int dtype, void* stream) {
-  int rc;
-  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache))) return rc;
-  if (cos_table == nullptr || sin_table == nullptr || idx_out == nullptr || workspace == nullptr) return LMK_ERR_NULL;
-  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row) || !aligned16(workspace))
-    return LMK_ERR_ALIGN;
-  if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
+  if (int rc = retrieve_topk_check(q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, B, H, T, S, D,
+                                   block, top_k, dtype))
+    return rc;
+  if (workspace == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(workspace)) return LMK_ERR_ALIGN;
   const RetrLayout l = retr_layout(B, H, T, S, D, block);
   if (workspace_bytes < l.total) return LMK_ERR_WORKSPACE;
   lmk::RetrParams p = {};
@@ -268,6 +313,23 @@ int lmk_retrieve_topk_reuse(const lmk_tensor4* q, const lmk_tensor4* kcache, con
                             int top_k, int dtype, void* stream) {
   return retrieve_topk_impl(true, q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, workspace,
                             workspace_bytes, B, H, T, S, D, block, top_k, dtype, stream);
+}
+
+size_t lmk_retrieve_static_max_bytes(void) { return LMK_STATIC_SCRATCH_BYTES; }
+
+int lmk_retrieve_topk_static(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
+                             const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out, int B,
+                             int H, int T, int S, int D, int block, int top_k, int dtype, void* stream) {
+  // every argument check runs on the host first, the size limit of the array among them
+  int rc = retrieve_topk_check(q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, B, H, T, S, D, block,
+                               top_k, dtype);
+  if (rc) return rc;
+  if (retr_layout(B, H, T, S, D, block).total > LMK_STATIC_SCRATCH_BYTES) return LMK_ERR_WORKSPACE;
+  void* ptr = static_scratch(&rc);
+  if (ptr == nullptr) return rc;
+  // same kernels, same layout: the device address of the array takes the place of the caller's workspace
+  return retrieve_topk_impl(false, q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, ptr,
+                            LMK_STATIC_SCRATCH_BYTES, B, H, T, S, D, block, top_k, dtype, stream);
 }
 
 int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,

@@ -63,6 +63,10 @@ def lib() -> ctypes.CDLL:
         L.lmk_retrieve_topk.argtypes = [T4, T4, vp, vp, i64, i64, vp, vp, sz, i, i, i, i, i, i, i, i, vp]
         L.lmk_retrieve_topk_reuse.restype = i
         L.lmk_retrieve_topk_reuse.argtypes = L.lmk_retrieve_topk.argtypes
+        L.lmk_retrieve_static_max_bytes.restype = sz
+        L.lmk_retrieve_static_max_bytes.argtypes = []
+        L.lmk_retrieve_topk_static.restype = i
+        L.lmk_retrieve_topk_static.argtypes = [T4, T4, vp, vp, i64, i64, vp, i, i, i, i, i, i, i, i, vp]
         L.lmk_gather_attend.restype = i
         L.lmk_gather_attend.argtypes = [T4, T4, T4, vp, vp, vp, i64, i64, T4, vp, vp, i64, T4,
                                         i, i, i, i, i, f, i, i, i, vp]

@@ -29,7 +29,7 @@ def _declared():
 def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
-            "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend",
+            "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend", "lmk_retrieve_topk_static", "lmk_retrieve_static_max_bytes",
             "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
@@ -106,7 +106,16 @@ def test_retrieval_argument_errors(lib):
     assert topk(wsb=64) == -8
     assert topk(D=96) == -3
     assert lib.lmk_retrieve_workspace_bytes(1, 32, 256, 32768, 128, 32) >= 32 * 1024 * 128 * 2 + 2 * 32 * 256 * 1024 * 4
-    # gather+attend is built for D=128 and blocks of 32/64 only
+    # the entry point whose workspace is a fixed array inside the library: same checks, all of them on the host
+    # before the array is looked up, and a size limit instead of a workspace argument
+    def static(S=64, T=8, H=1, top_k=4, cos=0x5000, idx=0x7000):
+        return lib.lmk_retrieve_topk_static(t, t, cos, 0x6000, 128, 1 << 20, idx, 1, H, T, S, 128, 32, top_k, 0, None)
+
+    assert lib.lmk_retrieve_static_max_bytes() == 16 << 20
+    assert static(cos=0) == -1 and static(idx=0) == -1 and static(S=16) == -9 and static(top_k=0) == -10
+    assert static(S=32768, T=256, H=32) == -8                 # benchmark config 4 needs 75 MB of workspace
+    assert lib.lmk_retrieve_workspace_bytes(1, 32, 1, 32768 + 7, 128, 32) < 16 << 20      # a decode step fits
+        # gather+attend is built for D=128 and blocks of 32/64 only
     rc = lib.lmk_gather_attend(t, t, t, 0x7000, 0x5000, 0x6000, 128, 4096, t, 0x2000, 0x3000, 8, t, 1, 1, 8, 64, 64, 0.1,
                                32, 4, 0, None)
     assert rc == -3
