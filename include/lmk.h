@@ -99,6 +99,39 @@ int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
                         int H, int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype, int phases,
                         void* stream);
 
+/* ---- landmark blocks of any size -------------------------------------------------------
+ * FusedLandmarkAttention.forward takes any block_size (llama/ltriton/flash_landmark_attention.py:318;
+ * the training models use mem_freq + 1 = 51, lm_benchmark/config/rotary.py:57).  The kernels work on
+ * blocks of 32, 64 or 128 slots, so a narrower block is stored PADDED: its block_real - 1 normal
+ * tokens in front, zero rows, and its landmark in the last of `block` slots.  The padded entry
+ * points mask the padding slots in every softmax, so the results at the real rows equal those of the
+ * unpadded problem; rows of o / dq / dk / dv at padding slots hold values of no meaning.
+ * block is 64 or 128 and 2 <= block_real <= block (block_real == block is the plain call, then 32
+ * is accepted too).  Lq, Lk and n_prefix count PADDED rows and stored blocks.
+ * dout must be zero at padding rows (lmk_pad_blocks writes zeros there). */
+
+/* Rows of a padded tensor that holds `rows` real rows: whole blocks widen to `block`, a partial
+ * last block keeps its length.  -1 for invalid sizes. */
+int64_t lmk_padded_rows(int64_t rows, int block_real, int block);
+
+/* dst (B,H,lmk_padded_rows(rows),D) <- src (B,H,rows,D): every row of dst is written. */
+int lmk_pad_blocks(const lmk_tensor4* src, const lmk_tensor4* dst, int B, int H, int64_t rows, int D,
+                   int block_real, int block, void* stream);
+/* dst (B,H,rows,D) <- src (B,H,lmk_padded_rows(rows),D): drops the padding rows. */
+int lmk_unpad_blocks(const lmk_tensor4* src, const lmk_tensor4* dst, int B, int H, int64_t rows, int D,
+                     int block_real, int block, void* stream);
+
+/* lmk_attn_fwd / lmk_attn_bwd on padded tensors (same kernels, same workspace formula with the
+ * padded sizes). */
+int lmk_attn_fwd_padded(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
+                        int block_real, int n_prefix, int dtype, void* stream);
+int lmk_attn_bwd_padded(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                        const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
+                        int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
+                        int dtype, void* stream);
+
 /* ---- mem-cache retrieval (inference) --------------------------------------------------
  * The reference has no function boundary here: scoring, selection and gather are inline in
  * LlamaAttention.forward (llama/llama_mem.py:318-430) and the attend step follows at :447-477.

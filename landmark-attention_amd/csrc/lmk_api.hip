@@ -174,16 +174,26 @@ const char* lmk_strerror(int code) {
 
 const char* lmk_version(void) { return "landmark_hip 0.1 gfx950"; }
 
-int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
-                 float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
-                 int n_prefix, int dtype, void* stream) {
+// block_real: tokens of each stored block that exist (== block for the plain entry points)
+static int check_block_real(int block, int block_real) {
+  if (block_real == block) return LMK_OK;
+  if (!(block == 64 || block == 128)) return LMK_ERR_UNSUPPORTED;      // the block-32 kernels carry no padding mask
+  if (block_real < 2 || block_real > block) return LMK_ERR_SHAPE;
+  return LMK_OK;
+}
+
+static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                         float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
+                         int block_real, int n_prefix, int dtype, void* stream) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o))) return rc;
   if (L == nullptr || M == nullptr) return LMK_ERR_NULL;
   if ((rc = check_common(B, H, Lq, Lk, D, sm_scale, block, n_prefix, dtype))) return rc;
+  if ((rc = check_block_real(block, block_real))) return rc;
   if (!slice_fits_32bit(q, Lq) || !slice_fits_32bit(o, Lq) || !slice_fits_32bit(k, Lk) || !slice_fits_32bit(v, Lk))
     return LMK_ERR_UNSUPPORTED;
   lmk::FwdParams p;
+  p.n_real = block_real;
   p.q = q->ptr; p.k = k->ptr; p.v = v->ptr; p.o = o->ptr;
   p.L = L; p.M = M;
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
@@ -195,6 +205,51 @@ int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
   p.os_b = o->stride_b; p.os_h = o->stride_h; p.os_r = o->stride_row;
   p.scale_log2 = sm_scale * 1.4426950408889634f;
   return lmk::launch_fwd(p, D, block, dtype, (hipStream_t)stream);
+}
+
+int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                 float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
+                 int n_prefix, int dtype, void* stream) {
+  return attn_fwd_impl(q, k, v, o, L, M, B, H, Lq, Lk, D, sm_scale, block, block, n_prefix, dtype, stream);
+}
+
+int lmk_attn_fwd_padded(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
+                        int block_real, int n_prefix, int dtype, void* stream) {
+  return attn_fwd_impl(q, k, v, o, L, M, B, H, Lq, Lk, D, sm_scale, block, block_real, n_prefix, dtype, stream);
+}
+
+int64_t lmk_padded_rows(int64_t rows, int block_real, int block) {
+  if (rows < 0 || block_real < 2 || block < block_real) return -1;
+  return rows / block_real * block + rows % block_real;
+}
+
+static int pad_impl(const lmk_tensor4* src, const lmk_tensor4* dst, int B, int H, int64_t rows, int D, int block_real,
+                    int block, bool unpad, void* stream) {
+  int rc;
+  if ((rc = check_tensor(src)) || (rc = check_tensor(dst))) return rc;
+  if (B <= 0 || H <= 0 || rows <= 0 || block_real < 2 || block < block_real) return LMK_ERR_SHAPE;
+  if (!(D == 64 || D == 128)) return LMK_ERR_UNSUPPORTED;
+  const int64_t rows_padded = lmk_padded_rows(rows, block_real, block);
+  if (rows_padded >= ((int64_t)1 << 31)) return LMK_ERR_UNSUPPORTED;
+  lmk::PadParams p;
+  p.src = src->ptr; p.dst = dst->ptr;
+  p.B = B; p.H = H; p.n_real = block_real; p.block = block;
+  p.L_src = (int)(unpad ? rows_padded : rows);
+  p.L_dst = (int)(unpad ? rows : rows_padded);
+  p.ss_b = src->stride_b; p.ss_h = src->stride_h; p.ss_r = src->stride_row;
+  p.ds_b = dst->stride_b; p.ds_h = dst->stride_h; p.ds_r = dst->stride_row;
+  return lmk::launch_pad_blocks(p, D, unpad, (hipStream_t)stream);
+}
+
+int lmk_pad_blocks(const lmk_tensor4* src, const lmk_tensor4* dst, int B, int H, int64_t rows, int D, int block_real,
+                   int block, void* stream) {
+  return pad_impl(src, dst, B, H, rows, D, block_real, block, false, stream);
+}
+
+int lmk_unpad_blocks(const lmk_tensor4* src, const lmk_tensor4* dst, int B, int H, int64_t rows, int D, int block_real,
+                     int block, void* stream) {
+  return pad_impl(src, dst, B, H, rows, D, block_real, block, true, stream);
 }
 
 size_t lmk_attn_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int block) {
@@ -212,11 +267,35 @@ int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
                              sm_scale, block, n_prefix, dtype, LMK_BWD_ALL, stream);
 }
 
+static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                         const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                         const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
+                         int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
+                         int dtype, int phases, void* stream);
+
 int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                         const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
                         const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
                         int H, int Lq, int Lk, int D, float sm_scale, int block, int n_prefix, int dtype, int phases,
                         void* stream) {
+  return attn_bwd_impl(q, k, v, o, dout, L, M, dq, dk, dv, workspace, workspace_bytes, B, H, Lq, Lk, D, sm_scale,
+                       block, block, n_prefix, dtype, phases, stream);
+}
+
+int lmk_attn_bwd_padded(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                        const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
+                        int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
+                        int dtype, void* stream) {
+  return attn_bwd_impl(q, k, v, o, dout, L, M, dq, dk, dv, workspace, workspace_bytes, B, H, Lq, Lk, D, sm_scale,
+                       block, block_real, n_prefix, dtype, LMK_BWD_ALL, stream);
+}
+
+static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                         const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                         const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
+                         int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
+                         int dtype, int phases, void* stream) {
   int rc;
   if (phases <= 0 || phases > LMK_BWD_ALL) return LMK_ERR_SHAPE;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o)) ||
@@ -224,6 +303,7 @@ int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
     return rc;
   if (L == nullptr || M == nullptr || workspace == nullptr) return LMK_ERR_NULL;
   if ((rc = check_common(B, H, Lq, Lk, D, sm_scale, block, n_prefix, dtype))) return rc;
+  if ((rc = check_block_real(block, block_real))) return rc;
   if (Lq % block != 0 || Lk % block != 0) return LMK_ERR_PARTIAL;
   if (!slice_fits_32bit(q, Lq) || !slice_fits_32bit(o, Lq) || !slice_fits_32bit(dout, Lq) || !slice_fits_32bit(dq, Lq) ||
       !slice_fits_32bit(k, Lk) || !slice_fits_32bit(v, Lk) || !slice_fits_32bit(dk, Lk) || !slice_fits_32bit(dv, Lk))
@@ -244,6 +324,7 @@ int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
   p.stat_l = w + 2 * rows + 2 * rows * nb;
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
   p.n_prefix = n_prefix; p.n_blocks = (int)nb;
+  p.n_real = block_real;
   p.n_qtiles = (Lq + 127) / 128; p.n_kvtiles = (Lk + 127) / 128;
   p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
   p.ks_b = k->stride_b; p.ks_h = k->stride_h; p.ks_r = k->stride_row;

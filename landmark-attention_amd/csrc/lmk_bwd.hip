@@ -195,6 +195,10 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dc][r] = 0.f;
   const float c2 = p.scale_log2;
+  // A block narrower than BS tokens is stored with its n_norm normal keys in front, its landmark in the
+  // last slot and padding in between: slots n_norm .. BS-2 hold no key and no query may see them.
+  const int n_norm = p.n_real - 1;
+  const bool padded = n_norm < BS - 1;                     // uniform over the launch
 
   // LDS byte offsets of this lane's operand fragments inside a 32-row tile: the swizzle repeats every 16
   // rows, so a tile at row 32u is the same offsets plus 32u rows -- an immediate of the LDS instruction
@@ -247,6 +251,15 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
       f32x16_t sc[C::NT], dp[C::KEEP_DP ? C::NT : 1];
 #pragma unroll
       for (int u = 0; u < C::NT; ++u) sc[u] = row_tile(kb + 32 * u * C::ROWB, qf);
+      if (padded) {                                        // padding slots leave the local softmax
+#pragma unroll
+        for (int u = 0; u < C::NT; ++u)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int kl = 32 * u + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (kl >= n_norm && kl < BS - 1) sc[u][r] = -INFINITY;
+          }
+      }
       const float s_last = sc[C::NT - 1][15];
       float mx = (h == 0) ? s_last : -INFINITY;
 #pragma unroll
@@ -305,7 +318,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int key = 8 * (r >> 2) + 4 * h + (r & 3);
-            const float pr = (u < tsub || key <= lim) ? fast_exp2(__builtin_fmaf(sc[r], c2, -mhat)) : 0.f;
+            const int kl = 32 * u + key;
+            const bool pad = padded && kl >= n_norm && kl < BS - 1;   // only the landmark query could reach one
+            const float pr = ((u < tsub || key <= lim) && !pad) ? fast_exp2(__builtin_fmaf(sc[r], c2, -mhat)) : 0.f;
             ds[r] = pr * (d[r] - delta);
           }
           dq_tile(kb + 32 * u * C::ROWB, ds);

@@ -34,6 +34,7 @@ struct FwdParams {
   int B, H, Lq, Lk;
   int n_prefix;   // history blocks in front of the queries
   int n_qtiles;   // ceil(Lq / 128)
+  int n_real;     // tokens of a block that exist (normal keys in front, landmark last); == block unless padded
   int64_t qs_b, qs_h, qs_r, ks_b, ks_h, ks_r, vs_b, vs_h, vs_r, os_b, os_h, os_r;  // element strides
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -50,6 +51,7 @@ struct BwdParams {
   int B, H, Lq, Lk;
   int n_prefix, n_blocks;        // history blocks; Lk / block
   int n_qtiles, n_kvtiles;       // ceil(Lq / 128), ceil(Lk / 128)
+  int n_real;                    // tokens of a block that exist; == block unless padded (blocks 64 and 128 only)
   int64_t qs_b, qs_h, qs_r, ks_b, ks_h, ks_r, vs_b, vs_h, vs_r, os_b, os_h, os_r, dos_b, dos_h, dos_r;
   int64_t dqs_b, dqs_h, dqs_r, dks_b, dks_h, dks_r, dvs_b, dvs_h, dvs_r;
   float scale, scale_log2;
@@ -102,6 +104,16 @@ struct RotaryParams {
   int B, H, L;
   int64_t xs_b, xs_h, xs_r, os_b, os_h, os_r, cs_r;
 };
+
+// Moves whole rows between a tensor with blocks of n_real tokens and one whose blocks are stored in `block`
+// slots (normal tokens in front, landmark in the last slot, zero rows in between).
+struct PadParams {
+  const void* src;
+  void* dst;
+  int B, H, L_src, L_dst, n_real, block;
+  int64_t ss_b, ss_h, ss_r, ds_b, ds_h, ds_r;
+};
+int launch_pad_blocks(const PadParams& p, int D, bool unpad, hipStream_t stream);
 
 int launch_rotary(const RotaryParams& p, int D, int dtype, hipStream_t stream);
 int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landmark_keys, hipStream_t stream);

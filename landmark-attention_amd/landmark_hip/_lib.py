@@ -57,6 +57,17 @@ def lib() -> ctypes.CDLL:
         L.lmk_attn_bwd_phases.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, ctypes.c_size_t,
                                           i, i, i, i, i, f, i, i, i, i, vp]
         i64, sz = ctypes.c_int64, ctypes.c_size_t
+        L.lmk_padded_rows.restype = i64
+        L.lmk_padded_rows.argtypes = [i64, i, i]
+        L.lmk_pad_blocks.restype = i
+        L.lmk_pad_blocks.argtypes = [T4, T4, i, i, i64, i, i, i, vp]
+        L.lmk_unpad_blocks.restype = i
+        L.lmk_unpad_blocks.argtypes = L.lmk_pad_blocks.argtypes
+        L.lmk_attn_fwd_padded.restype = i
+        L.lmk_attn_fwd_padded.argtypes = [T4, T4, T4, T4, vp, vp, i, i, i, i, i, f, i, i, i, i, vp]
+        L.lmk_attn_bwd_padded.restype = i
+        L.lmk_attn_bwd_padded.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, ctypes.c_size_t,
+                                          i, i, i, i, i, f, i, i, i, i, vp]
         L.lmk_retrieve_workspace_bytes.restype = sz
         L.lmk_retrieve_workspace_bytes.argtypes = [i, i, i, i, i, i]
         L.lmk_retrieve_topk.restype = i

@@ -1,6 +1,11 @@
 """``fused_landmark_attention`` with the reference's call surface
 (``llama/ltriton/flash_landmark_attention.py:308-403``), backed by the HIP kernels.
 
+Block sizes other than 32, 64 and 128 (the training models use ``mem_freq + 1 = 51``) run on the
+64- or 128-slot kernels: q, k, v and the incoming gradient are repacked so that every block has its
+normal tokens in front and its landmark in the last slot, the kernels mask the slots in between,
+and the results are packed back.  Blocks wider than 128 tokens are rejected.
+
 Differences a caller can observe, all of them relaxations:
 * ``is_mem=None`` is accepted and means "landmarks at fixed stride" (the reference's
   README promises this, its code dereferences ``is_mem.shape``, ``:393``);
@@ -15,35 +20,62 @@ import torch
 
 from . import _lib
 
-SUPPORTED_BLOCKS = (32, 64, 128)
+SUPPORTED_BLOCKS = (32, 64, 128)      # block sizes the kernels run without repacking
+MAX_BLOCK = 128
 SUPPORTED_HEAD_DIMS = (64, 128)
 
 
-def _launch_fwd(q, k, v, n_prefix, sm_scale, block):
+def storage_block(block_size: int) -> int:
+    """Slots per block the kernels work on for blocks of ``block_size`` tokens."""
+    if block_size in SUPPORTED_BLOCKS:
+        return block_size
+    if not 2 <= block_size <= MAX_BLOCK:
+        raise ValueError(f"block_size {block_size} is outside what the HIP kernels cover (2..{MAX_BLOCK})")
+    return 64 if block_size <= 64 else 128
+
+
+def _repack(x, block_size, block, unpad=False, rows=None):
+    """Pad (or, with ``unpad``, strip) the blocks of a (B, H, L, D) tensor; ``rows`` = real rows."""
+    B, H, _, D = x.shape
+    lib = _lib.lib()
+    rows = x.shape[2] if rows is None else rows
+    out_rows = rows if unpad else lib.lmk_padded_rows(rows, int(block_size), int(block))
+    out = torch.empty((B, H, out_rows, D), device=x.device, dtype=x.dtype)
+    fn = lib.lmk_unpad_blocks if unpad else lib.lmk_pad_blocks
+    _lib.check(fn(_lib.tensor4(x), _lib.tensor4(out), B, H, rows, D, int(block_size), int(block),
+                  _lib.current_stream(x.device)))
+    return out
+
+
+def _launch_fwd(q, k, v, n_prefix, sm_scale, block, block_real=None):
+    block_real = block if block_real is None else block_real
     B, H, Lq, D = q.shape
     Lk = k.shape[2]
     o = torch.empty_like(q)        # keeps q's memory layout: a (B,L,H,D)-backed q gives an output whose
     #                                transpose(1, 2).reshape(B, L, H*D) for o_proj (llama_mem.py:484-486) is a view
     L = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
     M = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
-    rc = _lib.lib().lmk_attn_fwd(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o),
-                                 L.data_ptr(), M.data_ptr(), B, H, Lq, Lk, D, float(sm_scale), int(block),
-                                 int(n_prefix), _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+    rc = _lib.lib().lmk_attn_fwd_padded(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o),
+                                        L.data_ptr(), M.data_ptr(), B, H, Lq, Lk, D, float(sm_scale), int(block),
+                                        int(block_real), int(n_prefix), _lib.DTYPE_CODES[q.dtype],
+                                        _lib.current_stream(q.device))
     _lib.check(rc)
     return o, L, M
 
 
-def _launch_bwd(q, k, v, o, do, L, M, n_prefix, sm_scale, block):
+def _launch_bwd(q, k, v, o, do, L, M, n_prefix, sm_scale, block, block_real=None):
+    block_real = block if block_real is None else block_real
     B, H, Lq, D = q.shape
     Lk = k.shape[2]
     lib = _lib.lib()
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)     # each in its input's layout
     nbytes = lib.lmk_attn_bwd_workspace_bytes(B, H, Lq, Lk, int(block))
     ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
-    rc = lib.lmk_attn_bwd(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o), _lib.tensor4(do),
-                          L.data_ptr(), M.data_ptr(), _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv),
-                          ws.data_ptr(), nbytes, B, H, Lq, Lk, D, float(sm_scale), int(block), int(n_prefix),
-                          _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+    rc = lib.lmk_attn_bwd_padded(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o),
+                                 _lib.tensor4(do), L.data_ptr(), M.data_ptr(), _lib.tensor4(dq), _lib.tensor4(dk),
+                                 _lib.tensor4(dv), ws.data_ptr(), nbytes, B, H, Lq, Lk, D, float(sm_scale),
+                                 int(block), int(block_real), int(n_prefix), _lib.DTYPE_CODES[q.dtype],
+                                 _lib.current_stream(q.device))
     _lib.check(rc)
     return dq, dk, dv
 
@@ -64,25 +96,41 @@ class FusedLandmarkAttention(torch.autograd.Function):
         assert q.is_cuda and k.is_cuda and v.is_cuda
         assert q.dtype in _lib.DTYPE_CODES, "HIP kernels are built for bf16 and fp16"
         assert d in SUPPORTED_HEAD_DIMS, f"HIP kernels are built for head dims {SUPPORTED_HEAD_DIMS}"
-        assert block_size in SUPPORTED_BLOCKS, f"HIP kernels are built for block sizes {SUPPORTED_BLOCKS}"
+        block = storage_block(block_size)
         q, k, v = _lib.kernel_ready(q), _lib.kernel_ready(k), _lib.kernel_ready(v)
-        with _lib.on_device(q.device):
-            o, L, m = _launch_fwd(q, k, v, n_prefix_q, sm_scale, block_size)
-        ctx.save_for_backward(q, k, v, o, L, m)
         ctx.sm_scale = sm_scale
         ctx.N_PREFIX_Q = n_prefix_q
         ctx.BLOCK = block_size
-        return o
+        ctx.real_rows = (seqlen_q, seqlen_k)
+        with _lib.on_device(q.device):
+            if block == block_size:
+                o, L, m = _launch_fwd(q, k, v, n_prefix_q, sm_scale, block_size)
+                ctx.save_for_backward(q, k, v, o, L, m)
+                return o
+            # the padded copies are what the backward kernels read, so they are what is kept
+            qp, kp, vp = (_repack(t, block_size, block) for t in (q, k, v))
+            op, L, m = _launch_fwd(qp, kp, vp, n_prefix_q, sm_scale, block, block_size)
+            ctx.save_for_backward(qp, kp, vp, op, L, m)
+            return _repack(op, block_size, block, unpad=True, rows=seqlen_q)
 
     @staticmethod
     def backward(ctx, do):
         BLOCK = ctx.BLOCK
         q, k, v, o, l, m = ctx.saved_tensors
-        assert q.shape[2] % BLOCK == 0, "Backward supported only for full blocks"
-        assert k.shape[2] % BLOCK == 0, "Backward supported only for full blocks"
+        rows_q, rows_k = ctx.real_rows
+        assert rows_q % BLOCK == 0, "Backward supported only for full blocks"
+        assert rows_k % BLOCK == 0, "Backward supported only for full blocks"
+        block = storage_block(BLOCK)
         do = _lib.kernel_ready(do)
         with _lib.on_device(q.device):
-            dq, dk, dv = _launch_bwd(q, k, v, o, do, l, m, ctx.N_PREFIX_Q, ctx.sm_scale, BLOCK)
+            if block == BLOCK:
+                dq, dk, dv = _launch_bwd(q, k, v, o, do, l, m, ctx.N_PREFIX_Q, ctx.sm_scale, BLOCK)
+            else:
+                dop = _repack(do, BLOCK, block)                     # zero rows at the padding slots
+                dq, dk, dv = _launch_bwd(q, k, v, o, dop, l, m, ctx.N_PREFIX_Q, ctx.sm_scale, block, BLOCK)
+                dq = _repack(dq, BLOCK, block, unpad=True, rows=rows_q)
+                dk = _repack(dk, BLOCK, block, unpad=True, rows=rows_k)
+                dv = _repack(dv, BLOCK, block, unpad=True, rows=rows_k)
         return dq, dk, dv, None, None, None
 
 
@@ -100,7 +148,9 @@ def _check_is_mem(is_mem, block_size):
     if key in _VALIDATED_MASKS:
         return
     expected_is_mem = torch.arange(0, is_mem.shape[-1], device=is_mem.device) % block_size == (block_size - 1)
-    assert (is_mem == expected_is_mem).all()
+    assert (is_mem == expected_is_mem).all(), (
+        f"is_mem must mark exactly the last token of every block of {block_size}: irregular landmark positions "
+        "and dropped landmarks are not covered by the fused kernels")
     if len(_VALIDATED_MASKS) >= _VALIDATED_MASKS_MAX:
         _VALIDATED_MASKS.clear()
     # the entry keeps the tensor alive, so its address cannot be handed to another mask meanwhile

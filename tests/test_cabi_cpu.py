@@ -30,6 +30,7 @@ def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
             "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend", "lmk_retrieve_topk_static", "lmk_retrieve_static_max_bytes",
+            "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded",
             "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
@@ -202,6 +203,51 @@ def test_python_shim_rejects_what_the_reference_rejects():
     with pytest.raises(AssertionError):                       # history not whole blocks (:397)
         fused_landmark_attention(q, torch.zeros(1, 1, 40, 128, dtype=torch.bfloat16), q, None, block_size=32)
     assert issubclass(FusedLandmarkAttention, torch.autograd.Function)
+
+
+def test_blocks_of_any_size_host_side(lib):
+    # a narrower block is stored in the next of 64 / 128 slots; whole blocks widen, a partial tail keeps its length
+    import torch
+    from landmark_hip import _lib, attention
+    L = _lib.lib()
+    assert L.lmk_padded_rows(510, 51, 64) == 640 and L.lmk_padded_rows(120, 51, 64) == 2 * 64 + 18
+    assert L.lmk_padded_rows(64, 64, 64) == 64 and L.lmk_padded_rows(0, 51, 64) == 0
+    assert L.lmk_padded_rows(10, 1, 64) == -1 and L.lmk_padded_rows(10, 65, 64) == -1 and L.lmk_padded_rows(-1, 51, 64) == -1
+    assert [attention.storage_block(b) for b in (2, 17, 32, 33, 51, 64, 65, 100, 128)] == [64, 64, 32, 64, 64, 64, 128, 128, 128]
+    for bad in (1, 0, 129, 256):
+        with pytest.raises(ValueError):
+            attention.storage_block(bad)
+    t = _lib.Tensor4(0x1000, 0, 0, 128)
+
+    def pad(fn=L.lmk_pad_blocks, src=t, rows=102, D=128, real=51, block=64):
+        return fn(src, t, 1, 1, rows, D, real, block, None)
+    assert pad(src=None) == -1 and pad(rows=0) == -2 and pad(real=1) == -2 and pad(real=65) == -2 and pad(D=96) == -3
+    assert pad(fn=L.lmk_unpad_blocks, rows=0) == -2 and pad(rows=1 << 31) == -3
+
+    def fwd(block, real, L_=128):
+        return L.lmk_attn_fwd_padded(t, t, t, t, 0x2000, 0x3000, 1, 1, L_, L_, 128, 0.1, block, real, 0, 0, None)
+    assert fwd(32, 17) == -3 and fwd(64, 1) == -2 and fwd(64, 65) == -2 and fwd(16, 16) == -3
+
+    def bwd(block, real, ws=1 << 30):
+        return L.lmk_attn_bwd_padded(t, t, t, t, t, 0x2000, 0x3000, t, t, t, 0x4000, ws, 1, 1, 128, 128, 128, 0.1, block,
+                                     real, 0, 0, None)
+    assert bwd(32, 17) == -3 and bwd(128, 1) == -2 and bwd(64, 51, ws=16) == -8
+
+
+def test_irregular_landmark_positions_are_rejected_with_a_message():
+    # landmarks anywhere but at the end of every block (irregular positions, group dropout) are outside the
+    # fused path, as in the reference (flash_landmark_attention.py:393-394)
+    import torch
+    from landmark_hip import attention
+    attention._VALIDATED_MASKS.clear()
+    mask = torch.arange(102) % 51 == 50
+    attention._check_is_mem(mask, 51)
+    dropped = mask.clone()
+    dropped[50] = False
+    with pytest.raises(AssertionError, match="last token of every block"):
+        attention._check_is_mem(dropped, 51)
+    with pytest.raises(AssertionError, match="last token of every block"):
+        attention._check_is_mem(torch.arange(102) % 51 == 49, 51)
 
 
 def test_is_mem_is_validated_once_per_mask_state():
