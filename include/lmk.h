@@ -221,6 +221,32 @@ int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, con
                             int reuse_landmark_keys, void* attend_workspace, size_t attend_workspace_bytes, int B,
                             int H, int T, int S, int D, float sm_scale, int block, int top_k, int dtype, void* stream);
 
+/* ---- ring cache of blocks (lm_benchmark) -----------------------------------------------
+ * Block selection of MemLMCacheStorage.retrieve_for_query
+ * (lm_benchmark/models/caches/mem_cache.py:50-85): the cache is a ring buffer of `n_blocks`
+ * filled block slots, slot `ring_start` (the reference's cache_iter once the ring is full, 0
+ * before) holding the OLDEST block.  Landmark keys are rotated at the positions of :56-61 (the
+ * top_k newest blocks at slots 1..top_k, every older block at slot 0, landmark token =
+ * slot*block + block-1), scored against the queries, soft-maxed over the blocks in fp32 and
+ * reduced as `method` says (:64-70); the top_k best slots are returned in order of age, oldest
+ * first -- what the order-restoring sort of :73-84 produces.
+ *   kring: (B,H,n_blocks*block,D) view of the filled slots, keys without rotary; the
+ *          reference's (B, slot, token, head, dim) buffer is such a view with
+ *          stride_row = H*D, stride_h = D.
+ *   idx_out: int64 slot numbers; (B,H,T,top_k) for PER_TOKEN_AND_HEAD, (B,T,top_k) for
+ *          MAX_OVER_HEADS (shared by the heads), (B,H,top_k) for MAX_OVER_TOKENS.
+ *   workspace: lmk_retrieve_workspace_bytes(B,H,T,n_blocks*block,D,block) bytes.
+ * top_k > n_blocks is an error (torch.topk raises there, :72).  Ties: (probability descending,
+ * slot ascending).  Tables in the half-split layout of the other entry points; the benchmark's
+ * interleaved pairs map onto it by moving the even head dims in front of the odd ones in q and k. */
+#define LMK_SELECT_PER_TOKEN_AND_HEAD 0
+#define LMK_SELECT_MAX_OVER_HEADS 1
+#define LMK_SELECT_MAX_OVER_TOKENS 2
+int lmk_ring_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kring, const void* cos_table,
+                           const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                           void* workspace, size_t workspace_bytes, int B, int H, int T, int n_blocks, int D, int block,
+                           int top_k, int ring_start, int method, int dtype, void* stream);
+
 /* Local window of the attend step when the cache ends in an incomplete block of
  * inc = S % block tokens (llama_mem.py:329-342; needs inc > 0 and T + inc <= block, the
  * reference's assert at :330).  Writes, each (B,H,inc+T,D):

@@ -471,6 +471,47 @@ int lmk_retrieve_topk_shared(const lmk_tensor4* q, const lmk_tensor4* kcache, co
   return lmk::launch_retrieve_topk_shared(p, D, dtype, (hipStream_t)stream);
 }
 
+int lmk_ring_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kring, const void* cos_table,
+                           const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                           void* workspace, size_t workspace_bytes, int B, int H, int T, int n_blocks, int D, int block,
+                           int top_k, int ring_start, int method, int dtype, void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kring))) return rc;
+  if (cos_table == nullptr || sin_table == nullptr || idx_out == nullptr || workspace == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row) || !aligned16(workspace))
+    return LMK_ERR_ALIGN;
+  if (B <= 0 || H <= 0 || T <= 0) return LMK_ERR_SHAPE;
+  if (n_blocks <= 0) return LMK_ERR_CACHE;
+  if (!(D == 64 || D == 128)) return LMK_ERR_UNSUPPORTED;
+  if (block < 2 || block > 4096 || (int64_t)n_blocks * block >= ((int64_t)1 << 31)) return LMK_ERR_UNSUPPORTED;
+  if (!(dtype == LMK_DTYPE_BF16 || dtype == LMK_DTYPE_F16)) return LMK_ERR_UNSUPPORTED;
+  if (method < LMK_SELECT_PER_TOKEN_AND_HEAD || method > LMK_SELECT_MAX_OVER_TOKENS) return LMK_ERR_UNSUPPORTED;
+  if (top_k < 1 || top_k > 64 || top_k > n_blocks) return LMK_ERR_TOPK;      // torch.topk raises for k > n (mem_cache.py:72)
+  if (ring_start < 0 || ring_start >= n_blocks) return LMK_ERR_SHAPE;
+  if (n_pos < (int64_t)(top_k + 1) * block) return LMK_ERR_TABLE;            // landmark positions end at top_k*block + block-1
+  const int S = n_blocks * block;
+  const RetrLayout l = retr_layout(B, H, T, S, D, block);
+  if (workspace_bytes < l.total) return LMK_ERR_WORKSPACE;
+  lmk::RetrParams p = {};
+  fill_retr_common(p, B, H, T, S, D, block, top_k);
+  p.prefix_len = 0;                                                          // mem_cache.py:60: slot * block + block - 1
+  p.ring_start = ring_start;
+  p.q = q->ptr; p.kcache = kring->ptr; p.cos = cos_table; p.sin = sin_table; p.idx = idx_out;
+  char* w = static_cast<char*>(workspace);
+  p.lk_rot = w + l.lk_rot;
+  p.lk_norm = reinterpret_cast<float*>(w + l.lk_norm);
+  p.approx = reinterpret_cast<float*>(w + l.approx);
+  p.exact = reinterpret_cast<float*>(w + l.exact);
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.kcs_b = kring->stride_b; p.kcs_h = kring->stride_h; p.kcs_r = kring->stride_row;
+  p.cs_r = table_stride_row;
+  if (method == LMK_SELECT_PER_TOKEN_AND_HEAD) return lmk::launch_retrieve_topk(p, D, dtype, false, (hipStream_t)stream);
+  p.agg = reinterpret_cast<uint32_t*>(w + l.exact);                          // B*T or B*H vectors of n_blocks words: fits
+  p.agg_over_heads = method == LMK_SELECT_MAX_OVER_HEADS;
+  p.prob32 = 1;                                                              // softmax output stays fp32 under autocast
+  return lmk::launch_retrieve_topk_shared(p, D, dtype, (hipStream_t)stream);
+}
+
 int lmk_local_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,
                      const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
                      int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win, const lmk_tensor4* k_win,

@@ -73,7 +73,9 @@ __global__ __launch_bounds__(256) void lmk_landmark_keys_kernel(RetrParams p) {
   if (row < total) {
     const int bh = (int)(row / p.num_mems), m = (int)(row % p.num_mems);
     const int b = bh / p.H, hh = bh % p.H;
-    const int slot = (m < p.num_mems - p.k) ? 0 : m - (p.num_mems - p.k) + 1;
+    int age = m - p.ring_start;                            // ring caches: slot ring_start holds the oldest block
+    age += age < 0 ? p.num_mems : 0;
+    const int slot = (age < p.num_mems - p.k) ? 0 : age - (p.num_mems - p.k) + 1;
     const int64_t pos = (int64_t)slot * p.block + (p.block - 1) + p.prefix_len;
     const char* src = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h + ((int64_t)m * p.block + p.block - 1) * p.kcs_r);
     const u32x4_t x = *(const u32x4_t*)(src + 16 * j);
@@ -136,12 +138,14 @@ __device__ __forceinline__ void wave_best(float& v, int& i) {
 // Every value is first clamped into the cache (a row whose scores are all NaN picks nothing, and a
 // pick left at its initial value must not become a block index), and equal values are ranked by
 // lane, so that all k slots of the row are always written with indices the gather may follow.
-__device__ __forceinline__ void write_ascending(int64_t* row_out, int mine, int lane, int k, int num_mems) {
+__device__ __forceinline__ void write_ascending(int64_t* row_out, int mine, int lane, int k, int num_mems, int ring_start) {
   mine = min(max(mine, 0), num_mems - 1);
+  int age = mine - ring_start;                             // oldest block first: slot order unless the cache is a ring
+  age += age < 0 ? num_mems : 0;
   int rank = 0;
   for (int j = 0; j < k; ++j) {
-    const int o = __shfl(mine, j, 64);
-    rank += (o < mine || (o == mine && j < lane)) ? 1 : 0;
+    const int o = __shfl(age, j, 64);
+    rank += (o < age || (o == age && j < lane)) ? 1 : 0;
   }
   if (lane < k) row_out[rank] = (int64_t)mine;
 }
@@ -280,8 +284,13 @@ __global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
   }
 #pragma unroll
   for (int msk = 32; msk >= 1; msk >>= 1) sum = sum + __shfl_xor(sum, msk, 64);
-  uint32_t* agg = p.agg + (int64_t)bh * NM;
-  for (int m = lane; m < NM; m += 64) atomicMax(agg + m, prob_bits<T>(__fdiv_rn(sc[m], sum)));
+  // one vector per (batch, head), maxima over the queries -- or per (batch, query), maxima over the heads;
+  // fp32 probabilities are positive, so their bit patterns order like the values
+  uint32_t* agg = p.agg + (int64_t)(p.agg_over_heads ? b * p.T + t : bh) * NM;
+  for (int m = lane; m < NM; m += 64) {
+    const float pr = __fdiv_rn(sc[m], sum);
+    atomicMax(agg + m, p.prob32 ? __float_as_uint(pr) : prob_bits<T>(pr));
+  }
 }
 
 // One workgroup per (batch, head): the k best blocks of agg under (value desc, index asc), ascending.
@@ -308,7 +317,8 @@ __global__ __launch_bounds__(256) void lmk_block_select_kernel(RetrParams p) {
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     for (int m = lane; m < NM; m += 64) {
-      const float x = (float)(in_lds ? cached[m] : agg[m]);       // 16-bit patterns: exact, order-preserving
+      const uint32_t u = in_lds ? cached[m] : agg[m];
+      const float x = p.prob32 ? __uint_as_float(u) : (float)u;   // 16-bit patterns as numbers: exact, order-preserving
       const bool after = (x < pv) || (x == pv && m > pi);
       if (after && (x > bv || (x == bv && m < bi))) {
         bv = x;
@@ -320,7 +330,7 @@ __global__ __launch_bounds__(256) void lmk_block_select_kernel(RetrParams p) {
     pi = bi;
     if (lane == j) mine = bi;
   }
-  write_ascending(p.idx + (int64_t)bh * p.k, mine, lane, p.k, p.num_mems);
+  write_ascending(p.idx + (int64_t)bh * p.k, mine, lane, p.k, p.num_mems, p.ring_start);
 }
 
 // ---------------------------------------------------------------------------
@@ -576,7 +586,7 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
             pick(bv, bi);
             if (lane == j) mine = bi;
           }
-          write_ascending(p.idx + ((int64_t)bh * p.T + t) * p.k, mine, lane, p.k, p.num_mems);
+          write_ascending(p.idx + ((int64_t)bh * p.T + t) * p.k, mine, lane, p.k, p.num_mems, p.ring_start);
         } else {
           float rv = -INFINITY;
           int rx = 0x7fffffff;
@@ -641,7 +651,7 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
 #pragma unroll
     for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
       if (i == ri) mine = run_i[i];
-    write_ascending(p.idx + ((int64_t)bh * p.T + t) * p.k, mine, lane, p.k, p.num_mems);
+    write_ascending(p.idx + ((int64_t)bh * p.T + t) * p.k, mine, lane, p.k, p.num_mems, p.ring_start);
   }
 }
 
@@ -816,7 +826,7 @@ __global__ __launch_bounds__(256) void lmk_topk_slice_merge_kernel(RetrParams p,
       if (own == bi && xi[w] == bi) x[w] = -INFINITY;
     if (lane == j) mine = bi;
   }
-  write_ascending(p.idx + row * p.k, mine, lane, p.k, p.num_mems);
+  write_ascending(p.idx + row * p.k, mine, lane, p.k, p.num_mems, p.ring_start);
 }
 
 // ---------------------------------------------------------------------------
@@ -1106,11 +1116,13 @@ static int launch_topk_shared_t(const RetrParams& p, hipStream_t stream) {
   int rc;
   hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
   if ((rc = (int)hipGetLastError())) return rc;
-  hipLaunchKernelGGL(lmk_fill_u32_kernel, dim3((unsigned)((lkrows + 255) / 256)), dim3(256), 0, stream, p.agg, lkrows, 0u);
+  const int64_t sel_rows = p.agg_over_heads ? (int64_t)p.B * p.T : (int64_t)p.B * p.H;   // vectors to pick from
+  const int64_t agg_words = sel_rows * p.num_mems;
+  hipLaunchKernelGGL(lmk_fill_u32_kernel, dim3((unsigned)((agg_words + 255) / 256)), dim3(256), 0, stream, p.agg, agg_words, 0u);
   if ((rc = (int)hipGetLastError())) return rc;
   hipLaunchKernelGGL((lmk_block_prob_kernel<T, D>), dim3((unsigned)(p.B * p.H * ((p.T + 3) / 4))), dim3(256), 0, stream, p);
   if ((rc = (int)hipGetLastError())) return rc;
-  hipLaunchKernelGGL(lmk_block_select_kernel, dim3(p.B * p.H), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL(lmk_block_select_kernel, dim3((unsigned)sel_rows), dim3(256), 0, stream, p);
   return (int)hipGetLastError();
 }
 

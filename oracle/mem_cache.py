@@ -1,0 +1,167 @@
+"""Ring cache of landmark blocks: storage bookkeeping and block selection.  TEST ORACLE.
+
+Restates ``MemLMCacheStorage`` of ``lm_benchmark/models/caches/mem_cache.py``: the ring-buffer
+bookkeeping of ``store_in_cache`` (``:111-158``) and the selection half of ``retrieve_for_query``
+(``:50-85``) -- landmark positions, scores, softmax, the three selection methods, top-k and the
+order-restoring sort -- plus the key positions of the gathered blocks (``:95-97``).  Nothing here is
+used by the library; the tests compare the HIP selection with it index for index.
+
+What the reference leaves to the libraries is fixed the same way as for the llama-flavour cache
+(``oracle/retrieval.py``): scores under the sequential-accumulation score contract, the softmax by
+``softmax_contract`` in fp32 (under the benchmark's autocast the score product is a 16-bit matmul and
+``softmax`` returns fp32, ``optim/base.py:49-50``), ties at the k-th place by (probability descending,
+slot ascending).  Positions use the kernels' half-split tables; the benchmark's interleaved pairs
+(``models/positional_encoders/rotary_utils.py:17-31``) are the same rotation with the even head dims
+moved in front of the odd ones, which leaves every q.k unchanged (checked in
+``tests/test_oracle_mem_cache.py`` against a restatement of the interleaved form).
+
+Pinned in ``tests/test_oracle_mem_cache.py``: the ring against a plain Python list of blocks that is
+appended to and truncated (contents, age order, slot of the oldest block, for chunks that wrap, fill
+exactly, and exceed the capacity); slot ages and landmark positions on hand-worked cases; the
+where/sort/where sequence against a brute-force sort by age; the selection of a ring against the
+already pinned flat-cache selection (``oracle/retrieval.py``) applied to the same blocks laid out oldest
+first; ``max_over_heads`` / ``max_over_tokens`` against literal loops; ``torch.topk`` on rows without a
+boundary tie.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .retrieval import sequential_dot_fp32, softmax_contract
+from .rotary import apply_rotary
+
+METHODS = ("per_token_and_head", "max_over_heads", "max_over_tokens")
+
+
+class RingStore:
+    """Buffers and counters of ``MemLMCacheStorage`` (``mem_cache.py:23-39``), CPU tensors.
+
+    ``cache_k/v``: (B, capacity, block, nh, hs); ``pending_*``: the tokens behind the last complete
+    block (``last_incomplete_*``).  ``cache_size`` keeps the reference's quirk of counting blocks that
+    were dropped or overwritten, so the number of filled slots is ``min(cache_size, capacity)``."""
+
+    def __init__(self, batch: int, capacity: int, block: int, heads: int, head_dim: int, dtype=torch.float32):
+        self.capacity, self.block = capacity, block
+        self.cache_k = torch.zeros(batch, capacity, block, heads, head_dim, dtype=dtype)
+        self.cache_v = torch.zeros_like(self.cache_k)
+        self.pending_k = torch.zeros(batch, heads, 0, head_dim, dtype=dtype)
+        self.pending_v = torch.zeros_like(self.pending_k)
+        self.pending_is_mem = torch.zeros(batch, 0, dtype=torch.bool)
+        self.cache_iter = 0
+        self.cache_size = 0
+
+    @property
+    def filled(self) -> int:
+        return min(self.cache_size, self.capacity)          # what ``[:, :self.cache_size]`` keeps (``:51``)
+
+    @property
+    def last_incomplete_len(self) -> int:
+        return self.pending_k.shape[2]
+
+    def store(self, keys, values, is_mem) -> None:
+        """``store_in_cache`` (``:111-158``): keys, values (B, nh, T, hs), is_mem (B, T)."""
+        k = torch.cat((self.pending_k, keys), dim=2)                                  # :114-116
+        v = torch.cat((self.pending_v, values), dim=2)
+        im = torch.cat((self.pending_is_mem, is_mem), dim=1)
+        B, nh, T, hs = k.shape
+        bs, cap = self.block, self.capacity
+        rest = T % bs                                                                 # :119-128
+        full = T - rest
+        self.pending_k, self.pending_v, self.pending_is_mem = k[:, :, full:], v[:, :, full:], im[:, full:]
+        blocks_mem = im[:, :full].reshape(B, -1, bs)                                  # :131-134
+        assert blocks_mem[..., -1].all() and not blocks_mem[..., :-1].any()
+        n_new = full // bs
+        kb = k[:, :, :full].transpose(1, 2).reshape(B, n_new, bs, nh, hs)             # :136-137
+        vb = v[:, :, :full].transpose(1, 2).reshape(B, n_new, bs, nh, hs)
+        kept = min(n_new, cap)                                                        # :138-143: only the newest fit
+        dropped = n_new - kept
+        kb, vb = kb[:, dropped:], vb[:, dropped:]
+        self.cache_iter = (self.cache_iter + dropped) % cap
+        self.cache_size += dropped
+        if self.cache_iter + kept >= cap:                                             # :146-152: the write wraps
+            head = cap - self.cache_iter
+            nxt = self.cache_iter + kept - cap
+            self.cache_k[:, self.cache_iter:] = kb[:, :head]
+            self.cache_v[:, self.cache_iter:] = vb[:, :head]
+            self.cache_k[:, :nxt] = kb[:, head:]
+            self.cache_v[:, :nxt] = vb[:, head:]
+        else:                                                                         # :153-156
+            nxt = self.cache_iter + kept
+            self.cache_k[:, self.cache_iter:nxt] = kb
+            self.cache_v[:, self.cache_iter:nxt] = vb
+        self.cache_iter = nxt                                                         # :158-159
+        self.cache_size += kept
+
+
+def slot_ages(n: int, cache_iter: int):
+    """Age rank of every filled slot, 0 = oldest (``mem_indices`` of ``mem_cache.py:52-55``)."""
+    return torch.cat((torch.arange(n - cache_iter, n), torch.arange(0, n - cache_iter)))
+
+
+def landmark_slots(n: int, cache_iter: int, top_k: int):
+    """Position slot of every filled block (``:57``): the ``top_k`` newest get 1..top_k, the rest 0."""
+    age = slot_ages(n, cache_iter)
+    return torch.where(age >= n - top_k, age - (n - top_k) + 1, 0)
+
+
+def landmark_token_positions(n: int, cache_iter: int, top_k: int, block: int):
+    """``mem_token_indices`` (``:58``)."""
+    return landmark_slots(n, cache_iter, top_k) * block + block - 1
+
+
+def ring_scores(q, cache_k, n: int, cache_iter: int, top_k: int, cos, sin):
+    """(B, nh, T, n) scores in q.dtype (``:51,59-60``) under the score contract.
+    q: (B, nh, T, hs) rotated; cache_k: (B, capacity, block, nh, hs)."""
+    block, hs = cache_k.shape[2], cache_k.shape[-1]
+    lk = cache_k[:, :n, -1].transpose(1, 2).to(q.dtype)                               # (B, nh, n, hs)
+    lk = apply_rotary(lk, cos, sin, landmark_token_positions(n, cache_iter, top_k, block))
+    dot = sequential_dot_fp32(q, lk)
+    return (dot.to(q.dtype).float() / torch.tensor(math.sqrt(hs), dtype=torch.float32)).to(q.dtype)
+
+
+def block_probabilities(scores, method: str):
+    """fp32 (B, nh, T, n): softmax over the blocks, reduced as ``cache_selection_method`` says (``:61-70``)."""
+    B, nh, T, n = scores.shape
+    prob = softmax_contract(scores, torch.float32)
+    if method == "max_over_heads":
+        return prob.amax(dim=1, keepdim=True).expand(B, nh, T, n)
+    if method == "max_over_tokens":
+        return prob.amax(dim=2, keepdim=True).expand(B, nh, T, n)
+    if method == "per_token_and_head":
+        return prob
+    raise NotImplementedError(method)
+
+
+def restore_order(picked, n: int, cache_iter: int):
+    """The order-restoring sort of ``:73-84`` applied to slot numbers (…, top_k): to age, sort, back to slots."""
+    if picked.shape[-1] == 1:
+        return picked
+    age = torch.where(picked < cache_iter, (n - cache_iter) + picked, picked - cache_iter)
+    age = age.sort(dim=-1).values
+    return torch.where(age >= n - cache_iter, age - (n - cache_iter), age + cache_iter)
+
+
+def select_blocks(scores, cache_iter: int, top_k: int, method: str):
+    """Slots (B, nh, T, top_k) int64, oldest block first; ties by (probability descending, slot ascending)."""
+    n = scores.shape[-1]
+    prob = block_probabilities(scores, method)
+    order = torch.sort(prob, dim=-1, descending=True, stable=True).indices[..., :top_k]
+    return restore_order(order, n, cache_iter)
+
+
+def boundary_tie_rows(scores, top_k: int, method: str):
+    """Bool (B, nh, T): rows whose k-th and (k+1)-th best probabilities are equal."""
+    prob = torch.sort(block_probabilities(scores, method), dim=-1, descending=True).values
+    if prob.shape[-1] <= top_k:
+        return torch.zeros(prob.shape[:-1], dtype=torch.bool)
+    return prob[..., top_k - 1] == prob[..., top_k]
+
+
+def gathered_key_positions(slots, n: int, cache_iter: int, top_k: int, block: int):
+    """``k_indices`` (``:95-97``): positions at which the gathered keys are rotated, (…, top_k * block).
+    The j-th picked block sits at tokens j*block .., one block further when it is one of the newest."""
+    chosen = landmark_slots(n, cache_iter, top_k)[slots]                               # position slot of each pick
+    base = torch.arange(top_k * block).view(top_k, block)
+    return (((chosen > 0) * block).unsqueeze(-1) + base).flatten(-2)

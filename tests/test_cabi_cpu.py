@@ -30,7 +30,7 @@ def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
             "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend", "lmk_retrieve_topk_static", "lmk_retrieve_static_max_bytes",
-            "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded",
+            "lmk_ring_retrieve_topk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded",
             "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
@@ -232,6 +232,21 @@ def test_blocks_of_any_size_host_side(lib):
         return L.lmk_attn_bwd_padded(t, t, t, t, t, 0x2000, 0x3000, t, t, t, 0x4000, ws, 1, 1, 128, 128, 128, 0.1, block,
                                      real, 0, 0, None)
     assert bwd(32, 17) == -3 and bwd(128, 1) == -2 and bwd(64, 51, ws=16) == -8
+
+
+def test_ring_selection_argument_errors(lib):
+    from landmark_hip import _lib
+    L = _lib.lib()
+    t = _lib.Tensor4(0x1000, 0, 0, 64)
+
+    def sel(q=t, idx=0x7000, ws=0x8000, nbytes=1 << 30, T=1, n=4, D=64, block=51, k=2, start=0, method=0, n_pos=1 << 20):
+        return L.lmk_ring_retrieve_topk(q, t, 0x5000, 0x6000, 64, n_pos, idx, ws, nbytes, 1, 2, T, n, D, block, k, start,
+                                        method, 0, None)
+    assert sel(q=None) == -1 and sel(idx=None) == -1 and sel(ws=None) == -1
+    assert sel(n=0) == -9 and sel(T=0) == -2 and sel(D=96) == -3 and sel(block=1) == -3 and sel(method=3) == -3
+    assert sel(k=5) == -10 and sel(k=0) == -10                    # more blocks asked for than cached: torch.topk raises
+    assert sel(start=4) == -2 and sel(start=-1) == -2
+    assert sel(n_pos=3 * 51 - 1) == -11 and sel(nbytes=16) == -8
 
 
 def test_irregular_landmark_positions_are_rejected_with_a_message():

@@ -27,3 +27,31 @@ def test_append_equals_torch_cat_and_views_share_storage():
     before = pk.data_ptr()
     cache.append(torch.zeros(B, H, 1, D), torch.zeros(B, H, 1, D))
     assert cache.past_key_value[0].data_ptr() == before
+
+
+def test_ring_storage_bookkeeping_matches_the_restated_store_in_cache():
+    # MemLMCacheStorage.store_in_cache on CPU tensors against oracle/mem_cache.RingStore
+    # (lm_benchmark/models/caches/mem_cache.py:111-158): counters and buffer contents after every chunk
+    from landmark_hip.mem_cache import MemLMCacheStorage
+    from oracle import mem_cache as omc
+    for cap, block, chunks in [(4, 3, [3, 3, 6, 3, 9]), (4, 3, [5, 2, 8, 1, 1, 1, 13]), (3, 4, [40]), (3, 4, [4, 20, 4]),
+                               (5, 2, [2] * 7)]:
+        B, nh, hs = 2, 3, 8
+        s = MemLMCacheStorage(B, cap, block - 1, nh, hs, dtype=torch.float32, device="cpu")
+        r = omc.RingStore(B, cap, block, nh, hs)
+        g = torch.Generator().manual_seed(cap)
+        seen = 0
+        for T in chunks:
+            k, v = torch.randn(B, nh, T, hs, generator=g), torch.randn(B, nh, T, hs, generator=g)
+            im = ((torch.arange(T) + seen) % block == block - 1)[None].expand(B, T)
+            s.store_in_cache(k, {"v": v, "is_mem": im})
+            r.store(k, v, im)
+            seen += T
+            n = r.filled
+            assert (s.cache_iter, s.cache_size, s.last_incomplete_len, s.filled) == \
+                (r.cache_iter, r.cache_size, r.last_incomplete_len, n)
+            assert torch.equal(s.cache_mem_k[:, :n], r.cache_k[:, :n]) and torch.equal(s.cache_mem_v[:, :n], r.cache_v[:, :n])
+            assert torch.equal(s.last_incomplete_k[:, :, :s.last_incomplete_len], r.pending_k)
+            assert s.oldest_slot == (int(omc.slot_ages(n, r.cache_iter).argmin()) if n else 0)
+        s.clear_state()
+        assert (s.cache_iter, s.cache_size, s.last_incomplete_len) == (0, 0, 0)
