@@ -24,6 +24,68 @@ for _p in (ROOT, os.path.join(ROOT, "landmark-attention_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_per_kernel.txt")
+COPY_KERNEL, COPY_BYTES = "__amd_rocclr_copyBuffer", 256 << 20      # the calibration copy of --traffic-probe
+
+
+def load_traffic(path=TRAFFIC_FILE):
+    """{kernel: (read_bytes, written_bytes)} per launch from the committed counter summary: lines
+    `kernel read_bytes written_bytes` behind `#` comments.  Empty when the file is missing."""
+    out = {}
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 3 and not line.startswith("#"):
+                    out[parts[0]] = (float(parts[1]), float(parts[2]))
+    except OSError:
+        pass
+    return out
+
+
+def traffic_summary(fetch_csv, write_csv):
+    """Turn the two rocprofv3 --pmc runs of `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE; counter
+    values are KiB per dispatch) into the text kept as profiles/hbm_traffic_per_kernel.txt: per kernel the
+    average over its dispatches, each counter scaled by what it reads for the 256 MiB device copy."""
+    import csv
+    import re
+
+    def per_kernel(path, counter):
+        acc = {}
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] != counter:
+                    continue
+                name = row["Kernel_Name"]
+                m = re.search(r"(lmk_\w+)", name)
+                key = m.group(1) if m else (COPY_KERNEL if COPY_KERNEL in name else None)
+                if key:
+                    acc.setdefault(key, []).append((int(row["Grid_Size"]), float(row["Counter_Value"])))
+        out = {}
+        for k, v in acc.items():       # a kernel launched at several sizes (the forward also serves the retrieval
+            big = max(g for g, _ in v)  # step's local chunk): the largest grid is the workload's own launch
+            vals = [x for g, x in v if g == big]
+            out[k] = (sum(vals) / len(vals), len(vals))
+        return out
+
+    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    f_scale = COPY_BYTES / 1024 / fetch[COPY_KERNEL][0]
+    w_scale = COPY_BYTES / 1024 / write[COPY_KERNEL][0]
+    lines = ["# HBM bytes per launch of each kernel, from two counter runs on an MI355X (one counter per run):",
+             "#   rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/pmc_fetch -o p -- python3 bench.py --traffic-probe",
+             "#   rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/pmc_write -o p -- python3 bench.py --traffic-probe",
+             "#   python3 bench.py --traffic-summary gpurun_out/pmc_fetch/p_counter_collection.csv "
+             "gpurun_out/pmc_write/p_counter_collection.csv",
+             f"# calibration: the 256 MiB device copy ({COPY_KERNEL}) reads {fetch[COPY_KERNEL][0]:.0f} KiB on FETCH_SIZE and "
+             f"{write[COPY_KERNEL][0]:.0f} KiB on WRITE_SIZE for 262144 KiB each way:",
+             f"#   FETCH_SIZE is scaled by {f_scale:.3f}, WRITE_SIZE by {w_scale:.3f}",
+             "# raw: " + "; ".join(f"{k} fetch {fetch[k][0]:.1f} KiB x{fetch[k][1]}, write {write.get(k, (0, 0))[0]:.1f} KiB"
+                                   for k in sorted(fetch) if k != COPY_KERNEL),
+             "# kernel read_bytes written_bytes"]
+    for k in sorted(fetch):
+        if k != COPY_KERNEL:
+            lines.append(f"{k} {fetch[k][0] * 1024 * f_scale:.4e} {write.get(k, (0.0, 0))[0] * 1024 * w_scale:.4e}")
+    return "\n".join(lines) + "\n"
 
 
 def _events(n):
@@ -126,10 +188,31 @@ def retrieval_bench(n=20, warm=3):
     t_step = _time_launches(lambda: retrieve_and_attend(q, (kc, vc), kl, vl, cos, sin, block, top_k), n, warm)
     gathered = H * T * top_k * block * D * 2 * 2
     alg = gathered + H * (S // block) * D * 2 + H * T * D * 2 + H * T * top_k * 8 + H * T * D * 2
+    # the dominant kernel alone: the local-chunk forward is a separate launch, so the attend step is timed with
+    # and without it through the C ABI (lmk_gather_attend against precomputed local statistics)
+    from landmark_hip import _lib
+    from landmark_hip.attention import _launch_fwd
+    lib, T4 = _lib.lib(), _lib.tensor4
+    scale = 1.0 / math.sqrt(D)
+    o_loc, L_loc, M_loc = _launch_fwd(q, kl, vl, 0, scale, block)
+    out = torch.empty_like(q)
+    stream = _lib.current_stream(dev)
+
+    def gather_only():
+        _lib.check(lib.lmk_gather_attend(T4(q), T4(kc), T4(vc), idx.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+                                         cos.stride(0), cos.shape[0], T4(o_loc), L_loc.data_ptr(), M_loc.data_ptr(), T,
+                                         T4(out), B, H, T, S, D, scale, block, top_k, 0, stream))
+    t_gather = _time_launches(gather_only, n, warm)
+    k_alg = gathered + 2 * H * T * D * 2 + H * T * top_k * 8 + H * T * D * 2     # K/V blocks, q, local out, idx; out
+    traffic = load_traffic().get("lmk_gather_attend_kernel")
     return {"workload": "config 4: H32 D128, cache 32768 tok (1024 blocks of 32), 256 queries, top-4",
             "topk_ms": t_topk, "gather_attend_ms": t_att, "whole_step_ms": t_step, "algorithmic_MB": alg / 1e6,
             "GBps_whole_step": alg / 1e6 / t_step, "GBps_gather_attend": gathered / 1e6 / t_att,
-            "frac_hbm_whole_step": alg / 1e6 / t_step / PEAK_HBM_GBS}
+            "frac_hbm_whole_step": alg / 1e6 / t_step / PEAK_HBM_GBS,
+            "roofline": {"bound": "hbm", "kernel": "lmk_gather_attend_kernel", "achieved": k_alg / 1e6 / t_gather,
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": k_alg / 1e6 / t_gather / PEAK_HBM_GBS,
+                         "traffic": sum(traffic) if traffic else None, "avg_launch_ms": t_gather,
+                         "algorithmic_MB_per_launch": k_alg / 1e6}}
 
 
 def decode_bench(n=50, warm=5):
@@ -201,10 +284,16 @@ def side_legs(n=30, warm=5):
     xq, xk = mk(Bq, H, Lq, D), mk(Bq, H, Lq, D)
     pos = torch.arange(Lq, device=dev)[None]
     t_rot = _time_launches(lambda: apply_rotary_pos_emb(xq, xk, cos, sin, pos), n, warm)
+
+    def one_tensor_at_a_time():
+        apply_rotary_pos_emb(None, xq, cos, sin, pos)
+        apply_rotary_pos_emb(None, xk, cos, sin, pos)
+    t_rot2 = _time_launches(one_tensor_at_a_time, n, warm)
     rot_bytes = 2 * 2 * xq.numel() * 2 + 2 * Lq * D * 2
     return {"per_head_selection": {"workload": "config 4 shapes, aggregate=max_over_tokens", "topk_ms": t_sel,
                                    "attend_ms": t_att},
-            "rotary": {"workload": "q and k of config 2, (2,32,2048,128) bf16 each", "ms": t_rot,
+            "rotary": {"workload": "q and k of config 2, (2,32,2048,128) bf16 each, one launch for both", "ms": t_rot,
+                       "one_launch_per_tensor_ms": t_rot2,
                        "GBps": rot_bytes / 1e6 / t_rot, "frac_hbm": rot_bytes / 1e6 / t_rot / PEAK_HBM_GBS}}
 
 
@@ -259,6 +348,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-retrieval", action="store_true")
+    ap.add_argument("--traffic-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="print the per-kernel HBM traffic table from two rocprofv3 counter CSVs and exit (no GPU needed)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="run a few steps plus a 256 MiB device copy and exit (for rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE runs: the copy's counters calibrate the kernels')")
@@ -266,6 +357,9 @@ def main():
                     help="time fwd+bwd and its three kernels at another shape instead of the headline run "
                          "(may be given several times)")
     a = ap.parse_args()
+    if a.traffic_summary:
+        sys.stdout.write(traffic_summary(*a.traffic_summary))
+        return
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; every (batch, head) slice is independent, so more GPUs "
                  "would only shard heads with no exchange step. Run with --gpus 1.")
@@ -309,6 +403,18 @@ def main():
         torch.cuda.synchronize()
         return
 
+    # Cold figure first: the same K steps timed straight after W warmup steps, with no spin-up in front, the way
+    # a caller that has just started sees them (reported as `cold_ms_per_step`; never the headline).
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    c0, c1 = _events(2)
+    c0.record()
+    for _ in range(a.steps):
+        step()
+    c1.record()
+    torch.cuda.synchronize()
+    cold_ms = c0.elapsed_time(c1) / a.steps
     # The GPU leaves its idle power state only after some tens of milliseconds of work (a 25-step run reads
     # 20 % slower than a 250-step one), so a fixed, untimed spin-up of the same step precedes the W warmup
     # steps; its length is reported as `spinup_steps`.
@@ -365,10 +471,11 @@ def main():
     t_dom, f_dom = kernels[dom]
     achieved = f_dom / (t_dom * 1e-3) / 1e12
     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --traffic-probe`,
-    # each scaled by what the same counter reads for a 256 MiB device copy (the summary is kept under profiles/)
-    measured_traffic = {"lmk_fwd32_kernel": 183.6e6, "lmk_bwd_dq32_kernel": 344.0e6, "lmk_bwd_dkdv32_kernel": 357.5e6}
+    # each scaled by what the same counter reads for a 256 MiB device copy: read from the committed summary
+    # (profiles/hbm_traffic_per_kernel.txt, written by `bench.py --traffic-summary`), null without it
+    traffic = load_traffic().get(dom)
     roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_BF16_TFLOPS, "traffic": measured_traffic.get(dom), "avg_launch_ms": t_dom,
+                "frac": achieved / PEAK_BF16_TFLOPS, "traffic": sum(traffic) if traffic else None, "avg_launch_ms": t_dom,
                 "algorithmic_gflop_per_launch": f_dom / 1e9}
     line = {
         "metric": "landmark-attn fwd+bwd TFLOP/s + % MFMA peak @ B2 H32 L2048 D128 bf16",
@@ -379,6 +486,7 @@ def main():
                                "block=32, q,k,v ~ N(0,1)*0.5, dO ~ N(0,1), seed 0"},
         "frac_of_mfma_peak": value / PEAK_BF16_TFLOPS,
         "spinup_steps": spinup_steps,
+        "cold_ms_per_step": cold_ms,
         "tokens_per_s": B * L / (ms_per_step * 1e-3),
         # block 32: delta and mhat (the reference's _bwd_preprocess) are computed inside the dQ kernel
         "kernel_ms": {"lmk_fwd32_kernel": t_fwd, "lmk_bwd_dq32_kernel": t_dq, "lmk_bwd_dkdv32_kernel": t_dkdv,

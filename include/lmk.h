@@ -306,6 +306,15 @@ int lmk_apply_rotary(const lmk_tensor4* x, const lmk_tensor4* out, const void* c
                      int64_t table_stride_row, int64_t n_pos, const int64_t* position_ids, int64_t pos_stride_b, int B,
                      int H, int L, int D, int dtype, void* stream);
 
+/* The layer's own call, apply_rotary_pos_emb(query_states, key_states, cos, sin, position_ids)
+ * (llama/llama_mem.py:298): q and k, both (B,H,L,D), rotated in ONE launch, each thread using the
+ * table rows it fetched for both tensors.  Same bits as two lmk_apply_rotary calls.  Outputs may
+ * alias their inputs. */
+int lmk_apply_rotary_qk(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* q_out, const lmk_tensor4* k_out,
+                        const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
+                        const int64_t* position_ids, int64_t pos_stride_b, int B, int H, int L, int D, int dtype,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -552,6 +552,30 @@ int lmk_apply_rotary(const lmk_tensor4* x, const lmk_tensor4* out, const void* c
   return lmk::launch_rotary(p, D, dtype, (hipStream_t)stream);
 }
 
+int lmk_apply_rotary_qk(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* q_out, const lmk_tensor4* k_out,
+                        const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
+                        const int64_t* position_ids, int64_t pos_stride_b, int B, int H, int L, int D, int dtype,
+                        void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(q_out)) || (rc = check_tensor(k_out))) return rc;
+  if (cos_table == nullptr || sin_table == nullptr || position_ids == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
+  if (B <= 0 || H <= 0 || L <= 0 || pos_stride_b < 0) return LMK_ERR_SHAPE;
+  if (!(D == 64 || D == 128)) return LMK_ERR_UNSUPPORTED;
+  if (!(dtype == LMK_DTYPE_BF16 || dtype == LMK_DTYPE_F16)) return LMK_ERR_UNSUPPORTED;
+  if (n_pos < 1) return LMK_ERR_TABLE;
+  lmk::RotaryParams p = {};
+  p.x = q->ptr; p.out = q_out->ptr; p.x2 = k->ptr; p.out2 = k_out->ptr; p.cos = cos_table; p.sin = sin_table;
+  p.pos = position_ids; p.pos_stride_b = pos_stride_b; p.n_pos = n_pos;
+  p.B = B; p.H = H; p.L = L;
+  p.xs_b = q->stride_b; p.xs_h = q->stride_h; p.xs_r = q->stride_row;
+  p.os_b = q_out->stride_b; p.os_h = q_out->stride_h; p.os_r = q_out->stride_row;
+  p.x2s_b = k->stride_b; p.x2s_h = k->stride_h; p.x2s_r = k->stride_row;
+  p.o2s_b = k_out->stride_b; p.o2s_h = k_out->stride_h; p.o2s_r = k_out->stride_row;
+  p.cs_r = table_stride_row;
+  return lmk::launch_rotary(p, D, dtype, (hipStream_t)stream);
+}
+
 // ---- the attend step as one call: local window, fused forward on it, gather + attend ----
 namespace {
 struct AttendLayout {

@@ -102,6 +102,9 @@ struct WindowParams {
 struct RotaryParams {
   const void *x, *cos, *sin;
   void* out;
+  const void* x2;                                 // optional second tensor of the same shape, rotated alongside
+  void* out2;
+  int64_t x2s_b, x2s_h, x2s_r, o2s_b, o2s_h, o2s_r;
   const int64_t* pos;
   int64_t pos_stride_b, n_pos;
   int B, H, L;

@@ -1233,8 +1233,10 @@ static int launch_window_t(const WindowParams& p, hipStream_t stream) {
 // (apply_rotary_pos_emb, llama_mem.py:134-149): x*cos + rotate_half(x)*sin with the model dtype's
 // rounding after each of the three elementwise operations.  One 16-byte chunk per thread; a row's
 // chunks sit in one wave and every lane loads before any lane stores, so out may be x itself.
+// PAIR: a second tensor of the same shape (the layer's q and k, :298) is rotated by the same thread with the
+// same table rows, in the same launch.
 // ---------------------------------------------------------------------------
-template <class T, int D>
+template <class T, int D, bool PAIR>
 __global__ __launch_bounds__(256) void lmk_rotary_kernel(RotaryParams p) {
   constexpr int LPR = D / 8;
   constexpr int RPW = 256 / LPR;
@@ -1249,19 +1251,32 @@ __global__ __launch_bounds__(256) void lmk_rotary_kernel(RotaryParams p) {
   const char* src = (const char*)p.x + 2 * (b * p.xs_b + hh * p.xs_h + (int64_t)l * p.xs_r);
   const u32x4_t x = *(const u32x4_t*)(src + 16 * j);
   const u32x4_t other = *(const u32x4_t*)(src + 16 * (j ^ (LPR / 2)));
+  u32x4_t x2 = {0, 0, 0, 0}, other2 = {0, 0, 0, 0};
+  if (PAIR) {                                                     // the second tensor's row at the same (b, h, l)
+    const char* src2 = (const char*)p.x2 + 2 * (b * p.x2s_b + hh * p.x2s_h + (int64_t)l * p.x2s_r);
+    x2 = *(const u32x4_t*)(src2 + 16 * j);
+    other2 = *(const u32x4_t*)(src2 + 16 * (j ^ (LPR / 2)));
+  }
   const u32x4_t c = *(const u32x4_t*)((const char*)p.cos + 2 * (pos * p.cs_r) + 16 * j);
   const u32x4_t s = *(const u32x4_t*)((const char*)p.sin + 2 * (pos * p.cs_r) + 16 * j);
   float o[8];
   rotate_chunk<T>(x, other, c, s, j >= LPR / 2, o);
   const u32x4_t r = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
   *(u32x4_t*)((char*)p.out + 2 * (b * p.os_b + hh * p.os_h + (int64_t)l * p.os_r) + 16 * j) = r;
+  if (PAIR) {
+    rotate_chunk<T>(x2, other2, c, s, j >= LPR / 2, o);
+    const u32x4_t r2 = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
+    *(u32x4_t*)((char*)p.out2 + 2 * (b * p.o2s_b + hh * p.o2s_h + (int64_t)l * p.o2s_r) + 16 * j) = r2;
+  }
 }
 
 template <class T, int D>
 static int launch_rotary_t(const RotaryParams& p, hipStream_t stream) {
   constexpr int RPW = 256 / (D / 8);
   const int64_t rows = (int64_t)p.B * p.H * p.L;
-  hipLaunchKernelGGL((lmk_rotary_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
+  const dim3 grid((unsigned)((rows + RPW - 1) / RPW));
+  if (p.x2 != nullptr) hipLaunchKernelGGL((lmk_rotary_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((lmk_rotary_kernel<T, D, false>), grid, dim3(256), 0, stream, p);
   return (int)hipGetLastError();
 }
 

@@ -3,7 +3,7 @@
 ``apply_rotary_pos_emb(q, k, cos, sin, position_ids)`` mirrors ``llama/llama_mem.py:134-149``:
 ``cos``/``sin`` are the ``(1, 1, n_pos, hd)`` (or ``(n_pos, hd)``) model-dtype tables of
 ``LlamaRotaryEmbedding`` (``:95-124``), ``position_ids`` is ``(bs, seq)`` or ``(1, seq)`` int64, ``q`` may
-be ``None`` (``:143-144``).  One launch per tensor replaces the reference's gather of the table rows,
+be ``None`` (``:143-144``).  One launch for q and k together (one per tensor when their shapes differ) replaces the reference's gather of the table rows,
 two products, ``rotate_half``'s concatenation and the sum, and gives the same bits: every one of the
 three elementwise operations rounds to the model dtype, as torch's 16-bit arithmetic does.
 """
@@ -37,5 +37,22 @@ def apply_rotary_pos_emb(q, k, cos, sin, position_ids):
     ``q`` is.  q, k: ``(B, nh, L, hd)`` bf16/fp16 on the GPU with hd 64 or 128."""
     assert k.is_cuda and k.dtype in _lib.DTYPE_CODES
     cos, sin = _tables(cos, sin, k.dtype)
-    q_embed = None if q is None else _rotate(q, cos, sin, position_ids)
-    return q_embed, _rotate(k, cos, sin, position_ids)
+    if q is None:
+        return None, _rotate(k, cos, sin, position_ids)
+    if q.shape != k.shape:                      # e.g. fewer key heads: one launch per tensor
+        return _rotate(q, cos, sin, position_ids), _rotate(k, cos, sin, position_ids)
+    B, H, L, D = q.shape
+    assert q.dtype == k.dtype and q.device == k.device
+    assert position_ids.dim() == 2 and position_ids.shape[1] == L and position_ids.shape[0] in (1, B)
+    assert position_ids.dtype == torch.int64 and position_ids.device == q.device
+    q, k = _lib.kernel_ready(q), _lib.kernel_ready(k)
+    position_ids = position_ids.contiguous()
+    q_embed, k_embed = torch.empty_like(q), torch.empty_like(k)
+    with _lib.on_device(q.device):
+        rc = _lib.lib().lmk_apply_rotary_qk(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(q_embed),
+                                            _lib.tensor4(k_embed), cos.data_ptr(), sin.data_ptr(), cos.stride(0),
+                                            cos.shape[0], position_ids.data_ptr(),
+                                            L if position_ids.shape[0] == B and B > 1 else 0, B, H, L, D,
+                                            _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+    _lib.check(rc)
+    return q_embed, k_embed
