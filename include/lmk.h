@@ -191,7 +191,7 @@ int lmk_retrieve_topk_static(const lmk_tensor4* q, const lmk_tensor4* kcache, co
  *   are dense; larger when they are the last T columns of a wider window's statistics)
  *   (q against the T new keys/values); out: (B,H,T,D) final attention output.
  * Blocks are read in place from the cache; nothing of size (T, k*block, D) is materialised.
- * Built for D = 128 and block 32, 64 or 128. */
+ * Built for D = 64 and 128 and block 32, 64 or 128. */
 int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
                       const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
                       const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, int64_t stat_stride,

@@ -426,7 +426,7 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
     return LMK_ERR_NULL;
   if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
   if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
-  if (D != 128 || !(block == 32 || block == 64 || block == 128)) return LMK_ERR_UNSUPPORTED;
+  if (!(block == 32 || block == 64 || block == 128)) return LMK_ERR_UNSUPPORTED;
   if (stat_stride < T) return LMK_ERR_SHAPE;
   if (!std::isfinite(sm_scale) || !(sm_scale > 0.f)) return LMK_ERR_SCALE;
   lmk::RetrParams p = {};
@@ -612,7 +612,7 @@ int attend_precheck(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_t
   if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row) || !aligned16(workspace))
     return LMK_ERR_ALIGN;
   if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
-  if (D != 128 || !(block == 32 || block == 64 || block == 128)) return LMK_ERR_UNSUPPORTED;   // gather + attend, fused forward
+  if (!(block == 32 || block == 64 || block == 128)) return LMK_ERR_UNSUPPORTED;   // gather + attend, fused forward
   if (!std::isfinite(sm_scale) || !(sm_scale > 0.f)) return LMK_ERR_SCALE;
   const int inc = S % block;
   if (inc && T + inc > block) return LMK_ERR_SHAPE;             // llama_mem.py:330

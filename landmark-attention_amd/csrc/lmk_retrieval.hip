@@ -844,7 +844,7 @@ __device__ __forceinline__ float sum8(float d) {                  // sum over th
 }
 
 // One wave per query row.  Eight lanes share a key: lane j of the group holds head dims 8j..8j+7 and
-// 64+8j..64+8j+7, i.e. both partners of the rotary pair, so the rotation needs no exchange between
+// 64+8j..64+8j+7 (head dim 128; 4j..4j+3 and 32+4j..32+4j+3 at head dim 64), i.e. both partners of the rotary pair, so the rotation needs no exchange between
 // lanes; the eight key groups of the wave take keys g, g+8, .. of a block.  Rotation and scores are
 // evaluated in fp32 from the 16-bit cache and table values (the reference rounds the rotated key to
 // the model dtype first; the difference is far inside the 2e-2 bound of this step, and selection --
@@ -853,9 +853,16 @@ __device__ __forceinline__ float sum8(float d) {                  // sum over th
 // (scores of the whole block, which the block's softmax needs before any weight is final), then the
 // values, so keys and values are never live together and the kernel keeps several waves per SIMD.  The
 // loads of the next chunk are issued before the arithmetic on the current one.
+template <int E> struct PieceVec;
+template <> struct PieceVec<8> { using type = u32x4_t; };
+template <> struct PieceVec<4> { using type = u32x2_t; };
+
 template <class T, int D, int BS, bool SPLIT>
 __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
-  static_assert(D == 128 && (BS == 32 || BS % 64 == 0), "16 chunks of 8 head dims per row; whole chunks of keys");
+  static_assert((D == 128 || D == 64) && (BS == 32 || BS % 64 == 0), "8 lanes x 2 pieces per row; whole chunks of keys");
+  constexpr int E = D / 16;                                       // head dims per lane and rotary half: 8 or 4
+  constexpr int PB = 2 * E;                                       // bytes of one piece
+  using vec_t = typename PieceVec<E>::type;                       // one piece: E 16-bit values
   constexpr int CK = BS < 64 ? BS : 64;                           // keys per chunk
   constexpr int KPG = CK / 8;                                     // keys per 8-lane group and chunk
   constexpr int NC = BS / CK;                                     // chunks per block
@@ -869,39 +876,39 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   const int bh = (int)(row / p.T), t = (int)(row % p.T);
   const int b = bh / p.H, hh = bh % p.H;
 
-  auto unpack8 = [](const u32x4_t u, float* o) {
+  auto unpack8 = [](const vec_t u, float* o) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < E / 2; ++i) {
       o[2 * i] = unpack_lo<T>(u[i]);
       o[2 * i + 1] = unpack_hi<T>(u[i]);
     }
   };
-  float qlo[8], qhi[8];
+  float qlo[E], qhi[E];
   {
     const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
-    unpack8(*(const u32x4_t*)(qp + 16 * j), qlo);
-    unpack8(*(const u32x4_t*)(qp + 128 + 16 * j), qhi);
+    unpack8(*(const vec_t*)(qp + PB * j), qlo);
+    unpack8(*(const vec_t*)(qp + D + PB * j), qhi);
   }
   const char* kc = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h);
   const char* vc = (const char*)p.vcache + 2 * (b * p.vcs_b + hh * p.vcs_h);
   const float c2 = p.scale_log2;
 
   float Mrun = -INFINITY, lrun = 0.f;
-  float alo[8], ahi[8];
+  float alo[E], ahi[E];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < E; ++i) {
     alo[i] = 0.f;
     ahi[i] = 0.f;
   }
 
   // one chunk = CK rows of K or of V: this lane's KPG rows (g, g+8, ..) x its two 16-byte pieces
-  u32x4_t clo[KPG], chi[KPG], nlo[KPG], nhi[KPG];
+  vec_t clo[KPG], chi[KPG], nlo[KPG], nhi[KPG];
   auto fetch = [&](const char* base, int64_t row_stride, int64_t key0) {
 #pragma unroll
     for (int i = 0; i < KPG; ++i) {
-      const char* r = base + 2 * ((key0 + g + 8 * i) * row_stride) + 16 * j;
-      nlo[i] = *(const u32x4_t*)(r);
-      nhi[i] = *(const u32x4_t*)(r + 128);
+      const char* r = base + 2 * ((key0 + g + 8 * i) * row_stride) + PB * j;
+      nlo[i] = *(const vec_t*)(r);
+      nhi[i] = *(const vec_t*)(r + D);
     }
   };
   auto take = [&]() {
@@ -928,18 +935,18 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
 #pragma unroll
       for (int i = 0; i < KPG; ++i) {
         const int kk = CK * c + g + 8 * i;
-        const char* cr = (const char*)p.cos + 2 * ((pos0 + kk) * p.cs_r) + 16 * j;
-        const char* sr = (const char*)p.sin + 2 * ((pos0 + kk) * p.cs_r) + 16 * j;
-        float kl[8], kh[8], cl[8], ch[8], sl[8], sh[8];
+        const char* cr = (const char*)p.cos + 2 * ((pos0 + kk) * p.cs_r) + PB * j;
+        const char* sr = (const char*)p.sin + 2 * ((pos0 + kk) * p.cs_r) + PB * j;
+        float kl[E], kh[E], cl[E], ch[E], sl[E], sh[E];
         unpack8(clo[i], kl);
         unpack8(chi[i], kh);
-        unpack8(*(const u32x4_t*)(cr), cl);
-        unpack8(*(const u32x4_t*)(cr + 128), ch);
-        unpack8(*(const u32x4_t*)(sr), sl);
-        unpack8(*(const u32x4_t*)(sr + 128), sh);
+        unpack8(*(const vec_t*)(cr), cl);
+        unpack8(*(const vec_t*)(cr + D), ch);
+        unpack8(*(const vec_t*)(sr), sl);
+        unpack8(*(const vec_t*)(sr + D), sh);
         float d = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < E; ++e) {
           const float rl = __builtin_fmaf(kl[e], cl[e], -kh[e] * sl[e]);
           const float rh = __builtin_fmaf(kh[e], ch[e], kl[e] * sh[e]);
           d = __builtin_fmaf(qlo[e], rl, d);
@@ -975,7 +982,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     Mrun = Mnew;
     const float f = gate / den;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
+    for (int e = 0; e < E; ++e) {
       alo[e] *= alpha;
       ahi[e] *= alpha;
     }
@@ -990,7 +997,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       for (int i = 0; i < KPG; ++i) {
         const float w = round_to<T>(sc[KPG * c + i] * f);         // weights enter PV in the model dtype
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
+        for (int e = 0; e < E / 2; ++e) {
           alo[2 * e] = __builtin_fmaf(w, unpack_lo<T>(clo[i][e]), alo[2 * e]);
           alo[2 * e + 1] = __builtin_fmaf(w, unpack_hi<T>(clo[i][e]), alo[2 * e + 1]);
           ahi[2 * e] = __builtin_fmaf(w, unpack_lo<T>(chi[i][e]), ahi[2 * e]);
@@ -1001,7 +1008,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     blk = blk_next;
   }
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {                                   // sum over the eight key groups
+  for (int e = 0; e < E; ++e) {                                   // sum over the eight key groups
     alo[e] += dpp_f<0x128>(alo[e]);
     ahi[e] += dpp_f<0x128>(ahi[e]);
     alo[e] += __shfl_xor(alo[e], 16, 64);
@@ -1010,13 +1017,13 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     ahi[e] += __shfl_xor(ahi[e], 32, 64);
   }
   if constexpr (SPLIT) {                                          // the four waves' partial (M, l, acc) -> wave 0
-    __shared__ float part_acc[4][128];
+    __shared__ float part_acc[4][D];
     __shared__ float part_ml[4][2];
     if (g == 0) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        part_acc[wave][8 * j + e] = alo[e];
-        part_acc[wave][64 + 8 * j + e] = ahi[e];
+      for (int e = 0; e < E; ++e) {
+        part_acc[wave][E * j + e] = alo[e];
+        part_acc[wave][D / 2 + E * j + e] = ahi[e];
       }
       if (j == 0) {
         part_ml[wave][0] = Mrun;
@@ -1030,7 +1037,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     for (int w = 1; w < 4; ++w) Mall = fmaxf(Mall, part_ml[w][0]);
     lrun = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
+    for (int e = 0; e < E; ++e) {
       alo[e] = 0.f;
       ahi[e] = 0.f;
     }
@@ -1039,9 +1046,9 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       const float sw = fast_exp2(part_ml[w][0] - Mall);           // 0 for a wave without blocks (M = -inf)
       lrun = __builtin_fmaf(part_ml[w][1], sw, lrun);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        alo[e] = __builtin_fmaf(part_acc[w][8 * j + e], sw, alo[e]);
-        ahi[e] = __builtin_fmaf(part_acc[w][64 + 8 * j + e], sw, ahi[e]);
+      for (int e = 0; e < E; ++e) {
+        alo[e] = __builtin_fmaf(part_acc[w][E * j + e], sw, alo[e]);
+        ahi[e] = __builtin_fmaf(part_acc[w][D / 2 + E * j + e], sw, ahi[e]);
       }
     }
     Mrun = Mall;
@@ -1053,19 +1060,22 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   const float wr = fast_exp2(Mrun - Mt), wl = fast_exp2(Ml - Mt) * Ll;
   const float inv = 1.0f / (lrun * wr + wl);
   if (g == 0) {
-    const char* olp = (const char*)p.o_loc + 2 * (b * p.ols_b + hh * p.ols_h + (int64_t)t * p.ols_r) + 16 * j;
-    char* outp = (char*)p.out + 2 * (b * p.outs_b + hh * p.outs_h + (int64_t)t * p.outs_r) + 16 * j;
-    float ol[8], o[8];
-    unpack8(*(const u32x4_t*)(olp), ol);
+    const char* olp = (const char*)p.o_loc + 2 * (b * p.ols_b + hh * p.ols_h + (int64_t)t * p.ols_r) + PB * j;
+    char* outp = (char*)p.out + 2 * (b * p.outs_b + hh * p.outs_h + (int64_t)t * p.outs_r) + PB * j;
+    float ol[E], o[E];
+    vec_t ov;
+    unpack8(*(const vec_t*)(olp), ol);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = (alo[i] * wr + ol[i] * wl) * inv;
-    u32x4_t ov = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
-    *(u32x4_t*)(outp) = ov;
-    unpack8(*(const u32x4_t*)(olp + 128), ol);
+    for (int i = 0; i < E; ++i) o[i] = (alo[i] * wr + ol[i] * wl) * inv;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = (ahi[i] * wr + ol[i] * wl) * inv;
-    u32x4_t ov2 = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
-    *(u32x4_t*)(outp + 128) = ov2;
+    for (int i = 0; i < E / 2; ++i) ov[i] = pack2<T>(o[2 * i], o[2 * i + 1]);
+    *(vec_t*)(outp) = ov;
+    unpack8(*(const vec_t*)(olp + D), ol);
+#pragma unroll
+    for (int i = 0; i < E; ++i) o[i] = (ahi[i] * wr + ol[i] * wl) * inv;
+#pragma unroll
+    for (int i = 0; i < E / 2; ++i) ov[i] = pack2<T>(o[2 * i], o[2 * i + 1]);
+    *(vec_t*)(outp + D) = ov;
   }
 }
 
@@ -1148,21 +1158,21 @@ int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landm
   return LMK_ERR_UNSUPPORTED;
 }
 
-template <class T>
+template <class T, int D>
 static int launch_gather_t(const RetrParams& p, int BS, hipStream_t stream) {
   const int64_t rows = (int64_t)p.B * p.H * p.T;
   if (rows <= 1024 && p.k > 1) {          // fewer rows than SIMDs: one workgroup per row, its waves share the blocks out
     const dim3 grid((unsigned)rows);
-    if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 32, true>), grid, dim3(256), 0, stream, p);
-    else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 64, true>), grid, dim3(256), 0, stream, p);
-    else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 128, true>), grid, dim3(256), 0, stream, p);
+    if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 32, true>), grid, dim3(256), 0, stream, p);
+    else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 64, true>), grid, dim3(256), 0, stream, p);
+    else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 128, true>), grid, dim3(256), 0, stream, p);
     else return LMK_ERR_UNSUPPORTED;
     return (int)hipGetLastError();
   }
   const dim3 grid((unsigned)((rows + 3) / 4));
-  if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 32, false>), grid, dim3(256), 0, stream, p);
-  else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 64, false>), grid, dim3(256), 0, stream, p);
-  else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, 128, 128, false>), grid, dim3(256), 0, stream, p);
+  if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 32, false>), grid, dim3(256), 0, stream, p);
+  else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 64, false>), grid, dim3(256), 0, stream, p);
+  else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 128, false>), grid, dim3(256), 0, stream, p);
   else return LMK_ERR_UNSUPPORTED;
   return (int)hipGetLastError();
 }
@@ -1303,9 +1313,13 @@ int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t str
 }
 
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream) {
-  if (D != 128) return LMK_ERR_UNSUPPORTED;
-  if (dtype == LMK_DTYPE_BF16) return launch_gather_t<bf16_t>(p, BS, stream);
-  if (dtype == LMK_DTYPE_F16) return launch_gather_t<f16_t>(p, BS, stream);
+  if (dtype == LMK_DTYPE_BF16) {
+    if (D == 128) return launch_gather_t<bf16_t, 128>(p, BS, stream);
+    if (D == 64) return launch_gather_t<bf16_t, 64>(p, BS, stream);
+  } else if (dtype == LMK_DTYPE_F16) {
+    if (D == 128) return launch_gather_t<f16_t, 128>(p, BS, stream);
+    if (D == 64) return launch_gather_t<f16_t, 64>(p, BS, stream);
+  }
   return LMK_ERR_UNSUPPORTED;
 }
 

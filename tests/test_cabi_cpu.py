@@ -116,10 +116,10 @@ def test_retrieval_argument_errors(lib):
     assert static(cos=0) == -1 and static(idx=0) == -1 and static(S=16) == -9 and static(top_k=0) == -10
     assert static(S=32768, T=256, H=32) == -8                 # benchmark config 4 needs 75 MB of workspace
     assert lib.lmk_retrieve_workspace_bytes(1, 32, 1, 32768 + 7, 128, 32) < 16 << 20      # a decode step fits
-        # gather+attend is built for D=128 and blocks of 32/64 only
-    rc = lib.lmk_gather_attend(t, t, t, 0x7000, 0x5000, 0x6000, 128, 4096, t, 0x2000, 0x3000, 8, t, 1, 1, 8, 64, 64, 0.1,
-                               32, 4, 0, None)
-    assert rc == -3
+    # gather+attend is built for head dims 64 and 128 and blocks of 32/64/128
+    ga = lambda D, block: lib.lmk_gather_attend(t, t, t, 0x7000, 0x5000, 0x6000, 128, 4096, t, 0x2000, 0x3000, 8, t, 1, 1,
+                                                8, 64, D, 0.1, block, 4, 0, None)
+    assert ga(96, 32) == -3 and ga(128, 16) == -3 and ga(64, 16) == -3
 
     # window of an incomplete cached block: needs a tail, and tail + new chunk within one block (llama_mem.py:330)
     def window(S, T):
@@ -162,7 +162,7 @@ def test_retrieval_argument_errors(lib):
                               block, 4, 0, None)
 
     for f in (both_x, attend_x):
-        assert f(D=64) == -3                                    # the gather kernel is built for D = 128
+        assert f(D=96) == -3                                    # head dims 64 and 128
         assert f(block=16) == -3                                # the fused forward for blocks of 32, 64, 128
         assert f(out=None) == -1
         assert f(idx=0) == -1

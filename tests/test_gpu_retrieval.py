@@ -96,14 +96,15 @@ def test_fp16_indices_bit_exact(T):
     assert torch.equal(got.cpu(), want)
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("B,H,T,S,block,top_k", [(1, 2, 64, 24 * 32, 32, 4), (1, 2, 128, 12 * 64, 64, 3),
                                                   (2, 2, 96, 3 * 32, 32, 5),
                                                   (1, 2, 1, 24 * 32, 32, 4),      # decode: first token of a new block
                                                   (1, 2, 5, 12 * 64, 64, 3),
                                                   (1, 2, 160, 9 * 128, 128, 3), (2, 2, 7, 2 * 128, 128, 4)])
-def test_gather_attend_matches_oracle(B, H, T, S, block, top_k):
+def test_gather_attend_matches_oracle(B, H, T, S, block, top_k, D):
     from landmark_hip.retrieval import retrieve_and_attend
-    D = 128
+    print(f"case gather B{B} H{H} T{T} S{S} bs{block} k{top_k} D{D}", flush=True)
     q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=S + T + 1)
     is_mem = (torch.arange(T) % block == block - 1)[None].expand(B, T)
     ref_bf16, idx_ref = oret.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, block, top_k)
@@ -133,11 +134,12 @@ def test_gather_attend_matches_oracle(B, H, T, S, block, top_k):
     (7, 100, 28, 128, 2),       # block 128, ends on the landmark
     (7, 5, 1, 128, 4),
 ])
-def test_incomplete_cached_block(n_mems, inc, T, block, top_k):
+@pytest.mark.parametrize("D", [128, 64])
+def test_incomplete_cached_block(n_mems, inc, T, block, top_k, D):
     from landmark_hip.retrieval import retrieve_and_attend
-    B, H, D = 2, 3, 128
+    B, H = 2, 3
     S = n_mems * block + inc
-    print(f"case tail n_mems{n_mems} inc{inc} T{T} bs{block} k{top_k}", flush=True)
+    print(f"case tail n_mems{n_mems} inc{inc} T{T} bs{block} k{top_k} D{D}", flush=True)
     q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=S + T + 2)
     is_mem = ((torch.arange(T) + inc) % block == block - 1)[None].expand(B, T)
     ref_bf16, idx_ref = oret.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, block, top_k)
