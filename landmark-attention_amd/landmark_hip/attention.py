@@ -6,6 +6,8 @@ Block sizes other than 32, 64 and 128 (the training models use ``mem_freq + 1 = 
 normal tokens in front and its landmark in the last slot, the kernels mask the slots in between,
 and the results are packed back.  Blocks wider than 128 tokens are rejected.
 
+Head dims 16 and 32 are zero-padded to 64 by ``fused_landmark_attention``.
+
 Differences a caller can observe, all of them relaxations:
 * ``is_mem=None`` is accepted and means "landmarks at fixed stride" (the reference's
   README promises this, its code dereferences ``is_mem.shape``, ``:393``);
@@ -23,6 +25,7 @@ from . import _lib
 SUPPORTED_BLOCKS = (32, 64, 128)      # block sizes the kernels run without repacking
 MAX_BLOCK = 128
 SUPPORTED_HEAD_DIMS = (64, 128)
+PADDED_HEAD_DIMS = (16, 32)          # accepted by fused_landmark_attention, zero-padded to 64
 
 
 def storage_block(block_size: int) -> int:
@@ -176,4 +179,12 @@ def fused_landmark_attention(q, k, v, is_mem, sm_scale=None, block_size=64):
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.size(-1))
 
+    d = q.size(-1)
+    if d in PADDED_HEAD_DIMS:
+        # head dims 16 and 32 (flash_landmark_attention.py:321) run on the 64-wide kernels: zero columns add
+        # nothing to a score and give zero output columns, which are dropped again; autograd differentiates
+        # through the padding and the slice
+        pad = (0, 64 - d)
+        q, k, v = (torch.nn.functional.pad(t, pad) for t in (q, k, v))
+        return FusedLandmarkAttention.apply(q, k, v, n_history_blocks, sm_scale, block_size)[..., :d]
     return FusedLandmarkAttention.apply(q, k, v, n_history_blocks, sm_scale, block_size)

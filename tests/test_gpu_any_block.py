@@ -147,3 +147,18 @@ def test_padded_entry_points_reject_what_the_kernels_do_not_cover():
     assert fwd(64, 1) == -2 and fwd(64, 65) == -2
     assert fwd(64, 64) == 0 and fwd(64, 51) == 0 and fwd(32, 32) == 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("D,block", [(32, 32), (16, 64), (32, 51)])
+def test_head_dims_16_and_32(D, block):
+    # the reference accepts head dims 16 and 32 as well (flash_landmark_attention.py:321)
+    B, H, L = 1, 3, 4 * block
+    q, k, v = make_qkv(B, H, L, L, D, seed=D + block)
+    do = torch.randn(B, H, L, D, generator=torch.Generator().manual_seed(5)).bfloat16()
+    ref, _, _ = oracle_forward(q, k, v, block)
+    rq, rk, rv = oracle_grads(q, k, v, do, block)
+    out, (gq, gk, gv) = _run(q, k, v, do, block)
+    assert out.shape == q.shape
+    assert (out.float().cpu() - ref).abs().max().item() <= TOL
+    for g, r in ((gq, rq), (gk, rk), (gv, rv)):
+        assert g.shape == r.shape and (g.float().cpu() - r).abs().max().item() <= TOL
