@@ -289,11 +289,28 @@ def side_legs(n=30, warm=5):
         apply_rotary_pos_emb(None, xq, cos, sin, pos)
         apply_rotary_pos_emb(None, xk, cos, sin, pos)
     t_rot2 = _time_launches(one_tensor_at_a_time, n, warm)
+    # inference prefill of config 2's shape: rotary of q and k, then the forward -- against rotary of k alone and the
+    # forward that rotates q as it loads it
+    from landmark_hip.attention import fused_landmark_attention_rotary_q
+    from ltriton.flash_landmark_attention import fused_landmark_attention
+    xv = mk(Bq, H, Lq, D)
+
+    def prefill_two_pass():
+        qr, kr = apply_rotary_pos_emb(xq, xk, cos, sin, pos)
+        fused_landmark_attention(qr, kr, xv, None, block_size=block)
+
+    def prefill_q_in_prologue():
+        _, kr = apply_rotary_pos_emb(None, xk, cos, sin, pos)
+        fused_landmark_attention_rotary_q(xq, kr, xv, cos, sin, pos, block_size=block)
+    with torch.no_grad():
+        t_pre2 = _time_launches(prefill_two_pass, n, warm)
+        t_pre1 = _time_launches(prefill_q_in_prologue, n, warm)
     rot_bytes = 2 * 2 * xq.numel() * 2 + 2 * Lq * D * 2
     return {"per_head_selection": {"workload": "config 4 shapes, aggregate=max_over_tokens", "topk_ms": t_sel,
                                    "attend_ms": t_att},
             "rotary": {"workload": "q and k of config 2, (2,32,2048,128) bf16 each, one launch for both", "ms": t_rot,
                        "one_launch_per_tensor_ms": t_rot2,
+                       "prefill_rotary_qk_then_forward_ms": t_pre2, "prefill_rotary_k_then_forward_rotating_q_ms": t_pre1,
                        "GBps": rot_bytes / 1e6 / t_rot, "frac_hbm": rot_bytes / 1e6 / t_rot / PEAK_HBM_GBS}}
 
 

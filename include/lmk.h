@@ -64,6 +64,17 @@ int lmk_attn_fwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* 
                  float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
                  int n_prefix, int dtype, void* stream);
 
+/* Forward pass for callers that do not differentiate (inference prefill): q arrives WITHOUT rotary and is
+ * rotated in registers as the kernel loads it, at positions position_ids[b*pos_stride_b + row] (device
+ * int64; pos_stride_b = 0 shares one row of positions over the batch), with the same three roundings
+ * as lmk_apply_rotary -- the output equals lmk_attn_fwd on the rotated q bit for bit, and q's own pass
+ * of apply_rotary_pos_emb (llama/llama_mem.py:298) disappears.  k must already carry its rotary (its
+ * rows reach LDS by direct loads that cannot rotate them).  Tables as for lmk_apply_rotary. */
+int lmk_attn_fwd_rotary_q(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                          float* L, float* M, const void* cos_table, const void* sin_table, int64_t table_stride_row,
+                          int64_t n_pos, const int64_t* position_ids, int64_t pos_stride_b, int B, int H, int Lq, int Lk,
+                          int D, float sm_scale, int block, int n_prefix, int dtype, void* stream);
+
 /* Bytes of device workspace lmk_attn_bwd needs (0 for invalid sizes):
  * 2*(B*H*Lq) floats of per-row terms + 3*(B*H*(Lk/block)*Lq) floats of per-(row, block)
  * terms handed from the dQ kernel to the dK/dV kernel. */

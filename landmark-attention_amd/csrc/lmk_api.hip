@@ -182,9 +182,16 @@ static int check_block_real(int block, int block_real) {
   return LMK_OK;
 }
 
+struct RopeArgs {
+  const void *cos, *sin;
+  int64_t stride_row, n_pos;
+  const int64_t* pos;
+  int64_t pos_stride_b;
+};
+
 static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                          float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
-                         int block_real, int n_prefix, int dtype, void* stream) {
+                         int block_real, int n_prefix, int dtype, void* stream, const RopeArgs* rope = nullptr) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o))) return rc;
   if (L == nullptr || M == nullptr) return LMK_ERR_NULL;
@@ -192,7 +199,17 @@ static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
   if ((rc = check_block_real(block, block_real))) return rc;
   if (!slice_fits_32bit(q, Lq) || !slice_fits_32bit(o, Lq) || !slice_fits_32bit(k, Lk) || !slice_fits_32bit(v, Lk))
     return LMK_ERR_UNSUPPORTED;
-  lmk::FwdParams p;
+  if (rope != nullptr) {
+    if (rope->cos == nullptr || rope->sin == nullptr || rope->pos == nullptr) return LMK_ERR_NULL;
+    if (!aligned16(rope->cos) || !aligned16(rope->sin) || !stride_ok(rope->stride_row)) return LMK_ERR_ALIGN;
+    if (rope->pos_stride_b < 0) return LMK_ERR_SHAPE;
+    if (rope->n_pos < 1) return LMK_ERR_TABLE;
+  }
+  lmk::FwdParams p = {};
+  if (rope != nullptr) {
+    p.rope_cos = rope->cos; p.rope_sin = rope->sin; p.rope_pos = rope->pos;
+    p.rope_pos_stride_b = rope->pos_stride_b; p.rope_cs_r = rope->stride_row; p.rope_n_pos = rope->n_pos;
+  }
   p.n_real = block_real;
   p.q = q->ptr; p.k = k->ptr; p.v = v->ptr; p.o = o->ptr;
   p.L = L; p.M = M;
@@ -217,6 +234,14 @@ int lmk_attn_fwd_padded(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
                         float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
                         int block_real, int n_prefix, int dtype, void* stream) {
   return attn_fwd_impl(q, k, v, o, L, M, B, H, Lq, Lk, D, sm_scale, block, block_real, n_prefix, dtype, stream);
+}
+
+int lmk_attn_fwd_rotary_q(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                          float* L, float* M, const void* cos_table, const void* sin_table, int64_t table_stride_row,
+                          int64_t n_pos, const int64_t* position_ids, int64_t pos_stride_b, int B, int H, int Lq, int Lk,
+                          int D, float sm_scale, int block, int n_prefix, int dtype, void* stream) {
+  const RopeArgs rope = {cos_table, sin_table, table_stride_row, n_pos, position_ids, pos_stride_b};
+  return attn_fwd_impl(q, k, v, o, L, M, B, H, Lq, Lk, D, sm_scale, block, block, n_prefix, dtype, stream, &rope);
 }
 
 int64_t lmk_padded_rows(int64_t rows, int block_real, int block) {

@@ -162,4 +162,50 @@ __device__ __forceinline__ u32x4_t load_row_frag(const unsigned char* kbuf, int 
   return *(const u32x4_t*)(kbuf + tile_off<D>(row, 2 * ks + (lane >> 5)));
 }
 
+template <class T>
+__device__ __forceinline__ float round_to(float x) {  // fp32 -> T (RNE) -> fp32
+  return unpack_lo<T>(pack2<T>(x, 0.f));
+}
+
+// rotary on 8 consecutive head dims held as 4 packed dwords; `other` holds the chunk D/2 away
+template <class T>
+__device__ __forceinline__ void rotate_chunk(const u32x4_t x, const u32x4_t other, const u32x4_t c, const u32x4_t s,
+                                             bool upper_half, float* out) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float x0 = unpack_lo<T>(x[i]), x1 = unpack_hi<T>(x[i]);
+    float r0 = unpack_lo<T>(other[i]), r1 = unpack_hi<T>(other[i]);
+    if (!upper_half) {  // rotate_half: first half gets -x[d + D/2], second half gets x[d - D/2]
+      r0 = -r0;
+      r1 = -r1;
+    }
+    float a0 = round_to<T>(x0 * unpack_lo<T>(c[i])), a1 = round_to<T>(x1 * unpack_hi<T>(c[i]));
+    float b0 = round_to<T>(r0 * unpack_lo<T>(s[i])), b1 = round_to<T>(r1 * unpack_hi<T>(s[i]));
+    // The rounded products are opaque to the compiler: with f16 it would otherwise turn
+    // round(round(x*c) + round(r*s)) into a half-precision fused multiply-add, which skips a rounding.
+    asm volatile("" : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
+    out[2 * i] = round_to<T>(a0 + b0);
+    out[2 * i + 1] = round_to<T>(a1 + b1);
+  }
+}
+
+// Rotary embedding of a wave's Q (or K) operand fragments in registers: fragment ks of a lane holds head dims
+// 16 ks + 8 h .. + 7 of its row, whose rotary partners (D/2 away) sit in fragment ks ^ (KS/2) of the same lane.
+// cos_row / sin_row: the row's table rows (D values each).  Same three roundings as rotate_chunk.
+template <class T, int KS>
+__device__ __forceinline__ void rotate_fragments(u32x4_t* f, const char* cos_row, const char* sin_row, int h) {
+  u32x4_t raw[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) raw[ks] = f[ks];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const u32x4_t c = *(const u32x4_t*)(cos_row + 16 * (2 * ks + h));
+    const u32x4_t s = *(const u32x4_t*)(sin_row + 16 * (2 * ks + h));
+    float o[8];
+    rotate_chunk<T>(raw[ks], raw[ks ^ (KS / 2)], c, s, ks >= KS / 2, o);
+    const u32x4_t r = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
+    f[ks] = r;
+  }
+}
+
 }  // namespace lmk

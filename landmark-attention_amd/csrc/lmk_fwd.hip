@@ -88,6 +88,11 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
     qf[ks] = z;
     if (qrow < p.Lq) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
   }
+  if (p.rope_cos != nullptr && qrow < p.Lq) {                      // q without rotary: rotate the fragments at the row's position
+    int64_t pos = p.rope_pos[(int64_t)b * p.rope_pos_stride_b + qrow];
+    pos = pos < 0 ? 0 : (pos >= p.rope_n_pos ? p.rope_n_pos - 1 : pos);
+    rotate_fragments<T, C::KS>(qf, (const char*)p.rope_cos + 2 * pos * p.rope_cs_r, (const char*)p.rope_sin + 2 * pos * p.rope_cs_r, h);
+  }
 
   // ---- stages of SK keys (one or two landmark blocks), up to the own block of the workgroup's last
   // query tile.  K and V rows come by direct global->LDS loads, requested one stage ahead, each wave its

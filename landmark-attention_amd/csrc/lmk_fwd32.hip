@@ -102,6 +102,11 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
     qf[ks] = z;
     if (rowok) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
   }
+  if (p.rope_cos != nullptr && rowok) {                      // q without rotary: rotate the fragments at the row's position
+    int64_t pos = p.rope_pos[(int64_t)b_ * p.rope_pos_stride_b + qrow];
+    pos = pos < 0 ? 0 : (pos >= p.rope_n_pos ? p.rope_n_pos - 1 : pos);
+    rotate_fragments<T, C::KS>(qf, (const char*)p.rope_cos + 2 * pos * p.rope_cs_r, (const char*)p.rope_sin + 2 * pos * p.rope_cs_r, h);
+  }
 
   // row fragment ks of a tile sits at tile_off(ql, 2 ks + h) = tile_off(ql, h) ^ (32 ks): the swizzle
   // is an XOR on the 16-byte chunk index and 2 ks only touches bits the row term leaves zero

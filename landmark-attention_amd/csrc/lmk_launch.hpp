@@ -35,6 +35,10 @@ struct FwdParams {
   int n_prefix;   // history blocks in front of the queries
   int n_qtiles;   // ceil(Lq / 128)
   int n_real;     // tokens of a block that exist (normal keys in front, landmark last); == block unless padded
+  // optional: q arrives without rotary and is rotated as it is loaded (null tables: q is used as it is)
+  const void *rope_cos, *rope_sin;
+  const int64_t* rope_pos;        // position of query row r of batch b: rope_pos[b * rope_pos_stride_b + r]
+  int64_t rope_pos_stride_b, rope_cs_r, rope_n_pos;
   int64_t qs_b, qs_h, qs_r, ks_b, ks_h, ks_r, vs_b, vs_h, vs_r, os_b, os_h, os_r;  // element strides
   float scale_log2;  // sm_scale * log2(e)
 };

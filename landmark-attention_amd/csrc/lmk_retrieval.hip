@@ -25,33 +25,6 @@
 
 namespace lmk {
 
-template <class T>
-__device__ __forceinline__ float round_to(float x) {  // fp32 -> T (RNE) -> fp32
-  return unpack_lo<T>(pack2<T>(x, 0.f));
-}
-
-// rotary on 8 consecutive head dims held as 4 packed dwords; `other` holds the chunk D/2 away
-template <class T>
-__device__ __forceinline__ void rotate_chunk(const u32x4_t x, const u32x4_t other, const u32x4_t c, const u32x4_t s,
-                                             bool upper_half, float* out) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float x0 = unpack_lo<T>(x[i]), x1 = unpack_hi<T>(x[i]);
-    float r0 = unpack_lo<T>(other[i]), r1 = unpack_hi<T>(other[i]);
-    if (!upper_half) {  // rotate_half: first half gets -x[d + D/2], second half gets x[d - D/2]
-      r0 = -r0;
-      r1 = -r1;
-    }
-    float a0 = round_to<T>(x0 * unpack_lo<T>(c[i])), a1 = round_to<T>(x1 * unpack_hi<T>(c[i]));
-    float b0 = round_to<T>(r0 * unpack_lo<T>(s[i])), b1 = round_to<T>(r1 * unpack_hi<T>(s[i]));
-    // The rounded products are opaque to the compiler: with f16 it would otherwise turn
-    // round(round(x*c) + round(r*s)) into a half-precision fused multiply-add, which skips a rounding.
-    asm volatile("" : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
-    out[2 * i] = round_to<T>(a0 + b0);
-    out[2 * i + 1] = round_to<T>(a1 + b1);
-  }
-}
-
 __device__ __forceinline__ u32x4_t shfl_xor4(u32x4_t v, int mask) {
   u32x4_t r;
 #pragma unroll

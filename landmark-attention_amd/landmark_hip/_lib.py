@@ -100,6 +100,8 @@ def lib() -> ctypes.CDLL:
                                         i, i, i, i, i, i, i, i, vp]
         L.lmk_apply_rotary.restype = i
         L.lmk_apply_rotary.argtypes = [T4, T4, vp, vp, i64, i64, vp, i64, i, i, i, i, i, vp]
+        L.lmk_attn_fwd_rotary_q.restype = i
+        L.lmk_attn_fwd_rotary_q.argtypes = [T4, T4, T4, T4, vp, vp, vp, vp, i64, i64, vp, i64, i, i, i, i, i, f, i, i, i, vp]
         L.lmk_apply_rotary_qk.restype = i
         L.lmk_apply_rotary_qk.argtypes = [T4, T4, T4, T4, vp, vp, i64, i64, vp, i64, i, i, i, i, i, vp]
         _lib = L

@@ -188,3 +188,40 @@ def fused_landmark_attention(q, k, v, is_mem, sm_scale=None, block_size=64):
         q, k, v = (torch.nn.functional.pad(t, pad) for t in (q, k, v))
         return FusedLandmarkAttention.apply(q, k, v, n_history_blocks, sm_scale, block_size)[..., :d]
     return FusedLandmarkAttention.apply(q, k, v, n_history_blocks, sm_scale, block_size)
+
+
+def fused_landmark_attention_rotary_q(q, k, v, cos, sin, position_ids, is_mem=None, sm_scale=None, block_size=64):
+    """Forward only (no autograd): ``fused_landmark_attention(rot(q), k, v, ...)`` with the rotary embedding of
+    ``q`` (``apply_rotary_pos_emb``, ``llama/llama_mem.py:298``) applied inside the kernel as it loads the
+    queries -- same bits as rotating first, one pass over ``q`` less.  ``k`` must already be rotated.
+
+    q: (B, H, Lq, D) without rotary; cos, sin: (n_pos, D) or (1, 1, n_pos, D) model-dtype tables;
+    position_ids: int64 (B, Lq) or (1, Lq), the positions of the query rows.  Native block sizes only."""
+    from .retrieval import _tables
+    assert not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)), \
+        "forward only: rotate q with apply_rotary_pos_emb and call fused_landmark_attention to differentiate"
+    if is_mem is not None:
+        _check_is_mem(is_mem, block_size)
+    B, H, Lq, D = q.shape
+    Lk = k.shape[2]
+    assert k.shape == v.shape == (B, H, Lk, D) and q.dtype == k.dtype == v.dtype and q.dtype in _lib.DTYPE_CODES
+    assert q.is_cuda and D in SUPPORTED_HEAD_DIMS and block_size in SUPPORTED_BLOCKS
+    assert (Lk - Lq) % block_size == 0
+    assert position_ids.dim() == 2 and position_ids.shape[1] == Lq and position_ids.shape[0] in (1, B)
+    assert position_ids.dtype == torch.int64 and position_ids.device == q.device
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    cos, sin = _tables(cos, sin, q.dtype)
+    q, k, v = _lib.kernel_ready(q), _lib.kernel_ready(k), _lib.kernel_ready(v)
+    position_ids = position_ids.contiguous()
+    o = torch.empty_like(q)
+    L = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+    M = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+    with _lib.on_device(q.device):
+        rc = _lib.lib().lmk_attn_fwd_rotary_q(
+            _lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o), L.data_ptr(), M.data_ptr(),
+            cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0], position_ids.data_ptr(),
+            Lq if position_ids.shape[0] == B and B > 1 else 0, B, H, Lq, Lk, D, float(sm_scale), int(block_size),
+            (Lk - Lq) // block_size, _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+    _lib.check(rc)
+    return o

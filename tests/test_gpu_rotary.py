@@ -77,3 +77,36 @@ def test_rotary_feeds_the_fused_attention_like_the_reference_layer():
     for h in range(H):
         ref = s1.s1_attention(pq[0, h].float(), pk[0, h].float(), v[0, h].float(), block)
         assert (out[0, h].float().cpu() - ref).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("B,H,Lq,Lk,D,block,dtype", [
+    (2, 3, 128, 128, 128, 32, torch.bfloat16),
+    (1, 2, 96, 224, 128, 32, torch.bfloat16),       # history: the queries sit at positions 128 ..
+    (2, 2, 128, 256, 64, 64, torch.float16),
+    (1, 2, 256, 256, 128, 128, torch.bfloat16),
+    (1, 2, 70, 70, 64, 32, torch.bfloat16),         # partial last block
+])
+def test_forward_with_q_rotated_in_the_prologue_is_bit_identical(B, H, Lq, Lk, D, block, dtype):
+    # lmk_attn_fwd_rotary_q == lmk_attn_fwd on apply_rotary_pos_emb(q): same output bits, one pass over q less
+    from landmark_hip.attention import fused_landmark_attention_rotary_q
+    from landmark_hip.rotary import apply_rotary_pos_emb
+    from ltriton.flash_landmark_attention import fused_landmark_attention
+    print(f"case rope-q B{B} H{H} Lq{Lq} Lk{Lk} D{D} bs{block} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(Lq + Lk + D)
+    q = (torch.randn(B, H, Lq, D, generator=g) * 0.5).to(dtype).cuda()
+    k = (torch.randn(B, H, Lk, D, generator=g) * 0.5).to(dtype).cuda()
+    v = (torch.randn(B, H, Lk, D, generator=g) * 0.5).to(dtype).cuda()
+    cos, sin = (t.cuda() for t in orot.rotary_tables(Lk + 40, D, dtype))
+    pos_q = (torch.arange(Lk - Lq, Lk)[None] + torch.tensor([[0], [7]])[:B]).cuda()      # per-batch offsets
+    pos_k = (torch.arange(Lk)[None] + torch.tensor([[0], [7]])[:B]).cuda()
+    q_rot, _ = apply_rotary_pos_emb(q, q, cos, sin, pos_q)
+    _, k_rot = apply_rotary_pos_emb(None, k, cos, sin, pos_k)
+    want = fused_landmark_attention(q_rot, k_rot, v, None, block_size=block)
+    got = fused_landmark_attention_rotary_q(q, k_rot, v, cos, sin, pos_q, block_size=block)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    # and against the oracle, end to end
+    ref = orot.apply_rotary(q.cpu(), cos.cpu(), sin.cpu(), pos_q.cpu()[:, None, :])
+    assert torch.equal(q_rot.cpu(), ref)
+    with pytest.raises(AssertionError):
+        fused_landmark_attention_rotary_q(q.clone().requires_grad_(True), k_rot, v, cos, sin, pos_q, block_size=block)
