@@ -22,6 +22,11 @@
 //     earlier block (query tile past the key tile):  x = a, y = nD, z = 0; at the block's landmark
 //         key W = 0 (x = 1e30) and z = the dS stored by the dQ kernel
 //     own block / not yet visible:  W = [key <= lim] exp2(s*c - mhat),  y = delta, z = 0
+//
+// A workgroup serves several 128-key tiles of one (batch, head) in a row when there are more tiles than CUs
+// (at most four, in a zig-zag over the head's tiles so that every workgroup gets the same work).  The ring does
+// not stop between them: behind a tile's last query tile the requests go on with the first query tiles of the
+// workgroup's next key tiles, so only the stationary operand and the accumulator change hands at the boundary.
 #include <type_traits>
 
 #include "lmk_common.hpp"
@@ -80,30 +85,50 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   const bool role_k = wave >= C::NKT;                      // false: S, W, dV; true: dP, dS, dK
   const int ql = lane & 31, h = lane >> 5;
 
-  int bh, kvt;                                             // (batch*head, 128-key tile); most work first
+  // A workgroup serves one (batch, head) and several 128-key tiles of it, one after the other ("items"):
+  // with G workgroups per head, workgroup g takes tiles g, 2G-1-g, 2G+g, 4G-1-g, .. (a zig-zag, so that
+  // every workgroup gets the same amount of work; tile 0 sees every query tile, the last one the fewest).
+  const int BH = p.B * p.H;
+  const int G = (int)gridDim.x / BH;                       // workgroups per head
+  const int n_c = (p.n_kvtiles + G - 1) / G;               // items per workgroup (some may fall past the last tile)
+  int bh, g_;
   {
-    const int bid = blockIdx.x, BH = p.B * p.H;
-    if ((BH & 7) == 0) {
+    const int bid = blockIdx.x;
+    if ((BH & 7) == 0) {                                   // all workgroups of a head on one XCD
       const int xcd = bid & 7, j = bid >> 3, ngrp = BH >> 3;
-      kvt = j / ngrp;
+      g_ = j / ngrp;
       bh = (j % ngrp) * 8 + xcd;
     } else {
-      kvt = bid / BH;
+      g_ = bid / BH;
       bh = bid % BH;
     }
   }
+  auto item_kvt = [&](int c) LMK_INL { return (c & 1) ? (c + 1) * G - 1 - g_ : c * G + g_; };
+  auto next_item = [&](int c) LMK_INL {                    // first item index >= c with a tile that exists, or n_c
+    while (c < n_c && item_kvt(c) >= p.n_kvtiles) ++c;
+    return c;
+  };
+  int kvt = item_kvt(0);                                   // item 0 always exists (g_ < G <= n_kvtiles)
   const int b_ = bh / p.H, hh = bh % p.H;
   const char* qp = (const char*)p.q + 2 * (b_ * p.qs_b + hh * p.qs_h);
   const char* gp = (const char*)p.dout + 2 * (b_ * p.dos_b + hh * p.dos_h);
 
   const int nkt = p.Lk >> 5;                               // key tiles (TPB per landmark block)
-  const int kt = kvt * C::NKT + tile;
-  const bool active = kt < nkt;
-  const int krow = kt * 32 + ql;
-  const bool lm_lane = (ql == 31) && (kt % C::TPB == C::TPB - 1);   // this lane's key is its block's landmark
   const int PT = p.n_prefix * C::TPB;                      // history tiles in front of the queries
-  const int kt_end = (kt / C::TPB + 1) * C::TPB;           // first tile behind this key tile's block
   const int nq = p.Lq >> 5;
+  // the item being computed
+  int kt, krow, kt_end, j_first;
+  bool active, lm_lane;
+  auto set_item = [&](int c) LMK_INL {
+    kvt = item_kvt(c);
+    kt = kvt * C::NKT + tile;
+    active = kt < nkt;
+    krow = kt * 32 + ql;
+    lm_lane = (ql == 31) && (kt % C::TPB == C::TPB - 1);   // this lane's key is its block's landmark
+    kt_end = (kt / C::TPB + 1) * C::TPB;                   // first tile behind this key tile's block
+    j_first = max(0, kvt * C::NKT - PT);                   // first query tile any wave here can see
+  };
+  set_item(0);
   const float c2 = p.scale_log2;
 
   u32x4_t bf[C::KS];                                       // stationary operand, loaded after the first requests
@@ -125,10 +150,15 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 
   // ---- loaders.  Wave pair t fetches rows RPD*(t*NDMA + d) .. of a query tile: the V-role wave those
   // of Q plus the terms of key tile t, the K-role wave those of dO.
-  const int j_first = max(0, kvt * C::NKT - PT);           // first query tile any wave here can see
-  static_assert(C::NDMA <= 2, "two running offsets per wave");
-  // per-lane source offset (bytes) of this wave's requests 0 and 1 inside its tensor: Q for the V role, dO for the K role
-  uint32_t src_vo0, src_vo1 = 0;
+  static_assert(C::NDMA <= 2, "two source offsets per wave");
+  // The requests run four to five query tiles ahead of the arithmetic and do not stop at the end of an item:
+  // behind an item's last query tile they go on with the first tiles of the workgroup's next item, so the ring
+  // is full when that item starts.  The stream's position is a handful of scalars: the tile it fetches next
+  // (j_req), the item's offset into the per-block planes (pl_req), and the same two for the item after it,
+  // which the arithmetic side fills in whenever it starts an item (every item but a workgroup's last has more
+  // query tiles than the stream runs ahead, so the entry is there before the stream needs it).
+  // per-lane source offset (bytes) of this wave's requests 0 and 1 inside tile 0 of its tensor: Q for the V role, dO for the K role
+  uint32_t lane_vo0, lane_vo1 = 0;
   const char* src_base = role_k ? gp : qp;                 // wave-uniform
   const int64_t src_rs = role_k ? p.dos_r : p.qs_r;
   {
@@ -136,43 +166,56 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     const int row0 = C::RPD * (tile * C::NDMA) + lane / C::CH, row1 = row0 + C::RPD;
     const int f0 = (((row0 & 3) << 2) | ((row0 >> 2) & 3)) & (C::CH - 1);
     const int f1 = (((row1 & 3) << 2) | ((row1 >> 2) & 3)) & (C::CH - 1);
-    src_vo0 = (uint32_t)(2 * (row0 * src_rs + 8 * (chp ^ f0)));   // the chunk that belongs at LDS position chp
-    if (C::NDMA > 1) src_vo1 = (uint32_t)(2 * (row1 * src_rs + 8 * (chp ^ f1)));
+    lane_vo0 = (uint32_t)(2 * (row0 * src_rs + 8 * (chp ^ f0)));   // the chunk that belongs at LDS position chp
+    if (C::NDMA > 1) lane_vo1 = (uint32_t)(2 * (row1 * src_rs + 8 * (chp ^ f1)));
   }
-  const float* st_src;                                     // this lane's 16 bytes of terms for query tile 0
-  {
-    const int arr = min(lane / 8, 4), part = lane % 8;     // 0: a, 1: nD, 2: dS at landmark, 3: mhat, 4..: delta
-    const int bk = min(kt / C::TPB, p.n_blocks - 1);
-    const int64_t plane_row = ((int64_t)bh * p.n_blocks + bk) * p.Lq, head_row = (int64_t)bh * p.Lq;
-    st_src = (arr == 0) ? p.stat_a + plane_row : (arr == 1) ? p.stat_n + plane_row : (arr == 2) ? p.stat_l + plane_row
-             : (arr == 3) ? p.mhat + head_row : p.delta + head_row;
-    st_src += 4 * part;
-  }
-  // Requests go out in tile order (j_first, j_first+1, ..), so the source position is a running
-  // offset: one vector add per request instead of 64-bit scalar multiplies per iteration.  Past the
-  // last tile it stops advancing and the last tile is re-read (never used).
-  int j_req = j_first;                                     // tile the next request fetches
   const uint32_t src_step = (uint32_t)(2 * 32 * src_rs);
-  src_vo0 += (uint32_t)j_first * src_step;
-  src_vo1 += (uint32_t)j_first * src_step;
-  st_src += 32 * (int64_t)j_first;
-  // One piece of this wave's share of query tile j_req -> ring slot.  A tile's pieces go out one per MFMA
+  // this lane's 16 bytes of a query tile's terms: lanes 0-7 a, 8-15 nD, 16-23 dS at the landmark (planes, one row
+  // of Lq per block), 24-31 mhat, 32-63 delta (one row per head)
+  const float* st_lane;                                    // its array at the head's first row, tile 0
+  {
+    const int arr = min(lane / 8, 4), part = lane % 8;
+    const int64_t plane0 = (int64_t)bh * p.n_blocks * p.Lq, head_row = (int64_t)bh * p.Lq;
+    st_lane = (arr == 0) ? p.stat_a + plane0 : (arr == 1) ? p.stat_n + plane0 : (arr == 2) ? p.stat_l + plane0
+              : (arr == 3) ? p.mhat + head_row : p.delta + head_row;
+    st_lane += 4 * part;
+  }
+  auto item_first = [&](int c) LMK_INL { return max(0, item_kvt(c) * C::NKT - PT); };
+  auto item_plane = [&](int c) LMK_INL {                   // element offset of this wave's key tile's block inside the planes
+    return (int64_t)min((item_kvt(c) * C::NKT + tile) / C::TPB, p.n_blocks - 1) * p.Lq;
+  };
+  int j_req = item_first(0), jf_nx = 0;
+  int64_t pl_req = item_plane(0), pl_nx = 0;
+  bool has_nx = false;
+  auto announce_next = [&](int c) LMK_INL {                // the arithmetic side starts item c: tell the stream what follows it
+    const int c2 = next_item(c + 1);
+    has_nx = c2 < n_c;
+    if (has_nx) {
+      jf_nx = item_first(c2);
+      pl_nx = item_plane(c2);
+    }
+  };
+  announce_next(0);
+  // One piece of this wave's share of the stream's tile -> ring slot.  A tile's pieces go out one per MFMA
   // slot of the first product rather than together: all eight waves asking at once queue up in front of
   // the address unit.  V role: pieces 0 .. NDMA-1 fetch Q rows, piece NDMA the terms; K role: dO rows.
   const int dst_off = (role_k ? C::TILE_BYTES : 0) + tile * C::NDMA * 1024;   // this wave's rows inside a slot
   auto request_piece = [&](int slot_bytes, auto Pc) LMK_INL {
     constexpr int P = decltype(Pc)::value;
-    const bool more = j_req < nq - 1;                      // wave-uniform
+    if constexpr (P == 0) {                                // a new tile: behind an item's last one, move to the next item
+      const bool past = j_req >= nq, take = past && has_nx;    // (or re-read the last tile, which nobody uses)
+      j_req = take ? jf_nx : (past ? nq - 1 : j_req);
+      pl_req = take ? pl_nx : pl_req;
+      has_nx = take ? false : has_nx;
+    }
     if constexpr (P < C::NDMA) {
-      uint32_t& vo = (P == 0) ? src_vo0 : src_vo1;
-      dma16_s(src_base, vo, slot_bytes + dst_off + P * 1024);
-      vo += more ? src_step : 0u;
-      if (P == C::NDMA - 1 && role_k) j_req += more ? 1 : 0;
+      dma16_s(src_base, ((P == 0) ? lane_vo0 : lane_vo1) + (uint32_t)j_req * src_step, slot_bytes + dst_off + P * 1024);
+      if (P == C::NDMA - 1 && role_k) ++j_req;
     } else if constexpr (P == C::NDMA) {
       if (!role_k) {
-        dma16_v(st_src, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
-        st_src += more ? 32 : 0;
-        j_req += more ? 1 : 0;
+        const int64_t off = 32 * (int64_t)j_req + ((lane < 24) ? pl_req : 0);
+        dma16_v(st_lane + off, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
+        ++j_req;
       }
     }
   };
@@ -339,100 +382,131 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     sync();
   };
 
-  // ---- prologue.  The stationary operand and the first two tiles are asked for first and awaited; tiles
-  // j_first+2, +3 go out behind that wait, so the workgroup does not sit through four tiles' worth of
-  // traffic (every workgroup of a launch round starts at the same moment) before its first product.
-  // this wave's stationary operand: K fragments (V role) or V fragments (K role), lane = key
-  {
+  // this wave's stationary operand of the current item: K fragments (V role) or V fragments (K role), lane = key
+  auto load_stationary = [&]() LMK_INL {
     const char* src = role_k ? (const char*)p.v + 2 * (b_ * p.vs_b + hh * p.vs_h)
                              : (const char*)p.k + 2 * (b_ * p.ks_b + hh * p.ks_h);
     const int64_t rs = role_k ? p.vs_r : p.ks_r;
+    int kr = krow, h8 = 8 * h;
+    asm volatile("" : "+v"(kr), "+v"(h8));                 // the address is formed here, not ahead of the loops (and spilled)
+    const char* row = src + 2 * ((int64_t)kr * rs + h8);
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) {
       u32x4_t z = {0, 0, 0, 0};
       bf[ks] = z;
-      if (active) bf[ks] = *(const u32x4_t*)(src + 2 * ((int64_t)krow * rs + 16 * ks + 8 * h));
+      if (active) bf[ks] = *(const u32x4_t*)(row + 32 * ks);
     }
-    request(0);
-    request(C::BUF_BYTES);
-    if (tid < 64) ((float*)(smem + C::CONST_OFF))[tid] = (tid < 32) ? 1e30f : 0.f;
-    // consume the operand here: no wait for these loads can then end up inside the loop, where it would
-    // drain the ring; the explicit wait covers the two requests, which the compiler does not count
+  };
+  // consume the operand at once: no wait for these loads can then end up inside the loop, where it would
+  // drain the ring; the explicit wait covers everything this wave has in flight, which the compiler does not count
+  auto await_stationary = [&]() LMK_INL {
     wait_vmcnt<0>();
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) asm volatile("" : "+v"(bf[ks]));
-    request(2 * C::BUF_BYTES);
-    request(3 * C::BUF_BYTES);
-  }
+  };
+
+  // ---- prologue of the first item.  The stationary operand and the first two tiles are asked for first and
+  // awaited; tiles j_first+2, +3 go out behind that wait, so the workgroup does not sit through four tiles'
+  // worth of traffic (every workgroup of a launch round starts at the same moment) before its first product.
+  load_stationary();
+  request(0);
+  request(C::BUF_BYTES);
+  if (tid < 64) ((float*)(smem + C::CONST_OFF))[tid] = (tid < 32) ? 1e30f : 0.f;
+  await_stationary();
+  request(2 * C::BUF_BYTES);
+  request(3 * C::BUF_BYTES);
 
   wait_tiles();
   __syncthreads();
 
-  // Iteration i = j_first .. nq, one barrier each, in both roles.  V role: tiles i (W, dV) and i+1 (S).
+  // Per item: iteration i = j_first .. nq, one barrier each, in both roles.  V role: tiles i (W, dV) and i+1 (S).
   // K role: tiles i (dP) and i-1 (dS, dK); it has nothing to finish in the first iteration and only
-  // finishes in the last.  The ring slot of tile i is a wave-uniform counter.
+  // finishes in the last.  The ring slot of tile i is a wave-uniform counter that runs on from item to item: the
+  // slots behind an item's last tile already hold the next item's first tiles.
   auto wrap = [](int x) LMK_INL { return x >= C::NBUF ? x - C::NBUF : x; };
   auto store_acc = [&](const f32x16_t* acc, char* dst, int64_t rs, float scl) LMK_INL {
+    int kr = krow, h4 = 4 * h;
+    asm volatile("" : "+v"(kr), "+v"(h4));                 // as in load_stationary
+    char* row = dst + 2 * ((int64_t)kr * rs + h4);
 #pragma unroll
     for (int dc = 0; dc < C::DC; ++dc)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * scl, acc[dc][4 * g + 1] * scl),
                       pack2<T>(acc[dc][4 * g + 2] * scl, acc[dc][4 * g + 3] * scl)};
-        *(u32x2_t*)(dst + 2 * ((int64_t)krow * rs + 32 * dc + 8 * g + 4 * h)) = o2;
+        *(u32x2_t*)(row + 2 * (32 * dc + 8 * g)) = o2;
       }
   };
   if (!role_k) {
     f32x16_t acc[C::DC];                                   // dV^T: rows = d, lane = key
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
     f32x16_t cur, nxt;                                      // S of tiles i and i+1
-    row_tile(0, cur);                                       // S of the first tile
-    int sc = 0;
-    auto step = [&](auto Mc, int i) LMK_INL {
-      // the barrier sits between the two products: the second one has its operands in registers, so
-      // its MFMAs run while the workgroup's stragglers arrive and the next tile's operands are fetched
-      auto sync = [&]() LMK_INL {
-        wait_vmcnt<2 * C::PER_TILE_V>();                    // tile i+2 has landed (tiles i+3, i+4 may be in flight)
-        __syncthreads();
+    int sc = 0;                                            // slot of the item's tile i
+    for (int c = 0; c < n_c; c = next_item(c + 1)) {
+      if (c > 0) {                                         // the ring already holds this item's first tiles
+        set_item(c);
+        announce_next(c);
+        load_stationary();
+        await_stationary();
+      }
+#pragma unroll
+      for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
+      row_tile(sc * C::BUF_BYTES, cur);                     // S of the first tile
+      auto step = [&](auto Mc, int i) LMK_INL {
+        // the barrier sits between the two products: the second one has its operands in registers, so
+        // its MFMAs run while the workgroup's stragglers arrive and the next tile's operands are fetched
+        auto sync = [&]() LMK_INL {
+          wait_vmcnt<2 * C::PER_TILE_V>();                  // tile i+2 has landed (tiles i+3, i+4 may be in flight)
+          __syncthreads();
+        };
+        body_v(Mc, i, sc * C::BUF_BYTES, wrap(sc + 1) * C::BUF_BYTES, wrap(sc + 4) * C::BUF_BYTES, (i - j_first) & 1, cur, nxt, acc, sync);
+        cur = nxt;
+        sc = wrap(sc + 1);
       };
-      body_v(Mc, i, sc * C::BUF_BYTES, wrap(sc + 1) * C::BUF_BYTES, wrap(sc + 4) * C::BUF_BYTES, (i - j_first) & 1, cur, nxt, acc, sync);
-      cur = nxt;
-      sc = wrap(sc + 1);
-    };
-    // own block and tiles that cannot see these keys yet come first, then every later tile sees all keys:
-    // two loops, so that each has one code path and the accumulators stay where they are
-    int i = j_first;
-    const int i_full = min(nq, max(j_first, kt_end - PT));
-    for (; i < i_full; ++i) step(std::true_type{}, i);
-    for (; i < nq; ++i) step(std::false_type{}, i);
-    request(wrap(sc + 4) * C::BUF_BYTES);                   // the K role finishes tile nq-1 in one more iteration
-    wait_vmcnt<2 * C::PER_TILE_V>();
-    __syncthreads();
+      // own block and tiles that cannot see these keys yet come first, then every later tile sees all keys:
+      // two loops, so that each has one code path and the accumulators stay where they are
+      int i = j_first;
+      const int i_full = min(nq, max(j_first, kt_end - PT));
+      for (; i < i_full; ++i) step(std::true_type{}, i);
+      for (; i < nq; ++i) step(std::false_type{}, i);
+      // the K role finishes tile nq-1 in one more iteration; nothing is requested here (the K role's request of
+      // that iteration is the one its first iteration of the next item leaves out)
+      wait_vmcnt<2 * C::PER_TILE_V>();
+      __syncthreads();
+      if (active) store_acc(acc, (char*)p.dv + 2 * (b_ * p.dvs_b + hh * p.dvs_h), p.dvs_r, 1.f);
+    }
     wait_vmcnt<0>();                                       // nothing may still be writing LDS when the wave ends
-    if (active) store_acc(acc, (char*)p.dv + 2 * (b_ * p.dvs_b + hh * p.dvs_h), p.dvs_r, 1.f);
   } else {
     f32x16_t acc[C::DC];                                   // dK^T: rows = d, lane = key
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
     f32x16_t prv, cur;                                      // dP of tiles i-1 and i
-    int sc = 0;
-    request(wrap(sc + 4) * C::BUF_BYTES);
-    row_tile(C::TILE_BYTES, prv);                           // dP of the first tile
-    wait_vmcnt<2 * C::PER_TILE_K>();
-    __syncthreads();
-    sc = 1;
-    for (int i = j_first + 1; i <= nq; ++i) {
-      auto sync = [&]() LMK_INL {
-        wait_vmcnt<2 * C::PER_TILE_K>();
-        __syncthreads();
-      };
-      body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, wrap(sc + 4) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc, sync);
-      prv = cur;
+    int sc = 0;                                            // slot of the item's first tile, then of tile i
+    for (int c = 0; c < n_c; c = next_item(c + 1)) {
+      if (c > 0) {
+        set_item(c);
+        announce_next(c);
+        load_stationary();
+        await_stationary();
+      } else {
+        request(wrap(sc + 4) * C::BUF_BYTES);               // the fifth tile; later items have it from the item before
+      }
+#pragma unroll
+      for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
+      row_tile(sc * C::BUF_BYTES + C::TILE_BYTES, prv);     // dP of the first tile
+      wait_vmcnt<2 * C::PER_TILE_K>();
+      __syncthreads();
       sc = wrap(sc + 1);
+      for (int i = j_first + 1; i <= nq; ++i) {
+        auto sync = [&]() LMK_INL {
+          wait_vmcnt<2 * C::PER_TILE_K>();
+          __syncthreads();
+        };
+        body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, wrap(sc + 4) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc, sync);
+        prv = cur;
+        sc = wrap(sc + 1);
+      }
+      sc = wrap(sc + C::NBUF - 1);                          // the slot behind the last tile: the next item's first tile
+      if (active) store_acc(acc, (char*)p.dk + 2 * (b_ * p.dks_b + hh * p.dks_h), p.dks_r, p.scale);
     }
     wait_vmcnt<0>();
-    if (active) store_acc(acc, (char*)p.dk + 2 * (b_ * p.dks_b + hh * p.dks_h), p.dks_r, p.scale);
   }
 }
 
@@ -444,7 +518,19 @@ static int launch_dkdv32_t(const BwdParams& p, hipStream_t stream) {
   auto kern = lmk_bwd_dkdv32_kernel<T, D, BS>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
-  hipLaunchKernelGGL(kern, dim3(p.n_kvtiles * p.B * p.H), dim3(C::NTHR), C::LDS_BYTES, stream, p);
+  // workgroups per head: enough for about one workgroup per CU, at most four 128-key tiles each
+  static std::atomic<int> n_cu{0};
+  if (n_cu.load() == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    n_cu.store(cus);
+  }
+  const int64_t items = (int64_t)p.n_kvtiles * p.B * p.H;
+  int per_wg = (int)(items / n_cu.load());
+  per_wg = per_wg < 1 ? 1 : (per_wg > 4 ? 4 : per_wg);
+  const int groups = (p.n_kvtiles + per_wg - 1) / per_wg;
+  hipLaunchKernelGGL(kern, dim3(groups * p.B * p.H), dim3(C::NTHR), C::LDS_BYTES, stream, p);
   return (int)hipGetLastError();
 }
 

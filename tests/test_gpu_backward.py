@@ -223,3 +223,24 @@ def test_reference_script_case():
     assert torch.allclose(out.float().cpu(), exact.detach(), rtol=1e-2, atol=1e-2)
     for name, a, b_ in zip("qkv", grads, exact_grads):
         assert torch.allclose(a.float().cpu(), b_, rtol=4e-2, atol=4e-2), f"d{name}"
+
+
+# Many heads: the dK/dV kernel then gives one workgroup several 128-key tiles of a head in a row (its requests
+# run on into the next tile while the current one finishes), in zig-zag order over the head's tiles.
+@pytest.mark.parametrize("B,H,Lq,Lk,D,block,dtype", [
+    (8, 32, 512, 512, 64, 32, torch.bfloat16),       # four tiles per workgroup, one workgroup per head
+    (8, 32, 384, 640, 64, 32, torch.bfloat16),       # history; five tiles over two workgroups (3 + 2)
+    (4, 32, 768, 768, 64, 64, torch.float16),        # three tiles per workgroup, blocks of two tiles
+    (8, 32, 512, 512, 128, 128, torch.bfloat16),     # blocks of four tiles
+    (6, 32, 416, 416, 128, 32, torch.bfloat16),      # last tile of a head partly empty (13 key tiles of 32)
+])
+def test_gradients_with_several_key_tiles_per_workgroup(B, H, Lq, Lk, D, block, dtype):
+    print(f"case multi-item B{B} H{H} Lq{Lq} Lk{Lk} D{D} bs{block} {dtype}", flush=True)
+    seed = B + Lq + Lk + D + block
+    q, k, v = make_qkv(B, H, Lq, Lk, D, seed=seed, dtype=dtype)
+    do = torch.randn(B, H, Lq, D, generator=torch.Generator().manual_seed(seed + 1)).to(dtype)
+    rq, rk, rv = oracle_grads(q, k, v, do, block, chunk=16)
+    gq, gk, gv = _grads(q, k, v, do, block)
+    for name, g, r in (("dq", gq, rq), ("dk", gk, rk), ("dv", gv, rv)):
+        err = (g.float().cpu() - r).abs().max().item()
+        assert err <= TOL, (name, err)
