@@ -519,15 +519,8 @@ static int launch_dkdv32_t(const BwdParams& p, hipStream_t stream) {
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   // workgroups per head: enough for about one workgroup per CU, at most four 128-key tiles each
-  static std::atomic<int> n_cu{0};
-  if (n_cu.load() == 0) {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-      cus = 256;
-    n_cu.store(cus);
-  }
   const int64_t items = (int64_t)p.n_kvtiles * p.B * p.H;
-  int per_wg = (int)(items / n_cu.load());
+  int per_wg = (int)(items / cu_count());
   per_wg = per_wg < 1 ? 1 : (per_wg > 4 ? 4 : per_wg);
   const int groups = (p.n_kvtiles + per_wg - 1) / per_wg;
   hipLaunchKernelGGL(kern, dim3(groups * p.B * p.H), dim3(C::NTHR), C::LDS_BYTES, stream, p);

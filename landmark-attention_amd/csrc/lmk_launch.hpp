@@ -27,6 +27,19 @@ inline int allow_dynamic_lds(K kern, int bytes, std::atomic<uint64_t>& done) {
   return 0;
 }
 
+// Compute units of the current device (looked up once; 256 if the query fails).
+inline int cu_count() {
+  static std::atomic<int> n{0};
+  int v = n.load(std::memory_order_relaxed);
+  if (v == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    n.store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
 struct FwdParams {
   const void *q, *k, *v;
   void* o;
