@@ -306,7 +306,21 @@ def side_legs(n=30, warm=5):
         t_pre2 = _time_launches(prefill_two_pass, n, warm)
         t_pre1 = _time_launches(prefill_q_in_prologue, n, warm)
     rot_bytes = 2 * 2 * xq.numel() * 2 + 2 * Lq * D * 2
-    return {"per_head_selection": {"workload": "config 4 shapes, aggregate=max_over_tokens", "topk_ms": t_sel,
+    # benchmark config 0 (the reference's CPU-runnable case: B2 H8 L510 D128, block 51) on the HIP path: inputs
+    # rounded to bf16, blocks repacked into 64 slots, forward and forward + backward through the autograd Function
+    q0, k0, v0, _, block0 = config0_inputs(0)
+    q0, k0, v0 = (t.bfloat16().to(dev).requires_grad_(True) for t in (q0, k0, v0))
+    do0 = torch.randn(q0.shape, generator=g).bfloat16().to(dev)
+
+    def config0_step():
+        out = fused_landmark_attention(q0, k0, v0, None, block_size=block0)
+        torch.autograd.grad(out, [q0, k0, v0], do0)
+    with torch.no_grad():
+        t_c0_fwd = _time_launches(lambda: fused_landmark_attention(q0, k0, v0, None, block_size=block0), n, warm)
+    t_c0_step = _time_launches(config0_step, n, warm)
+    return {"config0_on_hip": {"workload": "benchmark config 0 (B2 H8 L510 D128, block 51) in bf16, blocks padded to 64 slots",
+                               "forward_ms": t_c0_fwd, "forward_backward_ms": t_c0_step},
+            "per_head_selection": {"workload": "config 4 shapes, aggregate=max_over_tokens", "topk_ms": t_sel,
                                    "attend_ms": t_att},
             "rotary": {"workload": "q and k of config 2, (2,32,2048,128) bf16 each, one launch for both", "ms": t_rot,
                        "one_launch_per_tensor_ms": t_rot2,
