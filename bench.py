@@ -318,7 +318,23 @@ def side_legs(n=30, warm=5):
     with torch.no_grad():
         t_c0_fwd = _time_launches(lambda: fused_landmark_attention(q0, k0, v0, None, block_size=block0), n, warm)
     t_c0_step = _time_launches(config0_step, n, warm)
-    return {"config0_on_hip": {"workload": "benchmark config 0 (B2 H8 L510 D128, block 51) in bf16, blocks padded to 64 slots",
+    # the offloaded cache (keys and values of config 4's cache in pinned host memory, landmark keys on the GPU): one
+    # chunk of 256 queries and one single token, selection per head + attention over blocks read from host memory
+    from landmark_hip.cache import OffloadedLandmarkCache
+    oc = OffloadedLandmarkCache(B, H, D, block, torch.bfloat16, dev, capacity=S + 2 * T)
+    oc.append(kc, vc)
+    torch.cuda.synchronize()
+
+    def offloaded(tq):
+        out, _ = oc.step(q[:, :, :tq], kl[:, :, :tq], kl[:, :, :tq], vl[:, :, :tq], cos, sin, top_k)
+        oc.length = S                                      # the same step again: forget the appended rows
+        return out
+    t_off_chunk = _time_launches(lambda: offloaded(T), n, warm)
+    t_off_token = _time_launches(lambda: offloaded(1), n, warm)
+    return {"offloaded_cache": {"workload": "config 4's cache in pinned host memory (zero-copy reads of the selected blocks), "
+                                            "one selection per head; 256 queries / 1 query", "chunk_step_ms": t_off_chunk,
+                                "token_step_ms": t_off_token},
+            "config0_on_hip": {"workload": "benchmark config 0 (B2 H8 L510 D128, block 51) in bf16, blocks padded to 64 slots",
                                "forward_ms": t_c0_fwd, "forward_backward_ms": t_c0_step},
             "per_head_selection": {"workload": "config 4 shapes, aggregate=max_over_tokens", "topk_ms": t_sel,
                                    "attend_ms": t_att},

@@ -291,6 +291,15 @@ int lmk_retrieve_topk_shared(const lmk_tensor4* q, const lmk_tensor4* kcache, co
                              void* block_prob_out, void* workspace, size_t workspace_bytes, int B, int H, int T, int S,
                              int D, int block, int top_k, int dtype, void* stream);
 
+/* lmk_retrieve_topk_shared for a cache whose blocks live elsewhere (host memory, the reference's
+ * offload_cache_to_cpu branch, llama/llama_mem.py:326-328,344-356): landmark_keys is the tensor that branch
+ * keeps on the GPU as past_key_value[2] -- (B,H,n_blocks,D), one un-rotated landmark key per complete block.
+ * Same positions, contract, workspace (lmk_retrieve_workspace_bytes with S = n_blocks * block) and output. */
+int lmk_retrieve_topk_shared_landmarks(const lmk_tensor4* q, const lmk_tensor4* landmark_keys, const void* cos_table,
+                                       const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                                       void* block_prob_out, void* workspace, size_t workspace_bytes, int B, int H, int T,
+                                       int n_blocks, int D, int block, int top_k, int dtype, void* stream);
+
 /* Keys and values every query of a head attends to after a per-head selection
  * (llama_mem.py:386-388, 393-406): with k = min(top_k, S/block) and inc = S % block,
  *   k_win = [selected blocks' keys rotated at their slot positions ; tail keys rotated at

@@ -469,10 +469,34 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
   return lmk::launch_gather_attend(p, D, block, dtype, (hipStream_t)stream);
 }
 
+static int retrieve_topk_shared_impl(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
+                                     const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                                     void* block_prob_out, void* workspace, size_t workspace_bytes, int B, int H, int T,
+                                     int S, int D, int block, int top_k, int dtype, void* stream, bool lm_dense);
+
 int lmk_retrieve_topk_shared(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
                              const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
                              void* block_prob_out, void* workspace, size_t workspace_bytes, int B, int H, int T, int S,
                              int D, int block, int top_k, int dtype, void* stream) {
+  return retrieve_topk_shared_impl(q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, block_prob_out,
+                                   workspace, workspace_bytes, B, H, T, S, D, block, top_k, dtype, stream, false);
+}
+
+int lmk_retrieve_topk_shared_landmarks(const lmk_tensor4* q, const lmk_tensor4* landmark_keys, const void* cos_table,
+                                       const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                                       void* block_prob_out, void* workspace, size_t workspace_bytes, int B, int H, int T,
+                                       int n_blocks, int D, int block, int top_k, int dtype, void* stream) {
+  if (n_blocks <= 0) return LMK_ERR_CACHE;
+  if (block < 2 || (int64_t)n_blocks * block >= ((int64_t)1 << 31)) return LMK_ERR_UNSUPPORTED;
+  return retrieve_topk_shared_impl(q, landmark_keys, cos_table, sin_table, table_stride_row, n_pos, idx_out,
+                                   block_prob_out, workspace, workspace_bytes, B, H, T, n_blocks * block, D, block, top_k,
+                                   dtype, stream, true);
+}
+
+static int retrieve_topk_shared_impl(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
+                                     const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,
+                                     void* block_prob_out, void* workspace, size_t workspace_bytes, int B, int H, int T,
+                                     int S, int D, int block, int top_k, int dtype, void* stream, bool lm_dense) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(kcache))) return rc;
   if (cos_table == nullptr || sin_table == nullptr || idx_out == nullptr || workspace == nullptr) return LMK_ERR_NULL;
@@ -490,6 +514,7 @@ int lmk_retrieve_topk_shared(const lmk_tensor4* q, const lmk_tensor4* kcache, co
   p.approx = reinterpret_cast<float*>(w + l.approx);              // every query's scores, then exponentials
   p.agg = reinterpret_cast<uint32_t*>(w + l.exact);               // B*H*num_mems words: fits, T >= 1
   p.agg_out = static_cast<uint16_t*>(block_prob_out);
+  p.lm_dense = lm_dense ? 1 : 0;
   p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
   p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
   p.cs_r = table_stride_row;

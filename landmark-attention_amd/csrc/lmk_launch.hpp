@@ -95,6 +95,7 @@ struct RetrParams {
   int ring_start;                                 // slot of the oldest block (0 unless the cache is a ring buffer of blocks)
   int agg_over_heads;                             // shared selection: agg is (B*T, num_mems), maxima over the heads
   int prob32;                                     // shared selection: agg holds fp32 probabilities, not 16-bit ones
+  int lm_dense;                                   // kcache holds the landmark keys alone, one row per block
   int64_t prefix_len;                             // full_len - (k + 1) * block, may be -block
   int64_t qs_b, qs_h, qs_r, kcs_b, kcs_h, kcs_r, vcs_b, vcs_h, vcs_r, cs_r;
   int64_t ols_b, ols_h, ols_r, outs_b, outs_h, outs_r;

@@ -50,7 +50,9 @@ __global__ __launch_bounds__(256) void lmk_landmark_keys_kernel(RetrParams p) {
     age += age < 0 ? p.num_mems : 0;
     const int slot = (age < p.num_mems - p.k) ? 0 : age - (p.num_mems - p.k) + 1;
     const int64_t pos = (int64_t)slot * p.block + (p.block - 1) + p.prefix_len;
-    const char* src = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h + ((int64_t)m * p.block + p.block - 1) * p.kcs_r);
+    // the landmark is the last row of block m of the cache -- or row m of an array that holds the landmark keys alone
+    const int64_t lm_row = p.lm_dense ? (int64_t)m : (int64_t)m * p.block + p.block - 1;
+    const char* src = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h + lm_row * p.kcs_r);
     const u32x4_t x = *(const u32x4_t*)(src + 16 * j);
     const u32x4_t other = *(const u32x4_t*)(src + 16 * (j ^ (LPR / 2)));
     const u32x4_t c = *(const u32x4_t*)((const char*)p.cos + 2 * (pos * p.cs_r) + 16 * j);

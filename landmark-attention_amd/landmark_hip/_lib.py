@@ -93,6 +93,8 @@ def lib() -> ctypes.CDLL:
         L.lmk_local_window.argtypes = [T4, T4, T4, T4, T4, vp, vp, i64, i64, T4, T4, T4, i, i, i, i, i, i, i, vp]
         L.lmk_retrieve_topk_shared.restype = i
         L.lmk_retrieve_topk_shared.argtypes = [T4, T4, vp, vp, i64, i64, vp, vp, vp, sz, i, i, i, i, i, i, i, i, vp]
+        L.lmk_retrieve_topk_shared_landmarks.restype = i
+        L.lmk_retrieve_topk_shared_landmarks.argtypes = L.lmk_retrieve_topk_shared.argtypes
         L.lmk_ring_retrieve_topk.restype = i
         L.lmk_ring_retrieve_topk.argtypes = [T4, T4, vp, vp, i64, i64, vp, vp, sz, i, i, i, i, i, i, i, i, i, i, vp]
         L.lmk_gather_window.restype = i

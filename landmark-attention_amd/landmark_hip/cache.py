@@ -13,7 +13,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from .retrieval import retrieve_and_attend
+from .retrieval import attend_shared, retrieve_and_attend, retrieve_topk_from_landmarks
 
 
 class LandmarkKVCache:
@@ -75,5 +75,79 @@ class LandmarkKVCache:
                                        block, top_k, sm_scale, aggregate, workspace=self._ws,
                                        reuse_landmark_keys=reuse)
         self._ws_key = key if aggregate is None else None
+        self.append(key_states_before_pos, value_states)
+        return out, idx
+
+
+class OffloadedLandmarkCache:
+    """The cache of the reference's ``offload_cache_to_cpu`` branch (``llama/llama_mem.py:326-328,344-356,
+    427-428``): keys (without rotary) and values live in pinned host memory, only the landmark key of every
+    complete block stays on the GPU (``past_key_value[2]``), and every head retrieves one set of blocks per
+    step (``aggregate = "max_over_tokens"``, ``:369-372``).
+
+    The reference gathers the selected blocks on the CPU and copies them over (``:393-398``).  Here the
+    host buffers are mapped into the GPU's address space (pinned allocations are), so the kernel that builds
+    the key/value window reads the ``k`` selected blocks of each head -- and the few tokens of an incomplete
+    last block -- straight out of host memory: no index round trip to the host, no staging copy, and only
+    ``k * block`` rows per head cross the bus.  Appends are device-to-host copies of the new rows on the
+    caller's stream."""
+
+    def __init__(self, batch: int, heads: int, head_dim: int, block: int, dtype, device, capacity: int = 4096):
+        self.block = int(block)
+        self._k = torch.empty((batch, heads, capacity, head_dim), dtype=dtype, pin_memory=True)
+        self._v = torch.empty((batch, heads, capacity, head_dim), dtype=dtype, pin_memory=True)
+        self._lm = torch.empty((batch, heads, max(1, capacity // self.block), head_dim), dtype=dtype, device=device)
+        self.length = 0
+        self._ws = None
+
+    @property
+    def n_blocks(self) -> int:
+        return self.length // self.block
+
+    @property
+    def landmark_keys(self):
+        """``past_key_value[2]`` (``:344-347``): the un-rotated landmark keys of the complete blocks, on the GPU."""
+        return self._lm[:, :, : self.n_blocks]
+
+    @property
+    def host_key_value(self):
+        """Views of the filled part of the pinned host buffers, (B, nh, S, hd) each."""
+        return self._k[:, :, : self.length], self._v[:, :, : self.length]
+
+    def _reserve(self, rows: int) -> None:
+        if rows <= self._k.shape[2]:
+            return
+        cap = max(rows, 2 * self._k.shape[2])
+        torch.cuda.current_stream(self._lm.device).synchronize()     # copies into the old buffers have landed
+        for name in ("_k", "_v"):
+            old = getattr(self, name)
+            new = torch.empty(old.shape[:2] + (cap, old.shape[3]), dtype=old.dtype, pin_memory=True)
+            new[:, :, : self.length] = old[:, :, : self.length]
+            setattr(self, name, new)
+        lm = torch.empty(self._lm.shape[:2] + (cap // self.block, self._lm.shape[3]), dtype=self._lm.dtype,
+                         device=self._lm.device)
+        lm[:, :, : self.n_blocks] = self._lm[:, :, : self.n_blocks]
+        self._lm = lm
+
+    def append(self, key_states_before_pos, value_states) -> None:
+        """``:424-428``: the new rows go to the host buffers, landmark keys of blocks they complete to the GPU array."""
+        t = key_states_before_pos.shape[2]
+        self._reserve(self.length + t)
+        self._k[:, :, self.length: self.length + t].copy_(key_states_before_pos, non_blocking=True)
+        self._v[:, :, self.length: self.length + t].copy_(value_states, non_blocking=True)
+        first = (-(self.length + 1)) % self.block                    # offset of the first new landmark token, if any
+        if first < t:
+            n_new = (t - first + self.block - 1) // self.block
+            self._lm[:, :, self.n_blocks: self.n_blocks + n_new] = key_states_before_pos[:, :, first::self.block]
+        self.length += t
+
+    def step(self, query_states, key_states, key_states_before_pos, value_states, cos, sin, top_k: int, sm_scale=None):
+        """Attention of a new chunk against the offloaded cache, then the append; returns ``(out, idx)`` with
+        ``idx (B, nh, 1, k)``.  Needs at least one complete cached block."""
+        assert self.n_blocks >= 1, "no complete cached block yet"
+        idx = retrieve_topk_from_landmarks(query_states, self.landmark_keys, cos, sin, self.block, top_k, self._ws)
+        k_host, v_host = self.host_key_value
+        out = attend_shared(query_states, k_host, v_host, idx, key_states, value_states, cos, sin, self.block, top_k,
+                            sm_scale)
         self.append(key_states_before_pos, value_states)
         return out, idx

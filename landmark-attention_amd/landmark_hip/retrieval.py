@@ -88,6 +88,30 @@ def retrieve_topk(q, k_cache, cos, sin, block: int, top_k: int, aggregate=None, 
     return (idx, probs) if return_block_probs else idx
 
 
+def retrieve_topk_from_landmarks(q, landmark_keys, cos, sin, block: int, top_k: int, workspace=None):
+    """The ``max_over_tokens`` selection when the cached blocks are not on the GPU (``offload_cache_to_cpu``,
+    ``llama_mem.py:326-328,344-356``): ``landmark_keys (B, nh, n_blocks, hd)`` is ``past_key_value[2]`` of that
+    branch, the un-rotated landmark key of every complete block.  Returns ``(B, nh, 1, k)`` int64, as
+    ``retrieve_topk(..., aggregate="max_over_tokens")`` does for the same blocks."""
+    B, H, T, D = q.shape
+    n = landmark_keys.shape[2]
+    assert landmark_keys.shape == (B, H, n, D) and q.dtype == landmark_keys.dtype and q.is_cuda and landmark_keys.is_cuda
+    q, landmark_keys = _lib.kernel_ready(q), _lib.kernel_ready(landmark_keys)
+    cos, sin = _tables(cos, sin, q.dtype)
+    lib = _lib.lib()
+    idx = torch.empty((B, H, 1, min(top_k, n)), device=q.device, dtype=torch.int64)
+    nbytes = lib.lmk_retrieve_workspace_bytes(B, H, T, n * int(block), D, int(block))
+    with _lib.on_device(q.device):
+        ws = workspace if workspace is not None and workspace.numel() >= nbytes else \
+            torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+        rc = lib.lmk_retrieve_topk_shared_landmarks(
+            _lib.tensor4(q), _lib.tensor4(landmark_keys), cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0],
+            idx.data_ptr(), None, ws.data_ptr(), nbytes, B, H, T, n, D, int(block), int(top_k),
+            _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+    _lib.check(rc)
+    return idx
+
+
 def gather_attend(q, k_cache, v_cache, idx, k_loc, v_loc, cos, sin, block: int, top_k: int, sm_scale=None):
     """Attention output ``(B, nh, T, hd)`` over the blocks ``idx`` selects plus the local window
     (``llama_mem.py:386-412,447-477``).  The local window -- the new chunk, behind the tail of

@@ -30,7 +30,7 @@ def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
             "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend", "lmk_retrieve_topk_static", "lmk_retrieve_static_max_bytes",
-            "lmk_ring_retrieve_topk", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded",
+            "lmk_ring_retrieve_topk", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded",
             "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n

@@ -46,3 +46,45 @@ def test_decode_steps_match_the_oracle(aggregate):
         pk, pv = cache.past_key_value
         assert pk.shape[2] == S
     assert torch.equal(cache.past_key_value[0].cpu(), k_all) and torch.equal(cache.past_key_value[1].cpu(), v_all)
+
+
+def test_offloaded_cache_equals_the_device_cache_step_for_step():
+    """offload_cache_to_cpu (llama_mem.py:326-328,344-356): blocks in pinned host memory, landmark keys on the GPU,
+    one selection per head.  Same indices and bit-identical attention as the device-resident cache with
+    aggregate="max_over_tokens", over chunks and single tokens that cross landmarks and one regrowth of the buffers."""
+    from landmark_hip.cache import LandmarkKVCache, OffloadedLandmarkCache
+    from landmark_hip.rotary import apply_rotary_pos_emb
+    from oracle import rotary as orot
+    B, H, D, block, top_k = 2, 3, 128, 32, 3
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(11)
+    cos, sin = (t.to(dev) for t in orot.rotary_tables(4096, D, torch.bfloat16))
+    dcache = LandmarkKVCache(B, H, D, torch.bfloat16, dev, capacity=64)
+    ocache = OffloadedLandmarkCache(B, H, D, block, torch.bfloat16, dev, capacity=64)
+    prompt = 3 * block + 5
+    k0 = (torch.randn(B, H, prompt, D, generator=g) * 0.5).bfloat16().to(dev)
+    v0 = (torch.randn(B, H, prompt, D, generator=g) * 0.5).bfloat16().to(dev)
+    dcache.append(k0, v0)
+    ocache.append(k0, v0)
+    assert ocache.n_blocks == 3 and torch.equal(ocache.landmark_keys.cpu(), k0[:, :, block - 1::block].cpu())
+    for step, T in enumerate([1, 1, 20, 5, 1, 27, 4, 1, 1, 30, 2, 32 - 30]):
+        S = dcache.length
+        inc = S % block
+        assert inc == 0 or T + inc <= block
+        print(f"offload step {step}: S{S} T{T}", flush=True)
+        q = (torch.randn(B, H, T, D, generator=g) * 0.5).bfloat16().to(dev)
+        kn = (torch.randn(B, H, T, D, generator=g) * 0.5).bfloat16().to(dev)
+        v = (torch.randn(B, H, T, D, generator=g) * 0.5).bfloat16().to(dev)
+        pos = torch.arange(S, S + T, device=dev)[None]
+        q_rot, k_rot = apply_rotary_pos_emb(q, kn, cos, sin, pos)
+        want, want_idx = dcache.step(q_rot, k_rot, kn, v, cos, sin, block, top_k, aggregate="max_over_tokens")
+        got, got_idx = ocache.step(q_rot, k_rot, kn, v, cos, sin, top_k)
+        torch.cuda.synchronize()
+        assert torch.equal(got_idx, want_idx)
+        assert torch.equal(got, want)
+        assert ocache.length == dcache.length
+    kd, vd = dcache.past_key_value
+    kh, vh = ocache.host_key_value
+    assert torch.equal(kh, kd.cpu()) and torch.equal(vh, vd.cpu())
+    assert torch.equal(ocache.landmark_keys.cpu(), kd[:, :, block - 1::block].cpu())
+    assert ocache.n_blocks == dcache.length // block
