@@ -152,13 +152,15 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
     r_vo[d] = (uint32_t)(2 * (row * rs + 8 * (chp ^ f)));
     r_lds[d] = (r_isv[d] ? C::BLK_BYTES : 0) + part * 1024;
   }
+  static_assert((32 / C::RPD) % C::PER_TILE == 0, "all of a wave's requests read one tensor");
+  const bool rq_isv = wave * C::PER_TILE >= 32 / C::RPD;   // wave-uniform: this wave fetches V rows (else K rows)
+  const char* rq_base = rq_isv ? vp : kp;
+  const uint32_t rq_step = (uint32_t)(2 * 32 * (rq_isv ? p.vs_r : p.ks_r));   // bytes per block; a head's rows span < 4 GB (host check)
   auto request = [&](int slot_bytes, int blk) __attribute__((always_inline)) {
     const int bb = min(blk, nkb - 1);                      // past the end: re-read the last block (never used)
+    const char* base = rq_base + (uint32_t)bb * rq_step;
 #pragma unroll
-    for (int d = 0; d < C::PER_TILE; ++d) {
-      const char* base = r_isv[d] ? vp + 2 * ((int64_t)bb * 32 * p.vs_r) : kp + 2 * ((int64_t)bb * 32 * p.ks_r);
-      dq_dma16(base, r_vo[d], slot_bytes + r_lds[d]);
-    }
+    for (int d = 0; d < C::PER_TILE; ++d) dq_dma16(base, r_vo[d], slot_bytes + r_lds[d]);
   };
 
   f32x16_t acc[C::DC];
@@ -174,8 +176,8 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
     return l;
   };
   // flush: lane -> (block fl_bi of the group, queries 4 fl_part ..); wave-uniform base in SGPRs, one
-  // 32-bit lane offset shared by the three planes.  Lane-only values are recomputed at each use
-  // (see `fresh` below): held across the loop they cost registers the loop does not have.
+  // 32-bit lane offset shared by the three planes.  Lane-only values are recomputed at each use:
+  // held across the loop they cost registers the loop does not have.
   auto flush = [&](int blast) __attribute__((always_inline)) {   // blocks FL*(blast/FL) .. blast of this wave's terms
     const int ln = lane_now();
     const int fl_bi = ln >> 3, fl_part = ln & 7;
@@ -194,12 +196,6 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   };
 
   // ---- the stages
-  // addresses that depend only on the lane are recomputed where they are used: kept across the
-  // loop they would push the wave past its register budget
-  auto fresh = [](int x) __attribute__((always_inline)) {
-    asm volatile("" : "+v"(x));
-    return x;
-  };
   const int goff = C::GO_OFF + wave * C::BLK_BYTES;
   // row-fragment addresses of a tile at LDS address 0 (K, V: the slot is added as an immediate) and
   // of this wave's dO rows
@@ -208,6 +204,16 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   for (int ks = 0; ks < C::KS; ++ks) {
     kx[ks] = koff0 ^ (ks << 5);
     gx[ks] = goff + kx[ks];
+    // the compiler must not know the value's range: it would turn "offset + slot" into an OR computed by a
+    // vector instruction per read; as a plain sum the slot stays the read's immediate offset
+    asm volatile("" : "+v"(kx[ks]));
+  }
+  int zbc[2 * C::DC];                                       // the transposed-fragment offsets of a tile at LDS address 0;
+#pragma unroll                                              // slot and key step are immediate offsets of the reads
+  for (int dc = 0; dc < C::DC; ++dc) {
+    zbc[2 * dc] = voff0 ^ (dc << 6);
+    zbc[2 * dc + 1] = voff0 ^ ((dc << 6) | VOFF_HI);
+    asm volatile("" : "+v"(zbc[2 * dc]), "+v"(zbc[2 * dc + 1]));   // as for kx
   }
   auto zero16 = [](f32x16_t& x) __attribute__((always_inline)) {
 #pragma unroll
@@ -223,33 +229,23 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
       d = mfma32<T>(lds_ld128(kx[ks] + slot_bytes + C::BLK_BYTES), lds_ld128(gx[ks]), d);
     }
   };
-  auto zbase = [&](int slot_bytes, int* zb) __attribute__((always_inline)) {
-    const int b = fresh(voff0 + slot_bytes);
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc) {
-      zb[2 * dc] = b ^ (dc << 6);
-      zb[2 * dc + 1] = b ^ ((dc << 6) | VOFF_HI);
-    }
-  };
-  auto ztr = [&](const int* zb, int n) __attribute__((always_inline)) {   // A operand of the n-th dQ^T MFMA: K^T, keys 16 j ..
+  auto ztr = [&](int slot_bytes, int n) __attribute__((always_inline)) {   // A operand of the n-th dQ^T MFMA: K^T, keys 16 j ..
     const int j = n / C::DC, dc = n % C::DC;
-    const u32x2_t a0 = lds_ld_tr(16 * j * C::ROWB + zb[2 * dc]);
-    const u32x2_t a1 = lds_ld_tr(16 * j * C::ROWB + zb[2 * dc + 1]);
+    const u32x2_t a0 = lds_ld_tr(zbc[2 * dc] + (slot_bytes + 16 * j * C::ROWB));
+    const u32x2_t a1 = lds_ld_tr(zbc[2 * dc + 1] + (slot_bytes + 16 * j * C::ROWB));
     const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
     return a;
   };
   auto stage_z = [&](int slot_bytes) __attribute__((always_inline)) {     // dQ^T += K^T dS^T
-    int zb[2 * C::DC];
-    zbase(slot_bytes, zb);
     // operands are fetched PFZ MFMAs ahead: a fetch that is awaited at once costs the LDS latency per MFMA
     constexpr int NZ = 2 * C::DC, PFZ = 2;
     u32x4_t zf[NZ];
 #pragma unroll
-    for (int n = 0; n < PFZ; ++n) zf[n] = ztr(zb, n);
+    for (int n = 0; n < PFZ; ++n) zf[n] = ztr(slot_bytes, n);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int n = 0; n < NZ; ++n) {
-      if (n + PFZ < NZ) zf[n + PFZ] = ztr(zb, n + PFZ);
+      if (n + PFZ < NZ) zf[n + PFZ] = ztr(slot_bytes, n + PFZ);
       acc[n % C::DC] = mfma32<T>(zf[n], dsf[n / C::DC], acc[n % C::DC]);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -394,16 +390,19 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   zero16(dB);
   stage_x(0, sA, dA);
 
-  auto period = [&](auto Rc, int k) __attribute__((always_inline)) {
+  // ALL: block k lies in front of the whole workgroup and every wave has query rows, so no wave has
+  // anything to decide
+  auto period = [&](auto Rc, int k, auto all) __attribute__((always_inline)) {
     constexpr int R = decltype(Rc)::value;
+    constexpr bool ALL = decltype(all)::value;
     constexpr int CUR = R * C::BUF_BYTES, NXT = ((R + 1) % C::NBUF) * C::BUF_BYTES;
     request(((R + 3) % C::NBUF) * C::BUF_BYTES, k + 3);    // into the slot block k-1 has left
-    if (rowok && k <= cblk) {
+    if (ALL || (rowok && k <= cblk)) {
       f32x16_t& s = (R & 1) ? sB : sA;
       f32x16_t& d = (R & 1) ? dB : dA;
       f32x16_t& sn = (R & 1) ? sA : sB;
       f32x16_t& dn = (R & 1) ? dA : dB;
-      if (k < cblk) stage_xy(NXT, k, s, d, sn, dn);
+      if (ALL || k < cblk) stage_xy(NXT, k, s, d, sn, dn);
       else stage_y_diag(s, d);
       stage_z(CUR);
     }
@@ -414,11 +413,23 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
-  for (int k = 0; k < nblk; k += 4) {
-    period(I0{}, k);
-    if (k + 1 < nblk) period(I1{}, k + 1);
-    if (k + 2 < nblk) period(I2{}, k + 2);
-    if (k + 3 < nblk) period(I3{}, k + 3);
+  // The blocks in front of the workgroup's first query block, in whole turns of the ring, run as straight-line
+  // code without per-wave tests and their branches when every wave of the workgroup has query rows; the
+  // workgroup's own eight blocks and what is left of the turn take the general path.
+  const bool wg_full = (qtile + 1) * C::QT <= p.Lq;
+  const int n_all = wg_full ? (min(nblk, c0) & ~3) : 0;
+  int k = 0;
+  for (; k < n_all; k += 4) {
+    period(I0{}, k, std::true_type{});
+    period(I1{}, k + 1, std::true_type{});
+    period(I2{}, k + 2, std::true_type{});
+    period(I3{}, k + 3, std::true_type{});
+  }
+  for (; k < nblk; k += 4) {
+    period(I0{}, k, std::false_type{});
+    if (k + 1 < nblk) period(I1{}, k + 1, std::false_type{});
+    if (k + 2 < nblk) period(I2{}, k + 2, std::false_type{});
+    if (k + 3 < nblk) period(I3{}, k + 3, std::false_type{});
   }
   dq_wait_vmcnt<0>();                                      // nothing may still be writing LDS when the wave ends
 

@@ -113,7 +113,12 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
   const int koff0 = tile_off<D>(ql, h);
   int kx[C::KS];
 #pragma unroll
-  for (int ks = 0; ks < C::KS; ++ks) kx[ks] = koff0 ^ (ks << 5);
+  for (int ks = 0; ks < C::KS; ++ks) {
+    kx[ks] = koff0 ^ (ks << 5);
+    // the compiler must not know the value's range: it would turn "offset + slot" into an OR computed by a
+    // vector instruction per read; as a plain sum the slot stays the read's immediate offset
+    asm volatile("" : "+v"(kx[ks]));
+  }
   // transposed fragments: lane reads 8 bytes of row 4h + i/4 (+ 8 for the second half) at column
   // 32 dc + 16 g2 + 4 (i%4); dc and the second half are XORs on the dc = 0, first-half offset
   int voff0;
@@ -123,10 +128,13 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
     voff0 = tile_off<D>(4 * h + (i >> 2), col >> 3) + ((col >> 2) & 1) * 8;
   }
   constexpr int VOFF_HI = (8 * C::ROWB) | 32;
-  auto fresh = [](int x) LMK_INL {                         // recompute-at-use marker for lane-only values
-    asm volatile("" : "+v"(x));
-    return x;
-  };
+  int zbc[2 * C::DC];                                       // the transposed-fragment offsets of a tile at LDS address 0;
+#pragma unroll                                              // slot and key step are immediate offsets of the reads
+  for (int dc = 0; dc < C::DC; ++dc) {
+    zbc[2 * dc] = voff0 ^ (dc << 6);
+    zbc[2 * dc + 1] = voff0 ^ ((dc << 6) | VOFF_HI);
+    asm volatile("" : "+v"(zbc[2 * dc]), "+v"(zbc[2 * dc + 1]));   // as for kx
+  }
 
   // ---- requests: wave w issues request n = w*PER_TILE + d of each block (K first, then V).  In a
   // partial last block the rows past Lk re-read the last row (they are masked, but must be readable).
@@ -147,14 +155,16 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
     r_vo_last[d] = (uint32_t)(2 * (min(row, last_rows - 1) * rs + 8 * (chp ^ f)));
     r_lds[d] = (r_isv[d] ? C::BLK_BYTES : 0) + part * 1024;
   }
+  static_assert((32 / C::RPD) % C::PER_TILE == 0, "all of a wave's requests read one tensor");
+  const bool rq_isv = wave * C::PER_TILE >= 32 / C::RPD;   // wave-uniform: this wave fetches V rows (else K rows)
+  const char* rq_base = rq_isv ? vp : kp;
+  const uint32_t rq_step = (uint32_t)(2 * 32 * (rq_isv ? p.vs_r : p.ks_r));   // bytes per block; a head's rows span < 4 GB (host check)
   auto request = [&](int slot_bytes, int blk) LMK_INL {
     const int bb = min(blk, nkb - 1);                      // past the end: re-read the last block (never used)
     const bool last = bb == nkb - 1;                       // wave-uniform
+    const char* base = rq_base + (uint32_t)bb * rq_step;
 #pragma unroll
-    for (int d = 0; d < C::PER_TILE; ++d) {
-      const char* base = r_isv[d] ? vp + 2 * ((int64_t)bb * 32 * p.vs_r) : kp + 2 * ((int64_t)bb * 32 * p.ks_r);
-      fw_dma16(base, last ? r_vo_last[d] : r_vo[d], slot_bytes + r_lds[d]);
-    }
+    for (int d = 0; d < C::PER_TILE; ++d) fw_dma16(base, last ? r_vo_last[d] : r_vo[d], slot_bytes + r_lds[d]);
   };
   // first pass: tile lt holds the landmark keys (row 31) of blocks 32 lt .. 32 lt + 31, row j of the tile =
   // block 32 lt + j, same swizzle as a K block.  Every wave issues one request per tile (with D = 64 the
@@ -190,32 +200,22 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(lds_ld128(kx[ks] + tile_bytes), qf[ks], s);
   };
-  auto zbase = [&](int slot_bytes, int* zb) LMK_INL {
-    const int b = fresh(voff0 + slot_bytes);
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc) {
-      zb[2 * dc] = b ^ (dc << 6);
-      zb[2 * dc + 1] = b ^ ((dc << 6) | VOFF_HI);
-    }
-  };
-  auto ztr = [&](const int* zb, int n) LMK_INL {            // A operand of the n-th O^T MFMA: V^T, keys 16 j ..
+  auto ztr = [&](int tile_bytes, int n) LMK_INL {           // A operand of the n-th O^T MFMA: V^T, keys 16 j ..
     const int j = n / C::DC, dc = n % C::DC;
-    const u32x2_t a0 = lds_ld_tr(16 * j * C::ROWB + zb[2 * dc]);
-    const u32x2_t a1 = lds_ld_tr(16 * j * C::ROWB + zb[2 * dc + 1]);
+    const u32x2_t a0 = lds_ld_tr(zbc[2 * dc] + (tile_bytes + 16 * j * C::ROWB));
+    const u32x2_t a1 = lds_ld_tr(zbc[2 * dc + 1] + (tile_bytes + 16 * j * C::ROWB));
     const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
     return a;
   };
   auto stage_z = [&](int vtile_bytes) LMK_INL {            // O^T += V^T P^T
-    int zb[2 * C::DC];
-    zbase(vtile_bytes, zb);
     constexpr int NZ = 2 * C::DC, PFZ = 2;                  // operands fetched PFZ MFMAs ahead
     u32x4_t zf[NZ];
 #pragma unroll
-    for (int n = 0; n < PFZ; ++n) zf[n] = ztr(zb, n);
+    for (int n = 0; n < PFZ; ++n) zf[n] = ztr(vtile_bytes, n);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int n = 0; n < NZ; ++n) {
-      if (n + PFZ < NZ) zf[n + PFZ] = ztr(zb, n + PFZ);
+      if (n + PFZ < NZ) zf[n + PFZ] = ztr(vtile_bytes, n + PFZ);
       acc[n % C::DC] = mfma32<T>(zf[n], pf[n / C::DC], acc[n % C::DC]);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -350,14 +350,16 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
   zero16(sB);
   stage_x(0, sA);
 
-  auto period = [&](auto Rc, int k) LMK_INL {
+  // ALL: block k lies in front of the whole workgroup, so no wave has anything to decide
+  auto period = [&](auto Rc, int k, auto all) LMK_INL {
     constexpr int R = decltype(Rc)::value;
+    constexpr bool ALL = decltype(all)::value;
     constexpr int CUR = R * C::BUF_BYTES, NXT = ((R + 1) % C::NBUF) * C::BUF_BYTES;
     request(((R + 3) % C::NBUF) * C::BUF_BYTES, k + 3);    // into the slot block k-1 has left
-    if (waveok && k <= cblk) {
+    if (ALL || (waveok && k <= cblk)) {
       f32x16_t& s = (R & 1) ? sB : sA;
       f32x16_t& sn = (R & 1) ? sA : sB;
-      if (k < cblk) stage_xy(NXT, s, sn);
+      if (ALL || k < cblk) stage_xy(NXT, s, sn);
       else stage_y_diag(s);
       stage_z(CUR + C::BLK_BYTES);
     }
@@ -368,11 +370,22 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
-  for (int k = 0; k < nblk; k += 4) {
-    period(I0{}, k);
-    if (k + 1 < nblk) period(I1{}, k + 1);
-    if (k + 2 < nblk) period(I2{}, k + 2);
-    if (k + 3 < nblk) period(I3{}, k + 3);
+  // The blocks in front of the workgroup's first query block, in whole turns of the ring, run as straight-line
+  // code without per-wave tests and their branches (a wave past the last query row computes on zero queries
+  // and stores nothing); the workgroup's own eight blocks and what is left of the turn take the general path.
+  const int n_all = min(nblk, c0) & ~3;
+  int k = 0;
+  for (; k < n_all; k += 4) {
+    period(I0{}, k, std::true_type{});
+    period(I1{}, k + 1, std::true_type{});
+    period(I2{}, k + 2, std::true_type{});
+    period(I3{}, k + 3, std::true_type{});
+  }
+  for (; k < nblk; k += 4) {
+    period(I0{}, k, std::false_type{});
+    if (k + 1 < nblk) period(I1{}, k + 1, std::false_type{});
+    if (k + 2 < nblk) period(I2{}, k + 2, std::false_type{});
+    if (k + 3 < nblk) period(I3{}, k + 3, std::false_type{});
   }
   fw_wait_vmcnt<0>();                                      // nothing may still be writing LDS when the wave ends
 
