@@ -36,6 +36,12 @@ CASES = [
     (1, 2, 160, 256, 128, 32, torch.bfloat16),     # odd history (3 blocks), 5 query blocks
     (1, 2, 544, 544, 128, 32, torch.bfloat16),     # 17 blocks: the LDS rings wrap at every phase
     (1, 2, 544, 544, 64, 32, torch.float16),
+    # blocks in front of a workgroup run in a loop of their own, in whole turns of the 4-slot ring: history of
+    # 5, 6, 7 and 9 blocks leaves 1, 2, 3 and 1 of them to the general path, over two and three query tiles
+    (1, 2, 512, 672, 128, 32, torch.bfloat16),
+    (1, 2, 288, 480, 128, 32, torch.bfloat16),
+    (1, 1, 640, 864, 128, 32, torch.bfloat16),
+    (1, 2, 320, 608, 64, 32, torch.bfloat16),
     (1, 2, 256, 256, 128, 64, torch.bfloat16),
     (1, 2, 128, 320, 128, 64, torch.bfloat16),
     (1, 2, 512, 512, 128, 128, torch.bfloat16),

@@ -38,6 +38,13 @@ CASES = [
     (1, 2, 160, 256, 128, 32, torch.bfloat16),    # odd history (3 blocks)
     (1, 2, 544, 544, 128, 32, torch.bfloat16),    # 17 blocks: the LDS ring wraps at every phase
     (1, 2, 40, 104, 128, 32, torch.bfloat16),     # partial + history
+    # blocks in front of a workgroup run in a loop of their own (whole turns of the 4-slot ring): histories that
+    # leave 1, 2, 3 blocks of a turn to the general path, with and without a partial last block
+    (1, 2, 512, 672, 128, 32, torch.bfloat16),
+    (1, 2, 288, 480, 128, 32, torch.bfloat16),
+    (1, 1, 640, 864, 128, 32, torch.bfloat16),
+    (1, 2, 500, 660, 128, 32, torch.bfloat16),
+    (1, 2, 620, 844, 64, 32, torch.float16),
     (1, 2, 256, 256, 128, 64, torch.bfloat16),
     (1, 2, 256, 384, 128, 64, torch.bfloat16),
     (1, 2, 512, 512, 128, 128, torch.bfloat16),
