@@ -50,8 +50,8 @@ struct Dkv32Cfg {
   static constexpr int NBUF = 6;                           // ring slots: tiles i-1, i, i+1 in use, i+2 .. i+4 in flight
   static constexpr int RPD = 1024 / ROWB;                  // tile rows covered by one 1 KB request
   static constexpr int NDMA = 32 / RPD / NKT;              // requests per wave and tile for one tensor
-  static constexpr int PER_TILE_K = NDMA;                  // K-role waves fetch dO (the role with more arithmetic)
-  static constexpr int PER_TILE_V = NDMA + 1;              // V-role waves fetch Q and their key tile's terms
+  static constexpr int PER_TILE_V = 2 * NDMA + 1;          // the V-role waves fetch everything: Q rows, the key tile's terms,
+                                                           // dO rows (the K role is the longer chain of every iteration)
   static constexpr int XCH_OFF = NBUF * BUF_BYTES;         // W hand-over: [parity 2][key tile][piece 2][lane][16 B]
   static constexpr int XCH_TILE = 2048;
   static constexpr int CONST_OFF = XCH_OFF + 2 * NKT * XCH_TILE;   // 32 x 1e30f, then 32 x 0.0f
@@ -148,28 +148,30 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     }
   }
 
-  // ---- loaders.  Wave pair t fetches rows RPD*(t*NDMA + d) .. of a query tile: the V-role wave those
-  // of Q plus the terms of key tile t, the K-role wave those of dO.
-  static_assert(C::NDMA <= 2, "two source offsets per wave");
+  // ---- loaders.  The V-role wave of pair t fetches rows RPD*(t*NDMA + d) .. of a query tile's Q and dO and the
+  // terms of key tile t; the K-role waves fetch nothing.
+  static_assert(C::NDMA <= 2, "two source offsets per tensor");
   // The requests run four to five query tiles ahead of the arithmetic and do not stop at the end of an item:
   // behind an item's last query tile they go on with the first tiles of the workgroup's next item, so the ring
   // is full when that item starts.  The stream's position is a handful of scalars: the tile it fetches next
   // (j_req), the item's offset into the per-block planes (pl_req), and the same two for the item after it,
   // which the arithmetic side fills in whenever it starts an item (every item but a workgroup's last has more
   // query tiles than the stream runs ahead, so the entry is there before the stream needs it).
-  // per-lane source offset (bytes) of this wave's requests 0 and 1 inside tile 0 of its tensor: Q for the V role, dO for the K role
-  uint32_t lane_vo0, lane_vo1 = 0;
-  const char* src_base = role_k ? gp : qp;                 // wave-uniform
-  const int64_t src_rs = role_k ? p.dos_r : p.qs_r;
-  {
+  // per-lane source offsets (bytes) of this wave's requests 0 and 1 inside tile 0 of Q and of dO
+  uint32_t q_vo0 = 0, q_vo1 = 0, g_vo0 = 0, g_vo1 = 0;
+  if (!role_k) {
     const int chp = lane % C::CH;
     const int row0 = C::RPD * (tile * C::NDMA) + lane / C::CH, row1 = row0 + C::RPD;
     const int f0 = (((row0 & 3) << 2) | ((row0 >> 2) & 3)) & (C::CH - 1);
     const int f1 = (((row1 & 3) << 2) | ((row1 >> 2) & 3)) & (C::CH - 1);
-    lane_vo0 = (uint32_t)(2 * (row0 * src_rs + 8 * (chp ^ f0)));   // the chunk that belongs at LDS position chp
-    if (C::NDMA > 1) lane_vo1 = (uint32_t)(2 * (row1 * src_rs + 8 * (chp ^ f1)));
+    q_vo0 = (uint32_t)(2 * (row0 * p.qs_r + 8 * (chp ^ f0)));      // the chunk that belongs at LDS position chp
+    g_vo0 = (uint32_t)(2 * (row0 * p.dos_r + 8 * (chp ^ f0)));
+    if (C::NDMA > 1) {
+      q_vo1 = (uint32_t)(2 * (row1 * p.qs_r + 8 * (chp ^ f1)));
+      g_vo1 = (uint32_t)(2 * (row1 * p.dos_r + 8 * (chp ^ f1)));
+    }
   }
-  const uint32_t src_step = (uint32_t)(2 * 32 * src_rs);
+  const uint32_t q_step = (uint32_t)(2 * 32 * p.qs_r), g_step = (uint32_t)(2 * 32 * p.dos_r);
   // this lane's 16 bytes of a query tile's terms: lanes 0-7 a, 8-15 nD, 16-23 dS at the landmark (planes, one row
   // of Lq per block), 24-31 mhat, 32-63 delta (one row per head)
   const float* st_lane;                                    // its array at the head's first row, tile 0
@@ -197,9 +199,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   };
   announce_next(0);
   // One piece of this wave's share of the stream's tile -> ring slot.  A tile's pieces go out one per MFMA
-  // slot of the first product rather than together: all eight waves asking at once queue up in front of
-  // the address unit.  V role: pieces 0 .. NDMA-1 fetch Q rows, piece NDMA the terms; K role: dO rows.
-  const int dst_off = (role_k ? C::TILE_BYTES : 0) + tile * C::NDMA * 1024;   // this wave's rows inside a slot
+  // slot of the first product rather than together: all waves asking at once queue up in front of the
+  // address unit.  Pieces 0 .. NDMA-1 fetch Q rows, piece NDMA the terms, pieces NDMA+1 .. 2 NDMA dO rows.
+  const int dst_off = tile * C::NDMA * 1024;               // this wave's rows inside a tile of a slot
   auto request_piece = [&](int slot_bytes, auto Pc) LMK_INL {
     constexpr int P = decltype(Pc)::value;
     if constexpr (P == 0) {                                // a new tile: behind an item's last one, move to the next item
@@ -209,28 +211,31 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       has_nx = take ? false : has_nx;
     }
     if constexpr (P < C::NDMA) {
-      dma16_s(src_base, ((P == 0) ? lane_vo0 : lane_vo1) + (uint32_t)j_req * src_step, slot_bytes + dst_off + P * 1024);
-      if (P == C::NDMA - 1 && role_k) ++j_req;
+      dma16_s(qp, ((P == 0) ? q_vo0 : q_vo1) + (uint32_t)j_req * q_step, slot_bytes + dst_off + P * 1024);
     } else if constexpr (P == C::NDMA) {
-      if (!role_k) {
-        const int64_t off = 32 * (int64_t)j_req + ((lane < 24) ? pl_req : 0);
-        dma16_v(st_lane + off, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
-        ++j_req;
-      }
+      const int64_t off = 32 * (int64_t)j_req + ((lane < 24) ? pl_req : 0);
+      dma16_v(st_lane + off, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
+    } else if constexpr (P <= 2 * C::NDMA) {
+      constexpr int G = P - C::NDMA - 1;
+      dma16_s(gp, ((G == 0) ? g_vo0 : g_vo1) + (uint32_t)j_req * g_step, slot_bytes + C::TILE_BYTES + dst_off + G * 1024);
+      if (P == 2 * C::NDMA) ++j_req;
     }
   };
   using P0 = std::integral_constant<int, 0>;
   using P1 = std::integral_constant<int, 1>;
   using P2 = std::integral_constant<int, 2>;
-  static_assert(C::PER_TILE_V <= 3, "a tile's pieces are P0 .. P2");
-  auto request = [&](int slot_bytes) LMK_INL {             // the whole share at once (prologue, last iterations)
+  using P3 = std::integral_constant<int, 3>;
+  using P4 = std::integral_constant<int, 4>;
+  static_assert(C::PER_TILE_V <= 5 && C::PER_TILE_V <= C::KS, "a tile's pieces are P0 .. P4, one per MFMA slot");
+  auto request = [&](int slot_bytes) LMK_INL {             // the whole share at once (prologue); V role only
     request_piece(slot_bytes, P0{});
     request_piece(slot_bytes, P1{});
     request_piece(slot_bytes, P2{});
+    request_piece(slot_bytes, P3{});
+    request_piece(slot_bytes, P4{});
   };
   auto wait_tiles = [&]() LMK_INL {                        // all but this wave's two newest tiles have landed
-    if (role_k) wait_vmcnt<2 * C::PER_TILE_K>();
-    else wait_vmcnt<2 * C::PER_TILE_V>();
+    if (!role_k) wait_vmcnt<2 * C::PER_TILE_V>();
   };
 
   auto zero16 = [](f32x16_t& x) LMK_INL {
@@ -305,8 +310,10 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 #pragma unroll
       for (int n = (m * NB) / C::KS; n < ((m + 1) * NB) / C::KS; ++n) tf[n] = trfrag(cslot + C::TILE_BYTES, n);
       if (m == 0) request_piece(rslot, P0{});              // tile i+4, into the slot tile i-2 has left
-      if (m == 2) request_piece(rslot, P1{});
-      if (m == 4) request_piece(rslot, P2{});
+      if (m == 1) request_piece(rslot, P1{});
+      if (m == 2) request_piece(rslot, P2{});
+      if (m == 3) request_piece(rslot, P3{});
+      if (m == 4) request_piece(rslot, P4{});
       sn = mfma32<T>(fr[m], bf[m], sn);
 #pragma unroll
       for (int r = (m * 16) / C::KS; r < ((m + 1) * 16) / C::KS; ++r) elementwise(r);
@@ -321,7 +328,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   };
 
   // ---- K role: dP of tile i (slot cslot) interleaved with dS of tile i-1 (slot pslot), then dK of tile i-1.
-  auto body_k = [&](int i, int cslot, int pslot, int rslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc, auto sync) LMK_INL {
+  auto body_k = [&](int i, int cslot, int pslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc, auto sync) LMK_INL {
     const bool masked = PT + (i - 1) < kt_end;             // tile i-1: in the key tile's block or not yet visible
     const int CST = pslot + 2 * C::TILE_BYTES + tile * 1024;
     // y: subtrahend of dP, z: addend of dS  (byte offsets of 32-float arrays)
@@ -367,8 +374,6 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       if (m + 2 < C::KS && grp(m + 2) != grp(m + 1)) ldyz(grp(m + 2));
 #pragma unroll
       for (int n = (m * NB) / C::KS; n < ((m + 1) * NB) / C::KS; ++n) tf[n] = trfrag(pslot, n);
-      if (m == 1) request_piece(rslot, P0{});
-      if (m == 3) request_piece(rslot, P1{});
       dpn = mfma32<T>(fr[m], bf[m], dpn);
 #pragma unroll
       for (int r = (m * 16) / C::KS; r < ((m + 1) * 16) / C::KS; ++r) elementwise(r);
@@ -409,12 +414,16 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   // awaited; tiles j_first+2, +3 go out behind that wait, so the workgroup does not sit through four tiles'
   // worth of traffic (every workgroup of a launch round starts at the same moment) before its first product.
   load_stationary();
-  request(0);
-  request(C::BUF_BYTES);
+  if (!role_k) {
+    request(0);
+    request(C::BUF_BYTES);
+  }
   if (tid < 64) ((float*)(smem + C::CONST_OFF))[tid] = (tid < 32) ? 1e30f : 0.f;
   await_stationary();
-  request(2 * C::BUF_BYTES);
-  request(3 * C::BUF_BYTES);
+  if (!role_k) {
+    request(2 * C::BUF_BYTES);
+    request(3 * C::BUF_BYTES);
+  }
 
   wait_tiles();
   __syncthreads();
@@ -485,21 +494,15 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
         announce_next(c);
         load_stationary();
         await_stationary();
-      } else {
-        request(wrap(sc + 4) * C::BUF_BYTES);               // the fifth tile; later items have it from the item before
       }
 #pragma unroll
       for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
       row_tile(sc * C::BUF_BYTES + C::TILE_BYTES, prv);     // dP of the first tile
-      wait_vmcnt<2 * C::PER_TILE_K>();
-      __syncthreads();
+      __syncthreads();                                      // this role has no loads in flight: the V role's waits cover the ring
       sc = wrap(sc + 1);
       for (int i = j_first + 1; i <= nq; ++i) {
-        auto sync = [&]() LMK_INL {
-          wait_vmcnt<2 * C::PER_TILE_K>();
-          __syncthreads();
-        };
-        body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, wrap(sc + 4) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc, sync);
+        auto sync = [&]() LMK_INL { __syncthreads(); };
+        body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc, sync);
         prv = cur;
         sc = wrap(sc + 1);
       }
