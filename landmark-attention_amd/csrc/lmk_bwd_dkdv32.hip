@@ -328,8 +328,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   };
 
   // ---- K role: dP of tile i (slot cslot) interleaved with dS of tile i-1 (slot pslot), then dK of tile i-1.
-  auto body_k = [&](int i, int cslot, int pslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc, auto sync) LMK_INL {
-    const bool masked = PT + (i - 1) < kt_end;             // tile i-1: in the key tile's block or not yet visible
+  // MASKED: tile i-1 lies in the key tile's block or is not visible yet.
+  auto body_k = [&](auto Mc, int cslot, int pslot, int par_prev, f32x16_t& dpp, f32x16_t& dpn, f32x16_t* acc, auto sync) LMK_INL {
+    constexpr bool masked = decltype(Mc)::value;
     const int CST = pslot + 2 * C::TILE_BYTES + tile * 1024;
     // y: subtrahend of dP, z: addend of dS  (byte offsets of 32-float arrays)
     const int yoff = (masked ? CST + 512 : CST + 128) + 16 * h;
@@ -497,16 +498,38 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       }
 #pragma unroll
       for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
-      row_tile(sc * C::BUF_BYTES + C::TILE_BYTES, prv);     // dP of the first tile
+      int cs = sc * C::BUF_BYTES, ps;                       // byte offsets of the slots of tiles i and i-1
+      row_tile(cs + C::TILE_BYTES, prv);                    // dP of the first tile
       __syncthreads();                                      // this role has no loads in flight: the V role's waits cover the ring
-      sc = wrap(sc + 1);
-      for (int i = j_first + 1; i <= nq; ++i) {
-        auto sync = [&]() LMK_INL { __syncthreads(); };
-        body_k(i, sc * C::BUF_BYTES, wrap(sc + C::NBUF - 1) * C::BUF_BYTES, (i - 1 - j_first) & 1, prv, cur, acc, sync);
+      auto sync = [&]() LMK_INL { __syncthreads(); };
+      int par = 0;                                          // parity of tile i-1 in the W hand-over
+      auto advance = [&]() LMK_INL {
+        ps = cs;
+        cs = (cs == (C::NBUF - 1) * C::BUF_BYTES) ? 0 : cs + C::BUF_BYTES;
+      };
+      advance();
+      // iterations i = j_first+1 .. nq.  First those whose tile i-1 is masked (in the key tile's block or not
+      // visible yet; a handful), then the rest two at a time, so that dP of tiles i-1 and i swap registers
+      // instead of being copied.
+      int i = j_first + 1;
+      const int i_masked_end = min(nq, kt_end - PT);        // last i with PT + (i-1) < kt_end
+      for (; i <= i_masked_end; ++i) {
+        body_k(std::true_type{}, cs, ps, par, prv, cur, acc, sync);
         prv = cur;
-        sc = wrap(sc + 1);
+        par ^= 1;
+        advance();
       }
-      sc = wrap(sc + C::NBUF - 1);                          // the slot behind the last tile: the next item's first tile
+      for (; i + 1 <= nq; i += 2) {
+        body_k(std::false_type{}, cs, ps, par, prv, cur, acc, sync);
+        advance();
+        body_k(std::false_type{}, cs, ps, par ^ 1, cur, prv, acc, sync);
+        advance();
+      }
+      if (i <= nq) {
+        body_k(std::false_type{}, cs, ps, par, prv, cur, acc, sync);
+        advance();
+      }
+      sc = ps / C::BUF_BYTES;                               // the slot behind the last tile: the next item's first tile
       if (active) store_acc(acc, (char*)p.dk + 2 * (b_ * p.dks_b + hh * p.dks_h), p.dks_r, p.scale);
     }
     wait_vmcnt<0>();
