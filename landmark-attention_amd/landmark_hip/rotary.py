@@ -32,19 +32,8 @@ def _rotate(x, cos, sin, position_ids, out=None):
     return out
 
 
-def apply_rotary_pos_emb(q, k, cos, sin, position_ids):
-    """``(q_embed, k_embed)`` as ``llama_mem.py:134-149`` returns them; ``q_embed`` is ``None`` when
-    ``q`` is.  q, k: ``(B, nh, L, hd)`` bf16/fp16 on the GPU with hd 64 or 128."""
-    assert k.is_cuda and k.dtype in _lib.DTYPE_CODES
-    cos, sin = _tables(cos, sin, k.dtype)
-    if q is None:
-        return None, _rotate(k, cos, sin, position_ids)
-    if q.shape != k.shape:                      # e.g. fewer key heads: one launch per tensor
-        return _rotate(q, cos, sin, position_ids), _rotate(k, cos, sin, position_ids)
+def _rotate_qk(q, k, cos, sin, position_ids):
     B, H, L, D = q.shape
-    assert q.dtype == k.dtype and q.device == k.device
-    assert position_ids.dim() == 2 and position_ids.shape[1] == L and position_ids.shape[0] in (1, B)
-    assert position_ids.dtype == torch.int64 and position_ids.device == q.device
     q, k = _lib.kernel_ready(q), _lib.kernel_ready(k)
     position_ids = position_ids.contiguous()
     q_embed, k_embed = torch.empty_like(q), torch.empty_like(k)
@@ -56,3 +45,55 @@ def apply_rotary_pos_emb(q, k, cos, sin, position_ids):
                                             _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
     _lib.check(rc)
     return q_embed, k_embed
+
+
+def _transposed_sin(sin):
+    """The sine table of the transposed rotation.  ``y = x*cos + rotate_half(x)*sin`` is linear in x, and its
+    transpose is the same expression with ``sin`` replaced by ``-cat(sin[..., hd/2:], sin[..., :hd/2])``
+    (for LLaMA's tables, whose halves are equal, simply ``-sin``: the rotation by the opposite angle).  The
+    gradient therefore goes through the same kernel, with the same three roundings torch's autograd applies
+    to the reference expression in a 16-bit model."""
+    h = sin.shape[-1] // 2
+    return (-torch.cat((sin[..., h:], sin[..., :h]), dim=-1)).contiguous()
+
+
+class _Rotary(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, cos, sin, position_ids):
+        ctx.save_for_backward(cos, sin, position_ids)
+        return _rotate(x, cos, sin, position_ids)
+
+    @staticmethod
+    def backward(ctx, dy):
+        cos, sin, position_ids = ctx.saved_tensors
+        return _rotate(dy, cos, _transposed_sin(sin), position_ids), None, None, None
+
+
+class _RotaryQK(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, cos, sin, position_ids):
+        ctx.save_for_backward(cos, sin, position_ids)
+        return _rotate_qk(q, k, cos, sin, position_ids)
+
+    @staticmethod
+    def backward(ctx, dq, dk):
+        cos, sin, position_ids = ctx.saved_tensors
+        gq, gk = _rotate_qk(dq, dk, cos, _transposed_sin(sin), position_ids)
+        return gq, gk, None, None, None
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, position_ids):
+    """``(q_embed, k_embed)`` as ``llama_mem.py:134-149`` returns them; ``q_embed`` is ``None`` when
+    ``q`` is.  q, k: ``(B, nh, L, hd)`` bf16/fp16 on the GPU with hd 64 or 128.  Differentiable in q and k,
+    as the reference's expression is (the tables and positions get no gradient)."""
+    assert k.is_cuda and k.dtype in _lib.DTYPE_CODES
+    cos, sin = _tables(cos, sin, k.dtype)
+    if q is None:
+        return None, _Rotary.apply(k, cos, sin, position_ids)
+    if q.shape != k.shape:                      # e.g. fewer key heads: one launch per tensor
+        return _Rotary.apply(q, cos, sin, position_ids), _Rotary.apply(k, cos, sin, position_ids)
+    B, H, L, D = q.shape
+    assert q.dtype == k.dtype and q.device == k.device
+    assert position_ids.dim() == 2 and position_ids.shape[1] == L and position_ids.shape[0] in (1, B)
+    assert position_ids.dtype == torch.int64 and position_ids.device == q.device
+    return _RotaryQK.apply(q, k, cos, sin, position_ids)

@@ -55,3 +55,25 @@ def test_ring_storage_bookkeeping_matches_the_restated_store_in_cache():
             assert s.oldest_slot == (int(omc.slot_ages(n, r.cache_iter).argmin()) if n else 0)
         s.clear_state()
         assert (s.cache_iter, s.cache_size, s.last_incomplete_len) == (0, 0, 0)
+
+
+def test_transposed_rotation_table_gives_the_gradient_of_the_rotary_expression():
+    # the gradient of y = x*cos + rotate_half(x)*sin with respect to x is the same expression on dy with the
+    # table landmark_hip.rotary._transposed_sin(sin); checked in fp64 against torch autograd with tables whose
+    # two halves differ (LLaMA's are equal, which would hide a wrong swap)
+    import torch
+
+    from landmark_hip.rotary import _transposed_sin
+    from oracle import rotary as orot
+    g = torch.Generator().manual_seed(3)
+    n, D = 9, 16
+    cos, sin = (torch.randn(n, D, generator=g, dtype=torch.float64) for _ in range(2))
+    x = torch.randn(2, n, D, generator=g, dtype=torch.float64, requires_grad=True)
+    dy = torch.randn(2, n, D, generator=g, dtype=torch.float64)
+    y = x * cos + orot.rotate_half(x) * sin
+    (want,) = torch.autograd.grad(y, x, dy)
+    got = dy * cos + orot.rotate_half(dy) * _transposed_sin(sin)
+    assert torch.allclose(got, want, rtol=0, atol=1e-14)
+    # LLaMA's tables: the transposed rotation is the rotation by the opposite angle
+    c2, s2 = orot.rotary_tables(n, D, torch.float64)
+    assert torch.equal(_transposed_sin(s2), -s2)

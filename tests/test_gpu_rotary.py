@@ -110,3 +110,34 @@ def test_forward_with_q_rotated_in_the_prologue_is_bit_identical(B, H, Lq, Lk, D
     assert torch.equal(q_rot.cpu(), ref)
     with pytest.raises(AssertionError):
         fused_landmark_attention_rotary_q(q.clone().requires_grad_(True), k_rot, v, cos, sin, pos_q, block_size=block)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,L,D,share_pos", [(2, 3, 70, 128, False), (1, 2, 33, 64, True)])
+def test_rotary_gradients_match_torch_autograd_of_the_reference_expression(B, H, L, D, share_pos, dtype):
+    # apply_rotary_pos_emb is differentiable in q and k (llama_mem.py:134-149 is plain torch arithmetic); the
+    # gradient is the transposed rotation, through the same kernel.  Compared with torch's autograd through the
+    # reference expression evaluated in the model dtype on the CPU: one rounding per elementwise operation on
+    # both sides, so bit for bit.
+    from landmark_hip.rotary import apply_rotary_pos_emb
+    print(f"case grad B{B} H{H} L{L} D{D} {dtype}", flush=True)
+    q, k, cos, sin, n_pos, g = _case(B, H, L, D, dtype, seed=B * 10 + L)
+    pos = torch.randint(0, n_pos, (1 if share_pos else B, L), generator=g)
+    dq = torch.randn(B, H, L, D, generator=g).to(dtype)
+    dk = torch.randn(B, H, L, D, generator=g).to(dtype)
+    qc, kc = q.clone().requires_grad_(True), k.clone().requires_grad_(True)
+    c, s = cos[pos].unsqueeze(1), sin[pos].unsqueeze(1)
+    ref_q = (qc * c) + (orot.rotate_half(qc) * s)
+    ref_k = (kc * c) + (orot.rotate_half(kc) * s)
+    want_q, want_k = torch.autograd.grad([ref_q, ref_k], [qc, kc], [dq, dk])
+    qd, kd = q.cuda().requires_grad_(True), k.cuda().requires_grad_(True)
+    out_q, out_k = apply_rotary_pos_emb(qd, kd, cos.cuda(), sin.cuda(), pos.cuda())
+    assert out_q.requires_grad and out_k.requires_grad
+    got_q, got_k = torch.autograd.grad([out_q, out_k], [qd, kd], [dq.cuda(), dk.cuda()])
+    torch.cuda.synchronize()
+    assert torch.equal(got_q.cpu(), want_q) and torch.equal(got_k.cpu(), want_k)
+    # k alone (q is None), and through the fused attention: the gradient reaches the un-rotated projections
+    kd2 = k.cuda().requires_grad_(True)
+    _, only_k = apply_rotary_pos_emb(None, kd2, cos.cuda(), sin.cuda(), pos.cuda())
+    (g2,) = torch.autograd.grad(only_k, kd2, dk.cuda())
+    assert torch.equal(g2.cpu(), want_k)
