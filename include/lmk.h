@@ -80,13 +80,24 @@ int lmk_attn_fwd_rotary_q(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_
  * terms handed from the dQ kernel to the dK/dV kernel. */
 size_t lmk_attn_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int block);
 
+/* Bytes of workspace that select the HAND-OVER backward (block 32 only; 0 where it does not apply).
+ * Handed a workspace of at least this size, lmk_attn_bwd lets the dQ kernel leave dS of every
+ * (query tile, key block) pair behind as 16-bit tiles (2 KB per pair of 32 x 32, about Lq*(Lk+Lq)/2 * 2 bytes
+ * per (batch, head): 274 MB at B2 H32 L2048, 8.6 GB at B1 H32 L16384) and the dK/dV kernel reads them
+ * instead of forming dP and dS a second time -- each score and each dP is then formed twice per step, not
+ * three times.  With a smaller workspace (>= lmk_attn_bwd_workspace_bytes) the recomputing kernels run.
+ * The reference forms S and dP once in one kernel (flash_landmark_attention.py:246-299) and pays for it with
+ * one program per (batch, head). */
+size_t lmk_attn_bwd_handover_workspace_bytes(int B, int H, int Lq, int Lk, int block);
+
 /* Backward pass.  Replaces the launches of `_bwd_preprocess` and `_bwd_kernel` in
  * FusedLandmarkAttention.backward (llama/ltriton/flash_landmark_attention.py:356-389,
  * kernels :125-149 and :152-305).
  *   inputs: q, k, v, o (forward output), dout (gradient of o), L, M (forward statistics);
  *   outputs: dq (B,H,Lq,D), dk, dv (B,H,Lk,D) in the tensors' 16-bit dtype (accumulated in
  *   fp32, rounded once); every element is written, nothing needs zeroing.
- *   workspace: 16-byte aligned device memory of at least lmk_attn_bwd_workspace_bytes().
+ *   workspace: 16-byte aligned device memory of at least lmk_attn_bwd_workspace_bytes(); one of at least
+ *   lmk_attn_bwd_handover_workspace_bytes() (when that is not 0) selects the faster hand-over kernels.
  * Lq and Lk must be multiples of block (as in the reference, :359-360). */
 int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                  const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,

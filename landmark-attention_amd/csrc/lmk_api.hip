@@ -284,6 +284,21 @@ size_t lmk_attn_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int block) {
   return sizeof(float) * (2 * rows + 3 * rows * nb);
 }
 
+// hand-over layout: delta, mhat (rows floats each), the `a` plane (rows * nb floats), then the dS tiles at the
+// next multiple of 2 KB
+static size_t handover_tiles_offset(size_t rows, size_t nb) {
+  const size_t head = sizeof(float) * (2 * rows + rows * nb);
+  return (head + 2047) & ~(size_t)2047;
+}
+
+size_t lmk_attn_bwd_handover_workspace_bytes(int B, int H, int Lq, int Lk, int block) {
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0 || block != 32 || Lq % 32 != 0 || Lk % 32 != 0 || Lk < Lq) return 0;
+  const size_t rows = (size_t)B * H * Lq;
+  const size_t nb = (size_t)(Lk / 32);
+  const size_t tiles = (size_t)lmk::handover_tiles_per_head(Lq / 32, (Lk - Lq) / 32);
+  return handover_tiles_offset(rows, nb) + (size_t)B * H * tiles * 2048;
+}
+
 int lmk_attn_bwd(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                  const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
                  const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B, int H,
@@ -347,6 +362,13 @@ static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
   p.stat_a = w + 2 * rows;
   p.stat_n = w + 2 * rows + rows * nb;
   p.stat_l = w + 2 * rows + 2 * rows * nb;
+  // a workspace large enough for the dS tiles selects the hand-over backward (block 32, unpadded)
+  const size_t ho_bytes = (block_real == block) ? lmk_attn_bwd_handover_workspace_bytes(B, H, Lq, Lk, block) : 0;
+  p.ds_tiles = nullptr;
+  if (ho_bytes != 0 && workspace_bytes >= ho_bytes) {
+    p.ds_tiles = static_cast<char*>(workspace) + handover_tiles_offset(rows, nb);
+    p.stat_n = p.stat_l = nullptr;
+  }
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
   p.n_prefix = n_prefix; p.n_blocks = (int)nb;
   p.n_real = block_real;

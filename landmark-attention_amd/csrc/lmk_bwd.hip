@@ -368,6 +368,10 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
     }
   }
   if (phases & 4) {
+    if (p.ds_tiles != nullptr) {
+      if (BS != 32) return LMK_ERR_UNSUPPORTED;
+      return launch_bwd_dkdv32_handover(p, D, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream);
+    }
     return launch_bwd_dkdv32(p, D, BS, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream);
   }
   return 0;

@@ -55,7 +55,10 @@ __device__ __forceinline__ void dq_wait_vmcnt() {          // s_waitcnt vmcnt(N)
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <class T, int D>
+// HO: the hand-over variant.  dS^T of every (query tile, key block) pair also goes to p.ds_tiles as a 2 KB tile
+// [key step][query row][key of the step, in this kernel's register order], two 16-byte stores per lane and block, for the dK/dV
+// kernel that then forms neither dP nor dS; of the per-block terms only `a` is still needed.
+template <class T, int D, bool HO>
 __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   using C = Dq32Cfg<T, D>;
   extern __shared__ __align__(16) unsigned char smem[];   // used through LDS byte addresses (it starts at 0)
@@ -92,6 +95,21 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   const int nkb = p.Lk >> 5;
   const int nblk = min(nkb, c0 + C::NW);
   const float c2 = p.scale_log2;
+  // hand-over: this wave's tiles are consecutive, one per key block (wave-uniform address)
+  const char* ds_wave = nullptr;
+  if (HO) {
+    const int64_t j = qtile * C::NW + wave;
+    ds_wave = (const char*)p.ds_tiles +
+              (((int64_t)bh * handover_tiles_per_head(p.Lq >> 5, p.n_prefix) + j * (p.n_prefix + 1) + j * (j - 1) / 2) << 11);
+  }
+  auto store_ds = [&](int blk, const u32x4_t& d0, const u32x4_t& d1) __attribute__((always_inline)) {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    const uint32_t vo = (uint32_t)(((l & 31) << 5) | ((l >> 5) << 4));   // per key step 1 KB: row = query, 16 bytes per half-wave
+    const char* tb = ds_wave + ((int64_t)blk << 11);
+    asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(vo), "v"(d0), "s"(tb) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, %2 offset:1024" ::"v"(vo), "v"(d1), "s"(tb) : "memory");
+  };
 
   u32x4_t qf[C::KS];
 #pragma unroll
@@ -187,7 +205,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
     const int64_t ub = ((int64_t)bh * p.n_blocks + b0) * p.Lq + q0;
     if (b0 + fl_bi <= blast) {
 #pragma unroll
-      for (int pl = 0; pl < 3; ++pl) {
+      for (int pl = 0; pl < (HO ? 1 : 3); ++pl) {
         const float* base = (pl == 0 ? p.stat_a : pl == 1 ? p.stat_n : p.stat_l) + ub;
         const u32x4_t val = lds_ld128(fl_lds + pl * C::FL * 128);
         asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(fl_off), "v"(val), "s"(base) : "memory");
@@ -307,8 +325,10 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
           const int bi = blk & (C::FL - 1);
           const int sp = C::STAT_OFF + wave * C::STAT_WAVE + bi * 128 + ln * 4;
           lds_st32(sp + 0 * C::FL * 128, mloc + fast_log2(den) - glog);
-          lds_st32(sp + 1 * C::FL * 128, nD);
-          lds_st32(sp + 2 * C::FL * 128, dslm);
+          if (!HO) {
+            lds_st32(sp + 1 * C::FL * 128, nD);
+            lds_st32(sp + 2 * C::FL * 128, dslm);
+          }
         }
       } else {
 #pragma unroll
@@ -330,6 +350,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
       for (int u = (m * 16) / NX; u < ((m + 1) * 16) / NX; ++u) ywork(u);
       __builtin_amdgcn_sched_barrier(0);
     }
+    if (HO) store_ds(blk, dsf[0], dsf[1]);
     if ((blk & (C::FL - 1)) == C::FL - 1 || blk == cblk - 1) flush(blk);
   };
   auto stage_y_diag = [&](const f32x16_t& s, const f32x16_t& d) __attribute__((always_inline)) {   // the wave's own block
@@ -347,6 +368,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
                     pack2<T>(ds[8 * j + 4], ds[8 * j + 5]), pack2<T>(ds[8 * j + 6], ds[8 * j + 7])};
       dsf[j] = fr;
     }
+    if (HO) store_ds(cblk, dsf[0], dsf[1]);
   };
 
   // ---- prologue: this wave's dO rows -> LDS; blocks 0 .. 2 requested; blocks 0 and 1 must have landed
@@ -405,8 +427,13 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
       if (ALL || k < cblk) stage_xy(NXT, k, s, d, sn, dn);
       else stage_y_diag(s, d);
       stage_z(CUR);
+      // block k+2 has landed (k+3 may be in flight).  Behind its requests this wave has issued at least the two
+      // tile stores of the previous period (in the first period: the two row-term stores of the prologue), the
+      // requests of block k+3 and the two tile stores of this period; memory operations of a wave complete in order
+      dq_wait_vmcnt<C::PER_TILE + (HO ? 4 : 0)>();
+    } else {
+      dq_wait_vmcnt<C::PER_TILE>();
     }
-    dq_wait_vmcnt<C::PER_TILE>();                          // block k+2 has landed (k+3 may be in flight)
     __syncthreads();
   };
   using I0 = std::integral_constant<int, 0>;
@@ -446,15 +473,20 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   }
 }
 
-template <class T, int D>
-static int launch_dq32_t(const BwdParams& p, hipStream_t stream) {
+template <class T, int D, bool HO>
+static int launch_dq32_h(const BwdParams& p, hipStream_t stream) {
   using C = Dq32Cfg<T, D>;
-  auto kern = lmk_bwd_dq32_kernel<T, D>;
+  auto kern = lmk_bwd_dq32_kernel<T, D, HO>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   const int n_qt = (p.Lq + C::QT - 1) / C::QT;
   hipLaunchKernelGGL(kern, dim3(n_qt * p.B * p.H), dim3(C::NTHR), C::LDS_BYTES, stream, p);
   return (int)hipGetLastError();
+}
+
+template <class T, int D>
+static int launch_dq32_t(const BwdParams& p, hipStream_t stream) {
+  return p.ds_tiles != nullptr ? launch_dq32_h<T, D, true>(p, stream) : launch_dq32_h<T, D, false>(p, stream);
 }
 
 int launch_bwd_dq32(const BwdParams& p, int D, int dtype, hipStream_t stream) {

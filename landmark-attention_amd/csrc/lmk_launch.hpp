@@ -65,6 +65,11 @@ struct BwdParams {
   const float *L, *M;            // forward statistics, (B*H, Lq)
   float *delta, *mhat;           // (B*H, Lq) each, written by the pre kernel
   float *stat_a, *stat_n, *stat_l;   // (B*H, n_blocks, Lq) each, written by the dq kernel
+  // hand-over (block 32 only): the dq kernel leaves dS of every (query tile, key block) pair behind as a 2 KB
+  // 16-bit tile and the dK/dV kernel reads it instead of forming dP and dS again; then stat_n and stat_l are unused.
+  // Tiles of a head are ordered by query tile, then key block: tile (j, k), k <= n_prefix + j, is number
+  // j * (n_prefix + 1) + j * (j - 1) / 2 + k.  Null: no hand-over.
+  void* ds_tiles;
   int B, H, Lq, Lk;
   int n_prefix, n_blocks;        // history blocks; Lk / block
   int n_qtiles, n_kvtiles;       // ceil(Lq / 128), ceil(Lk / 128)
@@ -78,6 +83,12 @@ struct BwdParams {
 int launch_bwd(const BwdParams& p, int D, int BS, int dtype, int phases, hipStream_t stream);
 int launch_bwd_dq32(const BwdParams& p, int D, int dtype, hipStream_t stream);     // block 32 specialisation
 int launch_bwd_dkdv32(const BwdParams& p, int D, int BS, int dtype, hipStream_t stream);   // two-role kernel, all block sizes
+int launch_bwd_dkdv32_handover(const BwdParams& p, int D, int dtype, hipStream_t stream);  // block 32, dS read from p.ds_tiles
+
+// dS tiles (2 KB each) one (batch, head) leaves behind in the hand-over: query tile j sees key blocks 0 .. n_prefix + j
+__host__ __device__ inline int64_t handover_tiles_per_head(int64_t n_qtiles32, int64_t n_prefix) {
+  return n_qtiles32 * (n_prefix + 1) + n_qtiles32 * (n_qtiles32 - 1) / 2;
+}
 
 struct RetrParams {
   const void *q, *kcache, *vcache, *cos, *sin;   // q rotated; caches un-rotated; tables (n_pos, D)

@@ -50,6 +50,8 @@ def lib() -> ctypes.CDLL:
         L.lmk_attn_fwd.argtypes = [T4, T4, T4, T4, vp, vp, i, i, i, i, i, f, i, i, i, vp]
         L.lmk_attn_bwd_workspace_bytes.restype = ctypes.c_size_t
         L.lmk_attn_bwd_workspace_bytes.argtypes = [i, i, i, i, i]
+        L.lmk_attn_bwd_handover_workspace_bytes.restype = ctypes.c_size_t
+        L.lmk_attn_bwd_handover_workspace_bytes.argtypes = [i, i, i, i, i]
         L.lmk_attn_bwd.restype = i
         L.lmk_attn_bwd.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, ctypes.c_size_t,
                                    i, i, i, i, i, f, i, i, i, vp]

@@ -17,6 +17,7 @@ Differences a caller can observe, all of them relaxations:
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 
@@ -25,6 +26,13 @@ from . import _lib
 SUPPORTED_BLOCKS = (32, 64, 128)      # block sizes the kernels run without repacking
 MAX_BLOCK = 128
 SUPPORTED_HEAD_DIMS = (64, 128)
+# Two backward paths exist for block 32.  With a workspace of lmk_attn_bwd_handover_workspace_bytes() the dQ kernel
+# leaves dS behind for the dK/dV kernel (2 bytes per visible (query, key) pair), which then forms neither dP nor dS
+# again.  That pays while the tiles stay in the GPU's 256 MB last-level cache between the two kernels (measured:
+# backward 4 % faster at B1 H32 L2048, 154 MB) and loses once they have to travel through HBM (7 % slower at
+# B2 H32 L2048, 307 MB), so workspaces above this many bytes are not allocated and the recomputing kernels run
+# in 4 * (2 + 3 * Lk / block) bytes per query row.
+HANDOVER_MAX_BYTES = int(os.environ.get("LMK_BWD_HANDOVER_MAX_MB", "160")) << 20
 PADDED_HEAD_DIMS = (16, 32)          # accepted by fused_landmark_attention, zero-padded to 64
 
 
@@ -73,6 +81,10 @@ def _launch_bwd(q, k, v, o, do, L, M, n_prefix, sm_scale, block, block_real=None
     lib = _lib.lib()
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)     # each in its input's layout
     nbytes = lib.lmk_attn_bwd_workspace_bytes(B, H, Lq, Lk, int(block))
+    if block_real == block:
+        ho = lib.lmk_attn_bwd_handover_workspace_bytes(B, H, Lq, Lk, int(block))
+        if 0 < ho <= HANDOVER_MAX_BYTES:
+            nbytes = ho          # the library picks the hand-over kernels from the size it is handed
     ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
     rc = lib.lmk_attn_bwd_padded(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o),
                                  _lib.tensor4(do), L.data_ptr(), M.data_ptr(), _lib.tensor4(dq), _lib.tensor4(dk),

@@ -90,6 +90,12 @@ def test_backward_argument_errors(lib):
     need = lib.lmk_attn_bwd_workspace_bytes(2, 32, 2048, 2048, 32)
     assert need == 4 * (2 * 2 * 32 * 2048 + 3 * 2 * 32 * 2048 * 64)
     assert lib.lmk_attn_bwd_workspace_bytes(0, 1, 1, 1, 1) == 0
+    # hand-over workspace: row terms + one plane, rounded up to 2 KB, + one 2 KB tile per visible (query tile, block)
+    ho = lib.lmk_attn_bwd_handover_workspace_bytes(2, 32, 2048, 2048, 32)
+    assert ho == 4 * (2 * 2 * 32 * 2048 + 2 * 32 * 2048 * 64) + 64 * (64 * 65 // 2) * 2048
+    assert lib.lmk_attn_bwd_handover_workspace_bytes(1, 2, 64, 128, 32) == 4096 + 2 * (2 * 3 + 1) * 2048
+    assert lib.lmk_attn_bwd_handover_workspace_bytes(2, 32, 2048, 2048, 64) == 0     # block 32 only
+    assert lib.lmk_attn_bwd_handover_workspace_bytes(1, 1, 48, 48, 32) == 0          # whole blocks only
 
 
 def test_retrieval_argument_errors(lib):

@@ -14,6 +14,15 @@ pytestmark = pytest.mark.gpu
 TOL = 2e-2
 
 
+@pytest.fixture(params=["recompute", "handover"])
+def bwd_path(request, monkeypatch):
+    """Both backward paths of block 32: the kernels that form dS twice, and the hand-over of dS tiles from the
+    dQ kernel to the dK/dV kernel (chosen by the size of the workspace the shim allocates)."""
+    from landmark_hip import attention
+    monkeypatch.setattr(attention, "HANDOVER_MAX_BYTES", 0 if request.param == "recompute" else 1 << 40)
+    return request.param
+
+
 def _grads(q, k, v, do, block, scale=None):
     from ltriton.flash_landmark_attention import fused_landmark_attention
     dev = torch.device("cuda:0")
@@ -57,8 +66,10 @@ CASES = [
 
 
 @pytest.mark.parametrize("B,H,Lq,Lk,D,block,dtype", CASES)
-def test_gradients_match_oracle(B, H, Lq, Lk, D, block, dtype):
-    print(f"case B{B} H{H} Lq{Lq} Lk{Lk} D{D} bs{block} {dtype}", flush=True)
+def test_gradients_match_oracle(B, H, Lq, Lk, D, block, dtype, bwd_path):
+    if block != 32 and bwd_path == "handover":
+        pytest.skip("the hand-over exists for block 32 only; other sizes always recompute")
+    print(f"case B{B} H{H} Lq{Lq} Lk{Lk} D{D} bs{block} {dtype} {bwd_path}", flush=True)
     seed = Lq + Lk + D + block
     q, k, v = make_qkv(B, H, Lq, Lk, D, seed=seed, dtype=dtype)
     do = torch.randn(B, H, Lq, D, generator=torch.Generator().manual_seed(seed + 1)).to(dtype)
@@ -130,7 +141,7 @@ def test_partial_block_backward_is_rejected():
         out.sum().backward()
 
 
-def test_backward_deterministic_bitwise():
+def test_backward_deterministic_bitwise(bwd_path):
     B, H, L, D, block = 2, 8, 512, 128, 32
     q, k, v = make_qkv(B, H, L, L, D, seed=13)
     do = torch.randn(B, H, L, D, generator=torch.Generator().manual_seed(14)).bfloat16()
@@ -141,7 +152,9 @@ def test_backward_deterministic_bitwise():
 
 
 @pytest.mark.parametrize("seed", [0, 1, 2])
-def test_baseline_config2_full_size(seed):
+def test_baseline_config2_full_size(seed, bwd_path):
+    if bwd_path == "handover" and seed != 0:
+        pytest.skip("the hand-over path runs the full size once")
     # benchmark config 2: B2 H32 L2048 D128 block 32, dO ~ N(0,1); seed 0 is the benchmark's, 1 and 2 for robustness
     B, H, L, D, block = 2, 32, 2048, 128, 32
     q, k, v = make_qkv(B, H, L, L, D, seed=seed)
@@ -170,7 +183,7 @@ def test_gradients_with_a_custom_softmax_scale(scale, block, Lq, Lk):
 
 
 @pytest.mark.parametrize("Lq,Lk", [(256, 4352), (4608, 4608)])
-def test_gradients_beyond_64_blocks(Lq, Lk):
+def test_gradients_beyond_64_blocks(Lq, Lk, bwd_path):
     # 136 and 144 landmark blocks of 32: long history in front of few queries, and a long square problem
     B, H, D, block = 1, 2, 128, 32
     print(f"case long Lq{Lq} Lk{Lk}", flush=True)
@@ -240,7 +253,9 @@ def test_reference_script_case():
     (8, 32, 512, 512, 128, 128, torch.bfloat16),     # blocks of four tiles
     (6, 32, 416, 416, 128, 32, torch.bfloat16),      # last tile of a head partly empty (13 key tiles of 32)
 ])
-def test_gradients_with_several_key_tiles_per_workgroup(B, H, Lq, Lk, D, block, dtype):
+def test_gradients_with_several_key_tiles_per_workgroup(B, H, Lq, Lk, D, block, dtype, bwd_path):
+    if block != 32 and bwd_path == "handover":
+        pytest.skip("the hand-over exists for block 32 only")
     print(f"case multi-item B{B} H{H} Lq{Lq} Lk{Lk} D{D} bs{block} {dtype}", flush=True)
     seed = B + Lq + Lk + D + block
     q, k, v = make_qkv(B, H, Lq, Lk, D, seed=seed, dtype=dtype)
@@ -250,3 +265,42 @@ def test_gradients_with_several_key_tiles_per_workgroup(B, H, Lq, Lk, D, block, 
     for name, g, r in (("dq", gq, rq), ("dk", gk, rk), ("dv", gv, rv)):
         err = (g.float().cpu() - r).abs().max().item()
         assert err <= TOL, (name, err)
+
+
+def test_workspace_size_selects_the_backward_path():
+    # lmk_attn_bwd picks the hand-over kernels when the workspace reaches lmk_attn_bwd_handover_workspace_bytes and
+    # the recomputing kernels one byte below; both sides of the threshold give the oracle's gradients, and the two
+    # paths are different code (their dK differs in the last bits)
+    import math
+    from landmark_hip import _lib
+    from landmark_hip.attention import _launch_fwd
+    lib, T4 = _lib.lib(), _lib.tensor4
+    B, H, Lq, Lk, D, block = 1, 4, 256, 384, 128, 32
+    q, k, v = make_qkv(B, H, Lq, Lk, D, seed=77)
+    do = torch.randn(B, H, Lq, D, generator=torch.Generator().manual_seed(78)).bfloat16()
+    rq, rk, rv = oracle_grads(q, k, v, do, block)
+    dev = torch.device("cuda:0")
+    qd, kd, vd, dod = (t.to(dev) for t in (q, k, v, do))
+    scale = 1.0 / math.sqrt(D)
+    n_prefix = (Lk - Lq) // block
+    o, Ls, M = _launch_fwd(qd, kd, vd, n_prefix, scale, block)
+    small = lib.lmk_attn_bwd_workspace_bytes(B, H, Lq, Lk, block)
+    big = lib.lmk_attn_bwd_handover_workspace_bytes(B, H, Lq, Lk, block)
+    rows, nb, nq = B * H * Lq, Lk // block, Lq // block
+    tiles = nq * (n_prefix + 1) + nq * (nq - 1) // 2
+    assert big == ((4 * (2 * rows + rows * nb) + 2047) // 2048) * 2048 + B * H * tiles * 2048 and big > small
+    assert lib.lmk_attn_bwd_handover_workspace_bytes(B, H, Lq, Lk, 64) == 0
+    ws = torch.empty(big, device=dev, dtype=torch.uint8)
+    got = {}
+    for name, nbytes in (("below", big - 1), ("at", big), ("small", small)):
+        dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
+        ws.fill_(0xFF)                                        # NaN patterns: nothing may be read that was not written
+        _lib.check(lib.lmk_attn_bwd(T4(qd), T4(kd), T4(vd), T4(o), T4(dod), Ls.data_ptr(), M.data_ptr(), T4(dq), T4(dk),
+                                    T4(dv), ws.data_ptr(), nbytes, B, H, Lq, Lk, D, scale, block, n_prefix, 0,
+                                    _lib.current_stream(dev)))
+        torch.cuda.synchronize()
+        for nm, g, r in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+            assert (g.float().cpu() - r).abs().max().item() <= TOL, (name, nm)
+        got[name] = (dq, dk, dv)
+    assert all(torch.equal(a, b_) for a, b_ in zip(got["below"], got["small"]))
+    assert not torch.equal(got["at"][1], got["small"][1])
