@@ -269,6 +269,24 @@ int lmk_ring_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kring, const
                            void* workspace, size_t workspace_bytes, int B, int H, int T, int n_blocks, int D, int block,
                            int top_k, int ring_start, int method, int dtype, void* stream);
 
+/* Attention over the picked blocks of the ring, merged with the attention over the current chunk: the part of
+ * MemLMCacheStorage.retrieve_for_query behind the selection (lm_benchmark/models/caches/mem_cache.py:86-109:
+ * take_along_dim of the picked blocks' keys and values, keys rotated at k_indices = j*block + token, one block
+ * further for a block among the top_k newest (:95-97), scores q.k/sqrt(D), is_mem prefix) and what
+ * CausalSelfAttention.forward does with it (lm_benchmark/models/landmark.py:196-242: the picked blocks are earlier
+ * landmark groups in front of the chunk, grouped softmax, att_prefix @ cache_v added to att @ v).
+ *   q: (B,H,T,D) rotated queries; kring, vring: (B,H,n_blocks*block,D) views of the filled slots (keys without
+ *   rotary), as for lmk_ring_retrieve_topk; idx: the slots that call returned, in its shape for `method`;
+ *   o_loc, L_loc, M_loc, stat_stride: output and statistics of lmk_attn_fwd[_padded] over
+ *   [tokens behind the last complete block (last_incomplete_k, rotated; :43-46) ; the chunk], rows of the chunk --
+ *   as for lmk_gather_attend; out: (B,H,T,D).
+ * block: 2..128 tokens (the benchmark's 51 are worked on in 64 slots; nothing is repacked); D 64 or 128. */
+int lmk_ring_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kring, const lmk_tensor4* vring, const int64_t* idx,
+                           const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
+                           const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, int64_t stat_stride,
+                           const lmk_tensor4* out, int B, int H, int T, int n_blocks, int D, float sm_scale, int block,
+                           int top_k, int ring_start, int method, int dtype, void* stream);
+
 /* Local window of the attend step when the cache ends in an incomplete block of
  * inc = S % block tokens (llama_mem.py:329-342; needs inc > 0 and T + inc <= block, the
  * reference's assert at :330).  Writes, each (B,H,inc+T,D):

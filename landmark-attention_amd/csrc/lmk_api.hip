@@ -480,6 +480,7 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
   fill_retr_common(p, B, H, T, S, D, block, top_k);
   p.q = q->ptr; p.kcache = kcache->ptr; p.vcache = vcache->ptr; p.cos = cos_table; p.sin = sin_table;
   p.idx = const_cast<int64_t*>(idx);
+  p.idx_st = p.k; p.idx_sh = (int64_t)T * p.k; p.idx_sb = (int64_t)H * T * p.k;
   p.o_loc = o_loc->ptr; p.L_loc = L_loc; p.M_loc = M_loc; p.stat_stride = stat_stride; p.out = out->ptr;
   p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
   p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
@@ -582,6 +583,50 @@ int lmk_ring_retrieve_topk(const lmk_tensor4* q, const lmk_tensor4* kring, const
   p.agg_over_heads = method == LMK_SELECT_MAX_OVER_HEADS;
   p.prob32 = 1;                                                              // softmax output stays fp32 under autocast
   return lmk::launch_retrieve_topk_shared(p, D, dtype, (hipStream_t)stream);
+}
+
+int lmk_ring_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kring, const lmk_tensor4* vring, const int64_t* idx,
+                           const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
+                           const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, int64_t stat_stride,
+                           const lmk_tensor4* out, int B, int H, int T, int n_blocks, int D, float sm_scale, int block,
+                           int top_k, int ring_start, int method, int dtype, void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kring)) || (rc = check_tensor(vring)) || (rc = check_tensor(o_loc)) ||
+      (rc = check_tensor(out)))
+    return rc;
+  if (cos_table == nullptr || sin_table == nullptr || idx == nullptr || L_loc == nullptr || M_loc == nullptr)
+    return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
+  if (B <= 0 || H <= 0 || T <= 0 || stat_stride < T) return LMK_ERR_SHAPE;
+  if (n_blocks <= 0) return LMK_ERR_CACHE;
+  if (!(D == 64 || D == 128)) return LMK_ERR_UNSUPPORTED;
+  if (block < 2 || block > 128) return LMK_ERR_UNSUPPORTED;
+  if (!(dtype == LMK_DTYPE_BF16 || dtype == LMK_DTYPE_F16)) return LMK_ERR_UNSUPPORTED;
+  if (method < LMK_SELECT_PER_TOKEN_AND_HEAD || method > LMK_SELECT_MAX_OVER_TOKENS) return LMK_ERR_UNSUPPORTED;
+  if (top_k < 1 || top_k > 64 || top_k > n_blocks) return LMK_ERR_TOPK;
+  if (ring_start < 0 || ring_start >= n_blocks) return LMK_ERR_SHAPE;
+  if (n_pos < (int64_t)(top_k + 1) * block) return LMK_ERR_TABLE;            // key positions end at (top_k + 1) * block - 1
+  if (!std::isfinite(sm_scale) || !(sm_scale > 0.f)) return LMK_ERR_SCALE;
+  lmk::RetrParams p = {};
+  fill_retr_common(p, B, H, T, n_blocks * block, D, block, top_k);
+  p.prefix_len = 0;                                                          // mem_cache.py:95-97: k_indices start at 0
+  p.ring_start = ring_start;
+  p.q = q->ptr; p.kcache = kring->ptr; p.vcache = vring->ptr; p.cos = cos_table; p.sin = sin_table;
+  p.idx = const_cast<int64_t*>(idx);
+  const int64_t k = p.k;
+  if (method == LMK_SELECT_PER_TOKEN_AND_HEAD) { p.idx_st = k; p.idx_sh = T * k; p.idx_sb = (int64_t)H * T * k; }
+  else if (method == LMK_SELECT_MAX_OVER_HEADS) { p.idx_st = k; p.idx_sh = 0; p.idx_sb = T * k; }
+  else { p.idx_st = 0; p.idx_sh = k; p.idx_sb = H * k; }
+  p.o_loc = o_loc->ptr; p.L_loc = L_loc; p.M_loc = M_loc; p.stat_stride = stat_stride; p.out = out->ptr;
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.kcs_b = kring->stride_b; p.kcs_h = kring->stride_h; p.kcs_r = kring->stride_row;
+  p.vcs_b = vring->stride_b; p.vcs_h = vring->stride_h; p.vcs_r = vring->stride_row;
+  p.ols_b = o_loc->stride_b; p.ols_h = o_loc->stride_h; p.ols_r = o_loc->stride_row;
+  p.outs_b = out->stride_b; p.outs_h = out->stride_h; p.outs_r = out->stride_row;
+  p.cs_r = table_stride_row;
+  p.scale_log2 = sm_scale * 1.4426950408889634f;
+  const int slots = block == 32 ? 32 : (block <= 64 ? 64 : 128);
+  return lmk::launch_gather_attend(p, D, slots, dtype, (hipStream_t)stream);
 }
 
 int lmk_local_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,

@@ -97,6 +97,7 @@ struct RetrParams {
   int64_t stat_stride;                            // floats between consecutive (batch, head) rows of L_loc, M_loc
   void* out;
   int64_t* idx;                                   // (B, H, T, k) ascending block indices
+  int64_t idx_sb, idx_sh, idx_st;                 // gather step: elements between the index rows of batches, heads, queries
   void* lk_rot;                                   // (B*H, num_mems, D) rotated landmark keys
   float* lk_norm;                                 // (B*H, num_mems)
   float *approx, *exact;                          // (B*H*T, num_mems) each
@@ -154,6 +155,7 @@ int launch_rotary(const RotaryParams& p, int D, int dtype, hipStream_t stream);
 int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landmark_keys, hipStream_t stream);
 int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream_t stream);   // one selection per head
 int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t stream);
+// BS: slots per block (32, 64 or 128); p.block <= BS tokens per block in the cache
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream);
 
 }  // namespace lmk

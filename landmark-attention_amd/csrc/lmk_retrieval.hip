@@ -828,11 +828,17 @@ __device__ __forceinline__ float sum8(float d) {                  // sum over th
 // (scores of the whole block, which the block's softmax needs before any weight is final), then the
 // values, so keys and values are never live together and the kernel keeps several waves per SIMD.  The
 // loads of the next chunk are issued before the arithmetic on the current one.
+// PADDED: the cache's blocks hold p.block < BS tokens (the benchmark models' 51).  A block is then worked on in BS
+// slots: slot s < p.block - 1 is normal key s, the last slot is the landmark (token p.block - 1), the slots in
+// between re-read a normal key and get the score -inf, i.e. weight 0 in the block's softmax and in the output.
+// The picked blocks of a row are read at p.idx[b * idx_sb + h * idx_sh + t * idx_st + 0 .. k-1] (selections shared
+// by the heads or by the queries have a zero stride there); a block counts among the k newest, whose keys sit one
+// block further on, by its age in the ring (p.ring_start = slot of the oldest block, 0 for a flat cache).
 template <int E> struct PieceVec;
 template <> struct PieceVec<8> { using type = u32x4_t; };
 template <> struct PieceVec<4> { using type = u32x2_t; };
 
-template <class T, int D, int BS, bool SPLIT>
+template <class T, int D, int BS, bool SPLIT, bool PADDED>
 __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   static_assert((D == 128 || D == 64) && (BS == 32 || BS % 64 == 0), "8 lanes x 2 pieces per row; whole chunks of keys");
   constexpr int E = D / 16;                                       // head dims per lane and rotary half: 8 or 4
@@ -867,6 +873,17 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   const char* kc = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h);
   const char* vc = (const char*)p.vcache + 2 * (b * p.vcs_b + hh * p.vcs_h);
   const float c2 = p.scale_log2;
+  const int nreal = PADDED ? p.block : BS;                        // tokens of a block in the cache
+  auto token_of = [&](int slot) {                                 // slot of the block's BS -> token of the block it reads
+    if (!PADDED) return slot;
+    return slot == BS - 1 ? nreal - 1 : min(slot, nreal - 2);
+  };
+  const int64_t* idx_row = p.idx + (b * p.idx_sb + hh * p.idx_sh + (int64_t)t * p.idx_st);
+  auto newest = [&](int blk) {                                    // one of the k newest blocks: its keys sit one block further on
+    int age = blk - p.ring_start;
+    age += age < 0 ? p.num_mems : 0;
+    return age >= p.num_mems - p.k;
+  };
 
   float Mrun = -INFINITY, lrun = 0.f;
   float alo[E], ahi[E];
@@ -878,10 +895,10 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
 
   // one chunk = CK rows of K or of V: this lane's KPG rows (g, g+8, ..) x its two 16-byte pieces
   vec_t clo[KPG], chi[KPG], nlo[KPG], nhi[KPG];
-  auto fetch = [&](const char* base, int64_t row_stride, int64_t key0) {
+  auto fetch = [&](const char* base, int64_t row_stride, int64_t key0, int slot0) {
 #pragma unroll
     for (int i = 0; i < KPG; ++i) {
-      const char* r = base + 2 * ((key0 + g + 8 * i) * row_stride) + PB * j;
+      const char* r = base + 2 * ((key0 + token_of(slot0 + g + 8 * i)) * row_stride) + PB * j;
       nlo[i] = *(const vec_t*)(r);
       nhi[i] = *(const vec_t*)(r + D);
     }
@@ -895,21 +912,22 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   };
   int blk = 0;
   if (js0 < p.k) {
-    blk = min(max((int)p.idx[row * p.k + js0], 0), p.num_mems - 1);      // idx is a caller's array: never read outside the cache
-    fetch(kc, p.kcs_r, (int64_t)blk * BS);
+    blk = min(max((int)idx_row[js0], 0), p.num_mems - 1);      // idx is a caller's array: never read outside the cache
+    fetch(kc, p.kcs_r, (int64_t)blk * nreal, 0);
   }
   for (int js = js0; js < p.k; js += jstep) {
-    const int64_t key0 = (int64_t)blk * BS;
-    const int64_t pos0 = (int64_t)js * BS + ((blk >= p.num_mems - p.k) ? BS : 0) + p.prefix_len;
+    const int64_t key0 = (int64_t)blk * nreal;
+    const int64_t pos0 = (int64_t)js * nreal + (newest(blk) ? nreal : 0) + p.prefix_len;
     float sc[KPG * NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       take();
-      if (c + 1 < NC) fetch(kc, p.kcs_r, key0 + CK * (c + 1));
-      else fetch(vc, p.vcs_r, key0);
+      if (c + 1 < NC) fetch(kc, p.kcs_r, key0, CK * (c + 1));
+      else fetch(vc, p.vcs_r, key0, 0);
 #pragma unroll
       for (int i = 0; i < KPG; ++i) {
-        const int kk = CK * c + g + 8 * i;
+        const int slot = CK * c + g + 8 * i;
+        const int kk = token_of(slot);
         const char* cr = (const char*)p.cos + 2 * ((pos0 + kk) * p.cs_r) + PB * j;
         const char* sr = (const char*)p.sin + 2 * ((pos0 + kk) * p.cs_r) + PB * j;
         float kl[E], kh[E], cl[E], ch[E], sl[E], sh[E];
@@ -928,6 +946,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
           d = __builtin_fmaf(qhi[e], rh, d);
         }
         sc[KPG * c + i] = sum8(d) * c2;                           // log2 domain
+        if (PADDED && slot >= nreal - 1 && slot != BS - 1) sc[KPG * c + i] = -INFINITY;   // a slot without a token
       }
     }
     // landmark = key BS-1 = last chunk, group 7, last of the group's keys
@@ -962,12 +981,12 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       ahi[e] *= alpha;
     }
     int blk_next = blk;
-    if (js + jstep < p.k) blk_next = min(max((int)p.idx[row * p.k + js + jstep], 0), p.num_mems - 1);
+    if (js + jstep < p.k) blk_next = min(max((int)idx_row[js + jstep], 0), p.num_mems - 1);
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       take();
-      if (c + 1 < NC) fetch(vc, p.vcs_r, key0 + CK * (c + 1));
-      else if (js + jstep < p.k) fetch(kc, p.kcs_r, (int64_t)blk_next * BS);
+      if (c + 1 < NC) fetch(vc, p.vcs_r, key0, CK * (c + 1));
+      else if (js + jstep < p.k) fetch(kc, p.kcs_r, (int64_t)blk_next * nreal, 0);
 #pragma unroll
       for (int i = 0; i < KPG; ++i) {
         const float w = round_to<T>(sc[KPG * c + i] * f);         // weights enter PV in the model dtype
@@ -1133,23 +1152,31 @@ int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landm
   return LMK_ERR_UNSUPPORTED;
 }
 
-template <class T, int D>
-static int launch_gather_t(const RetrParams& p, int BS, hipStream_t stream) {
+template <class T, int D, int BS, bool PADDED>
+static int launch_gather_b(const RetrParams& p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.B * p.H * p.T;
   if (rows <= 1024 && p.k > 1) {          // fewer rows than SIMDs: one workgroup per row, its waves share the blocks out
-    const dim3 grid((unsigned)rows);
-    if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 32, true>), grid, dim3(256), 0, stream, p);
-    else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 64, true>), grid, dim3(256), 0, stream, p);
-    else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 128, true>), grid, dim3(256), 0, stream, p);
-    else return LMK_ERR_UNSUPPORTED;
-    return (int)hipGetLastError();
+    hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, true, PADDED>), dim3((unsigned)rows), dim3(256), 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, false, PADDED>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       stream, p);
   }
-  const dim3 grid((unsigned)((rows + 3) / 4));
-  if (BS == 32) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 32, false>), grid, dim3(256), 0, stream, p);
-  else if (BS == 64) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 64, false>), grid, dim3(256), 0, stream, p);
-  else if (BS == 128) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, 128, false>), grid, dim3(256), 0, stream, p);
-  else return LMK_ERR_UNSUPPORTED;
   return (int)hipGetLastError();
+}
+
+// BS: slots a block is worked on in (32, 64, 128); p.block: tokens of a block in the cache (<= BS)
+template <class T, int D>
+static int launch_gather_t(const RetrParams& p, int BS, hipStream_t stream) {
+  if (p.block > BS || p.block < 2) return LMK_ERR_UNSUPPORTED;
+  if (p.block == BS) {
+    if (BS == 32) return launch_gather_b<T, D, 32, false>(p, stream);
+    if (BS == 64) return launch_gather_b<T, D, 64, false>(p, stream);
+    if (BS == 128) return launch_gather_b<T, D, 128, false>(p, stream);
+  } else {
+    if (BS == 64) return launch_gather_b<T, D, 64, true>(p, stream);
+    if (BS == 128) return launch_gather_b<T, D, 128, true>(p, stream);
+  }
+  return LMK_ERR_UNSUPPORTED;
 }
 
 // ---------------------------------------------------------------------------

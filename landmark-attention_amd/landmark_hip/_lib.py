@@ -99,6 +99,9 @@ def lib() -> ctypes.CDLL:
         L.lmk_retrieve_topk_shared_landmarks.argtypes = L.lmk_retrieve_topk_shared.argtypes
         L.lmk_ring_retrieve_topk.restype = i
         L.lmk_ring_retrieve_topk.argtypes = [T4, T4, vp, vp, i64, i64, vp, vp, sz, i, i, i, i, i, i, i, i, i, i, vp]
+        L.lmk_ring_gather_attend.restype = i
+        L.lmk_ring_gather_attend.argtypes = [T4, T4, T4, vp, vp, vp, i64, i64, T4, vp, vp, i64, T4,
+                                             i, i, i, i, i, f, i, i, i, i, i, vp]
         L.lmk_gather_window.restype = i
         L.lmk_gather_window.argtypes = [T4, T4, T4, vp, T4, T4, vp, vp, i64, i64, T4, T4, T4,
                                         i, i, i, i, i, i, i, i, vp]

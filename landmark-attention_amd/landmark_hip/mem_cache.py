@@ -8,7 +8,10 @@ including the newest-blocks-win truncation of a chunk larger than the ring.  The
 ``retrieve_for_query`` (``:50-85``) runs in the HIP library: landmark keys are read from the ring in
 place, rotated at the positions of ``:56-58``, scored, soft-maxed, reduced by ``cache_selection_method``
 and the ``cache_topk`` best slots come back ordered by age, as the reference's order-restoring sort
-leaves them.  Buffers are kept in the 16-bit model dtype (the reference's are fp32 holding 16-bit values
+leaves them.  ``attend`` is the rest of ``retrieve_for_query`` (``:86-109``) together with the attention the
+layer computes over its result (``lm_benchmark/models/landmark.py:192-240``): the picked blocks are read in
+place from the ring, rotated at ``k_indices``, and merged with the chunk's own attention through the grouped
+softmax.  Buffers are kept in the 16-bit model dtype (the reference's are fp32 holding 16-bit values
 under autocast).
 """
 from __future__ import annotations
@@ -130,3 +133,68 @@ class MemLMCacheStorage:
         newest = age >= n - k
         base = torch.arange(k * bs, device=idx.device).view(k, bs)
         return (newest.to(torch.int64) * bs).unsqueeze(-1).add(base).flatten(-2)
+
+    # ------------------------------------------------------------ gather + attend
+    def attend(self, q, k, v, is_mem, cos, sin, start_index: int, sm_scale=None):
+        """Attention of a chunk over the cache and itself: ``retrieve_for_query`` (``mem_cache.py:41-109``)
+        followed by what ``CausalSelfAttention.forward`` does between ``adapt_keys`` and ``c_proj``
+        (``lm_benchmark/models/landmark.py:192-240``), without materialising the gathered blocks, the
+        (T, prefix + T) score matrix or its masks.
+
+        q, k: (B, nh, T, hs) rotated at positions ``start_index ..`` (``adapt_queries`` / ``adapt_keys``);
+        v: (B, nh, T, hs); is_mem: (B, T) bool, which must continue the stream's pattern (a landmark closes every
+        block of ``mem_cache_freq + 1`` tokens, counted from the first token behind the last complete block);
+        cos, sin: (n_pos, hs) half-split tables in q's dtype, ``n_pos >= start_index + T``.
+        Returns ``(y (B, nh, T, hs), slots)``: y is ``att @ v + att_prefix @ cache_v`` (``:235-240``), slots the
+        picked blocks in the shape of ``select_blocks`` (None while the cache holds no block or ``cache_topk`` is 0,
+        ``:48-49``).  Call ``store_in_cache`` afterwards, as the layer does (``:246-248``)."""
+        from .attention import _launch_fwd, _repack, storage_block
+        from .rotary import _rotate
+        import math
+        B, nh, T, hs = q.shape
+        block, tail = self.block, self.last_incomplete_len
+        assert q.dtype == self.cache_mem_k.dtype and q.is_cuda and k.shape == v.shape == q.shape
+        expected = (torch.arange(T, device=q.device) + tail) % block == block - 1
+        assert bool((is_mem == expected).all()), "is_mem must continue the stream: a landmark closes every block"
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(hs)
+        cos, sin = _tables(cos, sin, q.dtype)
+        if tail:
+            # the tokens behind the last complete block open the chunk's first block (:43-46): their keys rotated at
+            # start_index - tail .., zero rows standing in for their queries
+            pos = torch.arange(start_index - tail, start_index, device=q.device, dtype=torch.int64)[None]
+            k_tail = _rotate(self.last_incomplete_k[:B, :, :tail], cos, sin, pos)
+            k_win = torch.cat((k_tail, k), dim=2)
+            v_win = torch.cat((self.last_incomplete_v[:B, :, :tail], v), dim=2)
+            q_win = torch.cat((q.new_zeros(B, nh, tail, hs), q), dim=2)
+        else:
+            q_win, k_win, v_win = (_lib.kernel_ready(t) for t in (q, k, v))
+        W = tail + T
+        slots_per_block = storage_block(block)
+        with _lib.on_device(q.device):
+            if slots_per_block == block:
+                o_win, L, M = _launch_fwd(q_win, k_win, v_win, 0, sm_scale, block)
+                o_loc, L_loc, M_loc, stat_stride = o_win[:, :, tail:], L[:, tail:], M[:, tail:], W
+            else:
+                qp, kp, vp = (_repack(t, block, slots_per_block) for t in (q_win, k_win, v_win))
+                op, L, M = _launch_fwd(qp, kp, vp, 0, sm_scale, slots_per_block, block)
+                o_loc = _repack(op, block, slots_per_block, unpad=True, rows=W)[:, :, tail:]
+                r = torch.arange(tail, W, device=q.device)
+                r = r // block * slots_per_block + torch.where(r % block == block - 1, slots_per_block - 1, r % block)
+                L_loc, M_loc, stat_stride = L[:, r].contiguous(), M[:, r].contiguous(), T
+            n = self.filled
+            if n == 0 or self.cache_topk == 0:
+                return o_loc, None
+            slots = self.select_blocks(q, cos, sin)
+            q = _lib.kernel_ready(q)
+            out = torch.empty_like(q)
+            kring = self.cache_mem_k[:B, :n].flatten(1, 2).transpose(1, 2)    # (B, nh, n*block, hs) views, no copy
+            vring = self.cache_mem_v[:B, :n].flatten(1, 2).transpose(1, 2)
+            rc = _lib.lib().lmk_ring_gather_attend(
+                _lib.tensor4(q), _lib.tensor4(kring), _lib.tensor4(vring), slots.data_ptr(), cos.data_ptr(),
+                sin.data_ptr(), cos.stride(0), cos.shape[0], _lib.tensor4(o_loc), L_loc.data_ptr(), M_loc.data_ptr(),
+                stat_stride, _lib.tensor4(out), B, nh, T, n, hs, float(sm_scale), block, self.cache_topk,
+                self.oldest_slot, SELECTION_METHODS[self.cache_selection_method], _lib.DTYPE_CODES[q.dtype],
+                _lib.current_stream(q.device))
+        _lib.check(rc)
+        return out, slots

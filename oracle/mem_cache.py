@@ -1,10 +1,13 @@
 """Ring cache of landmark blocks: storage bookkeeping and block selection.  TEST ORACLE.
 
 Restates ``MemLMCacheStorage`` of ``lm_benchmark/models/caches/mem_cache.py``: the ring-buffer
-bookkeeping of ``store_in_cache`` (``:111-158``) and the selection half of ``retrieve_for_query``
+bookkeeping of ``store_in_cache`` (``:111-158``), the selection half of ``retrieve_for_query``
 (``:50-85``) -- landmark positions, scores, softmax, the three selection methods, top-k and the
-order-restoring sort -- plus the key positions of the gathered blocks (``:95-97``).  Nothing here is
-used by the library; the tests compare the HIP selection with it index for index.
+order-restoring sort -- the gather half (``:86-109``: picked blocks' keys rotated at ``k_indices``, their
+scores, values and ``is_mem`` prefix, the tokens behind the last complete block appended) and the attention
+``CausalSelfAttention.forward`` computes over that prefix and the current chunk
+(``lm_benchmark/models/landmark.py:181-236``).  Nothing here is used by the library; the tests compare the
+HIP selection with it index for index and the HIP attention with it to 2e-2.
 
 What the reference leaves to the libraries is fixed the same way as for the llama-flavour cache
 (``oracle/retrieval.py``): scores under the sequential-accumulation score contract, the softmax by
@@ -21,7 +24,10 @@ exactly, and exceed the capacity); slot ages and landmark positions on hand-work
 where/sort/where sequence against a brute-force sort by age; the selection of a ring against the
 already pinned flat-cache selection (``oracle/retrieval.py``) applied to the same blocks laid out oldest
 first; ``max_over_heads`` / ``max_over_tokens`` against literal loops; ``torch.topk`` on rows without a
-boundary tie.
+boundary tie; ``retrieve_for_query`` / ``attention_with_cache`` in float64 against the closed form
+(``oracle/s1.py``) on [picked blocks rotated at their positions ; tail ; chunk] and against the flat-cache
+step of ``oracle/retrieval.py`` on the same blocks laid out oldest first (rotary is relative, so the two
+position conventions agree when ``start_index`` is what ``MemLMCache.forward`` hands out, ``mem_cache.py:188``).
 """
 from __future__ import annotations
 
@@ -165,3 +171,81 @@ def gathered_key_positions(slots, n: int, cache_iter: int, top_k: int, block: in
     chosen = landmark_slots(n, cache_iter, top_k)[slots]                               # position slot of each pick
     base = torch.arange(top_k * block).view(top_k, block)
     return (((chosen > 0) * block).unsqueeze(-1) + base).flatten(-2)
+
+
+# ------------------------------------------------------------ gather + attend
+def gather_ring_blocks(cache, slots):
+    """``take_along_dim`` of ``mem_cache.py:87-92``: cache (B, n, block, nh, hs), slots (B, nh, T, k) ->
+    (B, nh, T, k * block, hs), the picked blocks of every (head, query) in the order of ``slots``."""
+    B, n, block, nh, hs = cache.shape
+    per_head = cache.permute(0, 3, 1, 2, 4)                                           # (B, nh, n, block, hs)
+    T, k = slots.shape[2], slots.shape[3]
+    wide = per_head[:, :, None].expand(B, nh, T, n, block, hs)
+    sel = slots[..., None, None].expand(B, nh, T, k, block, hs)
+    return torch.take_along_dim(wide, sel, dim=3).flatten(3, 4)
+
+
+def expand_slots(slots, method: str, B: int, nh: int, T: int):
+    """Slots in the shape a selection method returns them -> (B, nh, T, k)."""
+    k = slots.shape[-1]
+    if method == "max_over_heads":
+        return slots.reshape(B, 1, T, k).expand(B, nh, T, k)
+    if method == "max_over_tokens":
+        return slots.reshape(B, nh, 1, k).expand(B, nh, T, k)
+    return slots.reshape(B, nh, T, k)
+
+
+def retrieve_for_query(store: RingStore, q, cos, sin, top_k: int, method: str, start_index: int, slots=None):
+    """``MemLMCacheStorage.retrieve_for_query`` (``mem_cache.py:41-109``).
+
+    q: (B, nh, T, hs) already rotated at ``start_index ..``.  Returns ``(att_prefix (B, nh, T, P), v_prefix
+    (B, nh, T, P, hs), is_mem_prefix (B, P), slots)`` with ``P = top_k * block + last_incomplete_len``; without a
+    filled slot or with ``top_k == 0`` only the tokens behind the last complete block remain (``:48-49``).
+    Products run in the dtype of ``q`` (fp32 / fp64 for the closed-form comparisons, 16-bit for the kernels')."""
+    B, nh, T, hs = q.shape
+    block, tail = store.block, store.last_incomplete_len
+    inv = 1.0 / math.sqrt(hs)
+    tail_k = apply_rotary(store.pending_k.to(q.dtype), cos, sin, torch.arange(start_index - tail, start_index))   # :43
+    att_tail = (q @ tail_k.transpose(-2, -1)) * inv                                   # :44
+    v_tail = store.pending_v.to(q.dtype)[:, :, None].expand(B, nh, T, tail, hs)       # :45
+    mem_tail = store.pending_is_mem                                                   # :46
+    n = store.filled
+    if n == 0 or top_k == 0:
+        return att_tail, v_tail, mem_tail, None
+    if slots is None:
+        scores = ring_scores(q, store.cache_k, n, store.cache_iter, top_k, cos, sin)
+        slots = select_blocks(scores, store.cache_iter, top_k, method)
+    slots = expand_slots(slots, "per_token_and_head", B, nh, T)
+    mem_k = gather_ring_blocks(store.cache_k[:, :n].to(q.dtype), slots)               # :87-90
+    mem_v = gather_ring_blocks(store.cache_v[:, :n].to(q.dtype), slots)               # :91-92
+    k_indices = gathered_key_positions(slots, n, store.cache_iter, top_k, block)      # :94-96
+    mem_k = apply_rotary(mem_k, cos, sin, k_indices)                                  # :100
+    att_k = (q.unsqueeze(3) @ mem_k.transpose(-2, -1)).squeeze(3) * inv               # :101
+    is_mem = torch.zeros(top_k, block, dtype=torch.bool)
+    is_mem[:, -1] = True                                                              # :98
+    is_mem = is_mem.flatten().expand(B, top_k * block)
+    return (torch.cat((att_k, att_tail), dim=-1), torch.cat((mem_v, v_tail), dim=-2),
+            torch.cat((is_mem, mem_tail), dim=-1), slots)
+
+
+def attention_with_cache(store: RingStore, q, k, v, is_mem, cos, sin, top_k: int, method: str, start_index: int,
+                         n_buckets: int, slots=None):
+    """``CausalSelfAttention.forward`` between the projections and ``c_proj`` with a cache
+    (``lm_benchmark/models/landmark.py:181-236``).  q, k: (B, nh, T, hs) rotated at ``start_index ..``; v: (B, nh, T,
+    hs); is_mem: (B, T).  Returns ``(y (B, nh, T, hs), slots)``."""
+    from .highlevel import grouped_softmax, masks_from_is_mem
+    B, nh, T, hs = q.shape
+    att_prefix, v_prefix, mem_prefix, slots = retrieve_for_query(store, q, cos, sin, top_k, method, start_index, slots)
+    att = (q @ k.transpose(-2, -1)) * (1.0 / math.sqrt(hs))                           # :195
+    causal_masked = ~torch.tril(torch.ones(T, T, dtype=torch.bool))[None, None].expand(B, nh, T, T)
+    att = att.masked_fill(causal_masked, float("-inf"))                               # :197
+    P = att_prefix.shape[-1]
+    att = torch.cat((att_prefix, att), dim=-1)                                        # :202
+    mem_all = torch.cat((mem_prefix, is_mem), dim=-1)                                 # :204
+    attn_mask = torch.cat((torch.zeros(B, nh, T, P, dtype=torch.bool), causal_masked), dim=-1)   # :207
+    masked, im, ls = masks_from_is_mem(mem_all[:, None, None, :], attn_mask)          # :214-222
+    att = att.masked_fill(masked, float("-inf"))                                      # :223
+    w = grouped_softmax(att, im, ls, n_buckets, attn_mask=masked, guard_empty=True)   # :226-231
+    w_prefix, w_loc = w[..., :P], w[..., P:]                                          # :234
+    y = w_loc.to(v.dtype) @ v + (w_prefix.to(v.dtype).unsqueeze(3) @ v_prefix).squeeze(3)   # :235-240
+    return y, slots

@@ -272,7 +272,7 @@ def local_masks(is_mem_loc, T: int, dtype):
     """
     low = torch.finfo(dtype).min
     i = torch.arange(T)
-    add = torch.where(i[None, :] <= i[:, None], 0.0, low).to(dtype)[None, None]
+    add = torch.where(i[None, :] <= i[:, None], torch.zeros((), dtype=dtype), torch.full((), low, dtype=dtype))[None, None]
     add = add.expand(is_mem_loc.shape[0], 1, T, T).clone()
     im = is_mem_loc[:, None, None, :]
     ids = torch.where(add < -1, 0, torch.cumsum(im, -1) - im.int())

@@ -30,7 +30,7 @@ def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
             "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend", "lmk_retrieve_topk_static", "lmk_retrieve_static_max_bytes",
-            "lmk_ring_retrieve_topk", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded",
+            "lmk_ring_retrieve_topk", "lmk_ring_gather_attend", "lmk_attn_bwd_handover_workspace_bytes", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded",
             "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
@@ -253,6 +253,22 @@ def test_ring_selection_argument_errors(lib):
     assert sel(k=5) == -10 and sel(k=0) == -10                    # more blocks asked for than cached: torch.topk raises
     assert sel(start=4) == -2 and sel(start=-1) == -2
     assert sel(n_pos=3 * 51 - 1) == -11 and sel(nbytes=16) == -8
+
+
+def test_ring_attention_argument_errors(lib):
+    from landmark_hip import _lib
+    L = _lib.lib()
+    t = _lib.Tensor4(0x1000, 0, 0, 64)
+
+    def att(q=t, idx=0x7000, Ls=0x8000, T=1, n=4, D=64, block=51, k=2, start=0, method=0, n_pos=1 << 20, stride=1, scale=0.1):
+        return L.lmk_ring_gather_attend(q, t, t, idx, 0x5000, 0x6000, 64, n_pos, t, Ls, 0x9000, stride, t, 1, 2, T, n, D,
+                                        scale, block, k, start, method, 0, None)
+    assert att(q=None) == -1 and att(idx=None) == -1 and att(Ls=None) == -1
+    assert att(n=0) == -9 and att(T=0) == -2 and att(D=96) == -3 and att(method=3) == -3
+    assert att(block=1) == -3 and att(block=129) == -3           # blocks of 2..128 tokens
+    assert att(k=5) == -10 and att(k=0) == -10
+    assert att(start=4) == -2 and att(T=3, stride=2) == -2
+    assert att(n_pos=3 * 51 - 1) == -11 and att(scale=0.0) == -7
 
 
 def test_irregular_landmark_positions_are_rejected_with_a_message():

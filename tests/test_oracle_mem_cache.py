@@ -185,3 +185,110 @@ def test_interleaved_rotary_is_the_half_split_one_on_permuted_head_dims():
     assert torch.allclose(inter[:, perm], split, atol=1e-12)
     y = torch.randn(5, hs, generator=g, dtype=torch.float64)
     assert torch.allclose((inter * y).sum(-1), (split * y[:, perm]).sum(-1), atol=1e-12)
+
+
+# ---------------------------------------------------------------- gather + attend (mem_cache.py:86-109)
+def _filled_ring(B, nh, hs, block, capacity, n_tokens, g, dtype=torch.float64):
+    ring = mem_cache.RingStore(B, capacity, block, nh, hs, dtype=dtype)
+    k = torch.randn(B, nh, n_tokens, hs, generator=g, dtype=dtype) * 0.5
+    v = torch.randn(B, nh, n_tokens, hs, generator=g, dtype=dtype) * 0.5
+    im = (torch.arange(n_tokens) % block == block - 1)[None].expand(B, n_tokens)
+    ring.store(k, v, im)
+    return ring
+
+
+def _tables64(n_pos, hs):
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hs, 2, dtype=torch.float64) / hs))
+    ang = torch.outer(torch.arange(n_pos, dtype=torch.float64), inv)
+    ang = torch.cat((ang, ang), -1)
+    return ang.cos(), ang.sin()
+
+
+@pytest.mark.parametrize("method", mem_cache.METHODS)
+@pytest.mark.parametrize("capacity,block,n_tokens,top_k,T", [
+    (6, 5, 5 * 4 + 2, 2, 9),       # not yet full, tail of 2, chunk over two landmarks
+    (4, 5, 5 * 7 + 3, 3, 4),       # wrapped ring (oldest block at slot 3), chunk completes the tail's block exactly... minus one
+    (4, 7, 7 * 9, 2, 15),          # no tail, chunk of two blocks and one token
+    (5, 4, 4 * 6 + 1, 5, 6),       # top_k = filled slots
+])
+def test_attention_with_cache_is_the_closed_form_over_picked_blocks_tail_and_chunk(method, capacity, block, n_tokens, top_k, T):
+    # the picked blocks, rotated at k_indices, are earlier landmark blocks in front of [tail ; chunk]; zero rows stand
+    # in for the tail's queries.  float64, so only the mathematics is compared.
+    from oracle import s1
+    B, nh, hs = 2, 3, 8
+    g = torch.Generator().manual_seed(capacity * 31 + block + top_k)
+    ring = _filled_ring(B, nh, hs, block, capacity, n_tokens, g)
+    tail, n = ring.last_incomplete_len, ring.filled
+    start = (top_k + 1) * block + tail
+    cos, sin = _tables64(start + T, hs)
+    q0 = torch.randn(B, nh, T, hs, generator=g, dtype=torch.float64)
+    k0 = torch.randn(B, nh, T, hs, generator=g, dtype=torch.float64)
+    v = torch.randn(B, nh, T, hs, generator=g, dtype=torch.float64)
+    pos = torch.arange(start, start + T)
+    q, k = rotary.apply_rotary(q0, cos, sin, pos), rotary.apply_rotary(k0, cos, sin, pos)
+    is_mem = ((torch.arange(T) + tail) % block == block - 1)[None].expand(B, T)
+    y, slots = mem_cache.attention_with_cache(ring, q, k, v, is_mem, cos, sin, top_k, method, start, n_buckets=top_k + T // block + 3)
+    assert slots.shape == (B, nh, T, top_k)
+    tail_k = rotary.apply_rotary(ring.pending_k, cos, sin, torch.arange(start - tail, start))
+    newest = mem_cache.slot_ages(n, ring.cache_iter) >= n - top_k
+    for b, h, t in itertools.product(range(B), range(nh), range(T)):
+        ks, vs = [], []
+        for j, slot in enumerate(slots[b, h, t].tolist()):
+            p0 = j * block + (block if newest[slot] else 0)
+            ks.append(rotary.apply_rotary(ring.cache_k[b, slot, :, h], cos, sin, torch.arange(p0, p0 + block)))
+            vs.append(ring.cache_v[b, slot, :, h])
+        kk = torch.cat(ks + [tail_k[b, h], k[b, h]])
+        vv = torch.cat(vs + [ring.pending_v[b, h], v[b, h]])
+        qq = torch.cat((torch.zeros(tail, hs, dtype=torch.float64), q[b, h]))
+        want = s1.s1_attention(qq, kk, vv, block, rows=[tail + t])[0]
+        assert torch.allclose(y[b, h, t], want, atol=1e-12), (b, h, t)
+
+
+def test_ring_attention_equals_the_flat_cache_step_on_the_same_blocks():
+    # llama flavour (oracle/retrieval.py, llama_mem.py:386-477) on the ring's blocks laid out oldest first, with the
+    # ring's picks translated to ages: positions differ by a constant (prefix_len), which rotary does not see
+    B, nh, hs, block, capacity, top_k, T = 1, 2, 8, 6, 5, 2, 3
+    g = torch.Generator().manual_seed(5)
+    ring = _filled_ring(B, nh, hs, block, capacity, block * 8 + 2, g)          # wrapped, tail of 2; T + tail <= block
+    tail, n = ring.last_incomplete_len, ring.filled
+    ages = mem_cache.slot_ages(n, ring.cache_iter)
+    order = torch.argsort(ages)                                                  # slots, oldest first
+    flat_k = torch.cat([ring.cache_k[:, s].permute(0, 2, 1, 3) for s in order.tolist()] + [ring.pending_k], dim=2)
+    flat_v = torch.cat([ring.cache_v[:, s].permute(0, 2, 1, 3) for s in order.tolist()] + [ring.pending_v], dim=2)
+    S = flat_k.shape[2]
+    cos, sin = _tables64(S + T, hs)
+    q0 = torch.randn(B, nh, T, hs, generator=g, dtype=torch.float64)
+    k0 = torch.randn(B, nh, T, hs, generator=g, dtype=torch.float64)
+    v = torch.randn(B, nh, T, hs, generator=g, dtype=torch.float64)
+    is_mem = ((torch.arange(T) + tail) % block == block - 1)[None].expand(B, T)
+    start = (top_k + 1) * block + tail
+    q_ring = rotary.apply_rotary(q0, cos, sin, torch.arange(start, start + T))
+    k_ring = rotary.apply_rotary(k0, cos, sin, torch.arange(start, start + T))
+    slots = torch.randint(0, n, (B, nh, T, 1), generator=g)
+    slots = torch.cat((slots, (slots + 1 + torch.randint(0, n - 1, (B, nh, T, 1), generator=g)) % n), -1)   # two distinct slots
+    slots = mem_cache.restore_order(slots, n, ring.cache_iter)
+    y, _ = mem_cache.attention_with_cache(ring, q_ring, k_ring, v, is_mem, cos, sin, top_k, "per_token_and_head", start,
+                                          n_buckets=top_k + 3, slots=slots)
+    q_flat = rotary.apply_rotary(q0, cos, sin, torch.arange(S, S + T))
+    k_flat = rotary.apply_rotary(k0, cos, sin, torch.arange(S, S + T))
+    want, _ = retrieval.retrieve_and_attend(q_flat, flat_k, flat_v, k_flat, v, is_mem, cos, sin, block, top_k,
+                                            idx=ages[slots], n_buckets=top_k + 3)
+    assert torch.allclose(y, want, atol=1e-11)
+
+
+def test_without_blocks_only_the_tail_joins_the_chunk():
+    from oracle import s1
+    B, nh, hs, block, T = 1, 2, 8, 5, 7
+    g = torch.Generator().manual_seed(9)
+    ring = _filled_ring(B, nh, hs, block, 4, 3, g)                               # three tokens, no complete block
+    assert ring.filled == 0 and ring.last_incomplete_len == 3
+    cos, sin = _tables64(64, hs)
+    q, k, v = (torch.randn(B, nh, T, hs, generator=g, dtype=torch.float64) for _ in range(3))
+    is_mem = ((torch.arange(T) + 3) % block == block - 1)[None]
+    y, slots = mem_cache.attention_with_cache(ring, q, k, v, is_mem, cos, sin, 2, "per_token_and_head", 3, n_buckets=8)
+    assert slots is None
+    tail_k = rotary.apply_rotary(ring.pending_k, cos, sin, torch.arange(0, 3))
+    for h in range(nh):
+        qq = torch.cat((torch.zeros(3, hs, dtype=torch.float64), q[0, h]))
+        want = s1.s1_attention(qq, torch.cat((tail_k[0, h], k[0, h])), torch.cat((ring.pending_v[0, h], v[0, h])), block)[3:]
+        assert torch.allclose(y[0, h], want, atol=1e-12)
