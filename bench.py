@@ -334,7 +334,7 @@ def side_legs(n=30, warm=5):
     return {"offloaded_cache": {"workload": "config 4's cache in pinned host memory (zero-copy reads of the selected blocks), "
                                             "one selection per head; 256 queries / 1 query", "chunk_step_ms": t_off_chunk,
                                 "token_step_ms": t_off_token},
-            "config0_on_hip": {"workload": "benchmark config 0 (B2 H8 L510 D128, block 51) in bf16, blocks padded to 64 slots",
+            "config0_on_hip": {"workload": "benchmark config 0 (B2 H8 L510 D128, block 51) in bf16, blocks of 51 tokens worked on in 64 slots and read in place",
                                "forward_ms": t_c0_fwd, "forward_backward_ms": t_c0_step},
             "per_head_selection": {"workload": "config 4 shapes, aggregate=max_over_tokens", "topk_ms": t_sel,
                                    "attend_ms": t_att},

@@ -130,7 +130,10 @@ int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
  * unpadded problem; rows of o / dq / dk / dv at padding slots hold values of no meaning.
  * block is 64 or 128 and 2 <= block_real <= block (block_real == block is the plain call, then 32
  * is accepted too).  Lq, Lk and n_prefix count PADDED rows and stored blocks.
- * dout must be zero at padding rows (lmk_pad_blocks writes zeros there). */
+ * dout must be zero at padding rows (lmk_pad_blocks writes zeros there) and o at padding rows must be what
+ * lmk_attn_fwd_padded left there (finite): the dK/dV kernel carries no mask of its own and multiplies those rows
+ * by zero weights, so a NaN or Inf there would reach real rows of dk and dv.  lmk_attn_*_blocks below have no such
+ * requirement. */
 
 /* Rows of a padded tensor that holds `rows` real rows: whole blocks widen to `block`, a partial
  * last block keeps its length.  -1 for invalid sizes. */
@@ -153,6 +156,23 @@ int lmk_attn_bwd_padded(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
                         const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
                         int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
                         int dtype, void* stream);
+
+/* The same without any repacking: q, k, v, o (and dout, dq, dk, dv) keep their rows as they are -- Lq, Lk, L and M
+ * count TOKENS of blocks of block_tokens (2..128) -- and the kernels translate the slots they work on into token
+ * rows as they load and store (a slot without a token re-reads its block's first token and is masked).  This is what
+ * FusedLandmarkAttention.forward / backward do for a block_size that is not 32, 64 or 128
+ * (flash_landmark_attention.py:318; lm_benchmark's mem_freq + 1 = 51): no padded copies, no extra launches.
+ * block_tokens of 32, 64 or 128 is the plain call.  n_prefix = (Lk - Lq) / block_tokens; the backward needs whole
+ * blocks; its workspace (lmk_attn_bwd_blocks_workspace_bytes) is indexed by slots. */
+int lmk_attn_fwd_blocks(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block_tokens,
+                        int n_prefix, int dtype, void* stream);
+size_t lmk_attn_bwd_blocks_workspace_bytes(int B, int H, int Lq, int Lk, int block_tokens);
+int lmk_attn_bwd_blocks(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                        const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
+                        int H, int Lq, int Lk, int D, float sm_scale, int block_tokens, int n_prefix, int dtype,
+                        void* stream);
 
 /* ---- mem-cache retrieval (inference) --------------------------------------------------
  * The reference has no function boundary here: scoring, selection and gather are inline in
@@ -202,6 +222,11 @@ int lmk_retrieve_topk_reuse(const lmk_tensor4* q, const lmk_tensor4* kcache, con
  * GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls on one
  * stream are ordered.  Nothing in the array needs to start at zero (every kernel writes what it later reads). */
 size_t lmk_retrieve_static_max_bytes(void);
+/* Looks up the array's address on the CURRENT device (hipGetSymbolAddress, once per device; later calls return at
+ * once).  lmk_retrieve_topk_static does the same on its first call on a device, which is a runtime query and not a
+ * stream operation: a caller that records the entry point into a HIP graph calls this (or makes one eager call)
+ * on that device BEFORE the capture begins.  0, or a hipError_t. */
+int lmk_retrieve_static_init(void);
 int lmk_retrieve_topk_static(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
                              const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out, int B,
                              int H, int T, int S, int D, int block, int top_k, int dtype, void* stream);
@@ -259,7 +284,9 @@ int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, con
  *          MAX_OVER_HEADS (shared by the heads), (B,H,top_k) for MAX_OVER_TOKENS.
  *   workspace: lmk_retrieve_workspace_bytes(B,H,T,n_blocks*block,D,block) bytes.
  * top_k > n_blocks is an error (torch.topk raises there, :72).  Ties: (probability descending,
- * slot ascending).  Tables in the half-split layout of the other entry points; the benchmark's
+ * slot ascending) for the two aggregated methods; PER_TOKEN_AND_HEAD ranks by (16-bit score descending, slot
+ * ascending), which is the probability order wherever two probabilities differ and also orders scores whose
+ * exponentials collapse to one fp32 value, where torch.topk leaves the choice open.  Tables in the half-split layout of the other entry points; the benchmark's
  * interleaved pairs map onto it by moving the even head dims in front of the odd ones in q and k. */
 #define LMK_SELECT_PER_TOKEN_AND_HEAD 0
 #define LMK_SELECT_MAX_OVER_HEADS 1

@@ -189,9 +189,11 @@ struct RopeArgs {
   int64_t pos_stride_b;
 };
 
+// Lq_real, Lk_real > 0: the tensors are in token layout (rows = tokens of blocks of block_real), Lq and Lk count slots
 static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                          float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
-                         int block_real, int n_prefix, int dtype, void* stream, const RopeArgs* rope = nullptr) {
+                         int block_real, int n_prefix, int dtype, void* stream, const RopeArgs* rope = nullptr,
+                         int Lq_real = 0, int Lk_real = 0) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o))) return rc;
   if (L == nullptr || M == nullptr) return LMK_ERR_NULL;
@@ -211,6 +213,7 @@ static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
     p.rope_pos_stride_b = rope->pos_stride_b; p.rope_cs_r = rope->stride_row; p.rope_n_pos = rope->n_pos;
   }
   p.n_real = block_real;
+  p.Lq_real = Lq_real; p.Lk_real = Lk_real;
   p.q = q->ptr; p.k = k->ptr; p.v = v->ptr; p.o = o->ptr;
   p.L = L; p.M = M;
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
@@ -311,7 +314,7 @@ static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
                          const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
                          const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
                          int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
-                         int dtype, int phases, void* stream);
+                         int dtype, int phases, void* stream, int Lq_real = 0, int Lk_real = 0);
 
 int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                         const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
@@ -331,11 +334,59 @@ int lmk_attn_bwd_padded(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
                        block, block_real, n_prefix, dtype, LMK_BWD_ALL, stream);
 }
 
+// ---- blocks of any size on tensors in token layout
+static int slots_of(int block_tokens) {
+  if (block_tokens == 32 || block_tokens == 64 || block_tokens == 128) return block_tokens;
+  if (block_tokens < 2 || block_tokens > 128) return 0;
+  return block_tokens <= 64 ? 64 : 128;
+}
+
+int lmk_attn_fwd_blocks(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block_tokens,
+                        int n_prefix, int dtype, void* stream) {
+  const int slots = slots_of(block_tokens);
+  if (slots == 0) return LMK_ERR_UNSUPPORTED;
+  if (slots == block_tokens)
+    return attn_fwd_impl(q, k, v, o, L, M, B, H, Lq, Lk, D, sm_scale, slots, slots, n_prefix, dtype, stream);
+  if (Lq <= 0 || Lk < Lq || n_prefix < 0) return LMK_ERR_SHAPE;
+  if ((int64_t)Lk - Lq != (int64_t)n_prefix * block_tokens) return LMK_ERR_HISTORY;
+  const int64_t lq = lmk_padded_rows(Lq, block_tokens, slots), lk = (int64_t)n_prefix * slots + lq;
+  if (lk >= ((int64_t)1 << 31)) return LMK_ERR_UNSUPPORTED;
+  return attn_fwd_impl(q, k, v, o, L, M, B, H, (int)lq, (int)lk, D, sm_scale, slots, block_tokens, n_prefix, dtype, stream,
+                       nullptr, Lq, Lk);
+}
+
+size_t lmk_attn_bwd_blocks_workspace_bytes(int B, int H, int Lq, int Lk, int block_tokens) {
+  const int slots = slots_of(block_tokens);
+  if (slots == 0 || Lq <= 0 || Lk <= 0) return 0;
+  return lmk_attn_bwd_workspace_bytes(B, H, (int)lmk_padded_rows(Lq, block_tokens, slots),
+                                      (int)lmk_padded_rows(Lk, block_tokens, slots), slots);
+}
+
+int lmk_attn_bwd_blocks(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                        const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                        const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
+                        int H, int Lq, int Lk, int D, float sm_scale, int block_tokens, int n_prefix, int dtype,
+                        void* stream) {
+  const int slots = slots_of(block_tokens);
+  if (slots == 0) return LMK_ERR_UNSUPPORTED;
+  if (slots == block_tokens)
+    return attn_bwd_impl(q, k, v, o, dout, L, M, dq, dk, dv, workspace, workspace_bytes, B, H, Lq, Lk, D, sm_scale, slots,
+                         slots, n_prefix, dtype, LMK_BWD_ALL, stream);
+  if (Lq <= 0 || Lk < Lq || n_prefix < 0) return LMK_ERR_SHAPE;
+  if (Lq % block_tokens != 0 || Lk % block_tokens != 0) return LMK_ERR_PARTIAL;
+  if ((int64_t)Lk - Lq != (int64_t)n_prefix * block_tokens) return LMK_ERR_HISTORY;
+  const int64_t lq = (int64_t)Lq / block_tokens * slots, lk = (int64_t)Lk / block_tokens * slots;
+  if (lk >= ((int64_t)1 << 31)) return LMK_ERR_UNSUPPORTED;
+  return attn_bwd_impl(q, k, v, o, dout, L, M, dq, dk, dv, workspace, workspace_bytes, B, H, (int)lq, (int)lk, D, sm_scale,
+                       slots, block_tokens, n_prefix, dtype, LMK_BWD_ALL, stream, Lq, Lk);
+}
+
 static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                          const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
                          const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
                          int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
-                         int dtype, int phases, void* stream) {
+                         int dtype, int phases, void* stream, int Lq_real, int Lk_real) {
   int rc;
   if (phases <= 0 || phases > LMK_BWD_ALL) return LMK_ERR_SHAPE;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o)) ||
@@ -372,6 +423,7 @@ static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
   p.n_prefix = n_prefix; p.n_blocks = (int)nb;
   p.n_real = block_real;
+  p.Lq_real = Lq_real; p.Lk_real = Lk_real;
   p.n_qtiles = (Lq + 127) / 128; p.n_kvtiles = (Lk + 127) / 128;
   p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
   p.ks_b = k->stride_b; p.ks_h = k->stride_h; p.ks_r = k->stride_row;
@@ -444,6 +496,11 @@ int lmk_retrieve_topk_reuse(const lmk_tensor4* q, const lmk_tensor4* kcache, con
 }
 
 size_t lmk_retrieve_static_max_bytes(void) { return LMK_STATIC_SCRATCH_BYTES; }
+
+int lmk_retrieve_static_init(void) {
+  int rc = 0;
+  return static_scratch(&rc) != nullptr ? LMK_OK : rc;
+}
 
 int lmk_retrieve_topk_static(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
                              const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out, int B,

@@ -32,28 +32,37 @@ namespace lmk {
 // pre: delta and mhat
 // ---------------------------------------------------------------------------
 template <class T, int D>
-__global__ __launch_bounds__(256) void lmk_bwd_pre_kernel(BwdParams p) {
+__global__ __launch_bounds__(256) void lmk_bwd_pre_kernel(BwdParams p, int block_slots) {
   constexpr int LPR = D / 8;          // lanes per row (16 bytes each)
   constexpr int RPW = 256 / LPR;      // rows per workgroup
   const int tid = threadIdx.x;
   const int64_t row = (int64_t)blockIdx.x * RPW + tid / LPR;
   const int64_t total = (int64_t)p.B * p.H * p.Lq;
   float sum = 0.f;
+  int64_t li = row;                                         // index of the row in L and M; -1: a slot without a token
   if (row < total) {
-    const int bh = (int)(row / p.Lq), qi = (int)(row % p.Lq);
-    const int b = bh / p.H, hh = bh % p.H;
-    const int d0 = 8 * (tid % LPR);
-    const u32x4_t o4 = *(const u32x4_t*)((const char*)p.o + 2 * (b * p.os_b + hh * p.os_h + (int64_t)qi * p.os_r + d0));
-    const u32x4_t g4 = *(const u32x4_t*)((const char*)p.dout + 2 * (b * p.dos_b + hh * p.dos_h + (int64_t)qi * p.dos_r + d0));
+    const int bh = (int)(row / p.Lq);
+    int qi = (int)(row % p.Lq);
+    if (p.Lq_real > 0) {                                    // token layout: the workspace rows are slots
+      qi = block_slots == 64 ? slot_to_token_row<64>(qi, p.n_real, p.Lq_real / p.n_real)
+                             : slot_to_token_row<128>(qi, p.n_real, p.Lq_real / p.n_real);
+      li = qi < 0 ? -1 : (int64_t)bh * p.Lq_real + qi;
+    }
+    if (qi >= 0) {
+      const int b = bh / p.H, hh = bh % p.H;
+      const int d0 = 8 * (tid % LPR);
+      const u32x4_t o4 = *(const u32x4_t*)((const char*)p.o + 2 * (b * p.os_b + hh * p.os_h + (int64_t)qi * p.os_r + d0));
+      const u32x4_t g4 = *(const u32x4_t*)((const char*)p.dout + 2 * (b * p.dos_b + hh * p.dos_h + (int64_t)qi * p.dos_r + d0));
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      sum += unpack_lo<T>(o4[i]) * unpack_lo<T>(g4[i]) + unpack_hi<T>(o4[i]) * unpack_hi<T>(g4[i]);
+      for (int i = 0; i < 4; ++i)
+        sum += unpack_lo<T>(o4[i]) * unpack_lo<T>(g4[i]) + unpack_hi<T>(o4[i]) * unpack_hi<T>(g4[i]);
+    }
   }
 #pragma unroll
   for (int m = LPR / 2; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, 64);
   if (row < total && (tid % LPR) == 0) {
     p.delta[row] = sum;
-    p.mhat[row] = p.M[row] * kLog2e + fast_log2(p.L[row]);
+    p.mhat[row] = li < 0 ? 1e30f : p.M[li] * kLog2e + fast_log2(p.L[li]);
   }
 }
 
@@ -92,7 +101,9 @@ __device__ __forceinline__ void dq_dma16(const void* base_uniform, uint32_t voff
                :: "v"(voff), "s"(base_uniform), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory");
 }
 
-template <class T, int D, int BS>
+// VIRT: tensors in token layout (p.Lq_real > 0); a template parameter because the slot arithmetic costs the
+// slot-layout instantiations registers they do not have.
+template <class T, int D, int BS, bool VIRT>
 __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<T, D, BS>;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -125,6 +136,12 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   const int cblk = dt / C::NT, tsub = dt % C::NT;          // the wave's own block and its tile inside it
   const bool active = q0 < p.Lq;                           // Lq is a multiple of the block: whole tiles only
   const int qrow = q0 + ql;
+  // token layout: the tensors' rows are tokens, the kernel's rows (and the workspace's) are slots.  A slot without
+  // a token is a query row of zeros with mhat = 1e30: its gate, its weights and every term it leaves for the dK/dV
+  // kernel come out as exact zeros (a = 1e30), whatever that kernel reads for its Q and dO rows.
+  constexpr bool virt = VIRT;
+  const int nfull_k = virt ? p.Lk_real / p.n_real : 0;
+  const int qtok = !active ? -1 : (virt ? slot_to_token_row<BS>(qrow, p.n_real, p.Lq_real / p.n_real) : qrow);
 
   u32x4_t qf[C::KS], gf[C::KS];
 #pragma unroll
@@ -132,9 +149,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     u32x4_t z = {0, 0, 0, 0};
     qf[ks] = z;
     gf[ks] = z;
-    if (active) {
-      qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
-      gf[ks] = *(const u32x4_t*)(gp + 2 * ((int64_t)qrow * p.dos_r + 16 * ks + 8 * h));
+    if (qtok >= 0) {
+      qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qtok * p.qs_r + 16 * ks + 8 * h));
+      gf[ks] = *(const u32x4_t*)(gp + 2 * ((int64_t)qtok * p.dos_r + 16 * ks + 8 * h));
     }
   }
   // row terms (the reference's _bwd_preprocess, flash_landmark_attention.py:125-149): delta = rowsum(O * dO)
@@ -142,18 +159,22 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   // dK/dV kernel as well
   float mhat = 0.f, delta = 0.f;
   if (active) {
-    const char* orow = (const char*)p.o + 2 * (b * p.os_b + hh * p.os_h + (int64_t)qrow * p.os_r);
     float sum = 0.f;
+    mhat = 1e30f;
+    if (qtok >= 0) {
+      const char* orow = (const char*)p.o + 2 * (b * p.os_b + hh * p.os_h + (int64_t)qtok * p.os_r);
 #pragma unroll
-    for (int ks = 0; ks < C::KS; ++ks) {
-      const u32x4_t o4 = *(const u32x4_t*)(orow + 2 * (16 * ks + 8 * h));
+      for (int ks = 0; ks < C::KS; ++ks) {
+        const u32x4_t o4 = *(const u32x4_t*)(orow + 2 * (16 * ks + 8 * h));
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        sum += unpack_lo<T>(o4[i]) * unpack_lo<T>(gf[ks][i]) + unpack_hi<T>(o4[i]) * unpack_hi<T>(gf[ks][i]);
+        for (int i = 0; i < 4; ++i)
+          sum += unpack_lo<T>(o4[i]) * unpack_lo<T>(gf[ks][i]) + unpack_hi<T>(o4[i]) * unpack_hi<T>(gf[ks][i]);
+      }
+      const int64_t li = (int64_t)bh * (virt ? p.Lq_real : p.Lq) + qtok;   // L, M follow the tensors' layout
+      mhat = p.M[li] * kLog2e + fast_log2(p.L[li]);
     }
     delta = pair_sum(sum);
     const int64_t ri = (int64_t)bh * p.Lq + qrow;
-    mhat = p.M[ri] * kLog2e + fast_log2(p.L[ri]);
     if (h == 0) {
       p.delta[ri] = delta;
       p.mhat[ri] = mhat;
@@ -178,15 +199,24 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     src[i] = (uint32_t)(2 * ((int64_t)row * (is_v ? p.vs_r : p.ks_r) + 8 * (cp ^ f)));
   }
   const uint32_t step_k = (uint32_t)(2 * (int64_t)BS * p.ks_r), step_v = (uint32_t)(2 * (int64_t)BS * p.vs_r);
+  int blk_req = 0;                                         // block the next request fetches
   auto request = [&](int buf) {                            // next block in key order -> buffer buf
 #pragma unroll
     for (int i = 0; i < C::PER_WAVE; ++i) {
       const int r = wave * C::PER_WAVE + i;
       const bool is_v = r >= n_k;                          // wave-uniform
       const int dst = buf * C::STAGE_BYTES + (is_v ? C::TILE_BYTES : 0) + C::RPD * (r % n_k) * C::ROWB;
-      dq_dma16(is_v ? vp : kp, src[i], dst);
-      src[i] += is_v ? step_v : step_k;
+      if (virt) {                                          // the slot's token row, worked out per request
+        const int row = C::RPD * (r % n_k) + lane / C::CH, cp = lane % C::CH;
+        const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
+        const int tok = slot_to_token_row_clamped<BS>(blk_req * BS + row, p.n_real, nfull_k);
+        dq_dma16(is_v ? vp : kp, (uint32_t)(2 * ((int64_t)tok * (is_v ? p.vs_r : p.ks_r) + 8 * (cp ^ f))), dst);
+      } else {
+        dq_dma16(is_v ? vp : kp, src[i], dst);
+        src[i] += is_v ? step_v : step_k;
+      }
     }
+    ++blk_req;
   };
 
   f32x16_t acc[C::DC];
@@ -329,7 +359,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     }
   }
 
-  if (active) {
+  if (qtok >= 0) {
     const float sc = p.scale;
 #pragma unroll
     for (int dc = 0; dc < C::DC; ++dc)
@@ -337,7 +367,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
       for (int g = 0; g < 4; ++g) {
         u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * sc, acc[dc][4 * g + 1] * sc),
                       pack2<T>(acc[dc][4 * g + 2] * sc, acc[dc][4 * g + 3] * sc)};
-        *(u32x2_t*)(dqp + 2 * ((int64_t)qrow * p.dqs_r + 32 * dc + 8 * g + 4 * h)) = o2;
+        *(u32x2_t*)(dqp + 2 * ((int64_t)qtok * p.dqs_r + 32 * dc + 8 * g + 4 * h)) = o2;
       }
   }
 }
@@ -352,7 +382,7 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
   if ((phases & 1) && !(phases & 2)) {
     constexpr int RPW = 256 / (D / 8);
     const int64_t rows = (int64_t)p.B * p.H * p.Lq;
-    hipLaunchKernelGGL((lmk_bwd_pre_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((lmk_bwd_pre_kernel<T, D>), dim3((unsigned)((rows + RPW - 1) / RPW)), dim3(256), 0, stream, p, BS);
     if ((rc = (int)hipGetLastError())) return rc;
   }
   if (phases & 2) {
@@ -360,10 +390,18 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
       if ((rc = launch_bwd_dq32(p, D, std::is_same<T, bf16_t>::value ? LMK_DTYPE_BF16 : LMK_DTYPE_F16, stream))) return rc;
     } else {
       using C = DqCfg<T, D, BS>;
-      auto kern = lmk_bwd_dq_kernel<T, D, BS>;
-      static std::atomic<uint64_t> lds_ok{0};
-      if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
-      hipLaunchKernelGGL(kern, dim3(((p.Lq + 255) / 256) * p.B * p.H), dim3(64 * C::NW), C::LDS_BYTES, stream, p);
+      const dim3 grid(((p.Lq + 255) / 256) * p.B * p.H);
+      if (p.Lq_real > 0) {
+        auto kern = lmk_bwd_dq_kernel<T, D, BS, true>;
+        static std::atomic<uint64_t> lds_ok{0};
+        if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
+        hipLaunchKernelGGL(kern, grid, dim3(64 * C::NW), C::LDS_BYTES, stream, p);
+      } else {
+        auto kern = lmk_bwd_dq_kernel<T, D, BS, false>;
+        static std::atomic<uint64_t> lds_ok{0};
+        if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
+        hipLaunchKernelGGL(kern, grid, dim3(64 * C::NW), C::LDS_BYTES, stream, p);
+      }
       if ((rc = (int)hipGetLastError())) return rc;
     }
   }

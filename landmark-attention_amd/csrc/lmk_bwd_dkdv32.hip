@@ -75,7 +75,11 @@ __device__ __forceinline__ void wait_vmcnt() {             // s_waitcnt vmcnt(N)
 
 #define LMK_INL __attribute__((always_inline))
 
-template <class T, int D, int BS>
+// VIRT (blocks of 64 and 128 slots only): q, k, v, dout, dk, dv are in token layout (BwdParams::Lq_real > 0) while
+// p.Lq, p.Lk and the workspace count slots.  Slots without a token need no mask here: the dQ kernel left a = 1e30
+// and mhat = 1e30 for such query rows, so their W and dS are exact zeros whatever rows are read for them, and the
+// accumulator rows of such keys are not stored.
+template <class T, int D, int BS, bool VIRT = false>
 __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   using C = Dkv32Cfg<T, D, BS>;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -159,6 +163,8 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   // query tiles than the stream runs ahead, so the entry is there before the stream needs it).
   // per-lane source offsets (bytes) of this wave's requests 0 and 1 inside tile 0 of Q and of dO
   uint32_t q_vo0 = 0, q_vo1 = 0, g_vo0 = 0, g_vo1 = 0;
+  int vrow0 = 0, vcf0 = 0, vcf1 = 0;                       // VIRT: this lane's row inside a tile and its two chunk offsets
+  const int nfull_q = VIRT ? p.Lq_real / p.n_real : 0, nfull_k = VIRT ? p.Lk_real / p.n_real : 0;
   if (!role_k) {
     const int chp = lane % C::CH;
     const int row0 = C::RPD * (tile * C::NDMA) + lane / C::CH, row1 = row0 + C::RPD;
@@ -170,7 +176,15 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       q_vo1 = (uint32_t)(2 * (row1 * p.qs_r + 8 * (chp ^ f1)));
       g_vo1 = (uint32_t)(2 * (row1 * p.dos_r + 8 * (chp ^ f1)));
     }
+    vrow0 = row0;
+    vcf0 = 16 * (chp ^ f0);
+    vcf1 = 16 * (chp ^ f1);
   }
+  // VIRT: byte offset of this lane's chunk of slot row 32 j + its row (+ RPD for the second request) of a tensor
+  auto virt_off = [&](int j, int second, int64_t row_stride) LMK_INL {
+    const int tok = slot_to_token_row_clamped<BS>(32 * j + vrow0 + (second ? C::RPD : 0), p.n_real, nfull_q);
+    return 2u * (uint32_t)tok * (uint32_t)row_stride + (uint32_t)(second ? vcf1 : vcf0);
+  };
   const uint32_t q_step = (uint32_t)(2 * 32 * p.qs_r), g_step = (uint32_t)(2 * 32 * p.dos_r);
   // this lane's 16 bytes of a query tile's terms: lanes 0-7 a, 8-15 nD, 16-23 dS at the landmark (planes, one row
   // of Lq per block), 24-31 mhat, 32-63 delta (one row per head)
@@ -211,13 +225,15 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       has_nx = take ? false : has_nx;
     }
     if constexpr (P < C::NDMA) {
-      dma16_s(qp, ((P == 0) ? q_vo0 : q_vo1) + (uint32_t)j_req * q_step, slot_bytes + dst_off + P * 1024);
+      if constexpr (VIRT) dma16_s(qp, virt_off(j_req, P, p.qs_r), slot_bytes + dst_off + P * 1024);
+      else dma16_s(qp, ((P == 0) ? q_vo0 : q_vo1) + (uint32_t)j_req * q_step, slot_bytes + dst_off + P * 1024);
     } else if constexpr (P == C::NDMA) {
       const int64_t off = 32 * (int64_t)j_req + ((lane < 24) ? pl_req : 0);
       dma16_v(st_lane + off, slot_bytes + 2 * C::TILE_BYTES + tile * 1024);
     } else if constexpr (P <= 2 * C::NDMA) {
       constexpr int G = P - C::NDMA - 1;
-      dma16_s(gp, ((G == 0) ? g_vo0 : g_vo1) + (uint32_t)j_req * g_step, slot_bytes + C::TILE_BYTES + dst_off + G * 1024);
+      if constexpr (VIRT) dma16_s(gp, virt_off(j_req, G, p.dos_r), slot_bytes + C::TILE_BYTES + dst_off + G * 1024);
+      else dma16_s(gp, ((G == 0) ? g_vo0 : g_vo1) + (uint32_t)j_req * g_step, slot_bytes + C::TILE_BYTES + dst_off + G * 1024);
       if (P == 2 * C::NDMA) ++j_req;
     }
   };
@@ -395,6 +411,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     const int64_t rs = role_k ? p.vs_r : p.ks_r;
     int kr = krow, h8 = 8 * h;
     asm volatile("" : "+v"(kr), "+v"(h8));                 // the address is formed here, not ahead of the loops (and spilled)
+    if constexpr (VIRT) kr = slot_to_token_row_clamped<BS>(active ? kr : 0, p.n_real, nfull_k);
     const char* row = src + 2 * ((int64_t)kr * rs + h8);
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) {
@@ -437,15 +454,18 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   auto store_acc = [&](const f32x16_t* acc, char* dst, int64_t rs, float scl) LMK_INL {
     int kr = krow, h4 = 4 * h;
     asm volatile("" : "+v"(kr), "+v"(h4));                 // as in load_stationary
+    if constexpr (VIRT) kr = slot_to_token_row<BS>(kr, p.n_real, nfull_k);   // -1: a slot without a token, nothing to store
     char* row = dst + 2 * ((int64_t)kr * rs + h4);
+    if (!VIRT || kr >= 0) {
 #pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc)
+      for (int dc = 0; dc < C::DC; ++dc)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * scl, acc[dc][4 * g + 1] * scl),
-                      pack2<T>(acc[dc][4 * g + 2] * scl, acc[dc][4 * g + 3] * scl)};
-        *(u32x2_t*)(row + 2 * (32 * dc + 8 * g)) = o2;
-      }
+        for (int g = 0; g < 4; ++g) {
+          u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * scl, acc[dc][4 * g + 1] * scl),
+                        pack2<T>(acc[dc][4 * g + 2] * scl, acc[dc][4 * g + 3] * scl)};
+          *(u32x2_t*)(row + 2 * (32 * dc + 8 * g)) = o2;
+        }
+    }
   };
   if (!role_k) {
     f32x16_t acc[C::DC];                                   // dV^T: rows = d, lane = key
@@ -538,10 +558,10 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 
 #undef LMK_INL
 
-template <class T, int D, int BS>
+template <class T, int D, int BS, bool VIRT>
 static int launch_dkdv32_t(const BwdParams& p, hipStream_t stream) {
   using C = Dkv32Cfg<T, D, BS>;
-  auto kern = lmk_bwd_dkdv32_kernel<T, D, BS>;
+  auto kern = lmk_bwd_dkdv32_kernel<T, D, BS, VIRT>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   // workgroups per head: enough for about one workgroup per CU, at most four 128-key tiles each
@@ -555,9 +575,14 @@ static int launch_dkdv32_t(const BwdParams& p, hipStream_t stream) {
 
 template <class T, int D>
 static int launch_dkdv32_b(const BwdParams& p, int BS, hipStream_t stream) {
-  if (BS == 32) return launch_dkdv32_t<T, D, 32>(p, stream);
-  if (BS == 64) return launch_dkdv32_t<T, D, 64>(p, stream);
-  if (BS == 128) return launch_dkdv32_t<T, D, 128>(p, stream);
+  if (p.Lq_real > 0) {                                     // token layout: blocks narrower than their 64 or 128 slots
+    if (BS == 64) return launch_dkdv32_t<T, D, 64, true>(p, stream);
+    if (BS == 128) return launch_dkdv32_t<T, D, 128, true>(p, stream);
+    return LMK_ERR_UNSUPPORTED;
+  }
+  if (BS == 32) return launch_dkdv32_t<T, D, 32, false>(p, stream);
+  if (BS == 64) return launch_dkdv32_t<T, D, 64, false>(p, stream);
+  if (BS == 128) return launch_dkdv32_t<T, D, 128, false>(p, stream);
   return LMK_ERR_UNSUPPORTED;
 }
 

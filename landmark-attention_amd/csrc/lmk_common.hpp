@@ -162,6 +162,23 @@ __device__ __forceinline__ u32x4_t load_row_frag(const unsigned char* kbuf, int 
   return *(const u32x4_t*)(kbuf + tile_off<D>(row, 2 * ks + (lane >> 5)));
 }
 
+// Blocks of n tokens worked on in BS slots (n <= BS): slot s < n-1 of a complete block is its normal token s, the
+// last slot its landmark (token n-1), the slots in between hold nothing; a partial last block (n_full = number of
+// complete blocks) keeps its tokens in its first slots.  Slot row -> token row of the tensor, or -1.
+template <int BS>
+__device__ __forceinline__ int slot_to_token_row(int slot_row, int n, int n_full) {
+  const int blk = slot_row / BS, s = slot_row % BS;
+  int tok = s;
+  if (blk < n_full) tok = (s == BS - 1) ? n - 1 : (s < n - 1 ? s : -1);
+  return tok < 0 ? -1 : blk * n + tok;
+}
+// The same for loads whose result is masked afterwards: a slot without a token reads its block's first token.
+template <int BS>
+__device__ __forceinline__ int slot_to_token_row_clamped(int slot_row, int n, int n_full) {
+  const int r = slot_to_token_row<BS>(slot_row, n, n_full);
+  return r < 0 ? (slot_row / BS) * n : r;
+}
+
 template <class T>
 __device__ __forceinline__ float round_to(float x) {  // fp32 -> T (RNE) -> fp32
   return unpack_lo<T>(pack2<T>(x, 0.f));

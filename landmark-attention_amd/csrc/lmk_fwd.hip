@@ -79,6 +79,10 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   const int cblk = dt / C::NT, tsub = dt % C::NT;       // its landmark block and sub-tile
   const bool active = q0 < p.Lq;
   const int qrow = q0 + ql;
+  // token layout: the tensors' rows are tokens, the kernel's rows are slots
+  const bool virt = p.Lq_real > 0;                      // uniform over the launch
+  const int nfull_q = virt ? p.Lq_real / p.n_real : 0, nfull_k = virt ? p.Lk_real / p.n_real : 0;
+  const int qtok = !virt ? (qrow < p.Lq ? qrow : -1) : (qrow < p.Lq ? slot_to_token_row<BS>(qrow, p.n_real, nfull_q) : -1);
 
   // ---- Q fragments (B operand): query qrow, head dims 16*ks + 8h .. +7
   u32x4_t qf[C::KS];
@@ -86,10 +90,10 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   for (int ks = 0; ks < C::KS; ++ks) {
     u32x4_t z = {0, 0, 0, 0};
     qf[ks] = z;
-    if (qrow < p.Lq) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
+    if (qtok >= 0) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qtok * p.qs_r + 16 * ks + 8 * h));
   }
-  if (p.rope_cos != nullptr && qrow < p.Lq) {                      // q without rotary: rotate the fragments at the row's position
-    int64_t pos = p.rope_pos[(int64_t)b * p.rope_pos_stride_b + qrow];
+  if (p.rope_cos != nullptr && qtok >= 0) {                        // q without rotary: rotate the fragments at the row's position
+    int64_t pos = p.rope_pos[(int64_t)b * p.rope_pos_stride_b + qtok];
     pos = pos < 0 ? 0 : (pos >= p.rope_n_pos ? p.rope_n_pos - 1 : pos);
     rotate_fragments<T, C::KS>(qf, (const char*)p.rope_cos + 2 * pos * p.rope_cs_r, (const char*)p.rope_sin + 2 * pos * p.rope_cs_r, h);
   }
@@ -125,8 +129,15 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
       const int r = wave * C::PER_WAVE + i;
       const bool is_v = r >= n_k;                       // wave-uniform
       const int dst = buf * C::STAGE_BYTES + (is_v ? C::TILE_BYTES : 0) + C::RPD * (r % n_k) * C::ROWB;
-      fwd_dma16(is_v ? vp : kp, last ? src_last[i] : src[i], dst);
-      src[i] += is_v ? step_v : step_k;
+      if (virt) {                                       // the slot's token row, worked out per request
+        const int row = C::RPD * (r % n_k) + lane / C::CH, cp = lane % C::CH;
+        const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
+        const int tok = slot_to_token_row_clamped<BS>(min(blk_req * C::SK + row, p.Lk - 1), p.n_real, nfull_k);
+        fwd_dma16(is_v ? vp : kp, (uint32_t)(2 * ((int64_t)tok * (is_v ? p.vs_r : p.ks_r) + 8 * (cp ^ f))), dst);
+      } else {
+        fwd_dma16(is_v ? vp : kp, last ? src_last[i] : src[i], dst);
+        src[i] += is_v ? step_v : step_k;
+      }
     }
     ++blk_req;
   };
@@ -292,7 +303,7 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   }
 
   // ---- epilogue: out = acc / l, statistics in natural-log units like the reference
-  if (active && qrow < p.Lq) {
+  if (active && qtok >= 0) {
     const float inv = 1.0f / lrun;
 #pragma unroll
     for (int dc = 0; dc < C::DC; ++dc)
@@ -300,11 +311,12 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
       for (int g = 0; g < 4; ++g) {
         u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * inv, acc[dc][4 * g + 1] * inv),
                       pack2<T>(acc[dc][4 * g + 2] * inv, acc[dc][4 * g + 3] * inv)};
-        *(u32x2_t*)(op + 2 * ((int64_t)qrow * p.os_r + 32 * dc + 8 * g + 4 * h)) = o2;
+        *(u32x2_t*)(op + 2 * ((int64_t)qtok * p.os_r + 32 * dc + 8 * g + 4 * h)) = o2;
       }
-    if (h == 0) {
-      p.L[(int64_t)bh * p.Lq + qrow] = lrun;
-      p.M[(int64_t)bh * p.Lq + qrow] = Mrun * kLn2;
+    if (h == 0) {                                       // statistics follow the tensors' layout
+      const int64_t si = (int64_t)bh * (virt ? p.Lq_real : p.Lq) + qtok;
+      p.L[si] = lrun;
+      p.M[si] = Mrun * kLn2;
     }
   }
 }

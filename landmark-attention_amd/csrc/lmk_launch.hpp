@@ -48,6 +48,11 @@ struct FwdParams {
   int n_prefix;   // history blocks in front of the queries
   int n_qtiles;   // ceil(Lq / 128)
   int n_real;     // tokens of a block that exist (normal keys in front, landmark last); == block unless padded
+  // Lq_real > 0: q, k, v, o, L, M hold Lq_real / Lk_real rows of blocks of n_real tokens as they are ("token
+  // layout"), and Lq, Lk above count the slots the kernels work on (whole blocks widened to `block` slots, a
+  // partial last block keeps its length); the kernels translate slot rows to token rows themselves.
+  // 0: the tensors are stored in slots already (n_real < block: with padding rows).
+  int Lq_real, Lk_real;
   // optional: q arrives without rotary and is rotated as it is loaded (null tables: q is used as it is)
   const void *rope_cos, *rope_sin;
   const int64_t* rope_pos;        // position of query row r of batch b: rope_pos[b * rope_pos_stride_b + r]
@@ -74,6 +79,7 @@ struct BwdParams {
   int n_prefix, n_blocks;        // history blocks; Lk / block
   int n_qtiles, n_kvtiles;       // ceil(Lq / 128), ceil(Lk / 128)
   int n_real;                    // tokens of a block that exist; == block unless padded (blocks 64 and 128 only)
+  int Lq_real, Lk_real;          // > 0: tensors in token layout, as in FwdParams (the workspace stays indexed by slot rows)
   int64_t qs_b, qs_h, qs_r, ks_b, ks_h, ks_r, vs_b, vs_h, vs_r, os_b, os_h, os_r, dos_b, dos_h, dos_r;
   int64_t dqs_b, dqs_h, dqs_r, dks_b, dks_h, dks_r, dvs_b, dvs_h, dvs_r;
   float scale, scale_log2;

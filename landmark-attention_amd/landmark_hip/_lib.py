@@ -70,6 +70,12 @@ def lib() -> ctypes.CDLL:
         L.lmk_attn_bwd_padded.restype = i
         L.lmk_attn_bwd_padded.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, ctypes.c_size_t,
                                           i, i, i, i, i, f, i, i, i, i, vp]
+        L.lmk_attn_fwd_blocks.restype = i
+        L.lmk_attn_fwd_blocks.argtypes = [T4, T4, T4, T4, vp, vp, i, i, i, i, i, f, i, i, i, vp]
+        L.lmk_attn_bwd_blocks_workspace_bytes.restype = sz
+        L.lmk_attn_bwd_blocks_workspace_bytes.argtypes = [i, i, i, i, i]
+        L.lmk_attn_bwd_blocks.restype = i
+        L.lmk_attn_bwd_blocks.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, sz, i, i, i, i, i, f, i, i, i, vp]
         L.lmk_retrieve_workspace_bytes.restype = sz
         L.lmk_retrieve_workspace_bytes.argtypes = [i, i, i, i, i, i]
         L.lmk_retrieve_topk.restype = i
@@ -78,6 +84,8 @@ def lib() -> ctypes.CDLL:
         L.lmk_retrieve_topk_reuse.argtypes = L.lmk_retrieve_topk.argtypes
         L.lmk_retrieve_static_max_bytes.restype = sz
         L.lmk_retrieve_static_max_bytes.argtypes = []
+        L.lmk_retrieve_static_init.restype = i
+        L.lmk_retrieve_static_init.argtypes = []
         L.lmk_retrieve_topk_static.restype = i
         L.lmk_retrieve_topk_static.argtypes = [T4, T4, vp, vp, i64, i64, vp, i, i, i, i, i, i, i, i, vp]
         L.lmk_gather_attend.restype = i

@@ -2,9 +2,10 @@
 (``llama/ltriton/flash_landmark_attention.py:308-403``), backed by the HIP kernels.
 
 Block sizes other than 32, 64 and 128 (the training models use ``mem_freq + 1 = 51``) run on the
-64- or 128-slot kernels: q, k, v and the incoming gradient are repacked so that every block has its
-normal tokens in front and its landmark in the last slot, the kernels mask the slots in between,
-and the results are packed back.  Blocks wider than 128 tokens are rejected.
+64- or 128-slot kernels, which read and write the tensors as they are: a block's normal tokens occupy its
+first slots, its landmark the last one, and the kernels translate slots to token rows as they load and store
+and mask the slots in between (``lmk_attn_fwd_blocks`` / ``lmk_attn_bwd_blocks``).  Nothing is repacked or
+copied.  Blocks wider than 128 tokens are rejected.
 
 Head dims 16 and 32 are zero-padded to 64 by ``fused_landmark_attention``.
 
@@ -56,6 +57,35 @@ def _repack(x, block_size, block, unpad=False, rows=None):
     _lib.check(fn(_lib.tensor4(x), _lib.tensor4(out), B, H, rows, D, int(block_size), int(block),
                   _lib.current_stream(x.device)))
     return out
+
+
+def _launch_fwd_blocks(q, k, v, n_prefix, sm_scale, block_tokens):
+    """Forward for any block size 2..128 on the tensors as they are; L, M are indexed by token rows."""
+    B, H, Lq, D = q.shape
+    Lk = k.shape[2]
+    o = torch.empty_like(q)
+    L = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+    M = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+    rc = _lib.lib().lmk_attn_fwd_blocks(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o),
+                                        L.data_ptr(), M.data_ptr(), B, H, Lq, Lk, D, float(sm_scale), int(block_tokens),
+                                        int(n_prefix), _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+    _lib.check(rc)
+    return o, L, M
+
+
+def _launch_bwd_blocks(q, k, v, o, do, L, M, n_prefix, sm_scale, block_tokens):
+    B, H, Lq, D = q.shape
+    Lk = k.shape[2]
+    lib = _lib.lib()
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    nbytes = lib.lmk_attn_bwd_blocks_workspace_bytes(B, H, Lq, Lk, int(block_tokens))
+    ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+    rc = lib.lmk_attn_bwd_blocks(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o), _lib.tensor4(do),
+                                 L.data_ptr(), M.data_ptr(), _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv),
+                                 ws.data_ptr(), nbytes, B, H, Lq, Lk, D, float(sm_scale), int(block_tokens),
+                                 int(n_prefix), _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+    _lib.check(rc)
+    return dq, dk, dv
 
 
 def _launch_fwd(q, k, v, n_prefix, sm_scale, block, block_real=None):
@@ -120,13 +150,10 @@ class FusedLandmarkAttention(torch.autograd.Function):
         with _lib.on_device(q.device):
             if block == block_size:
                 o, L, m = _launch_fwd(q, k, v, n_prefix_q, sm_scale, block_size)
-                ctx.save_for_backward(q, k, v, o, L, m)
-                return o
-            # the padded copies are what the backward kernels read, so they are what is kept
-            qp, kp, vp = (_repack(t, block_size, block) for t in (q, k, v))
-            op, L, m = _launch_fwd(qp, kp, vp, n_prefix_q, sm_scale, block, block_size)
-            ctx.save_for_backward(qp, kp, vp, op, L, m)
-            return _repack(op, block_size, block, unpad=True, rows=seqlen_q)
+            else:
+                o, L, m = _launch_fwd_blocks(q, k, v, n_prefix_q, sm_scale, block_size)
+            ctx.save_for_backward(q, k, v, o, L, m)
+            return o
 
     @staticmethod
     def backward(ctx, do):
@@ -141,16 +168,13 @@ class FusedLandmarkAttention(torch.autograd.Function):
             if block == BLOCK:
                 dq, dk, dv = _launch_bwd(q, k, v, o, do, l, m, ctx.N_PREFIX_Q, ctx.sm_scale, BLOCK)
             else:
-                dop = _repack(do, BLOCK, block)                     # zero rows at the padding slots
-                dq, dk, dv = _launch_bwd(q, k, v, o, dop, l, m, ctx.N_PREFIX_Q, ctx.sm_scale, block, BLOCK)
-                dq = _repack(dq, BLOCK, block, unpad=True, rows=rows_q)
-                dk = _repack(dk, BLOCK, block, unpad=True, rows=rows_k)
-                dv = _repack(dv, BLOCK, block, unpad=True, rows=rows_k)
+                dq, dk, dv = _launch_bwd_blocks(q, k, v, o, do, l, m, ctx.N_PREFIX_Q, ctx.sm_scale, BLOCK)
         return dq, dk, dv, None, None, None
 
 
 # Masks that have already passed the check of ``flash_landmark_attention.py:393-394``, keyed by what
 # identifies a tensor's content without reading it: storage address, in-place version counter, layout.
+# (A write through ``.data`` or a custom kernel bypasses the counter; such a mask has to be a new tensor.)
 # A layer stack hands the same mask to every layer and every step, so the device->host sync of the
 # comparison is paid once per mask instead of once per call.
 _VALIDATED_MASKS: dict = {}
@@ -158,14 +182,20 @@ _VALIDATED_MASKS_MAX = 64
 
 
 def _check_is_mem(is_mem, block_size):
-    key = (is_mem.device, is_mem.data_ptr(), is_mem._version, tuple(is_mem.shape), tuple(is_mem.stride()),
-           is_mem.dtype, int(block_size))
-    if key in _VALIDATED_MASKS:
-        return
+    # tensors created under torch.inference_mode() track no version counter (reading it raises): they are checked
+    # on every call rather than cached
+    cacheable = not is_mem.is_inference()
+    if cacheable:
+        key = (is_mem.device, is_mem.data_ptr(), is_mem._version, tuple(is_mem.shape), tuple(is_mem.stride()),
+               is_mem.dtype, int(block_size))
+        if key in _VALIDATED_MASKS:
+            return
     expected_is_mem = torch.arange(0, is_mem.shape[-1], device=is_mem.device) % block_size == (block_size - 1)
     assert (is_mem == expected_is_mem).all(), (
         f"is_mem must mark exactly the last token of every block of {block_size}: irregular landmark positions "
         "and dropped landmarks are not covered by the fused kernels")
+    if not cacheable:
+        return
     if len(_VALIDATED_MASKS) >= _VALIDATED_MASKS_MAX:
         _VALIDATED_MASKS.clear()
     # the entry keeps the tensor alive, so its address cannot be handed to another mask meanwhile

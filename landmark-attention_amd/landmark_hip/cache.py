@@ -111,7 +111,9 @@ class OffloadedLandmarkCache:
 
     @property
     def host_key_value(self):
-        """Views of the filled part of the pinned host buffers, (B, nh, S, hd) each."""
+        """Views of the filled part of the pinned host buffers, (B, nh, S, hd) each.  ``append`` fills them with
+        asynchronous device->host copies on the caller's stream: synchronise that stream before reading the views
+        on the host (kernels on the same stream see the rows in order)."""
         return self._k[:, :, : self.length], self._v[:, :, : self.length]
 
     def _reserve(self, rows: int) -> None:
@@ -145,6 +147,11 @@ class OffloadedLandmarkCache:
         """Attention of a new chunk against the offloaded cache, then the append; returns ``(out, idx)`` with
         ``idx (B, nh, 1, k)``.  Needs at least one complete cached block."""
         assert self.n_blocks >= 1, "no complete cached block yet"
+        B, nh, T, hd = query_states.shape
+        nbytes = _lib.lib().lmk_retrieve_workspace_bytes(B, nh, T, self.n_blocks * self.block, hd, self.block)
+        if self._ws is None or self._ws.numel() < nbytes or self._ws.device != query_states.device:
+            self._ws = torch.empty(max(nbytes, 2 * (self._ws.numel() if self._ws is not None else 0)),
+                                   device=query_states.device, dtype=torch.uint8)     # grown on demand, kept between steps
         idx = retrieve_topk_from_landmarks(query_states, self.landmark_keys, cos, sin, self.block, top_k, self._ws)
         k_host, v_host = self.host_key_value
         out = attend_shared(query_states, k_host, v_host, idx, key_states, value_states, cos, sin, self.block, top_k,

@@ -148,7 +148,7 @@ class MemLMCacheStorage:
         Returns ``(y (B, nh, T, hs), slots)``: y is ``att @ v + att_prefix @ cache_v`` (``:235-240``), slots the
         picked blocks in the shape of ``select_blocks`` (None while the cache holds no block or ``cache_topk`` is 0,
         ``:48-49``).  Call ``store_in_cache`` afterwards, as the layer does (``:246-248``)."""
-        from .attention import _launch_fwd, _repack, storage_block
+        from .attention import _launch_fwd_blocks
         from .rotary import _rotate
         import math
         B, nh, T, hs = q.shape
@@ -170,18 +170,10 @@ class MemLMCacheStorage:
         else:
             q_win, k_win, v_win = (_lib.kernel_ready(t) for t in (q, k, v))
         W = tail + T
-        slots_per_block = storage_block(block)
         with _lib.on_device(q.device):
-            if slots_per_block == block:
-                o_win, L, M = _launch_fwd(q_win, k_win, v_win, 0, sm_scale, block)
-                o_loc, L_loc, M_loc, stat_stride = o_win[:, :, tail:], L[:, tail:], M[:, tail:], W
-            else:
-                qp, kp, vp = (_repack(t, block, slots_per_block) for t in (q_win, k_win, v_win))
-                op, L, M = _launch_fwd(qp, kp, vp, 0, sm_scale, slots_per_block, block)
-                o_loc = _repack(op, block, slots_per_block, unpad=True, rows=W)[:, :, tail:]
-                r = torch.arange(tail, W, device=q.device)
-                r = r // block * slots_per_block + torch.where(r % block == block - 1, slots_per_block - 1, r % block)
-                L_loc, M_loc, stat_stride = L[:, r].contiguous(), M[:, r].contiguous(), T
+            # blocks of any size up to 128 tokens, read as they are (the benchmark's 51 run in 64 slots)
+            o_win, L, M = _launch_fwd_blocks(q_win, k_win, v_win, 0, sm_scale, block)
+            o_loc, L_loc, M_loc, stat_stride = o_win[:, :, tail:], L[:, tail:], M[:, tail:], W
             n = self.filled
             if n == 0 or self.cache_topk == 0:
                 return o_loc, None

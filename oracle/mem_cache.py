@@ -152,7 +152,10 @@ def restore_order(picked, n: int, cache_iter: int):
 def select_blocks(scores, cache_iter: int, top_k: int, method: str):
     """Slots (B, nh, T, top_k) int64, oldest block first; ties by (probability descending, slot ascending)."""
     n = scores.shape[-1]
-    prob = block_probabilities(scores, method)
+    # per_token_and_head ranks by the score itself: softmax is monotone, so this is the probability order wherever
+    # two probabilities differ, and it also orders scores whose exponentials collapse to one fp32 value (underflow),
+    # where torch.topk on the probabilities (``:72``) leaves the choice open
+    prob = scores.float() if method == "per_token_and_head" else block_probabilities(scores, method)
     order = torch.sort(prob, dim=-1, descending=True, stable=True).indices[..., :top_k]
     return restore_order(order, n, cache_iter)
 

@@ -30,7 +30,7 @@ def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
             "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend", "lmk_retrieve_topk_static", "lmk_retrieve_static_max_bytes",
-            "lmk_ring_retrieve_topk", "lmk_ring_gather_attend", "lmk_attn_bwd_handover_workspace_bytes", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded",
+            "lmk_ring_retrieve_topk", "lmk_ring_gather_attend", "lmk_attn_bwd_handover_workspace_bytes", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded", "lmk_attn_fwd_blocks", "lmk_attn_bwd_blocks",
             "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
@@ -240,6 +240,28 @@ def test_blocks_of_any_size_host_side(lib):
     assert bwd(32, 17) == -3 and bwd(128, 1) == -2 and bwd(64, 51, ws=16) == -8
 
 
+def test_token_layout_entry_points_argument_errors(lib):
+    # lmk_attn_fwd_blocks / lmk_attn_bwd_blocks: blocks of 2..128 tokens on tensors that are not repacked
+    from landmark_hip import _lib
+    L = _lib.lib()
+    t = _lib.Tensor4(0x1000, 0, 0, 128)
+
+    def fwd(Lq=102, Lk=102, block=51, n_prefix=0, D=128):
+        return L.lmk_attn_fwd_blocks(t, t, t, t, 0x2000, 0x3000, 1, 1, Lq, Lk, D, 0.1, block, n_prefix, 0, None)
+
+    def bwd(Lq=102, Lk=102, block=51, n_prefix=0, ws=1 << 30):
+        return L.lmk_attn_bwd_blocks(t, t, t, t, t, 0x2000, 0x3000, t, t, t, 0x4000, ws, 1, 1, Lq, Lk, 128, 0.1, block,
+                                     n_prefix, 0, None)
+    assert fwd(block=1) == -3 and fwd(block=129) == -3 and fwd(D=96) == -3
+    assert fwd(Lk=153, n_prefix=0) == -5 and fwd(Lq=102, Lk=51) == -2        # history must be whole blocks; Lk >= Lq
+    assert bwd(Lq=100, Lk=100) == -6                                          # the backward needs whole blocks
+    assert bwd(Lk=153, n_prefix=2) == -5 and bwd(ws=16) == -8
+    # the workspace is indexed by slots: 51 tokens in 64 slots
+    assert L.lmk_attn_bwd_blocks_workspace_bytes(2, 8, 510, 510, 51) == L.lmk_attn_bwd_workspace_bytes(2, 8, 640, 640, 64)
+    assert L.lmk_attn_bwd_blocks_workspace_bytes(2, 8, 512, 512, 64) == L.lmk_attn_bwd_workspace_bytes(2, 8, 512, 512, 64)
+    assert L.lmk_attn_bwd_blocks_workspace_bytes(1, 1, 10, 10, 200) == 0
+
+
 def test_ring_selection_argument_errors(lib):
     from landmark_hip import _lib
     L = _lib.lib()
@@ -305,3 +327,21 @@ def test_is_mem_is_validated_once_per_mask_state():
         attention._check_is_mem(mask, 32)
     with pytest.raises(AssertionError):
         attention._check_is_mem(torch.zeros(128, dtype=torch.bool), 32)
+
+
+def test_is_mem_built_under_inference_mode_is_checked_without_a_version_counter():
+    # inference tensors track no version counter (reading it raises); such masks are validated on every call
+    import torch
+    from landmark_hip import attention
+    attention._VALIDATED_MASKS.clear()
+    with torch.inference_mode():
+        mask = torch.arange(128) % 32 == 31
+        bad = torch.zeros(128, dtype=torch.bool)
+    assert mask.is_inference()
+    attention._check_is_mem(mask, 32)
+    attention._check_is_mem(mask, 32)
+    assert len(attention._VALIDATED_MASKS) == 0
+    with pytest.raises(AssertionError):
+        attention._check_is_mem(bad, 32)
+    with torch.inference_mode():
+        attention._check_is_mem(mask, 32)

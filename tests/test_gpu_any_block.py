@@ -162,3 +162,58 @@ def test_head_dims_16_and_32(D, block):
     assert (out.float().cpu() - ref).abs().max().item() <= TOL
     for g, r in ((gq, rq), (gk, rk), (gv, rv)):
         assert g.shape == r.shape and (g.float().cpu() - r).abs().max().item() <= TOL
+
+
+@pytest.mark.parametrize("block,D,L,P", [(51, 128, 204, 1), (100, 64, 300, 0), (17, 128, 136, 2)])
+def test_token_layout_equals_the_repacked_path_bit_for_bit(block, D, L, P):
+    # the kernels reading the tensors as they are (lmk_attn_*_blocks) against the same kernels on repacked copies
+    # (lmk_pad_blocks + lmk_attn_*_padded + lmk_unpad_blocks): same arithmetic on the same values, so the same bits;
+    # and the autograd function keeps the caller's tensors, not padded copies
+    from landmark_hip import attention
+    from ltriton.flash_landmark_attention import fused_landmark_attention
+    B, H = 1, 2
+    Lk = L + P * block
+    q, k, v = (t.to(DEV) for t in make_qkv(B, H, L, Lk, D, seed=block + L))
+    do = torch.randn(B, H, L, D, generator=torch.Generator().manual_seed(3)).bfloat16().to(DEV)
+    scale = D ** -0.5
+    slots = attention.storage_block(block)
+    o, Ls, M = attention._launch_fwd_blocks(q, k, v, P, scale, block)
+    dq, dk, dv = attention._launch_bwd_blocks(q, k, v, o, do, Ls, M, P, scale, block)
+    qp, kp, vp, dop = (attention._repack(t, block, slots) for t in (q, k, v, do))
+    op, Lp, Mp = attention._launch_fwd(qp, kp, vp, P, scale, slots, block)
+    dqp, dkp, dvp = attention._launch_bwd(qp, kp, vp, op, dop, Lp, Mp, P, scale, slots, block)
+    torch.cuda.synchronize()
+    assert torch.equal(o, attention._repack(op, block, slots, unpad=True, rows=L))
+    assert torch.equal(dq, attention._repack(dqp, block, slots, unpad=True, rows=L))
+    assert torch.equal(dk, attention._repack(dkp, block, slots, unpad=True, rows=Lk))
+    assert torch.equal(dv, attention._repack(dvp, block, slots, unpad=True, rows=Lk))
+    r = torch.arange(L, device=DEV)
+    r = r // block * slots + torch.where(r % block == block - 1, slots - 1, r % block)
+    assert torch.equal(Ls, Lp[:, r]) and torch.equal(M, Mp[:, r])
+    qg = q.clone().requires_grad_(True)
+    out = fused_landmark_attention(qg, k, v, None, block_size=block)
+    assert all(t.shape[2] in (L, Lk) for t in out.grad_fn.saved_tensors[:4])
+
+
+def test_token_layout_ignores_what_lies_in_rows_it_does_not_own():
+    # the padded entry points need finite values in their padding rows; the token-layout ones have no such rows:
+    # NaNs around the tensors (strided views of a larger, poisoned buffer) must not reach any result
+    from landmark_hip import attention
+    B, H, L, D, block = 1, 2, 153, 128, 51
+    big = [torch.full((B, H, L + 64, D), float("nan"), dtype=torch.bfloat16, device=DEV) for _ in range(4)]
+    q, k, v, do = (make_qkv(B, H, L, L, D, seed=9)[i].to(DEV) if i < 3 else
+                   torch.randn(B, H, L, D, generator=torch.Generator().manual_seed(1)).bfloat16().to(DEV) for i in range(4))
+    views = []
+    for buf, t in zip(big, (q, k, v, do)):
+        buf[:, :, 32:32 + L] = t
+        views.append(buf[:, :, 32:32 + L])
+    qv, kv, vv, dov = views
+    scale = D ** -0.5
+    o, Ls, M = attention._launch_fwd_blocks(qv, kv, vv, 0, scale, block)
+    grads = attention._launch_bwd_blocks(qv, kv, vv, o, dov, Ls, M, 0, scale, block)
+    o2, L2, M2 = attention._launch_fwd_blocks(q, k, v, 0, scale, block)
+    grads2 = attention._launch_bwd_blocks(q, k, v, o2, do, L2, M2, 0, scale, block)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.equal(o, o2)
+    for a, b_ in zip(grads, grads2):
+        assert torch.isfinite(a.float()).all() and torch.equal(a, b_)

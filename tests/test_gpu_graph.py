@@ -54,8 +54,11 @@ def test_decode_step_replays_from_a_graph(aggregate):
     assert torch.equal(out_g, out2) and torch.equal(idx_g, idx2)
 
 
-def test_forward_backward_replays_from_a_graph():
+@pytest.mark.parametrize("path", ["recompute", "handover"])
+def test_forward_backward_replays_from_a_graph(path, monkeypatch):
+    from landmark_hip import attention
     from landmark_hip.attention import _launch_bwd, _launch_fwd
+    monkeypatch.setattr(attention, "HANDOVER_MAX_BYTES", 0 if path == "recompute" else 1 << 40)
     B, H, L, D, block = 1, 4, 256, 128, 32
     gen = torch.Generator().manual_seed(6)
     mk = lambda: (torch.randn(B, H, L, D, generator=gen) * 0.5).bfloat16().cuda()

@@ -292,3 +292,15 @@ def test_without_blocks_only_the_tail_joins_the_chunk():
         qq = torch.cat((torch.zeros(3, hs, dtype=torch.float64), q[0, h]))
         want = s1.s1_attention(qq, torch.cat((tail_k[0, h], k[0, h])), torch.cat((ring.pending_v[0, h], v[0, h])), block)[3:]
         assert torch.allclose(y[0, h], want, atol=1e-12)
+
+
+def test_per_token_and_head_orders_underflowed_probabilities_by_score():
+    # scores so far below the row maximum that their fp32 probabilities are all 0: the pick follows the scores
+    # (-150 before -200 before -300), not the slot numbers a tie on the probabilities would fall back to
+    scores = torch.tensor([0.0, -200.0, -150.0, -300.0]).bfloat16().view(1, 1, 1, 4)
+    prob = mem_cache.block_probabilities(scores, "per_token_and_head")
+    assert prob[0, 0, 0, 1:].tolist() == [0.0, 0.0, 0.0]
+    assert mem_cache.select_blocks(scores, 0, 2, "per_token_and_head").flatten().tolist() == [0, 2]
+    assert mem_cache.select_blocks(scores, 0, 3, "per_token_and_head").flatten().tolist() == [0, 1, 2]
+    # the aggregated methods do rank probabilities: equal ones fall back to the lower slot
+    assert mem_cache.select_blocks(scores, 0, 2, "max_over_tokens").flatten().tolist() == [0, 1]

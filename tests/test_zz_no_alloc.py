@@ -58,3 +58,48 @@ def test_static_scratch_rejects_sizes_beyond_its_array():
     assert rc == -8
     with pytest.raises(_lib.LmkError):
         _lib.check(rc)
+
+
+def test_static_scratch_selection_replays_from_a_graph():
+    # the array's address is resolved before the capture (lmk_retrieve_static_init); the captured call must then
+    # reproduce lmk_retrieve_topk on every replay, with eager work and new inputs in between
+    from landmark_hip import _lib
+    lib = _lib.lib()
+    _lib.check(lib.lmk_retrieve_static_init())
+    B, H, T, S, D, block, top_k = 1, 8, 1, 64 * 32 + 5, 128, 32, 4
+    g = torch.Generator().manual_seed(11)
+    mk = lambda *s_: (torch.randn(*s_, generator=g) * 0.5).bfloat16().cuda()
+    q, kc = mk(B, H, T, D), mk(B, H, S, D)
+    cos, sin = (t.cuda() for t in orot.rotary_tables(S + T, D, torch.bfloat16))
+    nbytes = lib.lmk_retrieve_workspace_bytes(B, H, T, S, D, block)
+    ws = torch.empty(nbytes, device="cuda", dtype=torch.uint8)
+    ref = torch.empty((B, H, T, top_k), device="cuda", dtype=torch.int64)
+    got = torch.empty_like(ref)
+
+    def eager_ref():
+        _lib.check(lib.lmk_retrieve_topk(_lib.tensor4(q), _lib.tensor4(kc), cos.data_ptr(), sin.data_ptr(), cos.stride(0),
+                                         cos.shape[0], ref.data_ptr(), ws.data_ptr(), nbytes, B, H, T, S, D, block, top_k, 0,
+                                         _lib.current_stream(q.device)))
+
+    def static_call():
+        _lib.check(lib.lmk_retrieve_topk_static(_lib.tensor4(q), _lib.tensor4(kc), cos.data_ptr(), sin.data_ptr(),
+                                                cos.stride(0), cos.shape[0], got.data_ptr(), B, H, T, S, D, block, top_k, 0,
+                                                _lib.current_stream(q.device)))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        static_call()                                            # kernel attributes are set outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_call()
+    for rep in range(4):
+        if rep:
+            q.copy_(mk(B, H, T, D))                              # new queries in the captured buffer
+        eager_ref()
+        got.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref), rep
