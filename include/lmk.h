@@ -174,6 +174,23 @@ int lmk_attn_bwd_blocks(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
                         int H, int Lq, int Lk, int D, float sm_scale, int block_tokens, int n_prefix, int dtype,
                         void* stream);
 
+/* Group dropout (lm_benchmark/models/landmark.py:110-113: `dropout(group_prob, p)` on the landmark probabilities
+ * that scale the earlier blocks, while the softmax over the landmarks itself stays as it is).  The random draw is
+ * the caller's: group_scale is (B*H, Lk/block_tokens, Lq) fp32, contiguous, and entry [bh][b][i] multiplies what
+ * earlier block b contributes to query row i -- 0 for a dropped block, 1/(1-p) for a kept one; entries of a row's
+ * own and later blocks are not read.  Same tensors, sizes and statistics as lmk_attn_*_blocks; block_tokens 2..128
+ * (32 included: it runs in 64 slots here, the block-32 kernels carry no such factor).  The backward must be given
+ * the forward's group_scale.  Workspace: lmk_attn_bwd_group_scale_workspace_bytes. */
+int lmk_attn_fwd_group_scale(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                             float* L, float* M, const float* group_scale, int B, int H, int Lq, int Lk, int D,
+                             float sm_scale, int block_tokens, int n_prefix, int dtype, void* stream);
+size_t lmk_attn_bwd_group_scale_workspace_bytes(int B, int H, int Lq, int Lk, int block_tokens);
+int lmk_attn_bwd_group_scale(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                             const lmk_tensor4* dout, const float* L, const float* M, const float* group_scale,
+                             const lmk_tensor4* dq, const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace,
+                             size_t workspace_bytes, int B, int H, int Lq, int Lk, int D, float sm_scale,
+                             int block_tokens, int n_prefix, int dtype, void* stream);
+
 /* ---- mem-cache retrieval (inference) --------------------------------------------------
  * The reference has no function boundary here: scoring, selection and gather are inline in
  * LlamaAttention.forward (llama/llama_mem.py:318-430) and the attend step follows at :447-477.

@@ -193,7 +193,7 @@ struct RopeArgs {
 static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                          float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
                          int block_real, int n_prefix, int dtype, void* stream, const RopeArgs* rope = nullptr,
-                         int Lq_real = 0, int Lk_real = 0) {
+                         int Lq_real = 0, int Lk_real = 0, const float* group_scale = nullptr) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o))) return rc;
   if (L == nullptr || M == nullptr) return LMK_ERR_NULL;
@@ -214,6 +214,12 @@ static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
   }
   p.n_real = block_real;
   p.Lq_real = Lq_real; p.Lk_real = Lk_real;
+  if (group_scale != nullptr) {                            // (B*H, Lk_real / block_real, Lq_real) floats
+    if (Lq_real <= 0) return LMK_ERR_UNSUPPORTED;
+    p.group_scale = group_scale;
+    p.gs_blk = Lq_real;
+    p.gs_bh = (int64_t)(Lk_real / block_real) * Lq_real;
+  }
   p.q = q->ptr; p.k = k->ptr; p.v = v->ptr; p.o = o->ptr;
   p.L = L; p.M = M;
   p.B = B; p.H = H; p.Lq = Lq; p.Lk = Lk;
@@ -314,7 +320,8 @@ static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
                          const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
                          const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
                          int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
-                         int dtype, int phases, void* stream, int Lq_real = 0, int Lk_real = 0);
+                         int dtype, int phases, void* stream, int Lq_real = 0, int Lk_real = 0,
+                         const float* group_scale = nullptr);
 
 int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                         const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
@@ -382,11 +389,56 @@ int lmk_attn_bwd_blocks(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
                        slots, block_tokens, n_prefix, dtype, LMK_BWD_ALL, stream, Lq, Lk);
 }
 
+// ---- group dropout: a caller-supplied factor per (query row, earlier block).  Always the slot kernels in token
+// layout: blocks of up to 64 tokens in 64 slots (block 32 included: its own kernels carry no such factor), wider in 128.
+static int slots_for_group_scale(int block_tokens) {
+  if (block_tokens < 2 || block_tokens > 128) return 0;
+  return block_tokens <= 64 ? 64 : 128;
+}
+
+int lmk_attn_fwd_group_scale(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                             float* L, float* M, const float* group_scale, int B, int H, int Lq, int Lk, int D,
+                             float sm_scale, int block_tokens, int n_prefix, int dtype, void* stream) {
+  const int slots = slots_for_group_scale(block_tokens);
+  if (slots == 0) return LMK_ERR_UNSUPPORTED;
+  if (group_scale == nullptr) return LMK_ERR_NULL;
+  if (Lq <= 0 || Lk < Lq || n_prefix < 0) return LMK_ERR_SHAPE;
+  if ((int64_t)Lk - Lq != (int64_t)n_prefix * block_tokens) return LMK_ERR_HISTORY;
+  const int64_t lq = lmk_padded_rows(Lq, block_tokens, slots), lk = (int64_t)n_prefix * slots + lq;
+  if (lk >= ((int64_t)1 << 31)) return LMK_ERR_UNSUPPORTED;
+  return attn_fwd_impl(q, k, v, o, L, M, B, H, (int)lq, (int)lk, D, sm_scale, slots, block_tokens, n_prefix, dtype, stream,
+                       nullptr, Lq, Lk, group_scale);
+}
+
+size_t lmk_attn_bwd_group_scale_workspace_bytes(int B, int H, int Lq, int Lk, int block_tokens) {
+  const int slots = slots_for_group_scale(block_tokens);
+  if (slots == 0 || Lq <= 0 || Lk <= 0) return 0;
+  return lmk_attn_bwd_workspace_bytes(B, H, (int)lmk_padded_rows(Lq, block_tokens, slots),
+                                      (int)lmk_padded_rows(Lk, block_tokens, slots), slots);
+}
+
+int lmk_attn_bwd_group_scale(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                             const lmk_tensor4* dout, const float* L, const float* M, const float* group_scale,
+                             const lmk_tensor4* dq, const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace,
+                             size_t workspace_bytes, int B, int H, int Lq, int Lk, int D, float sm_scale,
+                             int block_tokens, int n_prefix, int dtype, void* stream) {
+  const int slots = slots_for_group_scale(block_tokens);
+  if (slots == 0) return LMK_ERR_UNSUPPORTED;
+  if (group_scale == nullptr) return LMK_ERR_NULL;
+  if (Lq <= 0 || Lk < Lq || n_prefix < 0) return LMK_ERR_SHAPE;
+  if (Lq % block_tokens != 0 || Lk % block_tokens != 0) return LMK_ERR_PARTIAL;
+  if ((int64_t)Lk - Lq != (int64_t)n_prefix * block_tokens) return LMK_ERR_HISTORY;
+  const int64_t lq = (int64_t)Lq / block_tokens * slots, lk = (int64_t)Lk / block_tokens * slots;
+  if (lk >= ((int64_t)1 << 31)) return LMK_ERR_UNSUPPORTED;
+  return attn_bwd_impl(q, k, v, o, dout, L, M, dq, dk, dv, workspace, workspace_bytes, B, H, (int)lq, (int)lk, D, sm_scale,
+                       slots, block_tokens, n_prefix, dtype, LMK_BWD_ALL, stream, Lq, Lk, group_scale);
+}
+
 static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                          const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
                          const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
                          int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
-                         int dtype, int phases, void* stream, int Lq_real, int Lk_real) {
+                         int dtype, int phases, void* stream, int Lq_real, int Lk_real, const float* group_scale) {
   int rc;
   if (phases <= 0 || phases > LMK_BWD_ALL) return LMK_ERR_SHAPE;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o)) ||
@@ -424,6 +476,13 @@ static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
   p.n_prefix = n_prefix; p.n_blocks = (int)nb;
   p.n_real = block_real;
   p.Lq_real = Lq_real; p.Lk_real = Lk_real;
+  p.group_scale = nullptr; p.gs_bh = p.gs_blk = 0;
+  if (group_scale != nullptr) {
+    if (Lq_real <= 0) return LMK_ERR_UNSUPPORTED;
+    p.group_scale = group_scale;
+    p.gs_blk = Lq_real;
+    p.gs_bh = (int64_t)(Lk_real / block_real) * Lq_real;
+  }
   p.n_qtiles = (Lq + 127) / 128; p.n_kvtiles = (Lk + 127) / 128;
   p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
   p.ks_b = k->stride_b; p.ks_h = k->stride_h; p.ks_r = k->stride_row;

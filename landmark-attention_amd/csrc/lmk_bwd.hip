@@ -278,6 +278,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     const int kb = buf * C::STAGE_BYTES, vb = kb + C::TILE_BYTES;   // LDS byte addresses (the dynamic array starts at 0)
     if (!active) continue;
     if (s < cblk) {
+      float gscale = 1.f;                                  // group dropout: this block's factor for this query row
+      if constexpr (VIRT)
+        if (p.group_scale != nullptr && qtok >= 0) gscale = p.group_scale[(int64_t)bh * p.gs_bh + (int64_t)s * p.gs_blk + qtok];
       f32x16_t sc[C::NT], dp[C::KEEP_DP ? C::NT : 1];
 #pragma unroll
       for (int u = 0; u < C::NT; ++u) sc[u] = row_tile(kb + 32 * u * C::ROWB, qf);
@@ -320,12 +323,14 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
       const float nD = spd * invden;
       const float glog = t_lm - mhat;                      // log2 of the normalised gate
       const float g = fast_exp2(glog);
-      const float f = g * invden;
+      // out_i = .. + gscale * g * (P V): the weights carry the factor, the landmark's dS sees it through nD
+      const float f = g * invden * gscale;
+      const float dslm = g * (gscale * nD - delta);        // dS at the block's landmark key
       if (h == 0) {
         const int64_t si = ((int64_t)bh * p.n_blocks + s) * p.Lq + qrow;
-        p.stat_a[si] = mloc + fast_log2(den) - glog;
+        p.stat_a[si] = gscale > 0.f ? mloc + fast_log2(den) - glog - fast_log2(gscale) : 1e30f;
         p.stat_n[si] = nD;
-        p.stat_l[si] = g * (nD - delta);                   // dS at the block's landmark key
+        p.stat_l[si] = dslm;
       }
 #pragma unroll
       for (int u = 0; u < C::NT; ++u) {
@@ -334,7 +339,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
         float ds[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) ds[r] = sc[u][r] * f * (d[r] - nD);
-        if (u == C::NT - 1 && h == 1) ds[15] = g * (nD - delta);
+        if (u == C::NT - 1 && h == 1) ds[15] = dslm;
         dq_tile(kb + 32 * u * C::ROWB, ds);
       }
     } else if (s == cblk) {

@@ -217,6 +217,8 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
       const int kb = buf * C::STAGE_BYTES + jb * BS * C::ROWB, vb = kb + C::TILE_BYTES;
       if (blk < cblk) {
         // ---------------- earlier block: local softmax gated by its landmark
+        float gscale = 1.f;                               // group dropout: this block's factor for this query row
+        if (p.group_scale != nullptr && qtok >= 0) gscale = p.group_scale[(int64_t)bh * p.gs_bh + (int64_t)blk * p.gs_blk + qtok];
         f32x16_t sc[C::NT];
 #pragma unroll
         for (int u = 0; u < C::NT; ++u) sc[u] = qk_tile(kb + 32 * u * C::ROWB);
@@ -257,7 +259,7 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
         lrun = lrun * alpha + gate;
         Mrun = Mnew;
         rescale(alpha);
-        const float f = gate * fast_rcp(den);
+        const float f = gate * fast_rcp(den) * gscale;
 #pragma unroll
         for (int u = 0; u < C::NT; ++u) {
           float w[16];

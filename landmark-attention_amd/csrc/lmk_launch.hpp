@@ -53,6 +53,11 @@ struct FwdParams {
   // partial last block keeps its length); the kernels translate slot rows to token rows themselves.
   // 0: the tensors are stored in slots already (n_real < block: with padding rows).
   int Lq_real, Lk_real;
+  // optional (blocks of 64 / 128 slots, token layout only): factor of earlier block b's contribution to query row i,
+  // group_scale[bh * gs_bh + b * gs_blk + i] -- 0 drops the block for that row, 1 / (1 - p) keeps it under group
+  // dropout (lm_benchmark/models/landmark.py:110-113); the softmax over the landmarks is not renormalised
+  const float* group_scale;
+  int64_t gs_bh, gs_blk;
   // optional: q arrives without rotary and is rotated as it is loaded (null tables: q is used as it is)
   const void *rope_cos, *rope_sin;
   const int64_t* rope_pos;        // position of query row r of batch b: rope_pos[b * rope_pos_stride_b + r]
@@ -80,6 +85,8 @@ struct BwdParams {
   int n_qtiles, n_kvtiles;       // ceil(Lq / 128), ceil(Lk / 128)
   int n_real;                    // tokens of a block that exist; == block unless padded (blocks 64 and 128 only)
   int Lq_real, Lk_real;          // > 0: tensors in token layout, as in FwdParams (the workspace stays indexed by slot rows)
+  const float* group_scale;      // optional, as in FwdParams (token layout only)
+  int64_t gs_bh, gs_blk;
   int64_t qs_b, qs_h, qs_r, ks_b, ks_h, ks_r, vs_b, vs_h, vs_r, os_b, os_h, os_r, dos_b, dos_h, dos_r;
   int64_t dqs_b, dqs_h, dqs_r, dks_b, dks_h, dks_r, dvs_b, dvs_h, dvs_r;
   float scale, scale_log2;

@@ -76,6 +76,12 @@ def lib() -> ctypes.CDLL:
         L.lmk_attn_bwd_blocks_workspace_bytes.argtypes = [i, i, i, i, i]
         L.lmk_attn_bwd_blocks.restype = i
         L.lmk_attn_bwd_blocks.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, sz, i, i, i, i, i, f, i, i, i, vp]
+        L.lmk_attn_fwd_group_scale.restype = i
+        L.lmk_attn_fwd_group_scale.argtypes = [T4, T4, T4, T4, vp, vp, vp, i, i, i, i, i, f, i, i, i, vp]
+        L.lmk_attn_bwd_group_scale_workspace_bytes.restype = sz
+        L.lmk_attn_bwd_group_scale_workspace_bytes.argtypes = [i, i, i, i, i]
+        L.lmk_attn_bwd_group_scale.restype = i
+        L.lmk_attn_bwd_group_scale.argtypes = [T4, T4, T4, T4, T4, vp, vp, vp, T4, T4, T4, vp, sz, i, i, i, i, i, f, i, i, i, vp]
         L.lmk_retrieve_workspace_bytes.restype = sz
         L.lmk_retrieve_workspace_bytes.argtypes = [i, i, i, i, i, i]
         L.lmk_retrieve_topk.restype = i

@@ -172,6 +172,57 @@ class FusedLandmarkAttention(torch.autograd.Function):
         return dq, dk, dv, None, None, None
 
 
+class FusedLandmarkAttentionGroupScale(torch.autograd.Function):
+    """``FusedLandmarkAttention`` with group dropout (``lm_benchmark/models/landmark.py:110-113``): ``group_scale``
+    (B, H, Lk / block_size, Lq) fp32 multiplies what earlier block b contributes to query row i -- 0 for a dropped
+    block, 1 / (1 - p) for a kept one -- while the softmax over the landmarks is left as it is.  The draw is the
+    caller's (e.g. ``torch.nn.functional.dropout(torch.ones(...), p)``), so results are reproducible from the mask."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, group_scale, n_prefix_q, sm_scale, block_size):
+        B, H, Lq, D = q.shape
+        Lk = k.shape[2]
+        assert k.shape == v.shape == (B, H, Lk, D) and q.dtype == k.dtype == v.dtype and q.dtype in _lib.DTYPE_CODES
+        assert q.is_cuda and D in SUPPORTED_HEAD_DIMS and 2 <= block_size <= MAX_BLOCK
+        assert group_scale.shape == (B, H, Lk // block_size, Lq) and group_scale.dtype == torch.float32
+        assert group_scale.device == q.device
+        q, k, v = _lib.kernel_ready(q), _lib.kernel_ready(k), _lib.kernel_ready(v)
+        group_scale = group_scale.contiguous()
+        o = torch.empty_like(q)
+        L = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+        M = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+        with _lib.on_device(q.device):
+            rc = _lib.lib().lmk_attn_fwd_group_scale(
+                _lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o), L.data_ptr(), M.data_ptr(),
+                group_scale.data_ptr(), B, H, Lq, Lk, D, float(sm_scale), int(block_size), int(n_prefix_q),
+                _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+        _lib.check(rc)
+        ctx.save_for_backward(q, k, v, o, L, M, group_scale)
+        ctx.args = (n_prefix_q, sm_scale, block_size)
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, L, M, group_scale = ctx.saved_tensors
+        n_prefix_q, sm_scale, block_size = ctx.args
+        B, H, Lq, D = q.shape
+        Lk = k.shape[2]
+        assert Lq % block_size == 0 and Lk % block_size == 0, "Backward supported only for full blocks"
+        do = _lib.kernel_ready(do)
+        lib = _lib.lib()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        nbytes = lib.lmk_attn_bwd_group_scale_workspace_bytes(B, H, Lq, Lk, int(block_size))
+        ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+        with _lib.on_device(q.device):
+            rc = lib.lmk_attn_bwd_group_scale(
+                _lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o), _lib.tensor4(do), L.data_ptr(),
+                M.data_ptr(), group_scale.data_ptr(), _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv), ws.data_ptr(),
+                nbytes, B, H, Lq, Lk, D, float(sm_scale), int(block_size), int(n_prefix_q), _lib.DTYPE_CODES[q.dtype],
+                _lib.current_stream(q.device))
+        _lib.check(rc)
+        return dq, dk, dv, None, None, None, None
+
+
 # Masks that have already passed the check of ``flash_landmark_attention.py:393-394``, keyed by what
 # identifies a tensor's content without reading it: storage address, in-place version counter, layout.
 # (A write through ``.data`` or a custom kernel bypasses the counter; such a mask has to be a new tensor.)
@@ -202,14 +253,15 @@ def _check_is_mem(is_mem, block_size):
     _VALIDATED_MASKS[key] = is_mem
 
 
-def fused_landmark_attention(q, k, v, is_mem, sm_scale=None, block_size=64):
+def fused_landmark_attention(q, k, v, is_mem, sm_scale=None, block_size=64, group_scale=None):
     """Landmark grouped-softmax causal attention, landmarks at every ``block_size``-th key.
 
     q: (B, H, Lq, D); k, v: (B, H, Lk, D) with ``Lk - Lq`` a whole number of blocks of
     history.  ``is_mem`` (bool, last dim Lk) must mark exactly the positions
     ``j % block_size == block_size - 1`` (checked as in the reference, ``:393-394``; the check
     costs one device->host sync, paid once per distinct mask tensor state, not per call); pass
-    ``None`` to skip the check.
+    ``None`` to skip the check.  ``group_scale`` (not in the reference's signature): the group-dropout factors of
+    ``FusedLandmarkAttentionGroupScale``, (B, H, Lk / block_size, Lq) fp32, for head dims 64 and 128.
     """
     if is_mem is not None:
         _check_is_mem(is_mem, block_size)
@@ -220,6 +272,9 @@ def fused_landmark_attention(q, k, v, is_mem, sm_scale=None, block_size=64):
 
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(q.size(-1))
+
+    if group_scale is not None:
+        return FusedLandmarkAttentionGroupScale.apply(q, k, v, group_scale, n_history_blocks, sm_scale, block_size)
 
     d = q.size(-1)
     if d in PADDED_HEAD_DIMS:

@@ -55,8 +55,14 @@ def _bucketed_softmax(x, bucket, n_buckets: int, guard_empty: bool):
     return e / z
 
 
-def grouped_softmax(x, is_mem, last_section, n_buckets: int = 64, attn_mask=None, guard_empty: bool = False):
+def grouped_softmax(x, is_mem, last_section, n_buckets: int = 64, attn_mask=None, guard_empty: bool = False,
+                    group_keep=None):
     """Landmark grouped softmax over the last dim of ``x``.
+
+    ``group_keep`` (broadcastable to ``x.shape[:-1] + (n_buckets,)``), optional: the outcome of the group dropout
+    of ``landmark.py:110-113`` written as a factor per bucket -- ``dropout(group_prob, p)`` multiplies each
+    landmark probability by 0 or 1 / (1 - p) before it scales its block; the last bucket is overwritten
+    afterwards (``:112``), so its entry is not used.
 
     ``is_mem``        bool, True at visible landmark keys
     ``last_section``  bool, True at visible keys of the query's own block
@@ -75,6 +81,8 @@ def grouped_softmax(x, is_mem, last_section, n_buckets: int = 64, attn_mask=None
     slot = torch.where(is_mem, seen - 1, torch.full_like(seen, last)).expand(x.shape)
     by_block = torch.zeros(x.shape[:-1] + (n_buckets,), dtype=probs.dtype, device=x.device)
     by_block = by_block.scatter(-1, slot, probs)
+    if group_keep is not None:                                   # landmark.py:110-111
+        by_block = by_block * group_keep
     if attn_mask is not None:                                    # landmark.py:115
         by_block = by_block.clone()
         by_block[..., last] = (probs * last_section).sum(-1)

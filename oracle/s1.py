@@ -105,8 +105,12 @@ def _geometry(lq: int, lk: int, block: int, rows, device):
     return rows, cur, lim
 
 
-def s1_weights(q, k, block: int, scale: float | None = None, rows=None):
+def s1_weights(q, k, block: int, scale: float | None = None, rows=None, group_scale=None):
     """Attention weights (…, R, Lk) of S1 plus the global-bucket statistics.
+
+    ``group_scale`` (…, n_blocks, R), optional: factor of earlier block b's contribution to row i (group dropout,
+    ``lm_benchmark/models/landmark.py:110-113``: the landmark probabilities that scale the earlier blocks are
+    dropped or scaled by 1 / (1 - p), the softmax over the landmarks itself is not renormalised).
 
     q: (..., Lq, D), k: (..., Lk, D) in any float dtype; the arithmetic runs in
     that dtype.  ``rows`` optionally restricts the evaluation to some query rows
@@ -147,15 +151,17 @@ def s1_weights(q, k, block: int, scale: float | None = None, rows=None):
     zl = el.sum(-1, keepdim=True)
     pl = el / torch.where(zl > 0, zl, torch.ones_like(zl))
     gate = g.unflatten(-1, (nb, block))[..., block - 1:block]      # g at each block's landmark
+    if group_scale is not None:
+        gate = gate * group_scale.transpose(-1, -2).unsqueeze(-1).to(gate.dtype)
     w = (pl * gate).flatten(-2) + torch.where(same, g, torch.zeros_like(g))
     if pad:
         w = w[..., :lk]
     return w, L.squeeze(-1), M.squeeze(-1)
 
 
-def s1_attention(q, k, v, block: int, scale: float | None = None, rows=None, return_stats=False):
+def s1_attention(q, k, v, block: int, scale: float | None = None, rows=None, return_stats=False, group_scale=None):
     """out (…, R, D) of S1; differentiable through torch autograd."""
-    w, L, M = s1_weights(q, k, block, scale, rows)
+    w, L, M = s1_weights(q, k, block, scale, rows, group_scale)
     out = w @ v
     if return_stats:
         return out, L, M

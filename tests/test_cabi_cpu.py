@@ -30,7 +30,7 @@ def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
             "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend", "lmk_retrieve_topk_static", "lmk_retrieve_static_max_bytes",
-            "lmk_ring_retrieve_topk", "lmk_ring_gather_attend", "lmk_attn_bwd_handover_workspace_bytes", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded", "lmk_attn_fwd_blocks", "lmk_attn_bwd_blocks",
+            "lmk_ring_retrieve_topk", "lmk_ring_gather_attend", "lmk_attn_bwd_handover_workspace_bytes", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded", "lmk_attn_fwd_blocks", "lmk_attn_bwd_blocks", "lmk_attn_fwd_group_scale", "lmk_attn_bwd_group_scale",
             "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
@@ -260,6 +260,27 @@ def test_token_layout_entry_points_argument_errors(lib):
     assert L.lmk_attn_bwd_blocks_workspace_bytes(2, 8, 510, 510, 51) == L.lmk_attn_bwd_workspace_bytes(2, 8, 640, 640, 64)
     assert L.lmk_attn_bwd_blocks_workspace_bytes(2, 8, 512, 512, 64) == L.lmk_attn_bwd_workspace_bytes(2, 8, 512, 512, 64)
     assert L.lmk_attn_bwd_blocks_workspace_bytes(1, 1, 10, 10, 200) == 0
+
+
+def test_group_scale_and_rotary_q_argument_errors(lib):
+    from landmark_hip import _lib
+    L = _lib.lib()
+    t = _lib.Tensor4(0x1000, 0, 0, 128)
+
+    def fwd(gs=0x9000, Lq=102, Lk=102, block=51, n_prefix=0):
+        return L.lmk_attn_fwd_group_scale(t, t, t, t, 0x2000, 0x3000, gs, 1, 1, Lq, Lk, 128, 0.1, block, n_prefix, 0, None)
+
+    def bwd(gs=0x9000, Lq=102, Lk=102, block=51, ws=1 << 30):
+        return L.lmk_attn_bwd_group_scale(t, t, t, t, t, 0x2000, 0x3000, gs, t, t, t, 0x4000, ws, 1, 1, Lq, Lk, 128, 0.1,
+                                          block, 0, 0, None)
+    assert fwd(gs=None) == -1 and fwd(block=129) == -3 and fwd(Lk=150) == -5
+    assert bwd(gs=None) == -1 and bwd(Lq=100, Lk=100) == -6 and bwd(ws=8) == -8
+    # block 32 runs in 64 slots when group factors are given: the workspace is sized for that
+    assert L.lmk_attn_bwd_group_scale_workspace_bytes(1, 2, 64, 64, 32) == L.lmk_attn_bwd_workspace_bytes(1, 2, 128, 128, 64)
+    # the forward that rotates q in its prologue exists for the native block sizes only
+    rc = L.lmk_attn_fwd_rotary_q(t, t, t, t, 0x2000, 0x3000, 0x5000, 0x6000, 128, 4096, 0x7000, 0, 1, 1, 102, 102, 128, 0.1,
+                                 51, 0, 0, None)
+    assert rc == -3
 
 
 def test_ring_selection_argument_errors(lib):

@@ -304,3 +304,18 @@ def test_workspace_size_selects_the_backward_path():
         got[name] = (dq, dk, dv)
     assert all(torch.equal(a, b_) for a, b_ in zip(got["below"], got["small"]))
     assert not torch.equal(got["at"][1], got["small"][1])
+
+
+def test_gradients_at_8192_tokens():
+    # B1 H2 L8192, block 32: 256 landmark blocks, 32 query tiles per head.  The hand-over workspace (1.1 GB for two
+    # heads) is above the shim's default limit, so this is the recomputing pair, the path that serves this length
+    B, H, L, D, block = 1, 2, 8192, 128, 32
+    print("case L8192", flush=True)
+    q, k, v = make_qkv(B, H, L, L, D, seed=8192)
+    do = torch.randn(B, H, L, D, generator=torch.Generator().manual_seed(8193)).bfloat16()
+    rq, rk, rv = oracle_grads(q, k, v, do, block, chunk=1)
+    gq, gk, gv = _grads(q, k, v, do, block)
+    for name, g, r in (("dq", gq, rq), ("dk", gk, rk), ("dv", gv, rv)):
+        err = (g.float().cpu() - r).abs().max().item()
+        print("L8192", name, "max abs err", err, flush=True)
+        assert err <= TOL, (name, err)

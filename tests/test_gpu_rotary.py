@@ -141,3 +141,15 @@ def test_rotary_gradients_match_torch_autograd_of_the_reference_expression(B, H,
     _, only_k = apply_rotary_pos_emb(None, kd2, cos.cuda(), sin.cuda(), pos.cuda())
     (g2,) = torch.autograd.grad(only_k, kd2, dk.cuda())
     assert torch.equal(g2.cpu(), want_k)
+
+
+def test_rotary_q_forward_rejects_block_sizes_it_is_not_built_for():
+    # lmk_attn_fwd_rotary_q serves the native block sizes (32, 64, 128); other sizes rotate q with
+    # apply_rotary_pos_emb and call fused_landmark_attention
+    from landmark_hip.attention import fused_landmark_attention_rotary_q
+    B, H, L, D, block = 1, 2, 102, 128, 51
+    q, k, v = (torch.zeros(B, H, L, D, dtype=torch.bfloat16, device="cuda") for _ in range(3))
+    cos, sin = (t.cuda() for t in orot.rotary_tables(L, D, torch.bfloat16))
+    pos = torch.arange(L, device="cuda")[None]
+    with pytest.raises(AssertionError):
+        fused_landmark_attention_rotary_q(q, k, v, cos, sin, pos, block_size=block)

@@ -83,3 +83,41 @@ def test_benchmark_config0_full_size_restatement_equals_closed_form():
     a64 = highlevel.attention_lm_benchmark(q.double(), k.double(), v.double(), is_mem, n_buckets=16)
     assert (a64 - s1.s1_attention(q.double(), k.double(), v.double(), block)).abs().max().item() <= 1e-12
     assert (a64 - a).abs().max().item() <= 2e-5
+
+
+def test_group_dropout_scales_earlier_blocks_and_leaves_the_landmark_softmax_alone():
+    # landmark.py:110-113 with the dropout's outcome supplied as a factor per (row, block): the restated bucketed
+    # softmax, the closed form, and the plain statement "weights of a block's normal keys times its factor, every
+    # other weight unchanged" must agree (fp64)
+    import math
+    from oracle import highlevel, s1
+    torch.manual_seed(0)
+    B, H, L, D, block = 1, 2, 35, 8, 7
+    nb = L // block
+    q, k, v = (torch.randn(B, H, L, D, dtype=torch.float64) for _ in range(3))
+    p_drop = 0.4
+    keep = torch.nn.functional.dropout(torch.ones(B, H, nb, L, dtype=torch.float64), p_drop)     # {0, 1/(1-p)}
+    assert set(keep.unique().tolist()) <= {0.0, 1.0 / (1.0 - p_drop)} and (keep == 0).any() and (keep > 0).any()
+    w_plain, _, _ = s1.s1_weights(q, k, block)
+    w_drop, L_drop, M_drop = s1.s1_weights(q, k, block, group_scale=keep)
+    # plain statement: key j of an earlier block b (not its landmark) gets factor keep[b, i]; everything else stays
+    j = torch.arange(L)
+    i = torch.arange(L)
+    earlier_normal = ((j // block)[None, :] < (i // block)[:, None]) & ((j % block) != block - 1)[None, :]
+    per_key = keep.transpose(-1, -2)[..., j // block]                                   # (B, H, i, j)
+    want = torch.where(earlier_normal, w_plain * per_key, w_plain)
+    assert torch.allclose(w_drop, want, atol=1e-14)
+    _, L_plain, M_plain = s1.s1_weights(q, k, block)
+    assert torch.equal(L_drop, L_plain) and torch.equal(M_drop, M_plain)                # the global bucket is untouched
+    # the restated high-level path with the same outcome of the dropout
+    att = (q @ k.transpose(-2, -1)) / math.sqrt(D)
+    causal_masked = ~torch.tril(torch.ones(L, L, dtype=torch.bool))[None, None].expand(B, H, L, L)
+    att = att.masked_fill(causal_masked, float("-inf"))
+    is_mem = (j % block == block - 1)[None].expand(B, L)
+    masked, im, ls = highlevel.masks_from_is_mem(is_mem[:, None, None, :], causal_masked)
+    att = att.masked_fill(masked, float("-inf"))
+    n_buckets = nb + 3
+    keep_b = torch.ones(B, H, L, n_buckets, dtype=torch.float64)
+    keep_b[..., :nb] = keep.transpose(-1, -2)
+    w_high = highlevel.grouped_softmax(att, im, ls, n_buckets, attn_mask=masked, guard_empty=True, group_keep=keep_b)
+    assert torch.allclose(w_high, w_drop, atol=1e-14)
