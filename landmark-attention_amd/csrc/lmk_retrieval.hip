@@ -466,33 +466,40 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
       const float eps_q = sqrtf(qn) * 1.000001f * (1.0f / 16384.0f);
 
       float* srow = sc + qi * NMp;
-      float lo[NJ], hi[NJ];
+      // raw bracket of the fp32 dot product: [a - e, a + e] around the MFMA score a.  The contract (round, divide,
+      // round) is monotone, and so are the outward-rounded estimates T_lo / T_hi of it below, so the order
+      // statistics are taken on the raw ends and only the few values that matter go through T_lo / T_hi.
+      float up[NJ];
+      float lm = -INFINITY;                                         // this lane's best raw lower end
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        lo[j] = -INFINITY;
-        hi[j] = -INFINITY;
+        up[j] = -INFINITY;
         if (j < nj) {
           const float a = srow[64 * j + lane];
-          if (a > -INFINITY) {
-            const float e = eps_q * nrm[j];
-            const float cl = round_to<T>(a - e) * inv_sq, ch = round_to<T>(a + e) * inv_sq;
-            lo[j] = round_to<T>(cl - fabsf(cl) * 4.76837158203125e-7f);
-            hi[j] = round_to<T>(ch + fabsf(ch) * 4.76837158203125e-7f);
-          }
+          const float e = eps_q * nrm[j];
+          up[j] = a + e;                                            // -inf (no landmark) stays -inf
+          lm = fmaxf(lm, a - e);
         }
       }
-      // tau = the k-th best of the lanes' best lower ends: k different blocks reach it, so the k-th best
+      auto t_lo = [&](float x) {
+        const float cl = round_to<T>(x) * inv_sq;
+        return round_to<T>(cl - fabsf(cl) * 4.76837158203125e-7f);
+      };
+      auto t_hi = [&](float x) {
+        const float ch = round_to<T>(x) * inv_sq;
+        return round_to<T>(ch + fabsf(ch) * 4.76837158203125e-7f);
+      };
+      // tau = T_lo of the k-th best of the lanes' best lower ends: k different blocks reach it, so the k-th best
       // exact score does too (a little below the k-th best lower end itself, and k times cheaper to find)
-      float tau = -INFINITY;
-      {
-        float lm = -INFINITY;
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) lm = fmaxf(lm, lo[j]);
-        for (int j = 0; j < p.k; ++j) {
-          int bi;
-          take_one(lm, lane, tau, bi);
-        }
+      float tau_raw = -INFINITY;
+      for (int j = 0; j < p.k; ++j) {
+        int bi;
+        take_one(lm, lane, tau_raw, bi);
       }
+      const float tau = t_lo(tau_raw);
+      // T_hi(x) >= tau needs x >= tau_raw up to the roundings of both estimates (two roundings to 8 or 11 bits
+      // each, 3 % covers them; 1e-5 covers the subnormal range): everything below theta is out without being rounded
+      const float theta = tau_raw - (fabsf(tau_raw) * 0.03f + 1e-5f);
       // contenders: upper end reaches tau.  They are collected in a short list and evaluated exactly,
       // one lane per contender, whenever the list holds a wave's worth (and at the end).
       auto evaluate = [&](int count) {
@@ -534,8 +541,8 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
       bool flushed = false;                                         // wave-uniform: the list was emptied on the way
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        if (j < nj) {
-          const bool c = hi[j] >= tau && hi[j] > -INFINITY;
+        if (j < nj && __any(up[j] >= theta && up[j] > -INFINITY)) {   // wave-uniform: most slices hold no contender
+          const bool c = up[j] >= theta && up[j] > -INFINITY && t_hi(up[j]) >= tau;
           const uint64_t bal = __ballot(c);
           if (c) {
             cnd[count + __popcll(bal & ((1ull << lane) - 1))] = 64 * j + lane;
