@@ -193,7 +193,8 @@ struct RopeArgs {
 static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                          float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
                          int block_real, int n_prefix, int dtype, void* stream, const RopeArgs* rope = nullptr,
-                         int Lq_real = 0, int Lk_real = 0, const float* group_scale = nullptr) {
+                         int Lq_real = 0, int Lk_real = 0, const float* group_scale = nullptr,
+                         lmk::FwdParams* params_out = nullptr) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o))) return rc;
   if (L == nullptr || M == nullptr) return LMK_ERR_NULL;
@@ -230,6 +231,10 @@ static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
   p.vs_b = v->stride_b; p.vs_h = v->stride_h; p.vs_r = v->stride_row;
   p.os_b = o->stride_b; p.os_h = o->stride_h; p.os_r = o->stride_row;
   p.scale_log2 = sm_scale * 1.4426950408889634f;
+  if (params_out != nullptr) {                             // the caller launches (beside something else)
+    *params_out = p;
+    return LMK_OK;
+  }
   return lmk::launch_fwd(p, D, block, dtype, (hipStream_t)stream);
 }
 
@@ -516,7 +521,8 @@ static int retrieve_topk_check(const lmk_tensor4* q, const lmk_tensor4* kcache, 
 static int retrieve_topk_impl(bool reuse_landmark_keys, const lmk_tensor4* q, const lmk_tensor4* kcache,
                               const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
                               int64_t* idx_out, void* workspace, size_t workspace_bytes, int B, int H, int T, int S,
-                              int D, int block, int top_k, int dtype, void* stream) {
+                              int D, int block, int top_k, int dtype, void* stream,
+                              lmk::RetrParams* params_out = nullptr) {
   if (int rc = retrieve_topk_check(q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, B, H, T, S, D,
                                    block, top_k, dtype))
     return rc;
@@ -535,6 +541,10 @@ static int retrieve_topk_impl(bool reuse_landmark_keys, const lmk_tensor4* q, co
   p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
   p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
   p.cs_r = table_stride_row;
+  if (params_out != nullptr) {                             // the caller launches
+    *params_out = p;
+    return LMK_OK;
+  }
   return lmk::launch_retrieve_topk(p, D, dtype, reuse_landmark_keys, (hipStream_t)stream);
 }
 
@@ -906,6 +916,41 @@ int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, con
   if (retrieve_workspace == nullptr) return LMK_ERR_NULL;
   if (!aligned16(retrieve_workspace)) return LMK_ERR_ALIGN;
   if (retrieve_workspace_bytes < retr_layout(B, H, T, S, D, block).total) return LMK_ERR_WORKSPACE;
+  if (block == 32 && reuse_landmark_keys == 0) {
+    // The forward over the local window and the rotation of the landmark keys need nothing from each other and both
+    // stand in front of the selection and the gather; the forward alone fills a fraction of the chip (one workgroup
+    // per 256 query rows), so the two go out as one launch: window, forward || landmark keys, selection, gather.
+    int rc;
+    const int inc = S % block;
+    const AttendLayout l = attend_layout(B, H, T, S, D, block);
+    char* w = static_cast<char*>(attend_workspace);
+    const int64_t W = l.W;
+    auto win = [&](size_t off) { return lmk_tensor4{w + off, (int64_t)H * W * D, W * D, (int64_t)D}; };
+    const lmk_tensor4 q_win = win(l.q_win), k_win = win(l.k_win), v_win = win(l.v_win), o_win = win(l.o_win);
+    float* L = reinterpret_cast<float*>(w + l.L);
+    float* M = reinterpret_cast<float*>(w + l.M);
+    lmk::RetrParams pr;
+    if ((rc = retrieve_topk_impl(false, q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, retrieve_workspace,
+                                 retrieve_workspace_bytes, B, H, T, S, D, block, top_k, dtype, stream, &pr)))
+      return rc;
+    lmk::FwdParams pf;
+    if (inc) {
+      if ((rc = attn_fwd_impl(&q_win, &k_win, &v_win, &o_win, L, M, B, H, (int)W, (int)W, D, sm_scale, block, block, 0, dtype,
+                              stream, nullptr, 0, 0, nullptr, &pf)))
+        return rc;
+      if ((rc = lmk_local_window(q, kcache, vcache, k_loc, v_loc, cos_table, sin_table, table_stride_row, n_pos, &q_win,
+                                 &k_win, &v_win, B, H, T, S, D, block, dtype, stream)))
+        return rc;
+    } else if ((rc = attn_fwd_impl(q, k_loc, v_loc, &o_win, L, M, B, H, T, T, D, sm_scale, block, block, 0, dtype, stream,
+                                   nullptr, 0, 0, nullptr, &pf))) {
+      return rc;
+    }
+    if ((rc = lmk::launch_fwd32_landmark_keys(pf, pr, D, dtype, (hipStream_t)stream))) return rc;
+    if ((rc = lmk::launch_retrieve_topk(pr, D, dtype, true, (hipStream_t)stream))) return rc;   // keys are rotated already
+    const lmk_tensor4 o_loc = {w + l.o_win + (size_t)inc * D * 2, o_win.stride_b, o_win.stride_h, o_win.stride_row};
+    return lmk_gather_attend(q, kcache, vcache, idx_out, cos_table, sin_table, table_stride_row, n_pos, &o_loc, L + inc,
+                             M + inc, W, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream);
+  }
   if (int rc = retrieve_topk_impl(reuse_landmark_keys != 0, q, kcache, cos_table, sin_table, table_stride_row, n_pos,
                                   idx_out, retrieve_workspace, retrieve_workspace_bytes, B, H, T, S, D, block, top_k,
                                   dtype, stream))

@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "lmk_common.hpp"
+#include "lmk_landmark_keys.hpp"
 #include "lmk_launch.hpp"
 
 namespace lmk {
@@ -57,11 +58,11 @@ __device__ __forceinline__ void fw_wait_vmcnt() {          // s_waitcnt vmcnt(N)
 
 #define LMK_INL __attribute__((always_inline))
 
+// The whole forward of one workgroup; `bid` is its index among the forward's workgroups (the kernel's dynamic LDS
+// array is used through LDS byte addresses: it starts at 0).
 template <class T, int D>
-__global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
+__device__ __forceinline__ void fwd32_body(const FwdParams& p, const int bid_) {
   using C = Fwd32Cfg<T, D>;
-  extern __shared__ __align__(16) unsigned char smem[];   // used through LDS byte addresses (it starts at 0)
-  (void)smem;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ql = lane & 31, h = lane >> 5;
@@ -69,7 +70,7 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
   const int n_qt = (p.Lq + C::QT - 1) / C::QT;
   int bh, qtile;
   {
-    const int bid = blockIdx.x, BH = p.B * p.H;
+    const int bid = bid_, BH = p.B * p.H;
     if ((BH & 7) == 0) {                                   // all workgroups of a head on one XCD, longest first
       const int xcd = bid & 7, j = bid >> 3, ngrp = BH >> 3;
       qtile = n_qt - 1 - j / ngrp;
@@ -407,6 +408,49 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
 }
 
 #undef LMK_INL
+
+template <class T, int D>
+__global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  (void)smem;
+  fwd32_body<T, D>(p, (int)blockIdx.x);
+}
+
+// The forward over a retrieval step's local window and the rotation of the cache's landmark keys in one launch:
+// neither needs the other, the forward alone fills a fraction of the chip (one workgroup per 256 query rows), and
+// both stand in front of the selection and the gather.  Workgroups 0 .. n_fwd-1 run the forward, the rest rotate keys.
+template <class T, int D>
+__global__ __launch_bounds__(512, 2) void lmk_fwd32_landmark_keys_kernel(FwdParams pf, RetrParams pr, int n_fwd) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  (void)smem;
+  if ((int)blockIdx.x < n_fwd) fwd32_body<T, D>(pf, (int)blockIdx.x);
+  else landmark_keys_body<T, D, 512>(pr, (int)blockIdx.x - n_fwd);
+}
+
+template <class T, int D>
+static int launch_fwd32_lk_t(const FwdParams& pf, const RetrParams& pr, hipStream_t stream) {
+  using C = Fwd32Cfg<T, D>;
+  auto kern = lmk_fwd32_landmark_keys_kernel<T, D>;
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
+  const int n_fwd = ((pf.Lq + C::QT - 1) / C::QT) * pf.B * pf.H;
+  constexpr int RPW = 512 / (D / 8);
+  const int64_t lkrows = (int64_t)pr.B * pr.H * pr.num_mems;
+  const int n_lk = (int)((lkrows + RPW - 1) / RPW);
+  hipLaunchKernelGGL(kern, dim3(n_fwd + n_lk), dim3(C::NTHR), C::LDS_BYTES, stream, pf, pr, n_fwd);
+  return (int)hipGetLastError();
+}
+
+int launch_fwd32_landmark_keys(const FwdParams& pf, const RetrParams& pr, int D, int dtype, hipStream_t stream) {
+  if (dtype == LMK_DTYPE_BF16) {
+    if (D == 128) return launch_fwd32_lk_t<bf16_t, 128>(pf, pr, stream);
+    if (D == 64) return launch_fwd32_lk_t<bf16_t, 64>(pf, pr, stream);
+  } else if (dtype == LMK_DTYPE_F16) {
+    if (D == 128) return launch_fwd32_lk_t<f16_t, 128>(pf, pr, stream);
+    if (D == 64) return launch_fwd32_lk_t<f16_t, 64>(pf, pr, stream);
+  }
+  return LMK_ERR_UNSUPPORTED;
+}
 
 template <class T, int D>
 static int launch_fwd32_t(const FwdParams& p, hipStream_t stream) {

@@ -168,6 +168,8 @@ int launch_rotary(const RotaryParams& p, int D, int dtype, hipStream_t stream);
 int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landmark_keys, hipStream_t stream);
 int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream_t stream);   // one selection per head
 int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t stream);
+// block-32 forward (pf) and the rotation of the landmark keys (pr: what launch_retrieve_topk would do first) in one launch
+int launch_fwd32_landmark_keys(const FwdParams& pf, const RetrParams& pr, int D, int dtype, hipStream_t stream);
 // BS: slots per block (32, 64 or 128); p.block <= BS tokens per block in the cache
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream);
 
