@@ -203,8 +203,9 @@ int lmk_attn_bwd_group_scale(const lmk_tensor4* q, const lmk_tensor4* k, const l
  * the S - S % block tokens of the complete blocks, and the tail joins the local window of the
  * attend step (:329-342; see lmk_local_window). */
 
-/* Bytes of device workspace lmk_retrieve_topk needs: rotated landmark keys and their norms,
- * plus two fp32 planes of B*H*T*(S/block) that only lmk_retrieve_topk_shared writes. */
+/* Bytes of device workspace lmk_retrieve_topk needs: rotated landmark keys (kept in tiles of 32 keys,
+ * whole tiles per (batch, head)) and their norms, plus two fp32 planes of B*H*T*(S/block) for the
+ * per-head selections and the decode path. */
 size_t lmk_retrieve_workspace_bytes(int B, int H, int T, int S, int D, int block);
 
 /* Landmark scoring + top-k selection (llama_mem.py:344-384, aggregate=None branch).

@@ -75,7 +75,7 @@ RetrLayout retr_layout(int B, int H, int T, int S, int D, int block) {
   const size_t bh = (size_t)B * H, nm = (size_t)(S / block);
   RetrLayout l;
   l.lk_rot = 0;
-  l.lk_norm = align256(l.lk_rot + bh * nm * D * 2);
+  l.lk_norm = align256(l.lk_rot + bh * (size_t)lmk::lk_tiles((int)nm) * (size_t)lmk::lk_tile_bytes(D));   // whole tiles of 32 keys
   l.approx = align256(l.lk_norm + bh * nm * 4);
   l.exact = align256(l.approx + bh * T * nm * 4);
   l.total = align256(l.exact + bh * T * nm * 4);

@@ -19,6 +19,7 @@
 // (The reference kernel carries a running maximum and rescales per block,
 // llama/ltriton/flash_landmark_attention.py:64-76; the result is the same sum.)
 #include <type_traits>
+#include <utility>
 
 #include "lmk_common.hpp"
 #include "lmk_landmark_keys.hpp"
@@ -26,9 +27,9 @@
 
 namespace lmk {
 
-template <class T, int D>
+template <class T, int D, int NW_ = 8>
 struct Fwd32Cfg {
-  static constexpr int NW = 8;                             // waves per workgroup
+  static constexpr int NW = NW_;                           // waves per workgroup: 8, or 4 for launches that would not fill the chip
   static constexpr int NTHR = 64 * NW;
   static constexpr int QT = 32 * NW;                       // query rows per workgroup
   static constexpr int CH = D / 8;
@@ -37,12 +38,17 @@ struct Fwd32Cfg {
   static constexpr int ROWB = 2 * D;
   static constexpr int BLK_BYTES = 32 * ROWB;              // one block of K (or of V)
   static constexpr int BUF_BYTES = 2 * BLK_BYTES;          // K then V
-  static constexpr int NBUF = 4;                           // ring slots: blocks k, k+1 in use, k+2, k+3 in flight
+  // ring slots: blocks k, k+1 in use, the others in flight.  (A ring twice as deep does not help the short sequences
+  // that get the small workgroups: 12.3 -> 15.0 us for 256 rows per head, and whatever shares the launch loses LDS.)
+  static constexpr int NBUF = 4;
+  static constexpr int AHEAD = NBUF - 1;                   // a period requests the block this far in front of its own
   static constexpr int RPD = 1024 / ROWB;                  // block rows covered by one 1 KB request
   static constexpr int NREQ = 2 * (32 / RPD);              // requests per block (K and V)
   static constexpr int PER_TILE = NREQ / NW;               // requests per wave and block
+  static constexpr int WAIT_REQ = (AHEAD - 2) * PER_TILE;  // requests that may be in flight when block k+2 must have landed
   static constexpr int LM_OFF = NBUF * BUF_BYTES;          // two tiles of 32 landmark keys for the first pass
   static constexpr int LM_TILES = 2;
+  static constexpr int LM_REQ = (32 / RPD + NW - 1) / NW;  // requests per wave and landmark tile
   static constexpr int LDS_BYTES = LM_OFF + LM_TILES * BLK_BYTES;
 };
 
@@ -58,11 +64,17 @@ __device__ __forceinline__ void fw_wait_vmcnt() {          // s_waitcnt vmcnt(N)
 
 #define LMK_INL __attribute__((always_inline))
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <class F, int... R>
+__device__ __forceinline__ void fw_static_for(F&& f, std::integer_sequence<int, R...>) {
+  (f(std::integral_constant<int, R>{}), ...);
+}
+
 // The whole forward of one workgroup; `bid` is its index among the forward's workgroups (the kernel's dynamic LDS
 // array is used through LDS byte addresses: it starts at 0).
-template <class T, int D>
+template <class T, int D, int NW>
 __device__ __forceinline__ void fwd32_body(const FwdParams& p, const int bid_) {
-  using C = Fwd32Cfg<T, D>;
+  using C = Fwd32Cfg<T, D, NW>;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ql = lane & 31, h = lane >> 5;
@@ -168,19 +180,22 @@ __device__ __forceinline__ void fwd32_body(const FwdParams& p, const int bid_) {
     for (int d = 0; d < C::PER_TILE; ++d) fw_dma16(base, last ? r_vo_last[d] : r_vo[d], slot_bytes + r_lds[d]);
   };
   // first pass: tile lt holds the landmark keys (row 31) of blocks 32 lt .. 32 lt + 31, row j of the tile =
-  // block 32 lt + j, same swizzle as a K block.  Every wave issues one request per tile (with D = 64 the
-  // upper four waves repeat the lower four's, so that all waves count the same).  Only landmarks of
+  // block 32 lt + j, same swizzle as a K block.  Every wave issues LM_REQ requests per tile (with more waves than
+  // requests the upper waves repeat the lower ones', so that all waves count the same).  Only landmarks of
   // complete earlier blocks are ever used; rows past them re-read the last complete block's landmark.
   const int n_lm = min(c0 + C::NW - 1, p.Lk >> 5);          // landmarks any wave here can need: blocks 0 .. n_lm-1
   const int n_lt = (n_lm + 31) >> 5;
   auto request_lm = [&](int lt) LMK_INL {
     constexpr int per = 32 / C::RPD;
-    const int part = wave % per;
-    const int row = C::RPD * part + lane / C::CH, chp = lane % C::CH;
-    const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
-    const int blk = min(32 * lt + row, max(n_lm - 1, 0));
-    const uint32_t vo = (uint32_t)(2 * (((int64_t)blk * 32 + 31) * p.ks_r + 8 * (chp ^ f)));
-    fw_dma16(kp, vo, C::LM_OFF + (lt & 1) * C::BLK_BYTES + part * 1024);
+#pragma unroll
+    for (int i = 0; i < C::LM_REQ; ++i) {
+      const int part = (wave * C::LM_REQ + i) % per;
+      const int row = C::RPD * part + lane / C::CH, chp = lane % C::CH;
+      const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
+      const int blk = min(32 * lt + row, max(n_lm - 1, 0));
+      const uint32_t vo = (uint32_t)(2 * (((int64_t)blk * 32 + 31) * p.ks_r + 8 * (chp ^ f)));
+      fw_dma16(kp, vo, C::LM_OFF + (lt & 1) * C::BLK_BYTES + part * 1024);
+    }
   };
 
   f32x16_t acc[C::DC];
@@ -315,20 +330,20 @@ __device__ __forceinline__ void fwd32_body(const FwdParams& p, const int bid_) {
     }
   };
 
-  // ---- prologue: landmark tiles 0, 1 and blocks 0 .. 2 requested; all but block 2 must have landed
+  // ---- prologue: landmark tiles 0, 1 and blocks 0 .. NBUF-2 requested; the tiles and blocks 0, 1 must have landed
   if (n_lt > 0) request_lm(0);
   if (n_lt > 1) request_lm(1);
 #pragma unroll
-  for (int t = 0; t < C::NBUF - 1; ++t) request(t * C::BUF_BYTES, t);
-  fw_wait_vmcnt<C::PER_TILE>();
+  for (int t = 0; t < C::AHEAD; ++t) request(t * C::BUF_BYTES, t);
+  fw_wait_vmcnt<C::WAIT_REQ>();
   __syncthreads();
 
   // ---- first pass: R = max over the earlier blocks' landmark scores (log2 domain)
   {
     float mx = -1e30f;
     for (int lt = 0; lt < n_lt; ++lt) {
-      if (lt >= C::LM_TILES) {                             // requested one iteration ago, one newer request behind it
-        fw_wait_vmcnt<1>();
+      if (lt >= C::LM_TILES) {                             // requested one iteration ago, one newer tile's requests behind it
+        fw_wait_vmcnt<C::LM_REQ>();
         __syncthreads();
       }
       f32x16_t s;
@@ -356,7 +371,7 @@ __device__ __forceinline__ void fwd32_body(const FwdParams& p, const int bid_) {
     constexpr int R = decltype(Rc)::value;
     constexpr bool ALL = decltype(all)::value;
     constexpr int CUR = R * C::BUF_BYTES, NXT = ((R + 1) % C::NBUF) * C::BUF_BYTES;
-    request(((R + 3) % C::NBUF) * C::BUF_BYTES, k + 3);    // into the slot block k-1 has left
+    request(((R + C::AHEAD) % C::NBUF) * C::BUF_BYTES, k + C::AHEAD);   // into the slot block k-1 has left
     if (ALL || (waveok && k <= cblk)) {
       f32x16_t& s = (R & 1) ? sB : sA;
       f32x16_t& sn = (R & 1) ? sA : sB;
@@ -364,30 +379,21 @@ __device__ __forceinline__ void fwd32_body(const FwdParams& p, const int bid_) {
       else stage_y_diag(s);
       stage_z(CUR + C::BLK_BYTES);
     }
-    fw_wait_vmcnt<C::PER_TILE>();                          // block k+2 has landed (k+3 may be in flight)
+    fw_wait_vmcnt<C::WAIT_REQ>();                          // block k+2 has landed (the later ones may be in flight)
     __syncthreads();
   };
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
-  using I3 = std::integral_constant<int, 3>;
+  constexpr auto ring = std::make_integer_sequence<int, C::NBUF>{};
   // The blocks in front of the workgroup's first query block, in whole turns of the ring, run as straight-line
   // code without per-wave tests and their branches (a wave past the last query row computes on zero queries
-  // and stores nothing); the workgroup's own eight blocks and what is left of the turn take the general path.
-  const int n_all = min(nblk, c0) & ~3;
+  // and stores nothing); the workgroup's own blocks and what is left of the turn take the general path.
+  const int n_all = min(nblk, c0) & ~(C::NBUF - 1);
   int k = 0;
-  for (; k < n_all; k += 4) {
-    period(I0{}, k, std::true_type{});
-    period(I1{}, k + 1, std::true_type{});
-    period(I2{}, k + 2, std::true_type{});
-    period(I3{}, k + 3, std::true_type{});
-  }
-  for (; k < nblk; k += 4) {
-    period(I0{}, k, std::false_type{});
-    if (k + 1 < nblk) period(I1{}, k + 1, std::false_type{});
-    if (k + 2 < nblk) period(I2{}, k + 2, std::false_type{});
-    if (k + 3 < nblk) period(I3{}, k + 3, std::false_type{});
-  }
+  for (; k < n_all; k += C::NBUF)
+    fw_static_for([&](auto Rc) LMK_INL { period(Rc, k + decltype(Rc)::value, std::true_type{}); }, ring);
+  for (; k < nblk; k += C::NBUF)
+    fw_static_for([&](auto Rc) LMK_INL {
+      if (k + decltype(Rc)::value < nblk) period(Rc, k + decltype(Rc)::value, std::false_type{});   // uniform over the workgroup
+    }, ring);
   fw_wait_vmcnt<0>();                                      // nothing may still be writing LDS when the wave ends
 
   if (rowok) {
@@ -409,36 +415,49 @@ __device__ __forceinline__ void fwd32_body(const FwdParams& p, const int bid_) {
 
 #undef LMK_INL
 
-template <class T, int D>
-__global__ __launch_bounds__(512, 2) void lmk_fwd32_kernel(FwdParams p) {
+template <class T, int D, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void lmk_fwd32_kernel(FwdParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   (void)smem;
-  fwd32_body<T, D>(p, (int)blockIdx.x);
+  fwd32_body<T, D, NW>(p, (int)blockIdx.x);
 }
 
 // The forward over a retrieval step's local window and the rotation of the cache's landmark keys in one launch:
 // neither needs the other, the forward alone fills a fraction of the chip (one workgroup per 256 query rows), and
 // both stand in front of the selection and the gather.  Workgroups 0 .. n_fwd-1 run the forward, the rest rotate keys.
-template <class T, int D>
-__global__ __launch_bounds__(512, 2) void lmk_fwd32_landmark_keys_kernel(FwdParams pf, RetrParams pr, int n_fwd) {
+constexpr int kLkRowsPerThread = 4;   // landmark keys per thread of the workgroups that rotate them
+
+template <class T, int D, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void lmk_fwd32_landmark_keys_kernel(FwdParams pf, RetrParams pr, int n_fwd) {
   extern __shared__ __align__(16) unsigned char smem[];
   (void)smem;
-  if ((int)blockIdx.x < n_fwd) fwd32_body<T, D>(pf, (int)blockIdx.x);
-  else landmark_keys_body<T, D, 512>(pr, (int)blockIdx.x - n_fwd);
+  if ((int)blockIdx.x < n_fwd) fwd32_body<T, D, NW>(pf, (int)blockIdx.x);
+  else landmark_keys_body<T, D, 64 * NW, kLkRowsPerThread>(pr, (int)blockIdx.x - n_fwd);
 }
 
-template <class T, int D>
-static int launch_fwd32_lk_t(const FwdParams& pf, const RetrParams& pr, hipStream_t stream) {
-  using C = Fwd32Cfg<T, D>;
-  auto kern = lmk_fwd32_landmark_keys_kernel<T, D>;
+// Workgroups of 8 waves (256 query rows) share one K/V stream among the most rows; when that many rows per
+// workgroup would leave compute units without one, workgroups of 4 waves (128 rows, one wave per SIMD) are used.
+static bool fwd32_small_workgroups(const FwdParams& p) {
+  return (int64_t)((p.Lq + 255) / 256) * p.B * p.H < cu_count();
+}
+
+template <class T, int D, int NW>
+static int launch_fwd32_lk_w(const FwdParams& pf, const RetrParams& pr, hipStream_t stream) {
+  using C = Fwd32Cfg<T, D, NW>;
+  auto kern = lmk_fwd32_landmark_keys_kernel<T, D, NW>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   const int n_fwd = ((pf.Lq + C::QT - 1) / C::QT) * pf.B * pf.H;
-  constexpr int RPW = 512 / (D / 8);
+  constexpr int RPW = kLkRowsPerThread * C::NTHR / (D / 8);
   const int64_t lkrows = (int64_t)pr.B * pr.H * pr.num_mems;
   const int n_lk = (int)((lkrows + RPW - 1) / RPW);
   hipLaunchKernelGGL(kern, dim3(n_fwd + n_lk), dim3(C::NTHR), C::LDS_BYTES, stream, pf, pr, n_fwd);
   return (int)hipGetLastError();
+}
+
+template <class T, int D>
+static int launch_fwd32_lk_t(const FwdParams& pf, const RetrParams& pr, hipStream_t stream) {
+  return fwd32_small_workgroups(pf) ? launch_fwd32_lk_w<T, D, 4>(pf, pr, stream) : launch_fwd32_lk_w<T, D, 8>(pf, pr, stream);
 }
 
 int launch_fwd32_landmark_keys(const FwdParams& pf, const RetrParams& pr, int D, int dtype, hipStream_t stream) {
@@ -452,15 +471,20 @@ int launch_fwd32_landmark_keys(const FwdParams& pf, const RetrParams& pr, int D,
   return LMK_ERR_UNSUPPORTED;
 }
 
-template <class T, int D>
-static int launch_fwd32_t(const FwdParams& p, hipStream_t stream) {
-  using C = Fwd32Cfg<T, D>;
-  auto kern = lmk_fwd32_kernel<T, D>;
+template <class T, int D, int NW>
+static int launch_fwd32_w(const FwdParams& p, hipStream_t stream) {
+  using C = Fwd32Cfg<T, D, NW>;
+  auto kern = lmk_fwd32_kernel<T, D, NW>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   const int n_qt = (p.Lq + C::QT - 1) / C::QT;
   hipLaunchKernelGGL(kern, dim3(n_qt * p.B * p.H), dim3(C::NTHR), C::LDS_BYTES, stream, p);
   return (int)hipGetLastError();
+}
+
+template <class T, int D>
+static int launch_fwd32_t(const FwdParams& p, hipStream_t stream) {
+  return fwd32_small_workgroups(p) ? launch_fwd32_w<T, D, 4>(p, stream) : launch_fwd32_w<T, D, 8>(p, stream);
 }
 
 int launch_fwd32(const FwdParams& p, int D, int dtype, hipStream_t stream) {

@@ -103,6 +103,15 @@ __host__ __device__ inline int64_t handover_tiles_per_head(int64_t n_qtiles32, i
   return n_qtiles32 * (n_prefix + 1) + n_qtiles32 * (n_qtiles32 - 1) / 2;
 }
 
+// The rotated landmark keys are kept in tiles of 32 keys, 16-byte chunk c (8 head dims) of key n of the tile at byte
+// (32 c + n) * 16: every consumer gives a lane one landmark, so a wave reading chunk c of 32 or 64 consecutive
+// landmarks reads 512 contiguous bytes per tile -- as MFMA operand (lane = landmark, chunk = 8 of the 16 head dims
+// of a step) and in the sequential dot products alike.  Keys past num_mems in the last tile are never written.
+__host__ __device__ inline int64_t lk_tiles(int num_mems) { return ((int64_t)num_mems + 31) >> 5; }
+__host__ __device__ inline int64_t lk_tile_bytes(int D) { return 32 * 2 * (int64_t)D; }
+// byte offset of chunk 0 of landmark m inside one (batch, head)'s tiles; chunk c lies 512 c bytes further
+__host__ __device__ inline int64_t lk_key_offset(int m, int D) { return (int64_t)(m >> 5) * lk_tile_bytes(D) + 16 * (m & 31); }
+
 struct RetrParams {
   const void *q, *kcache, *vcache, *cos, *sin;   // q rotated; caches un-rotated; tables (n_pos, D)
   const void* o_loc;                              // attention over the local chunk (gather step)
@@ -111,7 +120,7 @@ struct RetrParams {
   void* out;
   int64_t* idx;                                   // (B, H, T, k) ascending block indices
   int64_t idx_sb, idx_sh, idx_st;                 // gather step: elements between the index rows of batches, heads, queries
-  void* lk_rot;                                   // (B*H, num_mems, D) rotated landmark keys
+  void* lk_rot;                                   // rotated landmark keys, (B*H, ceil(num_mems / 32)) tiles: see lk_tile_bytes
   float* lk_norm;                                 // (B*H, num_mems)
   float *approx, *exact;                          // (B*H*T, num_mems) each
   uint32_t* agg;                                  // (B*H, num_mems) per-head maxima of the 16-bit probabilities

@@ -81,6 +81,39 @@ __device__ __forceinline__ void wave_best(float& v, int& i) {
   i = bi;
 }
 
+// wave-wide maximum / minimum, every lane gets it (a NaN never wins against a number)
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));
+  v = fmaxf(v, dpp_f<0x4E>(v));
+  v = fmaxf(v, dpp_f<0x141>(v));
+  v = fmaxf(v, dpp_f<0x140>(v));                                  // every lane has its row's maximum
+  const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+  const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+  const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+  const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+  return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+__device__ __forceinline__ int wave_min(int v) {
+  v = min(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false));
+  v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false));
+  v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false));
+  v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, false));
+  return min(min(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+             min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+// wave-wide arg-best under (value desc, id asc) of one candidate per lane: the maximum first, the ids only where
+// several lanes hold it (seldom)
+__device__ __forceinline__ void wave_best_one(float v, int id, float& bv, int& bi) {
+  bv = wave_max(v);
+  const uint64_t eq = __ballot(v == bv);
+  if (__popcll(eq) == 1) bi = __builtin_amdgcn_readlane(id, __builtin_ctzll(eq));   // wave-uniform
+  else bi = wave_min(v == bv ? id : 0x7fffffff);                 // no lane at all (NaN everywhere): 0x7fffffff
+}
+
 // Lane j < k holds the j-th pick of a row; the k picks are written in ascending order as int64.
 // Every value is first clamped into the cache (a row whose scores are all NaN picks nothing, and a
 // pick left at its initial value must not become a block index), and equal values are ranked by
@@ -142,9 +175,8 @@ __global__ __launch_bounds__(256) void lmk_fill_u32_kernel(uint32_t* dst, int64_
 // One wave per (batch, head, query): scores -> softmax -> 16-bit probabilities -> maximum per block
 // into agg (B*H, num_mems), which holds zeros on entry.  A lane owns the blocks m = lane, lane + 64, ...;
 // the row's sum is each lane's running sum in that order, folded across lanes by halves.
-// A workgroup is four queries of one (batch, head): tiles of 128 rotated landmark keys are staged
-// through LDS with coalesced loads and shared by the four waves (a lane reading its own key row
-// straight from memory is one 64-byte request per lane and instruction); the query sits in registers.
+// A workgroup is four queries of one (batch, head): 128 rotated landmark keys at a time are staged
+// through LDS, fetched once in memory order and shared by the four waves; the query sits in registers.
 template <class T, int D>
 __global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
   constexpr int ROWB = 2 * D + 16;                                // padded key row: a 16-lane group reads 16 B each, all banks
@@ -173,14 +205,14 @@ __global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
   }
   const int64_t row = (int64_t)bh * p.T + (active ? t : 0);
   float* sc = p.approx + row * NM;                                // this row's scores, then its exponentials
-  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * NM * D);
+  const char* lk = (const char*)p.lk_rot + (int64_t)bh * lk_tiles(NM) * lk_tile_bytes(D);
 
   auto fetch = [&](int m0, u32x4_t* r) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = i * 256 + tid, kr = c / CPR, col = c % CPR;
+      const int c = i * 256 + tid;                                  // the tile's chunks in memory order: m0 is a multiple of 32
       u32x4_t z = {0, 0, 0, 0};
-      r[i] = (m0 + kr < NM) ? *(const u32x4_t*)(lk + 2 * ((int64_t)(m0 + kr) * D) + 16 * col) : z;
+      r[i] = (m0 + 32 * (c / (32 * CPR)) < NM) ? *(const u32x4_t*)(lk + lk_key_offset(m0, D) + 16 * (int64_t)c) : z;
     }
   };
   u32x4_t nxt[NCH];
@@ -190,8 +222,8 @@ __global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
     __syncthreads();                                              // the previous tile has been read by every wave
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = i * 256 + tid;
-      *(u32x4_t*)(tile + (c / CPR) * ROWB + 16 * (c % CPR)) = nxt[i];
+      const int c = i * 256 + tid, kr = 32 * (c / (32 * CPR)) + (c & 31), col = (c >> 5) % CPR;
+      *(u32x4_t*)(tile + kr * ROWB + 16 * col) = nxt[i];
     }
     __syncthreads();
     if (m0 + TM < NM) fetch(m0 + TM, nxt);                        // in flight during the arithmetic below
@@ -308,14 +340,16 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
   constexpr int NJ = kFusedMaxMems / 64;                          // scores per lane and row
   extern __shared__ __align__(16) unsigned char smem[];
   const int NMall = p.num_mems;
-  const int seg_cap = NMall < kFusedMaxMems ? NMall : kFusedMaxMems;
-  const int NMp = ((seg_cap + 63) & ~63) + 8;                     // row stride (words): the two half-waves of a store
-                                                                  // (rows 4 apart) then hit different banks
+  constexpr int NMp = kFusedMaxMems + 8;                          // row stride (words): the two half-waves of a store (rows 4
+                                                                  // apart) then hit different banks; a constant, so that the
+                                                                  // sixteen stores of a tile share their address registers
   float* sc = (float*)smem;                                       // [32][NMp]
   float* q_lds = sc + kFusedRows * NMp;                           // [waves][D]
   int* cand = (int*)(q_lds + kFusedWaves * D);                    // [waves][kFusedList]
-  unsigned char* q_raw = (unsigned char*)(cand + kFusedWaves * kFusedList);   // [32][D] in the model dtype
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  unsigned char* q_raw = (unsigned char*)(cand + kFusedWaves * kFusedList);   // [32][D] in the model dtype, rows of QROWB bytes
+  constexpr int QROWB = 2 * D + 16;                               // 16 lanes reading 16 B of 16 rows hit every bank once
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // in a scalar register: what depends on it alone is scalar too
   const int ql = lane & 31, h = lane >> 5;
   const int n_qt = (p.T + kFusedRows - 1) / kFusedRows;
   // Workgroups go to the eight XCDs in turn; the ones that read the same head's landmark keys are put on
@@ -324,16 +358,12 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
   const int bh = wg / n_qt, t0 = (wg % n_qt) * kFusedRows;
   const int b = bh / p.H, hh = bh % p.H;
   const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h);
-  const char* lk_all = (const char*)p.lk_rot + 2 * ((int64_t)bh * NMall * D);
+  const char* lk_all = (const char*)p.lk_rot + (int64_t)bh * lk_tiles(NMall) * lk_tile_bytes(D);
   const float* lkn_all = p.lk_norm + (int64_t)bh * NMall;
 
-  // ---- the 32 query rows -> LDS (the select phase reads them from there)
-  for (int c = tid; c < kFusedRows * (D / 8); c += 64 * kFusedWaves) {
-    const int r = c / (D / 8), ch = c % (D / 8);
-    u32x4_t v = {0, 0, 0, 0};
-    if (t0 + r < p.T) v = *(const u32x4_t*)(qp + 2 * ((int64_t)(t0 + r) * p.qs_r + 8 * ch));
-    *(u32x4_t*)(q_raw + r * 2 * D + 16 * ch) = v;
-  }
+  // ---- the 32 query rows -> LDS (MFMA operand of the score phase; the select phase reads them from there too):
+  // requested behind the first segment's landmark keys, so that one memory round trip lies in front of the first MFMA
+  static_assert(kFusedRows * (D / 8) <= 64 * kFusedWaves && kFusedRows * (D / 8) % 64 == 0, "one chunk of the query rows per thread, whole waves");
   // running k best of every row this wave owns (rows wave, wave + 16): lane j holds the j-th best so far
   float run_v[kFusedRows / kFusedWaves];
   int run_i[kFusedRows / kFusedWaves];
@@ -347,45 +377,58 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
   for (int seg = 0; seg < NMall; seg += kFusedMaxMems) {
     const int NM = min(NMall - seg, kFusedMaxMems);                 // landmarks of this segment
     const int NMr = (NM + 63) & ~63;                                // columns read by the select phase
-    const char* lk = lk_all + 2 * ((int64_t)seg * D);
+    const char* lk = lk_all + lk_key_offset(seg, D);                // a segment starts a tile
     const float* lkn = lkn_all + seg;
-    // ---- score: A = query rows (lane -> row), B = landmark keys (lane -> landmark)
+    float nrm[NJ];                                                  // |k_m| of this lane's landmarks, for the select phase:
+#pragma unroll                                                     // requested with the keys
+    for (int j = 0; j < NJ; ++j) {
+      const int m = 64 * j + lane;
+      nrm[j] = (m < NM) ? lkn[m] : 0.f;
+    }
+    // ---- score: A = query rows (lane -> row, from LDS), B = landmark keys (lane -> landmark).  A wave's tiles are
+    // 32 * kFusedWaves landmarks apart, at most two per segment, and both are requested before the first is used.
+    // MFMA step ks takes chunks 2 ks, 2 ks + 1 of the landmark in the lane: one load instruction reads 1 KB in a row.
     {
-      u32x4_t qf[KS];
-      const int qrow = t0 + ql;
+      constexpr int NT = kFusedMaxMems / (32 * kFusedWaves);
+      u32x4_t kf[NT][KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        u32x4_t z = {0, 0, 0, 0};
-        qf[ks] = z;
-        if (qrow < p.T) qf[ks] = *(const u32x4_t*)(qp + 2 * ((int64_t)qrow * p.qs_r + 16 * ks + 8 * h));
-      }
-      for (int m0 = 32 * wave; m0 < NMr; m0 += 32 * kFusedWaves) {
-        const int m = m0 + ql;
-        u32x4_t kf[KS];
+      for (int it = 0; it < NT; ++it) {
+        const int m0 = 32 * wave + 32 * kFusedWaves * it;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           u32x4_t z = {0, 0, 0, 0};
-          kf[ks] = z;
-          if (m < NM) kf[ks] = *(const u32x4_t*)(lk + 2 * ((int64_t)m * D + 16 * ks + 8 * h));
+          kf[it][ks] = z;
+          if (m0 < NM) kf[it][ks] = *(const u32x4_t*)(lk + lk_key_offset(m0 + ql, D) + 512 * (2 * ks + h));
         }
-        f32x16_t s;
+      }
+      if (seg == 0) {
+        if (wave < kFusedRows * (D / 8) / 64) {                     // wave-uniform
+          u32x4_t q_chunk = {0, 0, 0, 0};
+          if (t0 + tid / (D / 8) < p.T)
+            q_chunk = *(const u32x4_t*)(qp + 2 * ((int64_t)(t0 + tid / (D / 8)) * p.qs_r + 8 * (tid % (D / 8))));
+          *(u32x4_t*)(q_raw + (tid / (D / 8)) * QROWB + 16 * (tid % (D / 8))) = q_chunk;
+        }
+        __syncthreads();
+      }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+      for (int it = 0; it < NT; ++it) {
+        const int m0 = 32 * wave + 32 * kFusedWaves * it;
+        if (m0 < NMr) {                                             // wave-uniform
+          const int m = m0 + ql;
+          f32x16_t s;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = mfma32<T>(qf[ks], kf[ks], s);
+          for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sc[(8 * (r >> 2) + 4 * h + (r & 3)) * NMp + m] = (m < NM) ? s[r] : -INFINITY;
+          for (int ks = 0; ks < KS; ++ks)
+            s = mfma32<T>(*(const u32x4_t*)(q_raw + ql * QROWB + 32 * ks + 16 * h), kf[it][ks], s);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sc[(8 * (r >> 2) + 4 * h + (r & 3)) * NMp + m] = (m < NM) ? s[r] : -INFINITY;
+        }
       }
     }
     __syncthreads();
 
     // ---- select
-    float nrm[NJ];                                                  // |k_m| of this lane's landmarks
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int m = 64 * j + lane;
-      nrm[j] = (m < NM) ? lkn[m] : 0.f;
-    }
     const float sq = p.sqrt_hd, inv_sq = 1.0f / sq;
     float* qrow_lds = q_lds + wave * D;
     int* cnd = cand + wave * kFusedList;
@@ -412,19 +455,15 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
 
     // the same with one candidate (value v, index id, unique in the wave) per lane
     auto take_one = [&](float& v, int id, float& bv_out, int& bi_out) {
-      float bv = v;
-      int bi = id;
-      wave_best(bv, bi);
-      if (bi == id) v = -INFINITY;
-      bv_out = bv;
-      bi_out = bi;
+      wave_best_one(v, id, bv_out, bi_out);
+      if (bi_out == id) v = -INFINITY;
     };
 
     for (int qi = wave, ri = 0; qi < kFusedRows; qi += kFusedWaves, ++ri) {
       const int t = t0 + qi;
       if (t >= p.T) break;                                          // wave-uniform
       // q row -> fp32 in LDS (read back as a broadcast), and its norm
-      const unsigned char* qr = q_raw + qi * 2 * D;
+      const unsigned char* qr = q_raw + qi * QROWB;
       float qn = 0.f;
       for (int d = 2 * lane; d < D; d += 128) {
         const uint32_t u = *(const uint32_t*)(qr + 2 * d);
@@ -480,13 +519,13 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
         for (int c0 = 0; c0 < count; c0 += 64) {
           if (c0 + lane < count) {
             const int m = cnd[c0 + lane];
-            const char* kr = lk + 2 * ((int64_t)m * D);
+            const char* kr = lk + lk_key_offset(m, D);
             float acc = 0.f;
 #pragma unroll
             for (int g = 0; g < D / 64; ++g) {                      // 8 loads in flight, then their 64 dependent fmas
               u32x4_t kv[8];
 #pragma unroll
-              for (int i = 0; i < 8; ++i) kv[i] = *(const u32x4_t*)(kr + 16 * (8 * g + i));
+              for (int i = 0; i < 8; ++i) kv[i] = *(const u32x4_t*)(kr + 512 * (8 * g + i));
 #pragma unroll
               for (int i = 0; i < 8; ++i) {
                 const u32x4_t kk = kv[i];
@@ -622,13 +661,11 @@ constexpr int kSliceWaves = 4;
 constexpr int kSliceMems = 64 * kSliceWaves;                      // cached blocks per workgroup
 constexpr int kSliceMaxRows = 1024;                               // rows (batch x head x query) up to which this path is used
 constexpr int kSliceMaxCand = 1024;                               // candidates (slices x k) the merge holds, 16 per lane
-constexpr int kSliceRowB = 80;                                    // bytes per staged quarter row: 64 + 16, conflict-free b128 reads
 
 template <class T, int D>
 __global__ __launch_bounds__(64 * kSliceWaves) void lmk_topk_slice_kernel(RetrParams p, int n_slices) {
-  constexpr int NQ = D / 32;                                      // a key row passes through LDS in quarters of 32 dims
+  constexpr int NQ = D / 32;                                      // a key is worked on in quarters of 32 dims
   __shared__ __align__(16) float q_lds[D];
-  __shared__ __align__(16) unsigned char stage_all[kSliceWaves * 64 * kSliceRowB];
   __shared__ float list_v[kSliceWaves][64];
   __shared__ int list_i[kSliceWaves][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -638,20 +675,16 @@ __global__ __launch_bounds__(64 * kSliceWaves) void lmk_topk_slice_kernel(RetrPa
   const int bh = (int)(row / p.T), t = (int)(row % p.T);
   const int b = bh / p.H, hh = bh % p.H;
   const char* qr = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
-  const char* lk = (const char*)p.lk_rot + 2 * ((int64_t)bh * NM * D);
-  unsigned char* stage = stage_all + wave * 64 * kSliceRowB;
-  // The wave's 64 blocks (lane l scores block mw + l): the key rows come in with four lanes per row and
-  // quarter (64 contiguous bytes) and go through LDS to the lane that owns the row -- a lane reading its
-  // own 256-byte row would touch 64 cache lines per load instruction.
+  const char* lk = (const char*)p.lk_rot + (int64_t)bh * lk_tiles(NM) * lk_tile_bytes(D);
+  // The wave's 64 blocks (lane l scores block mw + l): in the tiled layout of the keys a load instruction
+  // brings one 16-byte chunk of each of them, 512 contiguous bytes per half-wave.
   const int mw = slice * kSliceMems + 64 * wave;
+  const char* kr = lk + lk_key_offset(min(mw + lane, (int)(32 * lk_tiles(NM)) - 1), D);   // past the last tile: a re-read whose score is dropped
   u32x4_t ld[NQ][4];
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int mr = min(mw + 16 * i + (lane >> 2), NM - 1);        // rows past the end re-read the last one; their score is dropped
-      ld[qt][i] = *(const u32x4_t*)(lk + 2 * ((int64_t)mr * D) + 64 * qt + 16 * (lane & 3));
-    }
+    for (int i = 0; i < 4; ++i) ld[qt][i] = *(const u32x4_t*)(kr + 512 * (4 * qt + i));
   if (tid < D / 2) {
     const uint32_t u = *(const uint32_t*)(qr + 4 * tid);
     q_lds[2 * tid] = unpack_lo<T>(u);
@@ -662,15 +695,11 @@ __global__ __launch_bounds__(64 * kSliceWaves) void lmk_topk_slice_kernel(RetrPa
   float acc = 0.f;
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *(u32x4_t*)(stage + (16 * i + (lane >> 2)) * kSliceRowB + 16 * (lane & 3)) = ld[qt][i];
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_s_waitcnt(0xc07f);
     int q0 = 0;
     asm volatile("" : "+v"(q0) : : "memory");                       // q is read from LDS quarter by quarter ...
 #pragma unroll
     for (int c = 0; c < 4; ++c) {                                   // the sequential dot product of the contract, d ascending
-      const u32x4_t kk = *(const u32x4_t*)(stage + lane * kSliceRowB + 16 * c);
+      const u32x4_t kk = ld[qt][c];
       const float4 qa = *(const float4*)&q_lds[q0 + 32 * qt + 8 * c];
       const float4 qb = *(const float4*)&q_lds[q0 + 32 * qt + 8 * c + 4];
       acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
@@ -683,9 +712,7 @@ __global__ __launch_bounds__(64 * kSliceWaves) void lmk_topk_slice_kernel(RetrPa
       acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
     }
     asm volatile("" : "+v"(acc));                                   // ... and its 32 fmas are done before the next one is read:
-                                                                    // left alone the compiler reads all of q and the keys first and spills
-    __builtin_amdgcn_wave_barrier();                                // the next quarter overwrites the rows
-    __builtin_amdgcn_s_waitcnt(0xc07f);
+                                                                    // left alone the compiler reads all of q first and spills
   }
   const int m = mw + lane;
   float cv = (m < NM) ? contract<T>(acc, p.sqrt_hd) : -INFINITY;
@@ -786,10 +813,6 @@ __global__ __launch_bounds__(256) void lmk_topk_slice_merge_kernel(RetrParams p,
 // ---------------------------------------------------------------------------
 // gather + attend over the selected blocks, merged with the local-chunk attention
 // ---------------------------------------------------------------------------
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
 __device__ __forceinline__ float sum8(float d) {                  // sum over the 8 lanes of a key group (lane & 7)
   d += dpp_f<0xB1>(d);                                            // quad_perm [1,0,3,2]
   d += dpp_f<0x4E>(d);                                            // quad_perm [2,3,0,1]
@@ -1072,10 +1095,8 @@ static int launch_topk_t(const RetrParams& p, bool reuse_landmark_keys, hipStrea
     hipLaunchKernelGGL(lmk_topk_slice_merge_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p, n_slices);
     return (int)hipGetLastError();
   }
-  const int seg_cap = p.num_mems < kFusedMaxMems ? p.num_mems : kFusedMaxMems;
-  const int NMr = (seg_cap + 63) & ~63;
-  const int lds = (kFusedRows * (NMr + 8) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
-  constexpr int lds_max = (kFusedRows * (kFusedMaxMems + 8) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * 2 * D;
+  constexpr int lds_max = (kFusedRows * (kFusedMaxMems + 8) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * (2 * D + 16);
+  constexpr int lds = lds_max;                                    // one workgroup of 16 waves per compute unit whatever it takes
   const int n_rt = (p.T + kFusedRows - 1) / kFusedRows;
   const dim3 grid(p.B * p.H * n_rt), block(64 * kFusedWaves);
   if (p.num_mems <= kFusedMaxMems) {
