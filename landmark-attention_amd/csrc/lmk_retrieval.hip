@@ -332,7 +332,7 @@ __global__ __launch_bounds__(256) void lmk_block_select_kernel(RetrParams p) {
 constexpr int kFusedMaxMems = 1024;
 constexpr int kFusedRows = 32;
 constexpr int kFusedWaves = 16;
-constexpr int kFusedList = 128;                                   // contender list per wave: flushed at 64, a ballot adds <= 64
+constexpr int kFusedList = 64;                                    // a row's contender list: what one pass of the exact evaluation takes
 
 template <class T, int D, bool SEGMENTS>
 __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrParams p) {
@@ -344,9 +344,9 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
                                                                   // apart) then hit different banks; a constant, so that the
                                                                   // sixteen stores of a tile share their address registers
   float* sc = (float*)smem;                                       // [32][NMp]
-  float* q_lds = sc + kFusedRows * NMp;                           // [waves][D]
-  int* cand = (int*)(q_lds + kFusedWaves * D);                    // [waves][kFusedList]
-  unsigned char* q_raw = (unsigned char*)(cand + kFusedWaves * kFusedList);   // [32][D] in the model dtype, rows of QROWB bytes
+  float* q_lds = sc + kFusedRows * NMp;                           // [32][D]: the query rows in fp32
+  unsigned short* cand = (unsigned short*)(q_lds + kFusedRows * D);   // [32][kFusedList]: a row's contenders (index in the segment)
+  unsigned char* q_raw = (unsigned char*)(cand + kFusedRows * kFusedList);    // [32][D] in the model dtype, rows of QROWB bytes
   constexpr int QROWB = 2 * D + 16;                               // 16 lanes reading 16 B of 16 rows hit every bank once
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // in a scalar register: what depends on it alone is scalar too
@@ -421,18 +421,29 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks)
             s = mfma32<T>(*(const u32x4_t*)(q_raw + ql * QROWB + 32 * ks + 16 * h), kf[it][ks], s);
+          // register r belongs to query row 8 (r / 4) + 4 h + r % 4: four address registers, made here and not kept,
+          // and the row within the four as the store's immediate offset (the score tile starts the LDS, at byte 0)
+          int base0 = (4 * h * NMp + m) * 4;
+          asm volatile("" : "+v"(base0));                           // opaque: what follows is computed here, each time
 #pragma unroll
-          for (int r = 0; r < 16; ++r) sc[(8 * (r >> 2) + 4 * h + (r & 3)) * NMp + m] = (m < NM) ? s[r] : -INFINITY;
+          for (int a = 0; a < 4; ++a) {
+            const int base = base0 + 8 * a * NMp * 4;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) lds_st32(base + b * NMp * 4, (m < NM) ? s[4 * a + b] : -INFINITY);
+          }
         }
       }
     }
     __syncthreads();
 
-    // ---- select
+    // ---- select.  A wave owns the rows wave and wave + 16: bracket, threshold and contender list of each, then
+    // ONE exact evaluation for the contenders of both (a lane per contender: the two short lists share a pass),
+    // then the k best of each.
     const float sq = p.sqrt_hd, inv_sq = 1.0f / sq;
-    float* qrow_lds = q_lds + wave * D;
-    int* cnd = cand + wave * kFusedList;
     const int nj = NMr >> 6;                                        // slices in use (wave-uniform)
+    constexpr int RPW = kFusedRows / kFusedWaves;
+    static_assert(RPW == 2, "two rows per wave");
+    auto row_of = [&](int ri) { return wave + kFusedWaves * ri; };
 
     // wave-wide arg-best of v[] under (value desc, index asc); the winner's slot is set to -inf
     auto take_best = [&](float* v, float& bv_out, int& bi_out) {
@@ -459,11 +470,59 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
       if (bi_out == id) v = -INFINITY;
     };
 
-    for (int qi = wave, ri = 0; qi < kFusedRows; qi += kFusedWaves, ++ri) {
-      const int t = t0 + qi;
-      if (t >= p.T) break;                                          // wave-uniform
-      // q row -> fp32 in LDS (read back as a broadcast), and its norm
+    // exact scores of the first cA contenders of row riA and the first cB of row riB, one lane per contender,
+    // written over their approximate scores
+    auto evaluate = [&](int cA, int riA, int cB, int riB) {
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);                           // this wave's LDS writes (q rows, lists) are visible
+      for (int c0 = 0; c0 < cA + cB; c0 += 64) {
+        const int c = c0 + lane;
+        if (c < cA + cB) {
+          const bool second = c >= cA;
+          const int qi = row_of(second ? riB : riA);
+          const int m = cand[qi * kFusedList + (second ? c - cA : c)];
+          const float* qrow = q_lds + qi * D;
+          const char* kr = lk + lk_key_offset(m, D);
+          float acc = 0.f;
+#pragma unroll
+          for (int g = 0; g < D / 64; ++g) {                        // 8 loads in flight, then their 64 dependent fmas
+            u32x4_t kv[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) kv[i] = *(const u32x4_t*)(kr + 512 * (8 * g + i));
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              const u32x4_t kk = kv[i];
+              const float4 qa = *(const float4*)&qrow[8 * (8 * g + i)];
+              const float4 qb = *(const float4*)&qrow[8 * (8 * g + i) + 4];
+              acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
+              acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
+              acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
+              acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
+              acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
+              acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
+              acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
+              acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
+            }
+          }
+          sc[qi * NMp + m] = contract<T>(acc, sq);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+    };
+
+    // what a row leaves for the steps behind its list: entries still in the list, whether the list was emptied
+    // on the way, the slices of this lane that hold a contender
+    int left[RPW] = {0, 0};
+    bool flushed[RPW] = {false, false};
+    uint32_t is_c[RPW] = {0u, 0u};
+#pragma unroll 1
+    for (int ri = 0; ri < RPW; ++ri) {
+      const int qi = row_of(ri);
+      if (t0 + qi >= p.T) break;                                    // wave-uniform
+      // q row -> fp32 in LDS (read back by the evaluation), and its norm
       const unsigned char* qr = q_raw + qi * QROWB;
+      float* qrow_lds = q_lds + qi * D;
       float qn = 0.f;
       for (int d = 2 * lane; d < D; d += 128) {
         const uint32_t u = *(const uint32_t*)(qr + 2 * d);
@@ -476,7 +535,7 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
       for (int m = 32; m >= 1; m >>= 1) qn += __shfl_xor(qn, m, 64);
       const float eps_q = sqrtf(qn) * 1.000001f * (1.0f / 16384.0f);
 
-      float* srow = sc + qi * NMp;
+      const float* srow = sc + qi * NMp;
       // raw bracket of the fp32 dot product: [a - e, a + e] around the MFMA score a.  The contract (round, divide,
       // round) is monotone, and so are the outward-rounded estimates T_lo / T_hi of it below, so the order
       // statistics are taken on the raw ends and only the few values that matter go through T_lo / T_hi.
@@ -511,63 +570,65 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
       // T_hi(x) >= tau needs x >= tau_raw up to the roundings of both estimates (two roundings to 8 or 11 bits
       // each, 3 % covers them; 1e-5 covers the subnormal range): everything below theta is out without being rounded
       const float theta = tau_raw - (fabsf(tau_raw) * 0.03f + 1e-5f);
-      // contenders: upper end reaches tau.  They are collected in a short list and evaluated exactly,
-      // one lane per contender, whenever the list holds a wave's worth (and at the end).
-      auto evaluate = [&](int count) {
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_s_waitcnt(0xc07f);                         // this wave's LDS writes (q row, list) are visible
-        for (int c0 = 0; c0 < count; c0 += 64) {
-          if (c0 + lane < count) {
-            const int m = cnd[c0 + lane];
-            const char* kr = lk + lk_key_offset(m, D);
-            float acc = 0.f;
-#pragma unroll
-            for (int g = 0; g < D / 64; ++g) {                      // 8 loads in flight, then their 64 dependent fmas
-              u32x4_t kv[8];
-#pragma unroll
-              for (int i = 0; i < 8; ++i) kv[i] = *(const u32x4_t*)(kr + 512 * (8 * g + i));
-#pragma unroll
-              for (int i = 0; i < 8; ++i) {
-                const u32x4_t kk = kv[i];
-                const float4 qa = *(const float4*)&qrow_lds[8 * (8 * g + i)];
-                const float4 qb = *(const float4*)&qrow_lds[8 * (8 * g + i) + 4];
-                acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
-                acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
-                acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
-                acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
-                acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
-                acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
-                acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
-                acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
-              }
-            }
-            srow[m] = contract<T>(acc, sq);
-          }
-        }
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-      };
-      uint32_t is_c = 0;
+      // contenders: upper end reaches tau.  They go into the row's list, which holds what one pass of the exact
+      // evaluation takes; the seldom row with more is evaluated here, a list at a time.
+      unsigned short* cnd = cand + qi * kFusedList;
+      uint32_t mine_c = 0;
       int count = 0;
-      bool flushed = false;                                         // wave-uniform: the list was emptied on the way
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         if (j < nj && __any(up[j] >= theta && up[j] > -INFINITY)) {   // wave-uniform: most slices hold no contender
           const bool c = up[j] >= theta && up[j] > -INFINITY && t_hi(up[j]) >= tau;
           const uint64_t bal = __ballot(c);
+          const int at = count + __popcll(bal & ((1ull << lane) - 1));
           if (c) {
-            cnd[count + __popcll(bal & ((1ull << lane) - 1))] = 64 * j + lane;
-            is_c |= 1u << j;
+            if (at < kFusedList) cnd[at] = (unsigned short)(64 * j + lane);
+            mine_c |= 1u << j;
           }
           count += __popcll(bal);
-          if (count >= 64) {                                        // wave-uniform
-            evaluate(count);
-            count = 0;
-            flushed = true;
-          }
         }
       }
-      if (count > 0) evaluate(count);
+      bool emptied = false;                                         // wave-uniform
+      if (count > kFusedList) {
+        const int total = count;
+#pragma unroll 1
+        for (int first = 0; first < total; first += kFusedList) {   // contenders first .. first + 63, in the order of above
+          __builtin_amdgcn_wave_barrier();                          // the list has been read
+          int seen = 0;
+#pragma unroll
+          for (int j = 0; j < NJ; ++j) {
+            const bool c = (mine_c >> j) & 1;
+            const uint64_t bal = __ballot(c);
+            const int at = seen + __popcll(bal & ((1ull << lane) - 1)) - first;
+            if (c && at >= 0 && at < kFusedList) cnd[at] = (unsigned short)(64 * j + lane);
+            seen += __popcll(bal);
+          }
+          evaluate(min(total - first, kFusedList), ri, 0, ri);
+        }
+        count = 0;
+        emptied = true;
+      }
+      if (ri == 0) {
+        left[0] = count;
+        flushed[0] = emptied;
+        is_c[0] = mine_c;
+      } else {
+        left[1] = count;
+        flushed[1] = emptied;
+        is_c[1] = mine_c;
+      }
+    }
+    if (left[0] + left[1] > 0) evaluate(left[0], 0, left[1], 1);
+
+#pragma unroll 1
+    for (int ri = 0; ri < RPW; ++ri) {
+      const int qi = row_of(ri);
+      const int t = t0 + qi;
+      if (t >= p.T) break;                                          // wave-uniform
+      const float* srow = sc + qi * NMp;
+      const int count = ri == 0 ? left[0] : left[1];
+      const bool emptied = ri == 0 ? flushed[0] : flushed[1];
+      const uint32_t mine_c = ri == 0 ? is_c[0] : is_c[1];
       // k best exact scores, best first, handed to `use`: in a single segment they are the row's (written
       // in ascending index order), otherwise each is inserted into the row's running list
       auto consume = [&](auto&& pick) {
@@ -581,14 +642,8 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
           }
           write_ascending(p.idx + ((int64_t)bh * p.T + t) * p.k, mine, lane, p.k, p.num_mems, p.ring_start);
         } else {
-          float rv = -INFINITY;
-          int rx = 0x7fffffff;
-#pragma unroll
-          for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
-            if (i == ri) {
-              rv = run_v[i];
-              rx = run_i[i];
-            }
+          float rv = ri == 0 ? run_v[0] : run_v[1];
+          int rx = ri == 0 ? run_i[0] : run_i[1];
           for (int j = 0; j < p.k; ++j) {
             float bv;
             int bi;
@@ -608,29 +663,29 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
               rx = bi;
             }
           }
-#pragma unroll
-          for (int i = 0; i < kFusedRows / kFusedWaves; ++i)
-            if (i == ri) {
-              run_v[i] = rv;
-              run_i[i] = rx;
-            }
+          if (ri == 0) {
+            run_v[0] = rv;
+            run_i[0] = rx;
+          } else {
+            run_v[1] = rv;
+            run_i[1] = rx;
+          }
         }
       };
-      if (!flushed) {                                               // the usual case: few contenders, still in the list
+      if (!emptied) {                                               // the usual case: few contenders, still in the list
         float cv = -INFINITY;
         int ci = 0x7fffffff;
         if (lane < count) {
-          ci = cnd[lane];
+          ci = cand[qi * kFusedList + lane];
           cv = srow[ci];
         }
         consume([&](float& bv, int& bi) { take_one(cv, ci, bv, bi); });
       } else {                                                      // exact scores picked up from the row, 16 per lane
         float x[NJ];
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) x[j] = (j < nj && ((is_c >> j) & 1)) ? srow[64 * j + lane] : -INFINITY;
+        for (int j = 0; j < NJ; ++j) x[j] = (j < nj && ((mine_c >> j) & 1)) ? srow[64 * j + lane] : -INFINITY;
         consume([&](float& bv, int& bi) { take_best(x, bv, bi); });
       }
-      __builtin_amdgcn_wave_barrier();                              // the next row reuses the q row and the list
     }
     __syncthreads();                                                // the next segment overwrites the score tile
   }
@@ -1095,7 +1150,8 @@ static int launch_topk_t(const RetrParams& p, bool reuse_landmark_keys, hipStrea
     hipLaunchKernelGGL(lmk_topk_slice_merge_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p, n_slices);
     return (int)hipGetLastError();
   }
-  constexpr int lds_max = (kFusedRows * (kFusedMaxMems + 8) + kFusedWaves * D + kFusedWaves * kFusedList) * 4 + kFusedRows * (2 * D + 16);
+  constexpr int lds_max = (kFusedRows * (kFusedMaxMems + 8) + kFusedRows * D) * 4 + kFusedRows * kFusedList * 2 + kFusedRows * (2 * D + 16);
+  static_assert(lds_max <= 160 * 1024, "the score tile, the query rows and the lists fill the LDS of a compute unit");
   constexpr int lds = lds_max;                                    // one workgroup of 16 waves per compute unit whatever it takes
   const int n_rt = (p.T + kFusedRows - 1) / kFusedRows;
   const dim3 grid(p.B * p.H * n_rt), block(64 * kFusedWaves);
