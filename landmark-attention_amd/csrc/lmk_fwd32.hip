@@ -38,8 +38,9 @@ struct Fwd32Cfg {
   static constexpr int ROWB = 2 * D;
   static constexpr int BLK_BYTES = 32 * ROWB;              // one block of K (or of V)
   static constexpr int BUF_BYTES = 2 * BLK_BYTES;          // K then V
-  // ring slots: blocks k, k+1 in use, the others in flight.  (A ring twice as deep does not help the short sequences
-  // that get the small workgroups: 12.3 -> 15.0 us for 256 rows per head, and whatever shares the launch loses LDS.)
+  // ring slots: blocks k, k+1 in use, the others in flight.  (A ring twice as deep helps neither the short sequences
+  // that get the small workgroups -- 12.3 -> 15.0 us for 256 rows per head, and whatever shares the launch loses
+  // LDS -- nor, with one barrier per two blocks, the long ones: 83.1 -> 84.1 us at B2 H32 L2048.)
   static constexpr int NBUF = 4;
   static constexpr int AHEAD = NBUF - 1;                   // a period requests the block this far in front of its own
   static constexpr int RPD = 1024 / ROWB;                  // block rows covered by one 1 KB request
