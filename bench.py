@@ -239,27 +239,33 @@ def decode_bench(n=50, warm=5):
     retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws)
     t_reuse = _time_launches(lambda: retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws,
                                                    reuse_landmark_keys=True), n, warm)
-    # the same step (selection with reused keys + attend, five launches) recorded once into a HIP graph and replayed
-    def step():
+    # the step a decode loop makes as its one host call (selection with reused keys + attend: window, forward beside
+    # the slice step of the selection, gather that merges the slices first -- three launches), eagerly and recorded
+    # once into a HIP graph and replayed; and the same work as the two separate calls above (five launches) from a graph
+    from landmark_hip.retrieval import retrieve_and_attend
+    one_call = lambda: retrieve_and_attend(q, (kc, vc), kl, vl, cos, sin, block, top_k, workspace=ws,
+                                           reuse_landmark_keys=True)
+    def two_calls():
         i = retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws, reuse_landmark_keys=True)
         return gather_attend(q, kc, vc, i, kl, vl, cos, sin, block, top_k)
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        step()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        step()
-    t_graph = _time_launches(graph.replay, n, warm)
-    # and called eagerly as the one host call a decode loop makes (selection with reused keys + attend)
-    from landmark_hip.retrieval import retrieve_and_attend
-    t_eager = _time_launches(lambda: retrieve_and_attend(q, (kc, vc), kl, vl, cos, sin, block, top_k, workspace=ws,
-                                                         reuse_landmark_keys=True), n, warm)
+    def from_graph(step):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        return _time_launches(graph.replay, n, warm)
+    t_graph = from_graph(one_call)
+    t_graph2 = from_graph(two_calls)
+    t_eager = _time_launches(one_call, n, warm)
     return {"workload": "decode: 1 new token, H32 D128, cache 32775 tok (1024 blocks of 32 + tail of 7), top-4",
             "topk_ms": t_topk, "topk_reusing_landmark_keys_ms": t_reuse, "gather_attend_ms": t_att,
-            "step_from_hip_graph_ms": t_graph, "step_eager_one_call_ms": t_eager}
+            "step_from_hip_graph_ms": t_graph, "step_eager_one_call_ms": t_eager,
+            "two_calls_from_hip_graph_ms": t_graph2}
 
 
 def side_legs(n=30, warm=5):

@@ -586,11 +586,13 @@ int lmk_retrieve_topk_static(const lmk_tensor4* q, const lmk_tensor4* kcache, co
                             LMK_STATIC_SCRATCH_BYTES, B, H, T, S, D, block, top_k, dtype, stream);
 }
 
-int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
-                      const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
-                      const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, int64_t stat_stride,
-                      const lmk_tensor4* out, int B, int H, int T, int S, int D, float sm_scale, int block, int top_k,
-                      int dtype, void* stream) {
+// `candidates`: the selection has stopped after its slice step (lmk::launch_fwd32_topk_slices) and the gather picks
+// a row's k best from what that step left, writing them to idx on the way; else idx holds the indices already.
+static int gather_attend_impl(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+                              const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
+                              const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, int64_t stat_stride,
+                              const lmk_tensor4* out, int B, int H, int T, int S, int D, float sm_scale, int block,
+                              int top_k, int dtype, void* stream, const lmk::RetrParams* candidates) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(kcache)) || (rc = check_tensor(vcache)) ||
       (rc = check_tensor(o_loc)) || (rc = check_tensor(out)))
@@ -615,7 +617,21 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
   p.outs_b = out->stride_b; p.outs_h = out->stride_h; p.outs_r = out->stride_row;
   p.cs_r = table_stride_row;
   p.scale_log2 = sm_scale * 1.4426950408889634f;
+  if (candidates != nullptr) {
+    p.merge_slices = lmk::topk_slices(*candidates);
+    p.approx = candidates->approx;
+    p.exact = candidates->exact;
+  }
   return lmk::launch_gather_attend(p, D, block, dtype, (hipStream_t)stream);
+}
+
+int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
+                      const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
+                      const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, int64_t stat_stride,
+                      const lmk_tensor4* out, int B, int H, int T, int S, int D, float sm_scale, int block, int top_k,
+                      int dtype, void* stream) {
+  return gather_attend_impl(q, kcache, vcache, idx, cos_table, sin_table, table_stride_row, n_pos, o_loc, L_loc, M_loc,
+                            stat_stride, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream, nullptr);
 }
 
 static int retrieve_topk_shared_impl(const lmk_tensor4* q, const lmk_tensor4* kcache, const void* cos_table,
@@ -916,10 +932,12 @@ int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, con
   if (retrieve_workspace == nullptr) return LMK_ERR_NULL;
   if (!aligned16(retrieve_workspace)) return LMK_ERR_ALIGN;
   if (retrieve_workspace_bytes < retr_layout(B, H, T, S, D, block).total) return LMK_ERR_WORKSPACE;
-  if (block == 32 && reuse_landmark_keys == 0) {
-    // The forward over the local window and the rotation of the landmark keys need nothing from each other and both
-    // stand in front of the selection and the gather; the forward alone fills a fraction of the chip (one workgroup
-    // per 256 query rows), so the two go out as one launch: window, forward || landmark keys, selection, gather.
+  if (block == 32) {
+    // The forward over the local window needs nothing from the selection and alone fills a fraction of the chip, so
+    // it shares a launch with a step of the selection that is as small:
+    //   many query rows   window, forward || rotation of the landmark keys, fused top-k, gather
+    //   a handful (decode) window, [rotation,] forward || slice step of the selection, gather that first picks a row's
+    //                     k best from the slices' candidates
     int rc;
     const int inc = S % block;
     const AttendLayout l = attend_layout(B, H, T, S, D, block);
@@ -945,11 +963,20 @@ int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, con
                                    nullptr, 0, 0, nullptr, &pf))) {
       return rc;
     }
-    if ((rc = lmk::launch_fwd32_landmark_keys(pf, pr, D, dtype, (hipStream_t)stream))) return rc;
-    if ((rc = lmk::launch_retrieve_topk(pr, D, dtype, true, (hipStream_t)stream))) return rc;   // keys are rotated already
+    const bool by_slices = lmk::topk_slices(pr) > 0;
+    if (by_slices) {
+      if (!reuse_landmark_keys && (rc = lmk::launch_landmark_keys(pr, D, dtype, (hipStream_t)stream))) return rc;
+      if ((rc = lmk::launch_fwd32_topk_slices(pf, pr, D, dtype, (hipStream_t)stream))) return rc;
+    } else {
+      if (reuse_landmark_keys) rc = lmk::launch_fwd(pf, D, block, dtype, (hipStream_t)stream);
+      else rc = lmk::launch_fwd32_landmark_keys(pf, pr, D, dtype, (hipStream_t)stream);
+      if (rc) return rc;
+      if ((rc = lmk::launch_retrieve_topk(pr, D, dtype, true, (hipStream_t)stream))) return rc;   // keys are rotated already
+    }
     const lmk_tensor4 o_loc = {w + l.o_win + (size_t)inc * D * 2, o_win.stride_b, o_win.stride_h, o_win.stride_row};
-    return lmk_gather_attend(q, kcache, vcache, idx_out, cos_table, sin_table, table_stride_row, n_pos, &o_loc, L + inc,
-                             M + inc, W, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream);
+    return gather_attend_impl(q, kcache, vcache, idx_out, cos_table, sin_table, table_stride_row, n_pos, &o_loc, L + inc,
+                              M + inc, W, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream,
+                              by_slices ? &pr : nullptr);
   }
   if (int rc = retrieve_topk_impl(reuse_landmark_keys != 0, q, kcache, cos_table, sin_table, table_stride_row, n_pos,
                                   idx_out, retrieve_workspace, retrieve_workspace_bytes, B, H, T, S, D, block, top_k,

@@ -24,6 +24,7 @@
 #include "lmk_common.hpp"
 #include "lmk_landmark_keys.hpp"
 #include "lmk_launch.hpp"
+#include "lmk_topk_slice.hpp"
 
 namespace lmk {
 
@@ -468,6 +469,41 @@ int launch_fwd32_landmark_keys(const FwdParams& pf, const RetrParams& pr, int D,
   } else if (dtype == LMK_DTYPE_F16) {
     if (D == 128) return launch_fwd32_lk_t<f16_t, 128>(pf, pr, stream);
     if (D == 64) return launch_fwd32_lk_t<f16_t, 64>(pf, pr, stream);
+  }
+  return LMK_ERR_UNSUPPORTED;
+}
+
+// The decode step: the forward over the local window (a row or a few per head) beside the slice step of the block
+// selection, which needs nothing from it; both are workgroups of four waves.
+template <class T, int D>
+__global__ __launch_bounds__(256, 2) void lmk_fwd32_topk_slices_kernel(FwdParams pf, RetrParams pr, int n_fwd, int n_slices) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  if ((int)blockIdx.x < n_fwd) fwd32_body<T, D, 4>(pf, (int)blockIdx.x);
+  else topk_slice_body<T, D>(pr, n_slices, (int)blockIdx.x - n_fwd, smem);
+}
+
+template <class T, int D>
+static int launch_fwd32_slices_t(const FwdParams& pf, const RetrParams& pr, hipStream_t stream) {
+  using C = Fwd32Cfg<T, D, 4>;
+  static_assert(C::NTHR == 64 * kSliceWaves && kSliceLdsBytes <= C::LDS_BYTES, "one workgroup shape for both");
+  const int n_slices = topk_slices(pr);
+  if (n_slices <= 0) return LMK_ERR_UNSUPPORTED;
+  auto kern = lmk_fwd32_topk_slices_kernel<T, D>;
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
+  const int n_fwd = ((pf.Lq + C::QT - 1) / C::QT) * pf.B * pf.H;
+  const int64_t n_sel = (int64_t)pr.B * pr.H * pr.T * n_slices;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(n_fwd + n_sel)), dim3(C::NTHR), C::LDS_BYTES, stream, pf, pr, n_fwd, n_slices);
+  return (int)hipGetLastError();
+}
+
+int launch_fwd32_topk_slices(const FwdParams& pf, const RetrParams& pr, int D, int dtype, hipStream_t stream) {
+  if (dtype == LMK_DTYPE_BF16) {
+    if (D == 128) return launch_fwd32_slices_t<bf16_t, 128>(pf, pr, stream);
+    if (D == 64) return launch_fwd32_slices_t<bf16_t, 64>(pf, pr, stream);
+  } else if (dtype == LMK_DTYPE_F16) {
+    if (D == 128) return launch_fwd32_slices_t<f16_t, 128>(pf, pr, stream);
+    if (D == 64) return launch_fwd32_slices_t<f16_t, 64>(pf, pr, stream);
   }
   return LMK_ERR_UNSUPPORTED;
 }

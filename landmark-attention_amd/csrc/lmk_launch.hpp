@@ -130,6 +130,8 @@ struct RetrParams {
   int agg_over_heads;                             // shared selection: agg is (B*T, num_mems), maxima over the heads
   int prob32;                                     // shared selection: agg holds fp32 probabilities, not 16-bit ones
   int lm_dense;                                   // kcache holds the landmark keys alone, one row per block
+  int merge_slices;                               // gather step: > 0 = approx / exact hold the candidates of so many slices per row (k each),
+                                                  // the k best of which are picked first and written to idx
   int64_t prefix_len;                             // full_len - (k + 1) * block, may be -block
   int64_t qs_b, qs_h, qs_r, kcs_b, kcs_h, kcs_r, vcs_b, vcs_h, vcs_r, cs_r;
   int64_t ols_b, ols_h, ols_r, outs_b, outs_h, outs_r;
@@ -174,11 +176,28 @@ struct PadParams {
 int launch_pad_blocks(const PadParams& p, int D, bool unpad, hipStream_t stream);
 
 int launch_rotary(const RotaryParams& p, int D, int dtype, hipStream_t stream);
+
+// Selection by slices, for a handful of query rows (decoding): a row's cached blocks are split into slices of 256
+// over as many workgroups of four waves, and a row's slices are merged afterwards.
+constexpr int kSliceWaves = 4;
+constexpr int kSliceMems = 64 * kSliceWaves;                      // cached blocks per workgroup
+constexpr int kSliceMaxRows = 1024;                               // rows (batch x head x query) up to which this path is used
+constexpr int kSliceMaxCand = 1024;                               // candidates (slices x k) the merge holds, 16 per lane
+// slices per row when launch_retrieve_topk selects that way, else 0
+inline int topk_slices(const RetrParams& p) {
+  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  const int n_slices = (p.num_mems + kSliceMems - 1) / kSliceMems;
+  return (rows <= kSliceMaxRows && (int64_t)n_slices * p.k <= kSliceMaxCand) ? n_slices : 0;
+}
 int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landmark_keys, hipStream_t stream);
 int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream_t stream);   // one selection per head
 int launch_local_window(const WindowParams& p, int D, int dtype, hipStream_t stream);
 // block-32 forward (pf) and the rotation of the landmark keys (pr: what launch_retrieve_topk would do first) in one launch
 int launch_fwd32_landmark_keys(const FwdParams& pf, const RetrParams& pr, int D, int dtype, hipStream_t stream);
+// block-32 forward (pf) and the slice step of the selection (pr, topk_slices(pr) > 0) in one launch: a row's candidates
+// are left in pr.approx / pr.exact for a gather step with merge_slices set
+int launch_fwd32_topk_slices(const FwdParams& pf, const RetrParams& pr, int D, int dtype, hipStream_t stream);
+int launch_landmark_keys(const RetrParams& p, int D, int dtype, hipStream_t stream);   // the rotation alone
 // BS: slots per block (32, 64 or 128); p.block <= BS tokens per block in the cache
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream);
 

@@ -23,6 +23,7 @@
 #include "lmk_common.hpp"
 #include "lmk_landmark_keys.hpp"
 #include "lmk_launch.hpp"
+#include "lmk_topk_slice.hpp"
 
 namespace lmk {
 
@@ -39,95 +40,6 @@ __device__ __forceinline__ u32x4_t shfl_xor4(u32x4_t v, int mask) {
 template <class T, int D>
 __global__ __launch_bounds__(256) void lmk_landmark_keys_kernel(RetrParams p) {
   landmark_keys_body<T, D, 256>(p, (int)blockIdx.x);
-}
-
-// ---------------------------------------------------------------------------
-// helpers of the selection: the rounding contract and a wave-wide arg-best
-// ---------------------------------------------------------------------------
-template <class T>
-__device__ __forceinline__ float contract(float dot, float sqrt_hd) {
-  return round_to<T>(__fdiv_rn(round_to<T>(dot), sqrt_hd));
-}
-
-// wave-wide arg-best under (value desc, index asc); every lane gets the winner.  Inside a row of 16
-// lanes the exchange partners come from DPP (no LDS round trip); the four row results are then read
-// as scalars.
-template <int CTRL>
-__device__ __forceinline__ void best_step_dpp(float& v, int& i) {
-  const float ov = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-  const int oi = __builtin_amdgcn_update_dpp(0, i, CTRL, 0xf, 0xf, false);
-  if (ov > v || (ov == v && oi < i)) {
-    v = ov;
-    i = oi;
-  }
-}
-__device__ __forceinline__ void wave_best(float& v, int& i) {
-  best_step_dpp<0xB1>(v, i);                                      // quad_perm [1,0,3,2]
-  best_step_dpp<0x4E>(v, i);                                      // quad_perm [2,3,0,1]
-  best_step_dpp<0x141>(v, i);                                     // row_half_mirror
-  best_step_dpp<0x140>(v, i);                                     // row_mirror: every lane has its row's best
-  float bv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
-  int bi = __builtin_amdgcn_readlane(i, 0);
-#pragma unroll
-  for (int r = 1; r < 4; ++r) {
-    const float ov = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16 * r));
-    const int oi = __builtin_amdgcn_readlane(i, 16 * r);
-    if (ov > bv || (ov == bv && oi < bi)) {
-      bv = ov;
-      bi = oi;
-    }
-  }
-  v = bv;
-  i = bi;
-}
-
-// wave-wide maximum / minimum, every lane gets it (a NaN never wins against a number)
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float wave_max(float v) {
-  v = fmaxf(v, dpp_f<0xB1>(v));
-  v = fmaxf(v, dpp_f<0x4E>(v));
-  v = fmaxf(v, dpp_f<0x141>(v));
-  v = fmaxf(v, dpp_f<0x140>(v));                                  // every lane has its row's maximum
-  const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
-  const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
-  const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
-  const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
-  return fmaxf(fmaxf(a, b), fmaxf(c, d));
-}
-__device__ __forceinline__ int wave_min(int v) {
-  v = min(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false));
-  v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false));
-  v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false));
-  v = min(v, __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, false));
-  return min(min(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
-             min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
-}
-// wave-wide arg-best under (value desc, id asc) of one candidate per lane: the maximum first, the ids only where
-// several lanes hold it (seldom)
-__device__ __forceinline__ void wave_best_one(float v, int id, float& bv, int& bi) {
-  bv = wave_max(v);
-  const uint64_t eq = __ballot(v == bv);
-  if (__popcll(eq) == 1) bi = __builtin_amdgcn_readlane(id, __builtin_ctzll(eq));   // wave-uniform
-  else bi = wave_min(v == bv ? id : 0x7fffffff);                 // no lane at all (NaN everywhere): 0x7fffffff
-}
-
-// Lane j < k holds the j-th pick of a row; the k picks are written in ascending order as int64.
-// Every value is first clamped into the cache (a row whose scores are all NaN picks nothing, and a
-// pick left at its initial value must not become a block index), and equal values are ranked by
-// lane, so that all k slots of the row are always written with indices the gather may follow.
-__device__ __forceinline__ void write_ascending(int64_t* row_out, int mine, int lane, int k, int num_mems, int ring_start) {
-  mine = min(max(mine, 0), num_mems - 1);
-  int age = mine - ring_start;                             // oldest block first: slot order unless the cache is a ring
-  age += age < 0 ? num_mems : 0;
-  int rank = 0;
-  for (int j = 0; j < k; ++j) {
-    const int o = __shfl(age, j, 64);
-    rank += (o < age || (o == age && j < lane)) ? 1 : 0;
-  }
-  if (lane < k) row_out[rank] = (int64_t)mine;
 }
 
 // ---------------------------------------------------------------------------
@@ -704,126 +616,12 @@ __global__ __launch_bounds__(64 * kFusedWaves) void lmk_topk_fused_kernel(RetrPa
 }
 
 // ---------------------------------------------------------------------------
-// select without the bracket, for a handful of query rows (decoding).  The fused kernel gives a
-// workgroup 32 rows and a row one wave: with one row per head fifteen of its sixteen waves idle and
-// the row's steps run one behind the other on 32 CUs.  Here a row's cached blocks are split into
-// slices of 256 over as many workgroups (one wave per SIMD, one block per thread): every score is
-// evaluated as the contract defines it (the sequential dot product of `evaluate` above), a workgroup
-// leaves its slice's k best (score, index) in the workspace, and a second small kernel merges a row's
-// slices.  Costs a launch, spreads the work over the chip.
+// select without the bracket, for a handful of query rows (decoding): see lmk_topk_slice.hpp
 // ---------------------------------------------------------------------------
-constexpr int kSliceWaves = 4;
-constexpr int kSliceMems = 64 * kSliceWaves;                      // cached blocks per workgroup
-constexpr int kSliceMaxRows = 1024;                               // rows (batch x head x query) up to which this path is used
-constexpr int kSliceMaxCand = 1024;                               // candidates (slices x k) the merge holds, 16 per lane
-
 template <class T, int D>
 __global__ __launch_bounds__(64 * kSliceWaves) void lmk_topk_slice_kernel(RetrParams p, int n_slices) {
-  constexpr int NQ = D / 32;                                      // a key is worked on in quarters of 32 dims
-  __shared__ __align__(16) float q_lds[D];
-  __shared__ float list_v[kSliceWaves][64];
-  __shared__ int list_i[kSliceWaves][64];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int NM = p.num_mems;
-  const int64_t row = blockIdx.x / n_slices;                      // (batch, head, query)
-  const int slice = blockIdx.x % n_slices;
-  const int bh = (int)(row / p.T), t = (int)(row % p.T);
-  const int b = bh / p.H, hh = bh % p.H;
-  const char* qr = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
-  const char* lk = (const char*)p.lk_rot + (int64_t)bh * lk_tiles(NM) * lk_tile_bytes(D);
-  // The wave's 64 blocks (lane l scores block mw + l): in the tiled layout of the keys a load instruction
-  // brings one 16-byte chunk of each of them, 512 contiguous bytes per half-wave.
-  const int mw = slice * kSliceMems + 64 * wave;
-  const char* kr = lk + lk_key_offset(min(mw + lane, (int)(32 * lk_tiles(NM)) - 1), D);   // past the last tile: a re-read whose score is dropped
-  u32x4_t ld[NQ][4];
-#pragma unroll
-  for (int qt = 0; qt < NQ; ++qt)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) ld[qt][i] = *(const u32x4_t*)(kr + 512 * (4 * qt + i));
-  if (tid < D / 2) {
-    const uint32_t u = *(const uint32_t*)(qr + 4 * tid);
-    q_lds[2 * tid] = unpack_lo<T>(u);
-    q_lds[2 * tid + 1] = unpack_hi<T>(u);
-  }
-  __syncthreads();
-
-  float acc = 0.f;
-#pragma unroll
-  for (int qt = 0; qt < NQ; ++qt) {
-    int q0 = 0;
-    asm volatile("" : "+v"(q0) : : "memory");                       // q is read from LDS quarter by quarter ...
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {                                   // the sequential dot product of the contract, d ascending
-      const u32x4_t kk = ld[qt][c];
-      const float4 qa = *(const float4*)&q_lds[q0 + 32 * qt + 8 * c];
-      const float4 qb = *(const float4*)&q_lds[q0 + 32 * qt + 8 * c + 4];
-      acc = __builtin_fmaf(qa.x, unpack_lo<T>(kk[0]), acc);
-      acc = __builtin_fmaf(qa.y, unpack_hi<T>(kk[0]), acc);
-      acc = __builtin_fmaf(qa.z, unpack_lo<T>(kk[1]), acc);
-      acc = __builtin_fmaf(qa.w, unpack_hi<T>(kk[1]), acc);
-      acc = __builtin_fmaf(qb.x, unpack_lo<T>(kk[2]), acc);
-      acc = __builtin_fmaf(qb.y, unpack_hi<T>(kk[2]), acc);
-      acc = __builtin_fmaf(qb.z, unpack_lo<T>(kk[3]), acc);
-      acc = __builtin_fmaf(qb.w, unpack_hi<T>(kk[3]), acc);
-    }
-    asm volatile("" : "+v"(acc));                                   // ... and its 32 fmas are done before the next one is read:
-                                                                    // left alone the compiler reads all of q first and spills
-  }
-  const int m = mw + lane;
-  float cv = (m < NM) ? contract<T>(acc, p.sqrt_hd) : -INFINITY;
-  int ci = (m < NM) ? m : 0x7fffffff;
-  // lane j <- the j-th best of the wave's 64 scores
-  float rv = -INFINITY;
-  int rx = 0x7fffffff;
-  for (int j = 0; j < p.k; ++j) {
-    float bv = cv;
-    int bi = ci;
-    wave_best(bv, bi);
-    if (bi == ci) cv = -INFINITY;
-    if (lane == j) {
-      rv = bv;
-      rx = bi;
-    }
-  }
-  list_v[wave][lane] = rv;
-  list_i[wave][lane] = rx;
-  __syncthreads();
-  if (wave != 0) return;
-
-  // lane j holds the j-th entry of every wave's list; k picks over the lists, pick j -> candidate j of the slice
-  float x[kSliceWaves];
-  int xi[kSliceWaves];
-#pragma unroll
-  for (int w = 0; w < kSliceWaves; ++w) {
-    x[w] = list_v[w][lane];
-    xi[w] = list_i[w][lane];
-  }
-  float out_v = -INFINITY;
-  int out_i = 0x7fffffff;
-  for (int j = 0; j < p.k; ++j) {
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-#pragma unroll
-    for (int w = 0; w < kSliceWaves; ++w)
-      if (x[w] > bv || (x[w] == bv && xi[w] < bi)) {
-        bv = x[w];
-        bi = xi[w];
-      }
-    const int own = bi;                                             // block indices are unique over the lists
-    wave_best(bv, bi);
-#pragma unroll
-    for (int w = 0; w < kSliceWaves; ++w)
-      if (own == bi && xi[w] == bi) x[w] = -INFINITY;
-    if (lane == j) {
-      out_v = bv;
-      out_i = bi;
-    }
-  }
-  if (lane < p.k) {
-    const int64_t at = row * NM + (int64_t)slice * p.k + lane;      // n_slices * k <= num_mems: a row of the score planes holds them
-    p.approx[at] = out_v;
-    ((int*)p.exact)[at] = out_i;
-  }
+  __shared__ __align__(16) unsigned char lds[kSliceLdsBytes];
+  topk_slice_body<T, D>(p, n_slices, (int)blockIdx.x, lds);
 }
 
 // One wave per query row: the k best of the row's n_slices * k candidates, written in ascending index order.
@@ -831,37 +629,7 @@ __global__ __launch_bounds__(256) void lmk_topk_slice_merge_kernel(RetrParams p,
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= (int64_t)p.B * p.H * p.T) return;                      // wave-uniform
-  const int n_cand = n_slices * p.k;
-  constexpr int NJ = kSliceMaxCand / 64;
-  float x[NJ];
-  int xi[NJ];
-#pragma unroll
-  for (int j = 0; j < NJ; ++j) {
-    const int c = 64 * j + lane;
-    x[j] = -INFINITY;
-    xi[j] = 0x7fffffff;
-    if (c < n_cand) {
-      x[j] = p.approx[row * p.num_mems + c];
-      xi[j] = ((const int*)p.exact)[row * p.num_mems + c];
-    }
-  }
-  int mine = 0x7fffffff;
-  for (int j = 0; j < p.k; ++j) {
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-#pragma unroll
-    for (int w = 0; w < NJ; ++w)
-      if (x[w] > bv || (x[w] == bv && xi[w] < bi)) {
-        bv = x[w];
-        bi = xi[w];
-      }
-    const int own = bi;
-    wave_best(bv, bi);
-#pragma unroll
-    for (int w = 0; w < NJ; ++w)
-      if (own == bi && xi[w] == bi) x[w] = -INFINITY;
-    if (lane == j) mine = bi;
-  }
+  const int mine = merge_slices_row(p, n_slices, row, lane);
   write_ascending(p.idx + row * p.k, mine, lane, p.k, p.num_mems, p.ring_start);
 }
 
@@ -936,6 +704,20 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     return slot == BS - 1 ? nreal - 1 : min(slot, nreal - 2);
   };
   const int64_t* idx_row = p.idx + (b * p.idx_sb + hh * p.idx_sh + (int64_t)t * p.idx_st);
+  // The decode-time selection leaves a row's candidates (k per slice of the cache) rather than its indices: the wave
+  // picks the k best first -- lane r of `sorted` gets the r-th block in the order of the output -- and one wave per
+  // row writes them where the caller expects the indices.
+  const bool merged = p.merge_slices > 0;                          // uniform over the launch
+  int sorted = 0;
+  if (merged) {
+    int mine = merge_slices_row(p, p.merge_slices, row, lane);
+    const int rank = rank_ascending(mine, lane, p.k, p.num_mems, p.ring_start);
+    sorted = __builtin_amdgcn_ds_permute(4 * (lane < p.k ? rank : lane), mine);
+    if (lane < p.k && (!SPLIT || wave == 0)) p.idx[b * p.idx_sb + hh * p.idx_sh + (int64_t)t * p.idx_st + rank] = (int64_t)mine;
+  }
+  auto picked = [&](int js) {                                      // idx is a caller's array: never read outside the cache
+    return merged ? __shfl(sorted, js, 64) : min(max((int)idx_row[js], 0), p.num_mems - 1);
+  };
   auto newest = [&](int blk) {                                    // one of the k newest blocks: its keys sit one block further on
     int age = blk - p.ring_start;
     age += age < 0 ? p.num_mems : 0;
@@ -969,7 +751,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   };
   int blk = 0;
   if (js0 < p.k) {
-    blk = min(max((int)idx_row[js0], 0), p.num_mems - 1);      // idx is a caller's array: never read outside the cache
+    blk = picked(js0);
     fetch(kc, p.kcs_r, (int64_t)blk * nreal, 0);
   }
   for (int js = js0; js < p.k; js += jstep) {
@@ -1038,7 +820,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       ahi[e] *= alpha;
     }
     int blk_next = blk;
-    if (js + jstep < p.k) blk_next = min(max((int)idx_row[js + jstep], 0), p.num_mems - 1);
+    if (js + jstep < p.k) blk_next = picked(js + jstep);
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       take();
@@ -1143,8 +925,8 @@ static int launch_topk_t(const RetrParams& p, bool reuse_landmark_keys, hipStrea
     if ((rc = (int)hipGetLastError())) return rc;
   }
   const int64_t rows = (int64_t)p.B * p.H * p.T;
-  const int n_slices = (p.num_mems + kSliceMems - 1) / kSliceMems;
-  if (rows <= kSliceMaxRows && (int64_t)n_slices * p.k <= kSliceMaxCand) {   // a handful of rows: every score exact, slices over the chip
+  const int n_slices = topk_slices(p);
+  if (n_slices > 0) {                                               // a handful of rows: every score exact, slices over the chip
     hipLaunchKernelGGL((lmk_topk_slice_kernel<T, D>), dim3((unsigned)(rows * n_slices)), dim3(64 * kSliceWaves), 0, stream, p, n_slices);
     if ((rc = (int)hipGetLastError())) return rc;
     hipLaunchKernelGGL(lmk_topk_slice_merge_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p, n_slices);
@@ -1193,6 +975,25 @@ int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream
   } else if (dtype == LMK_DTYPE_F16) {
     if (D == 128) return launch_topk_shared_t<f16_t, 128>(p, stream);
     if (D == 64) return launch_topk_shared_t<f16_t, 64>(p, stream);
+  }
+  return LMK_ERR_UNSUPPORTED;
+}
+
+template <class T, int D>
+static int launch_lk_t(const RetrParams& p, hipStream_t stream) {
+  constexpr int RPW = 256 / (D / 8);
+  const int64_t lkrows = (int64_t)p.B * p.H * p.num_mems;
+  hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+int launch_landmark_keys(const RetrParams& p, int D, int dtype, hipStream_t stream) {
+  if (dtype == LMK_DTYPE_BF16) {
+    if (D == 128) return launch_lk_t<bf16_t, 128>(p, stream);
+    if (D == 64) return launch_lk_t<bf16_t, 64>(p, stream);
+  } else if (dtype == LMK_DTYPE_F16) {
+    if (D == 128) return launch_lk_t<f16_t, 128>(p, stream);
+    if (D == 64) return launch_lk_t<f16_t, 64>(p, stream);
   }
   return LMK_ERR_UNSUPPORTED;
 }
