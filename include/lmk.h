@@ -278,7 +278,10 @@ int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor
 
 /* One inference step of the mem-cache path in one call: lmk_retrieve_topk (or lmk_retrieve_topk_reuse
  * when reuse_landmark_keys != 0) followed by lmk_attend on the indices it wrote -- llama_mem.py:321-412
- * and :447-477.  Same results as the two calls; idx_out (B,H,T,k) int64 is an output. */
+ * and :447-477.  Same results as the two calls; idx_out (B,H,T,k) int64 is an output.  With blocks of 32 the
+ * call takes fewer launches than the two: the forward over the local window shares one with a step of the
+ * selection (the rotation of the landmark keys when there are many query rows; the slice step when there are a
+ * handful, as in decoding, in which case the gather picks a row's k best from the slices' candidates itself). */
 int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,
                             const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table,
                             const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,

@@ -335,3 +335,24 @@ def test_gather_clamps_indices_outside_the_cache():
     torch.cuda.synchronize()
     assert torch.isfinite(got.float()).all()
     assert torch.equal(got, want)
+
+
+# The one-call step of a decode loop runs the selection's slice step beside the local forward and lets the gather
+# pick a row's k best from the slices' candidates; the separate calls run slice step, merge and gather as three
+# launches.  Same indices, same output bits -- with a candidate per lane (<= 64) and with several per lane.
+@pytest.mark.parametrize("n_mems,inc,T,top_k,reuse", [(1024, 7, 1, 4, True), (1024, 0, 3, 32, False),
+                                                      (700, 31, 1, 40, True), (40, 5, 2, 4, False)])
+def test_one_call_decode_step_equals_the_separate_calls(n_mems, inc, T, top_k, reuse):
+    from landmark_hip import _lib
+    from landmark_hip.retrieval import gather_attend, retrieve_and_attend, retrieve_topk
+    B, H, D, block = 1, 3, 128, 32
+    S = n_mems * block + inc
+    print(f"case one-call n_mems{n_mems} inc{inc} T{T} k{top_k} reuse{reuse}", flush=True)
+    q, kc, vc, kl, vl, cos, sin = (t.cuda() for t in _inputs(B, H, T, S, D, seed=n_mems + top_k))
+    ws = torch.empty(_lib.lib().lmk_retrieve_workspace_bytes(B, H, T, S, D, block), device="cuda", dtype=torch.uint8)
+    idx2 = retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws)
+    out2 = gather_attend(q, kc, vc, idx2, kl, vl, cos, sin, block, top_k)
+    out1, idx1 = retrieve_and_attend(q, (kc, vc), kl, vl, cos, sin, block, top_k, workspace=ws, reuse_landmark_keys=reuse)
+    torch.cuda.synchronize()
+    assert torch.equal(idx1, idx2)
+    assert torch.equal(out1.view(torch.int16), out2.view(torch.int16))
