@@ -181,13 +181,15 @@ int launch_rotary(const RotaryParams& p, int D, int dtype, hipStream_t stream);
 // over as many workgroups of four waves, and a row's slices are merged afterwards.
 constexpr int kSliceWaves = 4;
 constexpr int kSliceMems = 64 * kSliceWaves;                      // cached blocks per workgroup
-constexpr int kSliceMaxRows = 1024;                               // rows (batch x head x query) up to which this path is used
+constexpr int kSliceMaxRows = 1024;                               // rows (batch x head x query) up to which this path is used,
+constexpr int kSliceMaxRowsPerHead = 4;                           // or queries per (batch, head): the other path works on 32 at a time
 constexpr int kSliceMaxCand = 1024;                               // candidates (slices x k) the merge holds, 16 per lane
 // slices per row when launch_retrieve_topk selects that way, else 0
 inline int topk_slices(const RetrParams& p) {
   const int64_t rows = (int64_t)p.B * p.H * p.T;
   const int n_slices = (p.num_mems + kSliceMems - 1) / kSliceMems;
-  return (rows <= kSliceMaxRows && (int64_t)n_slices * p.k <= kSliceMaxCand) ? n_slices : 0;
+  const bool few = rows <= kSliceMaxRows || (p.T <= kSliceMaxRowsPerHead && rows * n_slices < ((int64_t)1 << 30));
+  return (few && (int64_t)n_slices * p.k <= kSliceMaxCand) ? n_slices : 0;
 }
 int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landmark_keys, hipStream_t stream);
 int launch_retrieve_topk_shared(const RetrParams& p, int D, int dtype, hipStream_t stream);   // one selection per head

@@ -32,6 +32,8 @@ CASES = [
     (1, 2, 1, 3000 * 32, 64, 32, 4),       # one query against a long cache
     (1, 2, 3, 1024 * 32, 128, 32, 64),     # few rows: four slices of 256 blocks, 256 candidates to merge
     (1, 1, 5, 4100 * 16, 128, 16, 60),     # few rows, 17 slices x 60 > 1024 candidates: back on the fused kernel
+    (36, 32, 1, 20 * 32, 128, 32, 4),      # batched decoding: more than 1024 rows but one per head: still by slices
+    (20, 32, 2, 300 * 32, 64, 32, 5),      # two per head, two slices
     # more than 1024 query rows (B * H * T): the fused score + select kernel
     (1, 2, 530, 33 * 32, 128, 32, 1),
     (2, 3, 200, 20 * 32, 128, 32, 5),
