@@ -337,7 +337,34 @@ def side_legs(n=30, warm=5):
         return out
     t_off_chunk = _time_launches(lambda: offloaded(T), n, warm)
     t_off_token = _time_launches(lambda: offloaded(1), n, warm)
-    return {"offloaded_cache": {"workload": "config 4's cache in pinned host memory (zero-copy reads of the selected blocks), "
+    # the benchmark's ring cache (lm_benchmark: 40 slots of 51 tokens, 12 heads of 64, chunk of 250 queries, top-4,
+    # cache filled past its capacity with a tail of 13 tokens): MemLMCacheStorage.attend = selection over the ring,
+    # forward over [tail ; chunk], gather + attend over the picked blocks, for the three selection methods
+    from landmark_hip.mem_cache import MemLMCacheStorage
+    rB, cap, freq, nh, hs, rk, rT = 2, 40, 50, 12, 64, 4, 250
+    rblock = freq + 1
+    ring_ms = {}
+    for method in ("per_token_and_head", "max_over_heads", "max_over_tokens"):
+        st = MemLMCacheStorage(rB, cap, freq, nh, hs, dtype=torch.bfloat16, device=dev, cache_topk=rk,
+                               cache_selection_method=method)
+        n_tok = rblock * 64 + 13
+        kk = (torch.randn(rB, nh, n_tok, hs, generator=g) * 0.5).bfloat16().to(dev)
+        vv = (torch.randn(rB, nh, n_tok, hs, generator=g) * 0.5).bfloat16().to(dev)
+        im = (torch.arange(n_tok) % rblock == rblock - 1)[None].expand(rB, n_tok).to(dev)
+        st.store_in_cache(kk, {"v": vv, "is_mem": im})
+        start = (rk + 1) * rblock + st.last_incomplete_len
+        rinv = 1.0 / (10000 ** (torch.arange(0, hs, 2).float() / hs))
+        rang = torch.outer(torch.arange(start + rT).float(), rinv)
+        rang = torch.cat((rang, rang), -1)
+        rcos, rsin = rang.cos().bfloat16().to(dev), rang.sin().bfloat16().to(dev)
+        rq, rkk, rv = ((torch.randn(rB, nh, rT, hs, generator=g) * 0.5).bfloat16().to(dev) for _ in range(3))
+        rim = ((torch.arange(rT) + st.last_incomplete_len) % rblock == rblock - 1)[None].expand(rB, rT).to(dev)
+        with torch.no_grad():
+            ring_ms[method] = _time_launches(lambda: st.attend(rq, rkk, rv, rim, rcos, rsin, start), n, warm)
+    return {"ring_cache": {"workload": "lm_benchmark's cache: 40 slots of 51 tokens, 12 heads of 64, B2, 250 queries, top-4; "
+                                       "MemLMCacheStorage.attend (selection + local forward + gather) per selection method",
+                           "attend_ms": ring_ms},
+            "offloaded_cache": {"workload": "config 4's cache in pinned host memory (zero-copy reads of the selected blocks), "
                                             "one selection per head; 256 queries / 1 query", "chunk_step_ms": t_off_chunk,
                                 "token_step_ms": t_off_token},
             "config0_on_hip": {"workload": "benchmark config 0 (B2 H8 L510 D128, block 51) in bf16, blocks of 51 tokens worked on in 64 slots and read in place",

@@ -351,6 +351,17 @@ int lmk_local_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_
                      int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win, const lmk_tensor4* k_win,
                      const lmk_tensor4* v_win, int B, int H, int T, int S, int D, int block, int dtype, void* stream);
 
+/* The same window for the ring cache of lm_benchmark, whose incomplete last block lives outside the ring
+ * (last_incomplete_k / last_incomplete_v, lm_benchmark/models/caches/mem_cache.py:43-46, 99-103): the first
+ * `tail` rows of k_tail (without positions) are rotated at positions tail_position .. tail_position + tail - 1
+ * and put in front of the chunk's keys; v_win = [tail values ; v_loc]; q_win = [tail zero rows ; q].
+ * Each window is (B,H,tail+T,D); tail > 0. */
+int lmk_ring_local_window(const lmk_tensor4* q, const lmk_tensor4* k_tail, const lmk_tensor4* v_tail,
+                          const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table,
+                          const void* sin_table, int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win,
+                          const lmk_tensor4* k_win, const lmk_tensor4* v_win, int B, int H, int T, int tail,
+                          int64_t tail_position, int D, int dtype, void* stream);
+
 /* Landmark scoring + ONE selection per (batch, head), shared by all T queries: the branch
  * `aggregate == "max_over_tokens"` of llama_mem.py:369-384, which the reference takes when the cache
  * is offloaded to the CPU (:369-370).  Per query: scores as in lmk_retrieve_topk, fp32 softmax over

@@ -127,6 +127,7 @@ int window_impl(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tenso
   p.q_win = q_win ? q_win->ptr : nullptr; p.k_win = k_win->ptr; p.v_win = v_win->ptr;
   p.B = B; p.H = H; p.T = T; p.inc = inc;
   p.full_len = (int64_t)S - inc;
+  p.tail_pos = p.full_len;
   p.block = block;
   p.num_mems = S / block;
   if (idx != nullptr) {
@@ -778,6 +779,42 @@ int lmk_local_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_
   if (q_win == nullptr) return LMK_ERR_NULL;
   return window_impl(q, kcache, vcache, nullptr, k_loc, v_loc, cos_table, sin_table, table_stride_row, n_pos, q_win,
                      k_win, v_win, B, H, T, S, D, block, 1, dtype, stream);
+}
+
+int lmk_ring_local_window(const lmk_tensor4* q, const lmk_tensor4* k_tail, const lmk_tensor4* v_tail,
+                          const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table,
+                          const void* sin_table, int64_t table_stride_row, int64_t n_pos, const lmk_tensor4* q_win,
+                          const lmk_tensor4* k_win, const lmk_tensor4* v_win, int B, int H, int T, int tail,
+                          int64_t tail_position, int D, int dtype, void* stream) {
+  int rc;
+  if ((rc = check_tensor(q)) || (rc = check_tensor(k_tail)) || (rc = check_tensor(v_tail)) ||
+      (rc = check_tensor(k_loc)) || (rc = check_tensor(v_loc)) || (rc = check_tensor(q_win)) ||
+      (rc = check_tensor(k_win)) || (rc = check_tensor(v_win)))
+    return rc;
+  if (cos_table == nullptr || sin_table == nullptr) return LMK_ERR_NULL;
+  if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
+  if (B <= 0 || H <= 0 || T <= 0 || tail <= 0) return LMK_ERR_SHAPE;
+  if (!(D == 64 || D == 128)) return LMK_ERR_UNSUPPORTED;
+  if (!(dtype == LMK_DTYPE_BF16 || dtype == LMK_DTYPE_F16)) return LMK_ERR_UNSUPPORTED;
+  if (tail_position < 0 || tail_position + tail > n_pos) return LMK_ERR_TABLE;
+  lmk::WindowParams p = {};
+  p.q = q->ptr; p.kcache = k_tail->ptr; p.vcache = v_tail->ptr; p.k_loc = k_loc->ptr; p.v_loc = v_loc->ptr;
+  p.cos = cos_table; p.sin = sin_table;
+  p.q_win = q_win->ptr; p.k_win = k_win->ptr; p.v_win = v_win->ptr;
+  p.B = B; p.H = H; p.T = T; p.inc = tail;
+  p.full_len = 0;                                          // the tail's rows are rows 0 .. tail-1 of k_tail, v_tail
+  p.tail_pos = tail_position;
+  p.block = 1; p.num_mems = 0;
+  p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
+  p.kcs_b = k_tail->stride_b; p.kcs_h = k_tail->stride_h; p.kcs_r = k_tail->stride_row;
+  p.vcs_b = v_tail->stride_b; p.vcs_h = v_tail->stride_h; p.vcs_r = v_tail->stride_row;
+  p.kls_b = k_loc->stride_b; p.kls_h = k_loc->stride_h; p.kls_r = k_loc->stride_row;
+  p.vls_b = v_loc->stride_b; p.vls_h = v_loc->stride_h; p.vls_r = v_loc->stride_row;
+  p.qws_b = q_win->stride_b; p.qws_h = q_win->stride_h; p.qws_r = q_win->stride_row;
+  p.kws_b = k_win->stride_b; p.kws_h = k_win->stride_h; p.kws_r = k_win->stride_row;
+  p.vws_b = v_win->stride_b; p.vws_h = v_win->stride_h; p.vws_r = v_win->stride_row;
+  p.cs_r = table_stride_row;
+  return lmk::launch_local_window(p, D, dtype, (hipStream_t)stream);
 }
 
 int lmk_gather_window(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,

@@ -147,7 +147,8 @@ struct WindowParams {
   int B, H, T, inc;
   int n_sel, k, block, num_mems;                  // n_sel = k * block rows of selected blocks in front, or 0
   int64_t prefix_len;
-  int64_t full_len;                               // first cached row of the tail = its rotary position
+  int64_t full_len;                               // first cached row of the tail
+  int64_t tail_pos;                               // its rotary position (the same number in the llama cache)
   int64_t qs_b, qs_h, qs_r, kcs_b, kcs_h, kcs_r, vcs_b, vcs_h, vcs_r, kls_b, kls_h, kls_r, vls_b, vls_h, vls_r;
   int64_t qws_b, qws_h, qws_r, kws_b, kws_h, kws_r, vws_b, vws_h, vws_r, cs_r;
 };

@@ -1066,7 +1066,8 @@ __global__ __launch_bounds__(256) void lmk_local_window_kernel(WindowParams p) {
       src_row = blk * p.block + tok;
       pos = (int64_t)r + (blk >= p.num_mems - p.k ? p.block : 0) + p.prefix_len;   // llama_mem.py:386-388
     } else {
-      src_row = pos = p.full_len + (r - p.n_sel);
+      src_row = p.full_len + (r - p.n_sel);
+      pos = p.tail_pos + (r - p.n_sel);
     }
     const char* src = (const char*)p.kcache + 2 * (b * p.kcs_b + hh * p.kcs_h + src_row * p.kcs_r);
     const u32x4_t x = *(const u32x4_t*)(src + 16 * j);

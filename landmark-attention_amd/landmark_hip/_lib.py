@@ -107,6 +107,8 @@ def lib() -> ctypes.CDLL:
                                               i, i, i, i, i, f, i, i, i, vp]
         L.lmk_local_window.restype = i
         L.lmk_local_window.argtypes = [T4, T4, T4, T4, T4, vp, vp, i64, i64, T4, T4, T4, i, i, i, i, i, i, i, vp]
+        L.lmk_ring_local_window.restype = i
+        L.lmk_ring_local_window.argtypes = [T4, T4, T4, T4, T4, vp, vp, i64, i64, T4, T4, T4, i, i, i, i, i64, i, i, vp]
         L.lmk_retrieve_topk_shared.restype = i
         L.lmk_retrieve_topk_shared.argtypes = [T4, T4, vp, vp, i64, i64, vp, vp, vp, sz, i, i, i, i, i, i, i, i, vp]
         L.lmk_retrieve_topk_shared_landmarks.restype = i

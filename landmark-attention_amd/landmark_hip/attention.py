@@ -232,16 +232,17 @@ _VALIDATED_MASKS: dict = {}
 _VALIDATED_MASKS_MAX = 64
 
 
-def _check_is_mem(is_mem, block_size):
+def _check_is_mem(is_mem, block_size, offset=0):
+    # offset: tokens of the first block that lie in front of the mask (a stream cut between two landmarks)
     # tensors created under torch.inference_mode() track no version counter (reading it raises): they are checked
     # on every call rather than cached
     cacheable = not is_mem.is_inference()
     if cacheable:
         key = (is_mem.device, is_mem.data_ptr(), is_mem._version, tuple(is_mem.shape), tuple(is_mem.stride()),
-               is_mem.dtype, int(block_size))
+               is_mem.dtype, int(block_size), int(offset))
         if key in _VALIDATED_MASKS:
             return
-    expected_is_mem = torch.arange(0, is_mem.shape[-1], device=is_mem.device) % block_size == (block_size - 1)
+    expected_is_mem = (torch.arange(0, is_mem.shape[-1], device=is_mem.device) + offset) % block_size == (block_size - 1)
     assert (is_mem == expected_is_mem).all(), (
         f"is_mem must mark exactly the last token of every block of {block_size}: irregular landmark positions "
         "and dropped landmarks are not covered by the fused kernels")

@@ -148,25 +148,30 @@ class MemLMCacheStorage:
         Returns ``(y (B, nh, T, hs), slots)``: y is ``att @ v + att_prefix @ cache_v`` (``:235-240``), slots the
         picked blocks in the shape of ``select_blocks`` (None while the cache holds no block or ``cache_topk`` is 0,
         ``:48-49``).  Call ``store_in_cache`` afterwards, as the layer does (``:246-248``)."""
-        from .attention import _launch_fwd_blocks
-        from .rotary import _rotate
+        from .attention import _check_is_mem, _launch_fwd_blocks
         import math
         B, nh, T, hs = q.shape
         block, tail = self.block, self.last_incomplete_len
         assert q.dtype == self.cache_mem_k.dtype and q.is_cuda and k.shape == v.shape == q.shape
-        expected = (torch.arange(T, device=q.device) + tail) % block == block - 1
-        assert bool((is_mem == expected).all()), "is_mem must continue the stream: a landmark closes every block"
+        # is_mem must continue the stream (a landmark closes every block); the check costs a device->host sync, paid
+        # once per mask tensor state and tail length, not per call
+        _check_is_mem(is_mem, block, offset=tail)
         if sm_scale is None:
             sm_scale = 1.0 / math.sqrt(hs)
         cos, sin = _tables(cos, sin, q.dtype)
         if tail:
             # the tokens behind the last complete block open the chunk's first block (:43-46): their keys rotated at
-            # start_index - tail .., zero rows standing in for their queries
-            pos = torch.arange(start_index - tail, start_index, device=q.device, dtype=torch.int64)[None]
-            k_tail = _rotate(self.last_incomplete_k[:B, :, :tail], cos, sin, pos)
-            k_win = torch.cat((k_tail, k), dim=2)
-            v_win = torch.cat((self.last_incomplete_v[:B, :, :tail], v), dim=2)
-            q_win = torch.cat((q.new_zeros(B, nh, tail, hs), q), dim=2)
+            # start_index - tail .., zero rows standing in for their queries -- one launch writes the three windows
+            assert start_index >= tail
+            q, k, v = (_lib.kernel_ready(t) for t in (q, k, v))
+            q_win, k_win, v_win = (torch.empty((B, nh, tail + T, hs), dtype=q.dtype, device=q.device) for _ in range(3))
+            with _lib.on_device(q.device):
+                rc = _lib.lib().lmk_ring_local_window(
+                    _lib.tensor4(q), _lib.tensor4(self.last_incomplete_k[:B]), _lib.tensor4(self.last_incomplete_v[:B]),
+                    _lib.tensor4(k), _lib.tensor4(v), cos.data_ptr(), sin.data_ptr(), cos.stride(0), cos.shape[0],
+                    _lib.tensor4(q_win), _lib.tensor4(k_win), _lib.tensor4(v_win), B, nh, T, tail,
+                    int(start_index - tail), hs, _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+            _lib.check(rc)
         else:
             q_win, k_win, v_win = (_lib.kernel_ready(t) for t in (q, k, v))
         W = tail + T

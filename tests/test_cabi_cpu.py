@@ -28,7 +28,7 @@ def _declared():
 
 def test_every_declared_symbol_is_exported(lib):
     names = _declared()
-    assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window",
+    assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window", "lmk_ring_local_window",
             "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend", "lmk_retrieve_topk_static", "lmk_retrieve_static_max_bytes",
             "lmk_ring_retrieve_topk", "lmk_ring_gather_attend", "lmk_attn_bwd_handover_workspace_bytes", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded", "lmk_attn_fwd_blocks", "lmk_attn_bwd_blocks", "lmk_attn_fwd_group_scale", "lmk_attn_bwd_group_scale",
             "lmk_strerror"} <= set(names)
@@ -134,6 +134,14 @@ def test_retrieval_argument_errors(lib):
     assert window(64, 4) == -9
     assert window(70, 27) == -2
     assert window(20, 4) == -9
+
+    # the ring cache's window: the tail lives outside the ring and is rotated at positions the caller names
+    def ring_window(tail=5, pos=100, D=128, kt=None):
+        return lib.lmk_ring_local_window(t, kt or t, t, t, t, 0x5000, 0x6000, 128, 4096, t, t, t, 1, 1, 8, tail, pos, D,
+                                         0, None)
+
+    assert ring_window(tail=0) == -2 and ring_window(pos=-1) == -11 and ring_window(pos=4092) == -11
+    assert ring_window(D=96) == -3 and ring_window(kt=_t4(ptr=0)) == -1
 
     # the attend step as one call: workspace and tail are checked before anything is launched
     def attend(S=64, T=8, ws=0x4000, wsb=1 << 30):
