@@ -174,6 +174,28 @@ int lmk_attn_bwd_blocks(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_te
                         int H, int Lq, int Lk, int D, float sm_scale, int block_tokens, int n_prefix, int dtype,
                         void* stream);
 
+/* Landmarks at irregular positions: blocks of unequal length.  The reference's fused kernel rejects such masks
+ * (flash_landmark_attention.py:393-394); its high-level path takes any is_mem
+ * (llama_mem.py:222-243, lm_benchmark/models/landmark.py:88-119) and this is that semantics on the fused kernels.
+ * The keys' blocks are described by a table of n_blocks + 1 token offsets: seg[b] = first token of block b,
+ * seg[0] = 0, seg[n_blocks] = Lk; every block ends in its landmark except, with last_is_partial, the last one
+ * (tokens behind the last landmark, at most max_block_tokens - 1 of them).  A complete block holds
+ * 2 .. max_block_tokens (<= 128) tokens.  The table is
+ * passed twice: seg_host is read and checked by the call itself (monotone, lengths in range, history made of whole
+ * blocks: Lk - Lq == seg[n_prefix]), seg_dev is the copy in device memory the kernels read -- the caller keeps the
+ * two identical.  Tensors, L and M are in token rows as in lmk_attn_fwd_blocks; the blocks are worked on in 64 or
+ * 128 slots.  The backward needs complete blocks only; workspace: lmk_attn_bwd_segments_workspace_bytes. */
+int lmk_attn_fwd_segments(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                          float* L, float* M, const int32_t* seg_host, const int32_t* seg_dev, int n_blocks,
+                          int max_block_tokens, int last_is_partial, int B, int H, int Lq, int Lk, int D,
+                          float sm_scale, int n_prefix, int dtype, void* stream);
+size_t lmk_attn_bwd_segments_workspace_bytes(int B, int H, int n_blocks, int n_prefix, int max_block_tokens);
+int lmk_attn_bwd_segments(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                          const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                          const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes,
+                          const int32_t* seg_host, const int32_t* seg_dev, int n_blocks, int max_block_tokens, int B,
+                          int H, int Lq, int Lk, int D, float sm_scale, int n_prefix, int dtype, void* stream);
+
 /* Group dropout (lm_benchmark/models/landmark.py:110-113: `dropout(group_prob, p)` on the landmark probabilities
  * that scale the earlier blocks, while the softmax over the landmarks itself stays as it is).  The random draw is
  * the caller's: group_scale is (B*H, Lk/block_tokens, Lq) fp32, contiguous, and entry [bh][b][i] multiplies what

@@ -191,11 +191,18 @@ struct RopeArgs {
 };
 
 // Lq_real, Lk_real > 0: the tensors are in token layout (rows = tokens of blocks of block_real), Lq and Lk count slots
+// Blocks of unequal length: the device copy of the table the kernels read and the number of complete blocks among
+// the keys' (validated on the host by the entry points that take one).
+struct SegArgs {
+  const int* seg_dev;
+  int n_full_k;
+};
+
 static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                          float* L, float* M, int B, int H, int Lq, int Lk, int D, float sm_scale, int block,
                          int block_real, int n_prefix, int dtype, void* stream, const RopeArgs* rope = nullptr,
                          int Lq_real = 0, int Lk_real = 0, const float* group_scale = nullptr,
-                         lmk::FwdParams* params_out = nullptr) {
+                         lmk::FwdParams* params_out = nullptr, const SegArgs* segs = nullptr) {
   int rc;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o))) return rc;
   if (L == nullptr || M == nullptr) return LMK_ERR_NULL;
@@ -216,6 +223,15 @@ static int attn_fwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
   }
   p.n_real = block_real;
   p.Lq_real = Lq_real; p.Lk_real = Lk_real;
+  if (segs != nullptr) {
+    if (Lq_real <= 0 || group_scale != nullptr) return LMK_ERR_UNSUPPORTED;
+    p.seg = segs->seg_dev;
+    p.n_full_k = segs->n_full_k;
+    p.n_full_q = segs->n_full_k - n_prefix;
+  } else if (Lq_real > 0) {
+    p.n_full_q = Lq_real / block_real;
+    p.n_full_k = Lk_real / block_real;
+  }
   if (group_scale != nullptr) {                            // (B*H, Lk_real / block_real, Lq_real) floats
     if (Lq_real <= 0) return LMK_ERR_UNSUPPORTED;
     p.group_scale = group_scale;
@@ -327,7 +343,7 @@ static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
                          const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
                          int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
                          int dtype, int phases, void* stream, int Lq_real = 0, int Lk_real = 0,
-                         const float* group_scale = nullptr);
+                         const float* group_scale = nullptr, const SegArgs* segs = nullptr);
 
 int lmk_attn_bwd_phases(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                         const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
@@ -402,6 +418,68 @@ static int slots_for_group_scale(int block_tokens) {
   return block_tokens <= 64 ? 64 : 128;
 }
 
+// Host-side check of a table of blocks of unequal length and the geometry that follows from it: slots per block,
+// rows of slots of the keys and of the queries.  `complete_only`: the backward's restriction.
+struct SegGeometry {
+  int slots, n_full_k;
+  int64_t lq_slots, lk_slots;
+};
+
+static int check_segments(const int32_t* seg_host, const void* seg_dev, int n_blocks, int max_block_tokens, int n_prefix,
+                          int Lq, int Lk, bool last_is_partial, bool complete_only, SegGeometry* g) {
+  if (seg_host == nullptr || seg_dev == nullptr) return LMK_ERR_NULL;
+  if (n_blocks <= 0 || n_prefix < 0 || n_prefix >= n_blocks || Lq <= 0 || Lk < Lq) return LMK_ERR_SHAPE;
+  if (max_block_tokens < 2 || max_block_tokens > 128) return LMK_ERR_UNSUPPORTED;
+  if (last_is_partial && complete_only) return LMK_ERR_PARTIAL;
+  const int n_full = n_blocks - (last_is_partial ? 1 : 0);
+  if (seg_host[0] != 0 || seg_host[n_blocks] != Lk) return LMK_ERR_SHAPE;
+  for (int b = 0; b < n_blocks; ++b) {
+    const int64_t len = (int64_t)seg_host[b + 1] - seg_host[b];
+    // a complete block: a key and its landmark at least; the block without landmark must leave the last slot free
+    if (len > max_block_tokens - (b < n_full ? 0 : 1) || len < (b < n_full ? 2 : 1)) return LMK_ERR_SHAPE;
+  }
+  if ((int64_t)Lk - Lq != seg_host[n_prefix]) return LMK_ERR_HISTORY;                 // the history is whole blocks
+  g->slots = max_block_tokens <= 64 ? 64 : 128;
+  g->n_full_k = n_full;
+  g->lk_slots = (int64_t)n_full * g->slots + (last_is_partial ? seg_host[n_blocks] - seg_host[n_blocks - 1] : 0);
+  g->lq_slots = g->lk_slots - (int64_t)n_prefix * g->slots;
+  if (g->lk_slots >= ((int64_t)1 << 31) || g->lq_slots <= 0) return LMK_ERR_UNSUPPORTED;
+  return LMK_OK;
+}
+
+int lmk_attn_fwd_segments(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                          float* L, float* M, const int32_t* seg_host, const int32_t* seg_dev, int n_blocks,
+                          int max_block_tokens, int last_is_partial, int B, int H, int Lq, int Lk, int D,
+                          float sm_scale, int n_prefix, int dtype, void* stream) {
+  SegGeometry g;
+  if (int rc = check_segments(seg_host, seg_dev, n_blocks, max_block_tokens, n_prefix, Lq, Lk, last_is_partial != 0, false, &g))
+    return rc;
+  const SegArgs segs = {seg_dev, g.n_full_k};
+  return attn_fwd_impl(q, k, v, o, L, M, B, H, (int)g.lq_slots, (int)g.lk_slots, D, sm_scale, g.slots, g.slots, n_prefix,
+                       dtype, stream, nullptr, Lq, Lk, nullptr, nullptr, &segs);
+}
+
+size_t lmk_attn_bwd_segments_workspace_bytes(int B, int H, int n_blocks, int n_prefix, int max_block_tokens) {
+  if (n_blocks <= 0 || n_prefix < 0 || n_prefix >= n_blocks || max_block_tokens < 2 || max_block_tokens > 128) return 0;
+  const int slots = max_block_tokens <= 64 ? 64 : 128;
+  const int64_t lk = (int64_t)n_blocks * slots, lq = (int64_t)(n_blocks - n_prefix) * slots;
+  if (lk >= ((int64_t)1 << 31)) return 0;
+  return lmk_attn_bwd_workspace_bytes(B, H, (int)lq, (int)lk, slots);
+}
+
+int lmk_attn_bwd_segments(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
+                          const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
+                          const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes,
+                          const int32_t* seg_host, const int32_t* seg_dev, int n_blocks, int max_block_tokens, int B,
+                          int H, int Lq, int Lk, int D, float sm_scale, int n_prefix, int dtype, void* stream) {
+  SegGeometry g;
+  if (int rc = check_segments(seg_host, seg_dev, n_blocks, max_block_tokens, n_prefix, Lq, Lk, false, true, &g)) return rc;
+  const SegArgs segs = {seg_dev, g.n_full_k};
+  return attn_bwd_impl(q, k, v, o, dout, L, M, dq, dk, dv, workspace, workspace_bytes, B, H, (int)g.lq_slots,
+                       (int)g.lk_slots, D, sm_scale, g.slots, g.slots, n_prefix, dtype, LMK_BWD_ALL, stream, Lq, Lk, nullptr,
+                       &segs);
+}
+
 int lmk_attn_fwd_group_scale(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_tensor4* v, const lmk_tensor4* o,
                              float* L, float* M, const float* group_scale, int B, int H, int Lq, int Lk, int D,
                              float sm_scale, int block_tokens, int n_prefix, int dtype, void* stream) {
@@ -444,7 +522,8 @@ static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
                          const lmk_tensor4* dout, const float* L, const float* M, const lmk_tensor4* dq,
                          const lmk_tensor4* dk, const lmk_tensor4* dv, void* workspace, size_t workspace_bytes, int B,
                          int H, int Lq, int Lk, int D, float sm_scale, int block, int block_real, int n_prefix,
-                         int dtype, int phases, void* stream, int Lq_real, int Lk_real, const float* group_scale) {
+                         int dtype, int phases, void* stream, int Lq_real, int Lk_real, const float* group_scale,
+                         const SegArgs* segs) {
   int rc;
   if (phases <= 0 || phases > LMK_BWD_ALL) return LMK_ERR_SHAPE;
   if ((rc = check_tensor(q)) || (rc = check_tensor(k)) || (rc = check_tensor(v)) || (rc = check_tensor(o)) ||
@@ -482,6 +561,16 @@ static int attn_bwd_impl(const lmk_tensor4* q, const lmk_tensor4* k, const lmk_t
   p.n_prefix = n_prefix; p.n_blocks = (int)nb;
   p.n_real = block_real;
   p.Lq_real = Lq_real; p.Lk_real = Lk_real;
+  p.seg = nullptr; p.n_full_q = p.n_full_k = 0;
+  if (segs != nullptr) {
+    if (Lq_real <= 0 || group_scale != nullptr) return LMK_ERR_UNSUPPORTED;
+    p.seg = segs->seg_dev;
+    p.n_full_k = segs->n_full_k;
+    p.n_full_q = segs->n_full_k - n_prefix;
+  } else if (Lq_real > 0) {
+    p.n_full_q = Lq_real / block_real;
+    p.n_full_k = Lk_real / block_real;
+  }
   p.group_scale = nullptr; p.gs_bh = p.gs_blk = 0;
   if (group_scale != nullptr) {
     if (Lq_real <= 0) return LMK_ERR_UNSUPPORTED;

@@ -44,8 +44,9 @@ __global__ __launch_bounds__(256) void lmk_bwd_pre_kernel(BwdParams p, int block
     const int bh = (int)(row / p.Lq);
     int qi = (int)(row % p.Lq);
     if (p.Lq_real > 0) {                                    // token layout: the workspace rows are slots
-      qi = block_slots == 64 ? slot_to_token_row<64>(qi, p.n_real, p.Lq_real / p.n_real)
-                             : slot_to_token_row<128>(qi, p.n_real, p.Lq_real / p.n_real);
+      const int* seg_q = p.seg != nullptr ? p.seg + p.n_prefix : nullptr;   // the queries' first block
+      qi = block_slots == 64 ? slot_to_token_row<64>(qi, p.n_real, p.n_full_q, seg_q)
+                             : slot_to_token_row<128>(qi, p.n_real, p.n_full_q, seg_q);
       li = qi < 0 ? -1 : (int64_t)bh * p.Lq_real + qi;
     }
     if (qi >= 0) {
@@ -103,8 +104,10 @@ __device__ __forceinline__ void dq_dma16(const void* base_uniform, uint32_t voff
 
 // VIRT: tensors in token layout (p.Lq_real > 0); a template parameter because the slot arithmetic costs the
 // slot-layout instantiations registers they do not have.
-template <class T, int D, int BS, bool VIRT>
+// SEG (with VIRT): blocks of unequal length, looked up in p.seg -- a template parameter for the same reason.
+template <class T, int D, int BS, bool VIRT, bool SEG = false>
 __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
+  static_assert(VIRT || !SEG, "the table describes tensors in token layout");
   using C = DqCfg<T, D, BS>;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -140,8 +143,10 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   // a token is a query row of zeros with mhat = 1e30: its gate, its weights and every term it leaves for the dK/dV
   // kernel come out as exact zeros (a = 1e30), whatever that kernel reads for its Q and dO rows.
   constexpr bool virt = VIRT;
-  const int nfull_k = virt ? p.Lk_real / p.n_real : 0;
-  const int qtok = !active ? -1 : (virt ? slot_to_token_row<BS>(qrow, p.n_real, p.Lq_real / p.n_real) : qrow);
+  const int nfull_k = p.n_full_k;
+  const int* seg_k = SEG ? p.seg : nullptr;
+  const int* seg_q = SEG ? p.seg + p.n_prefix : nullptr;   // the queries' first block
+  const int qtok = !active ? -1 : (virt ? slot_to_token_row<BS>(qrow, p.n_real, p.n_full_q, seg_q) : qrow);
 
   u32x4_t qf[C::KS], gf[C::KS];
 #pragma unroll
@@ -209,7 +214,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
       if (virt) {                                          // the slot's token row, worked out per request
         const int row = C::RPD * (r % n_k) + lane / C::CH, cp = lane % C::CH;
         const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
-        const int tok = slot_to_token_row_clamped<BS>(blk_req * BS + row, p.n_real, nfull_k);
+        const int tok = slot_to_token_row_clamped<BS>(blk_req * BS + row, p.n_real, nfull_k, seg_k);
         dq_dma16(is_v ? vp : kp, (uint32_t)(2 * ((int64_t)tok * (is_v ? p.vs_r : p.ks_r) + 8 * (cp ^ f))), dst);
       } else {
         dq_dma16(is_v ? vp : kp, src[i], dst);
@@ -227,8 +232,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   const float c2 = p.scale_log2;
   // A block narrower than BS tokens is stored with its n_norm normal keys in front, its landmark in the
   // last slot and padding in between: slots n_norm .. BS-2 hold no key and no query may see them.
-  const int n_norm = p.n_real - 1;
-  const bool padded = n_norm < BS - 1;                     // uniform over the launch
+  // With blocks of unequal length n_norm is the stage's block's (uniform over the workgroup).
+  const int n_norm_all = p.n_real - 1;
+  const bool padded = n_norm_all < BS - 1 || seg_k != nullptr;   // uniform over the launch
 
   // LDS byte offsets of this lane's operand fragments inside a 32-row tile: the swizzle repeats every 16
   // rows, so a tile at row 32u is the same offsets plus 32u rows -- an immediate of the LDS instruction
@@ -277,6 +283,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     if (s + 1 < n_stages) request(buf ^ 1);
     const int kb = buf * C::STAGE_BYTES, vb = kb + C::TILE_BYTES;   // LDS byte addresses (the dynamic array starts at 0)
     if (!active) continue;
+    int n_norm = n_norm_all;
+    if constexpr (SEG)
+      if (s <= cblk) n_norm = block_normal_keys<BS>(s, p.n_real, nfull_k, seg_k);
     if (s < cblk) {
       float gscale = 1.f;                                  // group dropout: this block's factor for this query row
       if constexpr (VIRT)
@@ -396,7 +405,12 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
     } else {
       using C = DqCfg<T, D, BS>;
       const dim3 grid(((p.Lq + 255) / 256) * p.B * p.H);
-      if (p.Lq_real > 0) {
+      if (p.Lq_real > 0 && p.seg != nullptr) {
+        auto kern = lmk_bwd_dq_kernel<T, D, BS, true, true>;
+        static std::atomic<uint64_t> lds_ok{0};
+        if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
+        hipLaunchKernelGGL(kern, grid, dim3(64 * C::NW), C::LDS_BYTES, stream, p);
+      } else if (p.Lq_real > 0) {
         auto kern = lmk_bwd_dq_kernel<T, D, BS, true>;
         static std::atomic<uint64_t> lds_ok{0};
         if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;

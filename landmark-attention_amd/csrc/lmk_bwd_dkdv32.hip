@@ -164,7 +164,9 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   // per-lane source offsets (bytes) of this wave's requests 0 and 1 inside tile 0 of Q and of dO
   uint32_t q_vo0 = 0, q_vo1 = 0, g_vo0 = 0, g_vo1 = 0;
   int vrow0 = 0, vcf0 = 0, vcf1 = 0;                       // VIRT: this lane's row inside a tile and its two chunk offsets
-  const int nfull_q = VIRT ? p.Lq_real / p.n_real : 0, nfull_k = VIRT ? p.Lk_real / p.n_real : 0;
+  const int nfull_q = p.n_full_q, nfull_k = p.n_full_k;
+  const int* seg_k = VIRT ? p.seg : nullptr;            // blocks of unequal length (null: n_real tokens each)
+  const int* seg_q = (VIRT && p.seg != nullptr) ? p.seg + p.n_prefix : nullptr;   // the queries' first block
   if (!role_k) {
     const int chp = lane % C::CH;
     const int row0 = C::RPD * (tile * C::NDMA) + lane / C::CH, row1 = row0 + C::RPD;
@@ -182,7 +184,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   }
   // VIRT: byte offset of this lane's chunk of slot row 32 j + its row (+ RPD for the second request) of a tensor
   auto virt_off = [&](int j, int second, int64_t row_stride) LMK_INL {
-    const int tok = slot_to_token_row_clamped<BS>(32 * j + vrow0 + (second ? C::RPD : 0), p.n_real, nfull_q);
+    const int tok = slot_to_token_row_clamped<BS>(32 * j + vrow0 + (second ? C::RPD : 0), p.n_real, nfull_q, seg_q);
     return 2u * (uint32_t)tok * (uint32_t)row_stride + (uint32_t)(second ? vcf1 : vcf0);
   };
   const uint32_t q_step = (uint32_t)(2 * 32 * p.qs_r), g_step = (uint32_t)(2 * 32 * p.dos_r);
@@ -411,7 +413,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     const int64_t rs = role_k ? p.vs_r : p.ks_r;
     int kr = krow, h8 = 8 * h;
     asm volatile("" : "+v"(kr), "+v"(h8));                 // the address is formed here, not ahead of the loops (and spilled)
-    if constexpr (VIRT) kr = slot_to_token_row_clamped<BS>(active ? kr : 0, p.n_real, nfull_k);
+    if constexpr (VIRT) kr = slot_to_token_row_clamped<BS>(active ? kr : 0, p.n_real, nfull_k, seg_k);
     const char* row = src + 2 * ((int64_t)kr * rs + h8);
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) {
@@ -454,7 +456,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   auto store_acc = [&](const f32x16_t* acc, char* dst, int64_t rs, float scl) LMK_INL {
     int kr = krow, h4 = 4 * h;
     asm volatile("" : "+v"(kr), "+v"(h4));                 // as in load_stationary
-    if constexpr (VIRT) kr = slot_to_token_row<BS>(kr, p.n_real, nfull_k);   // -1: a slot without a token, nothing to store
+    if constexpr (VIRT) kr = slot_to_token_row<BS>(kr, p.n_real, nfull_k, seg_k);   // -1: a slot without a token, nothing to store
     char* row = dst + 2 * ((int64_t)kr * rs + h4);
     if (!VIRT || kr >= 0) {
 #pragma unroll

@@ -179,6 +179,32 @@ __device__ __forceinline__ int slot_to_token_row_clamped(int slot_row, int n, in
   return r < 0 ? (slot_row / BS) * n : r;
 }
 
+// Blocks of unequal length (landmarks at irregular positions): seg[b] is the first token of block b and
+// seg[b + 1] - seg[b] its length, at most BS; the first n_full blocks end in their landmark, a last block behind
+// them has none.  `seg` points at the entry of the first block of the tensor whose rows are asked for (the queries
+// of a call with history start n_prefix blocks into the keys' table).  Null: every block holds n tokens.
+template <int BS>
+__device__ __forceinline__ int slot_to_token_row(int slot_row, int n, int n_full, const int* seg) {
+  if (seg == nullptr) return slot_to_token_row<BS>(slot_row, n, n_full);
+  const int blk = slot_row / BS, s = slot_row % BS;
+  const int first = seg[blk], len = seg[blk + 1] - first;
+  int tok = s < len ? s : -1;
+  if (blk < n_full) tok = (s == BS - 1) ? len - 1 : (s < len - 1 ? s : -1);
+  return tok < 0 ? -1 : first - seg[0] + tok;
+}
+template <int BS>
+__device__ __forceinline__ int slot_to_token_row_clamped(int slot_row, int n, int n_full, const int* seg) {
+  if (seg == nullptr) return slot_to_token_row_clamped<BS>(slot_row, n, n_full);
+  const int r = slot_to_token_row<BS>(slot_row, n, n_full, seg);
+  return r < 0 ? seg[slot_row / BS] - seg[0] : r;
+}
+// normal keys of block blk of the keys (slots behind them, up to the landmark's, hold nothing)
+template <int BS>
+__device__ __forceinline__ int block_normal_keys(int blk, int n, int n_full, const int* seg) {
+  if (seg == nullptr) return n - 1;
+  return blk < n_full ? seg[blk + 1] - seg[blk] - 1 : BS - 1;
+}
+
 template <class T>
 __device__ __forceinline__ float round_to(float x) {  // fp32 -> T (RNE) -> fp32
   return unpack_lo<T>(pack2<T>(x, 0.f));

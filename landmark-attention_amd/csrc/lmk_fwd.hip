@@ -81,8 +81,9 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   const int qrow = q0 + ql;
   // token layout: the tensors' rows are tokens, the kernel's rows are slots
   const bool virt = p.Lq_real > 0;                      // uniform over the launch
-  const int nfull_q = virt ? p.Lq_real / p.n_real : 0, nfull_k = virt ? p.Lk_real / p.n_real : 0;
-  const int qtok = !virt ? (qrow < p.Lq ? qrow : -1) : (qrow < p.Lq ? slot_to_token_row<BS>(qrow, p.n_real, nfull_q) : -1);
+  const int nfull_q = p.n_full_q, nfull_k = p.n_full_k;
+  const int* seg_q = p.seg != nullptr ? p.seg + p.n_prefix : nullptr;   // the queries' first block
+  const int qtok = !virt ? (qrow < p.Lq ? qrow : -1) : (qrow < p.Lq ? slot_to_token_row<BS>(qrow, p.n_real, nfull_q, seg_q) : -1);
 
   // ---- Q fragments (B operand): query qrow, head dims 16*ks + 8h .. +7
   u32x4_t qf[C::KS];
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
       if (virt) {                                       // the slot's token row, worked out per request
         const int row = C::RPD * (r % n_k) + lane / C::CH, cp = lane % C::CH;
         const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
-        const int tok = slot_to_token_row_clamped<BS>(min(blk_req * C::SK + row, p.Lk - 1), p.n_real, nfull_k);
+        const int tok = slot_to_token_row_clamped<BS>(min(blk_req * C::SK + row, p.Lk - 1), p.n_real, nfull_k, p.seg);
         fwd_dma16(is_v ? vp : kp, (uint32_t)(2 * ((int64_t)tok * (is_v ? p.vs_r : p.ks_r) + 8 * (cp ^ f))), dst);
       } else {
         fwd_dma16(is_v ? vp : kp, last ? src_last[i] : src[i], dst);
@@ -153,8 +154,9 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   const float c2 = p.scale_log2;
   // A block narrower than BS tokens is stored with its n_norm normal keys in front, its landmark in the
   // last slot and padding in between: slots n_norm .. BS-2 hold no key and no query may see them.
-  const int n_norm = p.n_real - 1;
-  const bool padded = n_norm < BS - 1;                  // uniform over the launch
+  // With blocks of unequal length n_norm is the block's at hand (uniform over the workgroup).
+  const int n_norm_all = p.n_real - 1;
+  const bool padded = n_norm_all < BS - 1 || p.seg != nullptr;   // uniform over the launch
 
   // LDS byte offsets of this lane's operand fragments inside a 32-row tile: the swizzle repeats every 16
   // rows, so a tile at row 32u is the same offsets plus 32u rows -- an immediate of the LDS instruction
@@ -215,6 +217,9 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
       const int blk = s * C::NB + jb;                     // absolute landmark block
       // LDS byte addresses of the block's K and V rows (the dynamic array starts at 0)
       const int kb = buf * C::STAGE_BYTES + jb * BS * C::ROWB, vb = kb + C::TILE_BYTES;
+      // (a stage may reach past the wave's own block, and past the table: those blocks are not looked at)
+      int n_norm = n_norm_all;
+      if (p.seg != nullptr && blk <= cblk) n_norm = block_normal_keys<BS>(blk, p.n_real, nfull_k, p.seg);
       if (blk < cblk) {
         // ---------------- earlier block: local softmax gated by its landmark
         float gscale = 1.f;                               // group dropout: this block's factor for this query row

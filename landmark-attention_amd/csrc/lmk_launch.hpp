@@ -53,6 +53,11 @@ struct FwdParams {
   // partial last block keeps its length); the kernels translate slot rows to token rows themselves.
   // 0: the tensors are stored in slots already (n_real < block: with padding rows).
   int Lq_real, Lk_real;
+  // token layout with blocks of unequal length (landmarks at irregular positions): seg[b] = first token of key block
+  // b, n_blocks + 1 entries in device memory, n_full_k of the blocks complete (ending in their landmark); null:
+  // every block holds n_real tokens.  n_full_q, n_full_k are set in both cases.
+  const int* seg;
+  int n_full_q, n_full_k;
   // optional (blocks of 64 / 128 slots, token layout only): factor of earlier block b's contribution to query row i,
   // group_scale[bh * gs_bh + b * gs_blk + i] -- 0 drops the block for that row, 1 / (1 - p) keeps it under group
   // dropout (lm_benchmark/models/landmark.py:110-113); the softmax over the landmarks is not renormalised
@@ -85,6 +90,8 @@ struct BwdParams {
   int n_qtiles, n_kvtiles;       // ceil(Lq / 128), ceil(Lk / 128)
   int n_real;                    // tokens of a block that exist; == block unless padded (blocks 64 and 128 only)
   int Lq_real, Lk_real;          // > 0: tensors in token layout, as in FwdParams (the workspace stays indexed by slot rows)
+  const int* seg;                // blocks of unequal length, as in FwdParams (null: n_real tokens each)
+  int n_full_q, n_full_k;
   const float* group_scale;      // optional, as in FwdParams (token layout only)
   int64_t gs_bh, gs_blk;
   int64_t qs_b, qs_h, qs_r, ks_b, ks_h, ks_r, vs_b, vs_h, vs_r, os_b, os_h, os_r, dos_b, dos_h, dos_r;

@@ -107,6 +107,13 @@ def lib() -> ctypes.CDLL:
                                               i, i, i, i, i, f, i, i, i, vp]
         L.lmk_local_window.restype = i
         L.lmk_local_window.argtypes = [T4, T4, T4, T4, T4, vp, vp, i64, i64, T4, T4, T4, i, i, i, i, i, i, i, vp]
+        L.lmk_attn_fwd_segments.restype = i
+        L.lmk_attn_fwd_segments.argtypes = [T4, T4, T4, T4, vp, vp, vp, vp, i, i, i, i, i, i, i, i, f, i, i, vp]
+        L.lmk_attn_bwd_segments_workspace_bytes.restype = sz
+        L.lmk_attn_bwd_segments_workspace_bytes.argtypes = [i, i, i, i, i]
+        L.lmk_attn_bwd_segments.restype = i
+        L.lmk_attn_bwd_segments.argtypes = [T4, T4, T4, T4, T4, vp, vp, T4, T4, T4, vp, sz, vp, vp, i, i, i, i, i, i, i, f,
+                                            i, i, vp]
         L.lmk_ring_local_window.restype = i
         L.lmk_ring_local_window.argtypes = [T4, T4, T4, T4, T4, vp, vp, i64, i64, T4, T4, T4, i, i, i, i, i64, i, i, vp]
         L.lmk_retrieve_topk_shared.restype = i

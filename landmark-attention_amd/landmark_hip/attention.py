@@ -223,6 +223,84 @@ class FusedLandmarkAttentionGroupScale(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None
 
 
+class LandmarkSegments:
+    """Blocks of unequal length cut out by a mask with landmarks at irregular positions: ``seg[b]`` is the first
+    token of block b, every block ends in its landmark except -- ``last_is_partial`` -- the tokens behind the last
+    landmark.  Held on the host (checked by every call of the library) and on the device (read by the kernels)."""
+
+    def __init__(self, is_mem_row, device):
+        import ctypes
+        marks = [bool(x) for x in is_mem_row]
+        ends = [j + 1 for j, m in enumerate(marks) if m]
+        self.last_is_partial = not marks or not marks[-1]
+        seg = [0] + ends + ([len(marks)] if self.last_is_partial else [])
+        self.n_blocks = len(seg) - 1
+        lengths = [b - a for a, b in zip(seg[:-1], seg[1:])]
+        n_full = self.n_blocks - int(self.last_is_partial)
+        # the tokens behind the last landmark count one more: their block must leave its last slot, the landmark's, free
+        widths = lengths[:n_full] + ([lengths[-1] + 1] if self.last_is_partial else [])
+        assert self.n_blocks > 0 and max(widths) <= MAX_BLOCK, \
+            f"a block of more than {MAX_BLOCK} tokens between two landmarks is outside what the HIP kernels cover"
+        assert all(n >= 2 for n in lengths[:n_full]), "two landmarks in a row (a block without a normal token) are not covered"
+        self.max_len = max(max(widths), 2)
+        self.seg = seg
+        self.seg_host = (ctypes.c_int32 * len(seg))(*seg)
+        self.seg_dev = torch.tensor(seg, dtype=torch.int32, device=device)
+
+    def history_blocks(self, n_history_tokens: int) -> int:
+        assert n_history_tokens in self.seg[:-1], "the keys in front of the first query must be whole blocks"
+        return self.seg.index(n_history_tokens)
+
+
+class FusedLandmarkAttentionSegments(torch.autograd.Function):
+    """``FusedLandmarkAttention`` for landmarks at irregular positions (blocks of unequal length, each at most 128
+    tokens): the grouped softmax of the reference's high-level path (``llama/llama_mem.py:222-243``) on the fused
+    kernels.  The reference's own fused path rejects such masks (``flash_landmark_attention.py:393-394``)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, segments, sm_scale):
+        B, H, Lq, D = q.shape
+        Lk = k.shape[2]
+        assert k.shape == v.shape == (B, H, Lk, D) and q.dtype == k.dtype == v.dtype and q.dtype in _lib.DTYPE_CODES
+        assert q.is_cuda and D in SUPPORTED_HEAD_DIMS and segments.seg[-1] == Lk
+        n_prefix = segments.history_blocks(Lk - Lq)
+        q, k, v = _lib.kernel_ready(q), _lib.kernel_ready(k), _lib.kernel_ready(v)
+        o = torch.empty_like(q)
+        L = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+        M = torch.empty((B * H, Lq), device=q.device, dtype=torch.float32)
+        with _lib.on_device(q.device):
+            rc = _lib.lib().lmk_attn_fwd_segments(
+                _lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o), L.data_ptr(), M.data_ptr(),
+                segments.seg_host, segments.seg_dev.data_ptr(), segments.n_blocks, segments.max_len,
+                int(segments.last_is_partial), B, H, Lq, Lk, D, float(sm_scale), n_prefix, _lib.DTYPE_CODES[q.dtype],
+                _lib.current_stream(q.device))
+        _lib.check(rc)
+        ctx.save_for_backward(q, k, v, o, L, M)
+        ctx.args = (segments, n_prefix, sm_scale)
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, L, M = ctx.saved_tensors
+        segments, n_prefix, sm_scale = ctx.args
+        assert not segments.last_is_partial, "Backward supported only for full blocks"
+        B, H, Lq, D = q.shape
+        Lk = k.shape[2]
+        do = _lib.kernel_ready(do)
+        lib = _lib.lib()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        nbytes = lib.lmk_attn_bwd_segments_workspace_bytes(B, H, segments.n_blocks, n_prefix, segments.max_len)
+        ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+        with _lib.on_device(q.device):
+            rc = lib.lmk_attn_bwd_segments(
+                _lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o), _lib.tensor4(do), L.data_ptr(),
+                M.data_ptr(), _lib.tensor4(dq), _lib.tensor4(dk), _lib.tensor4(dv), ws.data_ptr(), nbytes,
+                segments.seg_host, segments.seg_dev.data_ptr(), segments.n_blocks, segments.max_len, B, H, Lq, Lk, D,
+                float(sm_scale), n_prefix, _lib.DTYPE_CODES[q.dtype], _lib.current_stream(q.device))
+        _lib.check(rc)
+        return dq, dk, dv, None, None
+
+
 # Masks that have already passed the check of ``flash_landmark_attention.py:393-394``, keyed by what
 # identifies a tensor's content without reading it: storage address, in-place version counter, layout.
 # (A write through ``.data`` or a custom kernel bypasses the counter; such a mask has to be a new tensor.)
@@ -232,8 +310,11 @@ _VALIDATED_MASKS: dict = {}
 _VALIDATED_MASKS_MAX = 64
 
 
-def _check_is_mem(is_mem, block_size, offset=0):
-    # offset: tokens of the first block that lie in front of the mask (a stream cut between two landmarks)
+def _check_is_mem(is_mem, block_size, offset=0, irregular_ok=False):
+    """None when ``is_mem`` marks exactly the last token of every block of ``block_size`` (the check of
+    ``flash_landmark_attention.py:393-394``); otherwise an AssertionError -- or, with ``irregular_ok``, the
+    ``LandmarkSegments`` of the mask.  offset: tokens of the first block that lie in front of the mask (a stream
+    cut between two landmarks)."""
     # tensors created under torch.inference_mode() track no version counter (reading it raises): they are checked
     # on every call rather than cached
     cacheable = not is_mem.is_inference()
@@ -241,31 +322,49 @@ def _check_is_mem(is_mem, block_size, offset=0):
         key = (is_mem.device, is_mem.data_ptr(), is_mem._version, tuple(is_mem.shape), tuple(is_mem.stride()),
                is_mem.dtype, int(block_size), int(offset))
         if key in _VALIDATED_MASKS:
-            return
+            found = _VALIDATED_MASKS[key][1]
+            assert found is None or irregular_ok, _IRREGULAR_MESSAGE.format(block_size)
+            return found
     expected_is_mem = (torch.arange(0, is_mem.shape[-1], device=is_mem.device) + offset) % block_size == (block_size - 1)
-    assert (is_mem == expected_is_mem).all(), (
-        f"is_mem must mark exactly the last token of every block of {block_size}: irregular landmark positions "
-        "and dropped landmarks are not covered by the fused kernels")
-    if not cacheable:
-        return
-    if len(_VALIDATED_MASKS) >= _VALIDATED_MASKS_MAX:
-        _VALIDATED_MASKS.clear()
-    # the entry keeps the tensor alive, so its address cannot be handed to another mask meanwhile
-    _VALIDATED_MASKS[key] = is_mem
+    found = None
+    if not bool((is_mem == expected_is_mem).all()):
+        assert irregular_ok, _IRREGULAR_MESSAGE.format(block_size)
+        rows = is_mem.reshape(-1, is_mem.shape[-1])
+        assert bool((rows == rows[:1]).all()), "landmarks at irregular positions must be the same for every sequence of the batch"
+        found = LandmarkSegments(rows[0].tolist(), is_mem.device)
+    if cacheable:
+        if len(_VALIDATED_MASKS) >= _VALIDATED_MASKS_MAX:
+            _VALIDATED_MASKS.clear()
+        # the entry keeps the tensor alive, so its address cannot be handed to another mask meanwhile
+        _VALIDATED_MASKS[key] = (is_mem, found)
+    return found
+
+
+_IRREGULAR_MESSAGE = ("is_mem must mark exactly the last token of every block of {}: landmarks at irregular positions "
+                      "are covered by fused_landmark_attention only (head dims 64 and 128, no group dropout)")
 
 
 def fused_landmark_attention(q, k, v, is_mem, sm_scale=None, block_size=64, group_scale=None):
     """Landmark grouped-softmax causal attention, landmarks at every ``block_size``-th key.
 
     q: (B, H, Lq, D); k, v: (B, H, Lk, D) with ``Lk - Lq`` a whole number of blocks of
-    history.  ``is_mem`` (bool, last dim Lk) must mark exactly the positions
-    ``j % block_size == block_size - 1`` (checked as in the reference, ``:393-394``; the check
-    costs one device->host sync, paid once per distinct mask tensor state, not per call); pass
-    ``None`` to skip the check.  ``group_scale`` (not in the reference's signature): the group-dropout factors of
+    history.  ``is_mem`` (bool, last dim Lk) marks the positions ``j % block_size == block_size - 1``
+    (checked as in the reference, ``:393-394``; the check costs one device->host sync, paid once per
+    distinct mask tensor state, not per call); pass ``None`` to skip the check.  A mask with landmarks
+    at other positions -- which the reference's fused path rejects and only its high-level path takes --
+    runs on the same kernels with blocks of unequal length (``FusedLandmarkAttentionSegments``: every
+    block at most 128 tokens and at least one normal token, the same mask for every sequence of the
+    batch, the keys in front of the first query whole blocks).  ``group_scale`` (not in the reference's signature): the group-dropout factors of
     ``FusedLandmarkAttentionGroupScale``, (B, H, Lk / block_size, Lq) fp32, for head dims 64 and 128.
     """
     if is_mem is not None:
-        _check_is_mem(is_mem, block_size)
+        segments = _check_is_mem(is_mem, block_size, irregular_ok=group_scale is None)
+        if segments is not None:
+            # not in the reference's fused path (its check rejects the mask): blocks of unequal length, what its
+            # high-level path computes for such a mask; block_size plays no part
+            if sm_scale is None:
+                sm_scale = 1.0 / math.sqrt(q.size(-1))
+            return FusedLandmarkAttentionSegments.apply(q, k, v, segments, sm_scale)
 
     n_history_kv = k.shape[-2] - q.shape[-2]
     assert n_history_kv % block_size == 0

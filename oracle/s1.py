@@ -89,6 +89,65 @@ def s1_rows_python(q, k, v, block: int, scale: float | None = None):
     return outs, ls, ms
 
 
+def s1_rows_python_irregular(q, k, v, is_mem, scale: float | None = None):
+    """S1 for landmarks at arbitrary positions, row by row in Python floats: what the reference's high-level
+    path computes for any ``is_mem`` (``llama/llama_mem.py:222-243,807-815``;
+    ``lm_benchmark/models/landmark.py:88-119,216-224``).
+
+    q: (Lq, D), k, v: (Lk, D); is_mem: Lk booleans.  A block is a run of tokens that ends in a landmark; the
+    tokens behind the last landmark form a last block without one.  Query row i sits at key position
+    ``p = i + Lk - Lq``; it sees the keys of its own block up to ``p`` (a landmark query: up to ``p - 1``) and
+    every earlier block through that block's landmark.  Returns ``out`` as lists.  Shares no code with
+    :mod:`oracle.highlevel`.
+    """
+    q = [[float(x) for x in row] for row in q]
+    k = [[float(x) for x in row] for row in k]
+    v = [[float(x) for x in row] for row in v]
+    is_mem = [bool(x) for x in is_mem]
+    lq, lk, d = len(q), len(k), len(q[0])
+    assert len(is_mem) == lk
+    if scale is None:
+        scale = default_scale(d)
+    block_of, b = [], 0
+    for j in range(lk):
+        block_of.append(b)
+        if is_mem[j]:
+            b += 1
+    members = {}
+    for j in range(lk):
+        members.setdefault(block_of[j], []).append(j)
+    outs = []
+    for i in range(lq):
+        p = i + lk - lq
+        c = block_of[p]
+        lim = p - 1 if is_mem[p] else p
+        s = [scale * sum(x * y for x, y in zip(q[i], k[j])) for j in range(lk)]
+        own = [j for j in members[c] if j <= lim]
+        landmarks = [members[bb][-1] for bb in range(c)]            # every earlier block ends in its landmark
+        bucket = landmarks + own
+        o = [0.0] * d
+        if bucket:
+            m = max(s[j] for j in bucket)
+            e = {j: math.exp(s[j] - m) for j in bucket}
+            ell = sum(e.values())
+            for j in own:
+                for t in range(d):
+                    o[t] += e[j] / ell * v[j][t]
+            for bb in range(c):
+                normal = members[bb][:-1]
+                if not normal:
+                    continue                                         # a block of a landmark alone carries nothing
+                mb = max(s[j] for j in normal)
+                eb = [math.exp(s[j] - mb) for j in normal]
+                zb = sum(eb)
+                gate = e[members[bb][-1]] / ell
+                for j, ej in zip(normal, eb):
+                    for t in range(d):
+                        o[t] += gate * ej / zb * v[j][t]
+        outs.append(o)
+    return outs
+
+
 # --------------------------------------------------------------------------
 # vectorised, differentiable form
 # --------------------------------------------------------------------------

@@ -30,7 +30,7 @@ def test_every_declared_symbol_is_exported(lib):
     names = _declared()
     assert {"lmk_attn_fwd", "lmk_attn_bwd", "lmk_retrieve_topk", "lmk_gather_attend", "lmk_local_window", "lmk_ring_local_window",
             "lmk_retrieve_topk_shared", "lmk_retrieve_topk_reuse", "lmk_gather_window", "lmk_apply_rotary", "lmk_attend", "lmk_retrieve_and_attend", "lmk_retrieve_topk_static", "lmk_retrieve_static_max_bytes",
-            "lmk_ring_retrieve_topk", "lmk_ring_gather_attend", "lmk_attn_bwd_handover_workspace_bytes", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded", "lmk_attn_fwd_blocks", "lmk_attn_bwd_blocks", "lmk_attn_fwd_group_scale", "lmk_attn_bwd_group_scale",
+            "lmk_ring_retrieve_topk", "lmk_ring_gather_attend", "lmk_attn_bwd_handover_workspace_bytes", "lmk_retrieve_topk_shared_landmarks", "lmk_attn_fwd_rotary_q", "lmk_apply_rotary_qk", "lmk_padded_rows", "lmk_pad_blocks", "lmk_unpad_blocks", "lmk_attn_fwd_padded", "lmk_attn_bwd_padded", "lmk_attn_fwd_blocks", "lmk_attn_bwd_blocks", "lmk_attn_fwd_segments", "lmk_attn_bwd_segments", "lmk_attn_fwd_group_scale", "lmk_attn_bwd_group_scale",
             "lmk_strerror"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
@@ -323,8 +323,8 @@ def test_ring_attention_argument_errors(lib):
 
 
 def test_irregular_landmark_positions_are_rejected_with_a_message():
-    # landmarks anywhere but at the end of every block (irregular positions, group dropout) are outside the
-    # fused path, as in the reference (flash_landmark_attention.py:393-394)
+    # landmarks anywhere but at the end of every block are rejected where the caller has not asked for them
+    # (the rotary-q forward, the ring cache, group dropout), as in the reference (flash_landmark_attention.py:393-394)
     import torch
     from landmark_hip import attention
     attention._VALIDATED_MASKS.clear()
@@ -374,3 +374,58 @@ def test_is_mem_built_under_inference_mode_is_checked_without_a_version_counter(
         attention._check_is_mem(bad, 32)
     with torch.inference_mode():
         attention._check_is_mem(mask, 32)
+
+
+def test_irregular_landmark_positions_become_a_table_of_blocks():
+    import torch
+    from landmark_hip import attention
+    attention._VALIDATED_MASKS.clear()
+    mask = torch.zeros(20, dtype=torch.bool)
+    mask[[3, 9, 11, 16]] = True
+    seg = attention._check_is_mem(mask, 5, irregular_ok=True)
+    assert seg.seg == [0, 4, 10, 12, 17, 20] and seg.n_blocks == 5 and seg.last_is_partial and seg.max_len == 6
+    assert list(seg.seg_host) == seg.seg and seg.seg_dev.tolist() == seg.seg
+    assert attention._check_is_mem(mask, 5, irregular_ok=True) is seg            # remembered with the mask
+    assert seg.history_blocks(10) == 2 and seg.history_blocks(0) == 0
+    with pytest.raises(AssertionError, match="whole blocks"):
+        seg.history_blocks(5)
+    with pytest.raises(AssertionError, match="last token of every block"):
+        attention._check_is_mem(mask, 5)                                         # the same mask where it is not wanted
+    two_in_a_row = mask.clone()
+    two_in_a_row[4] = True
+    with pytest.raises(AssertionError, match="two landmarks in a row"):
+        attention._check_is_mem(two_in_a_row, 5, irregular_ok=True)
+    wide = torch.zeros(300, dtype=torch.bool)
+    wide[[200, 299]] = True
+    with pytest.raises(AssertionError, match="more than 128"):
+        attention._check_is_mem(wide, 5, irregular_ok=True)
+    per_sequence = torch.stack((mask, mask.roll(1)))
+    with pytest.raises(AssertionError, match="same for every sequence"):
+        attention._check_is_mem(per_sequence, 5, irregular_ok=True)
+    assert attention._check_is_mem(torch.arange(20) % 5 == 4, 5, irregular_ok=True) is None   # a regular mask stays one
+
+
+def test_block_table_is_checked_on_the_host(lib):
+    import ctypes
+    t = _t4()
+
+    def fwd(seg=(0, 4, 10, 12), n_blocks=3, max_len=6, partial=0, Lq=12, Lk=12, n_prefix=0, dev=0x9000, host=True):
+        arr = (ctypes.c_int32 * len(seg))(*seg)
+        return lib.lmk_attn_fwd_segments(t, t, t, t, 0x2000, 0x3000, arr if host else None, dev, n_blocks, max_len,
+                                         partial, 1, 1, Lq, Lk, 128, 0.1, n_prefix, 0, None)
+
+    assert fwd(host=False) == -1 and fwd(dev=0) == -1
+    assert fwd(seg=(1, 4, 10, 12)) == -2                       # the first block starts at token 0
+    assert fwd(seg=(0, 4, 10, 13)) == -2                       # the last one ends at Lk
+    assert fwd(seg=(0, 4, 11, 12)) == -2                       # longer than max_block_tokens
+    assert fwd(seg=(0, 4, 5, 12), max_len=8) == -2             # a landmark alone
+    assert fwd(seg=(0, 4, 4, 12), max_len=8) == -2             # not increasing
+    assert fwd(max_len=129) == -3 and fwd(max_len=1) == -3
+    assert fwd(Lq=7, n_prefix=1) == -5                         # the history is not whole blocks
+    assert fwd(n_prefix=3) == -2
+    assert lib.lmk_attn_bwd_segments_workspace_bytes(1, 1, 3, 0, 6) == lib.lmk_attn_bwd_workspace_bytes(1, 1, 192, 192, 64)
+    assert lib.lmk_attn_bwd_segments_workspace_bytes(1, 1, 3, 1, 100) == lib.lmk_attn_bwd_workspace_bytes(1, 1, 256, 384, 128)
+    arr = (ctypes.c_int32 * 4)(0, 4, 10, 12)
+    bwd = lib.lmk_attn_bwd_segments(t, t, t, t, t, 0x2000, 0x3000, t, t, t, 0x4000, 16, arr, 0x9000, 3, 6, 1, 1, 12, 12, 128,
+                                    0.1, 0, 0, None)
+    assert bwd == -8                                           # workspace too small: nothing is launched

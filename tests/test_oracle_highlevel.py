@@ -121,3 +121,40 @@ def test_group_dropout_scales_earlier_blocks_and_leaves_the_landmark_softmax_alo
     keep_b[..., :nb] = keep.transpose(-1, -2)
     w_high = highlevel.grouped_softmax(att, im, ls, n_buckets, attn_mask=masked, guard_empty=True, group_keep=keep_b)
     assert torch.allclose(w_high, w_drop, atol=1e-14)
+
+
+def _irregular_mask(T, seed, tail):
+    """Landmarks at irregular positions, never two in a row; `tail` tokens without a landmark at the end."""
+    g = torch.Generator().manual_seed(seed)
+    marks, j = [False] * T, 0
+    while True:
+        j += int(torch.randint(2, 7, (1,), generator=g))
+        if j >= T - tail:
+            break
+        marks[j - 1] = True
+    if tail == 0:
+        marks[T - 1] = True
+        if T >= 2 and marks[T - 2]:
+            marks[T - 2] = False
+    return torch.tensor(marks)
+
+
+@pytest.mark.parametrize("T,tail,seed", [(23, 0, 1), (23, 3, 2), (40, 1, 3), (9, 0, 4)])
+def test_irregular_landmarks_equal_the_row_by_row_evaluation(T, tail, seed):
+    # the restatement of the reference's scatter/gather grouped softmax against a literal per-row loop that
+    # shares no code with it: blocks of unequal length, with and without a trailing block without landmark
+    d = 5
+    q, k, v = _rand(1, 1, T, d, seed=20 + seed), _rand(1, 1, T, d, seed=30 + seed), _rand(1, 1, T, d, seed=40 + seed)
+    is_mem = _irregular_mask(T, seed, tail)
+    got = highlevel.attention_lm_benchmark(q, k, v, is_mem[None], n_buckets=int(is_mem.sum()) + 3)
+    want = torch.tensor(s1.s1_rows_python_irregular(q[0, 0], k[0, 0], v[0, 0], is_mem.tolist()), dtype=torch.float64)
+    assert torch.allclose(got[0, 0], want, atol=1e-12)
+
+
+def test_row_by_row_evaluation_for_irregular_landmarks_reduces_to_the_regular_one():
+    T, d, block = 24, 4, 6
+    q, k, v = _rand(1, 1, 12, d, seed=51)[0, 0], _rand(1, 1, T, d, seed=52)[0, 0], _rand(1, 1, T, d, seed=53)[0, 0]
+    is_mem = [(j % block) == block - 1 for j in range(T)]
+    want, _, _ = s1.s1_rows_python(q, k, v, block)
+    got = s1.s1_rows_python_irregular(q, k, v, is_mem)
+    assert torch.allclose(torch.tensor(got), torch.tensor(want), atol=1e-13)
