@@ -79,7 +79,9 @@ __device__ __forceinline__ void wait_vmcnt() {             // s_waitcnt vmcnt(N)
 // p.Lq, p.Lk and the workspace count slots.  Slots without a token need no mask here: the dQ kernel left a = 1e30
 // and mhat = 1e30 for such query rows, so their W and dS are exact zeros whatever rows are read for them, and the
 // accumulator rows of such keys are not stored.
-template <class T, int D, int BS, bool VIRT = false>
+// SEG (with VIRT): blocks of unequal length, rows looked up in p.seg (a template parameter: the lookup in the
+// request stream costs the other variants 5 us at B2 H8 L510 when it is decided at run time).
+template <class T, int D, int BS, bool VIRT = false, bool SEG = false>
 __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   using C = Dkv32Cfg<T, D, BS>;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -165,8 +167,8 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   uint32_t q_vo0 = 0, q_vo1 = 0, g_vo0 = 0, g_vo1 = 0;
   int vrow0 = 0, vcf0 = 0, vcf1 = 0;                       // VIRT: this lane's row inside a tile and its two chunk offsets
   const int nfull_q = p.n_full_q, nfull_k = p.n_full_k;
-  const int* seg_k = VIRT ? p.seg : nullptr;            // blocks of unequal length (null: n_real tokens each)
-  const int* seg_q = (VIRT && p.seg != nullptr) ? p.seg + p.n_prefix : nullptr;   // the queries' first block
+  const int* seg_k = SEG ? p.seg : nullptr;             // blocks of unequal length (null: n_real tokens each)
+  const int* seg_q = SEG ? p.seg + p.n_prefix : nullptr;   // the queries' first block
   if (!role_k) {
     const int chp = lane % C::CH;
     const int row0 = C::RPD * (tile * C::NDMA) + lane / C::CH, row1 = row0 + C::RPD;
@@ -560,10 +562,10 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
 
 #undef LMK_INL
 
-template <class T, int D, int BS, bool VIRT>
+template <class T, int D, int BS, bool VIRT, bool SEG = false>
 static int launch_dkdv32_t(const BwdParams& p, hipStream_t stream) {
   using C = Dkv32Cfg<T, D, BS>;
-  auto kern = lmk_bwd_dkdv32_kernel<T, D, BS, VIRT>;
+  auto kern = lmk_bwd_dkdv32_kernel<T, D, BS, VIRT, SEG>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   // workgroups per head: enough for about one workgroup per CU, at most four 128-key tiles each
@@ -577,6 +579,11 @@ static int launch_dkdv32_t(const BwdParams& p, hipStream_t stream) {
 
 template <class T, int D>
 static int launch_dkdv32_b(const BwdParams& p, int BS, hipStream_t stream) {
+  if (p.Lq_real > 0 && p.seg != nullptr) {                 // token layout, blocks of unequal length
+    if (BS == 64) return launch_dkdv32_t<T, D, 64, true, true>(p, stream);
+    if (BS == 128) return launch_dkdv32_t<T, D, 128, true, true>(p, stream);
+    return LMK_ERR_UNSUPPORTED;
+  }
   if (p.Lq_real > 0) {                                     // token layout: blocks narrower than their 64 or 128 slots
     if (BS == 64) return launch_dkdv32_t<T, D, 64, true>(p, stream);
     if (BS == 128) return launch_dkdv32_t<T, D, 128, true>(p, stream);

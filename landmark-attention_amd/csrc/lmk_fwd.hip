@@ -44,9 +44,12 @@ __device__ __forceinline__ void fwd_dma16(const void* base_uniform, uint32_t vof
                :: "v"(voff), "s"(base_uniform), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory");
 }
 
-template <class T, int D, int BS>
+// SEG: token layout with blocks of unequal length, looked up in p.seg (a template parameter: decided at run time
+// the lookup costs the other launches 7 %).
+template <class T, int D, int BS, bool SEG = false>
 __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   using C = FwdCfg<T, D, BS>;
+  const int* const seg_k = SEG ? p.seg : nullptr;
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -82,7 +85,7 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   // token layout: the tensors' rows are tokens, the kernel's rows are slots
   const bool virt = p.Lq_real > 0;                      // uniform over the launch
   const int nfull_q = p.n_full_q, nfull_k = p.n_full_k;
-  const int* seg_q = p.seg != nullptr ? p.seg + p.n_prefix : nullptr;   // the queries' first block
+  const int* seg_q = SEG ? p.seg + p.n_prefix : nullptr;   // the queries' first block
   const int qtok = !virt ? (qrow < p.Lq ? qrow : -1) : (qrow < p.Lq ? slot_to_token_row<BS>(qrow, p.n_real, nfull_q, seg_q) : -1);
 
   // ---- Q fragments (B operand): query qrow, head dims 16*ks + 8h .. +7
@@ -133,7 +136,7 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
       if (virt) {                                       // the slot's token row, worked out per request
         const int row = C::RPD * (r % n_k) + lane / C::CH, cp = lane % C::CH;
         const int f = (((row & 3) << 2) | ((row >> 2) & 3)) & (C::CH - 1);
-        const int tok = slot_to_token_row_clamped<BS>(min(blk_req * C::SK + row, p.Lk - 1), p.n_real, nfull_k, p.seg);
+        const int tok = slot_to_token_row_clamped<BS>(min(blk_req * C::SK + row, p.Lk - 1), p.n_real, nfull_k, seg_k);
         fwd_dma16(is_v ? vp : kp, (uint32_t)(2 * ((int64_t)tok * (is_v ? p.vs_r : p.ks_r) + 8 * (cp ^ f))), dst);
       } else {
         fwd_dma16(is_v ? vp : kp, last ? src_last[i] : src[i], dst);
@@ -156,7 +159,7 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   // last slot and padding in between: slots n_norm .. BS-2 hold no key and no query may see them.
   // With blocks of unequal length n_norm is the block's at hand (uniform over the workgroup).
   const int n_norm_all = p.n_real - 1;
-  const bool padded = n_norm_all < BS - 1 || p.seg != nullptr;   // uniform over the launch
+  const bool padded = n_norm_all < BS - 1 || SEG;      // uniform over the launch
 
   // LDS byte offsets of this lane's operand fragments inside a 32-row tile: the swizzle repeats every 16
   // rows, so a tile at row 32u is the same offsets plus 32u rows -- an immediate of the LDS instruction
@@ -219,7 +222,8 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
       const int kb = buf * C::STAGE_BYTES + jb * BS * C::ROWB, vb = kb + C::TILE_BYTES;
       // (a stage may reach past the wave's own block, and past the table: those blocks are not looked at)
       int n_norm = n_norm_all;
-      if (p.seg != nullptr && blk <= cblk) n_norm = block_normal_keys<BS>(blk, p.n_real, nfull_k, p.seg);
+      if constexpr (SEG)
+        if (blk <= cblk) n_norm = block_normal_keys<BS>(blk, p.n_real, nfull_k, seg_k);
       if (blk < cblk) {
         // ---------------- earlier block: local softmax gated by its landmark
         float gscale = 1.f;                               // group dropout: this block's factor for this query row
@@ -328,15 +332,20 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   }
 }
 
-template <class T, int D, int BS>
-static int launch_fwd_t(const FwdParams& p, hipStream_t stream) {
+template <class T, int D, int BS, bool SEG>
+static int launch_fwd_s(const FwdParams& p, hipStream_t stream) {
   using C = FwdCfg<T, D, BS>;
-  auto kern = lmk_fwd_kernel<T, D, BS>;
+  auto kern = lmk_fwd_kernel<T, D, BS, SEG>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   const int grid = ((p.Lq + 255) / 256) * p.B * p.H;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * C::NW), C::LDS_BYTES, stream, p);
   return (int)hipGetLastError();
+}
+
+template <class T, int D, int BS>
+static int launch_fwd_t(const FwdParams& p, hipStream_t stream) {
+  return p.seg != nullptr ? launch_fwd_s<T, D, BS, true>(p, stream) : launch_fwd_s<T, D, BS, false>(p, stream);
 }
 
 template <class T>
