@@ -663,7 +663,9 @@ template <int E> struct PieceVec;
 template <> struct PieceVec<8> { using type = u32x4_t; };
 template <> struct PieceVec<4> { using type = u32x2_t; };
 
-template <class T, int D, int BS, bool SPLIT, bool PADDED>
+// MERGE: the row's blocks are picked from the slices' candidates first (p.merge_slices > 0); a template parameter
+// because the four registers it holds on to would cost the plain kernel its third wave per SIMD (172 against 168).
+template <class T, int D, int BS, bool SPLIT, bool PADDED, bool MERGE = false>
 __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   static_assert((D == 128 || D == 64) && (BS == 32 || BS % 64 == 0), "8 lanes x 2 pieces per row; whole chunks of keys");
   constexpr int E = D / 16;                                       // head dims per lane and rotary half: 8 or 4
@@ -707,9 +709,9 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   // The decode-time selection leaves a row's candidates (k per slice of the cache) rather than its indices: the wave
   // picks the k best first -- lane r of `sorted` gets the r-th block in the order of the output -- and one wave per
   // row writes them where the caller expects the indices.
-  const bool merged = p.merge_slices > 0;                          // uniform over the launch
+  constexpr bool merged = MERGE;
   int sorted = 0;
-  if (merged) {
+  if constexpr (MERGE) {
     int mine = merge_slices_row(p, p.merge_slices, row, lane);
     const int rank = rank_ascending(mine, lane, p.k, p.num_mems, p.ring_start);
     sorted = __builtin_amdgcn_ds_permute(4 * (lane < p.k ? rank : lane), mine);
@@ -1012,6 +1014,18 @@ int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landm
 template <class T, int D, int BS, bool PADDED>
 static int launch_gather_b(const RetrParams& p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.B * p.H * p.T;
+  if (p.merge_slices > 0) {               // the selection stopped after its slice step: blocks of 32 as they are only
+    if constexpr (BS == 32 && !PADDED) {
+      if (rows <= 1024 && p.k > 1)
+        hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, true, PADDED, true>), dim3((unsigned)rows), dim3(256), 0, stream, p);
+      else
+        hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, false, PADDED, true>), dim3((unsigned)((rows + 3) / 4)), dim3(256),
+                           0, stream, p);
+      return (int)hipGetLastError();
+    } else {
+      return LMK_ERR_UNSUPPORTED;
+    }
+  }
   if (rows <= 1024 && p.k > 1) {          // fewer rows than SIMDs: one workgroup per row, its waves share the blocks out
     hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, true, PADDED>), dim3((unsigned)rows), dim3(256), 0, stream, p);
   } else {
