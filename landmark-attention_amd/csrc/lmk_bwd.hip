@@ -98,8 +98,11 @@ struct DqCfg {
 // One 1 KB direct global->LDS request of a wave: lane i's 16 bytes land at lds_off + 16*i.
 // lds_off must be wave-uniform (it travels in M0).
 __device__ __forceinline__ void dq_dma16(const void* base_uniform, uint32_t voff, uint32_t lds_off) {
+  const uint64_t b = (uint64_t)base_uniform;
+  const uint64_t base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b >> 32)) << 32) |
+                        (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :: "v"(voff), "s"(base_uniform), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory");
+               :: "v"(voff), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory");
 }
 
 // VIRT: tensors in token layout (p.Lq_real > 0); a template parameter because the slot arithmetic costs the
@@ -205,7 +208,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   }
   const uint32_t step_k = (uint32_t)(2 * (int64_t)BS * p.ks_r), step_v = (uint32_t)(2 * (int64_t)BS * p.vs_r);
   int blk_req = 0;                                         // block the next request fetches
-  auto request = [&](int buf) {                            // next block in key order -> buffer buf
+  auto request = [&](int buf) __attribute__((always_inline)) {   // next block in key order -> buffer buf
 #pragma unroll
     for (int i = 0; i < C::PER_WAVE; ++i) {
       const int r = wave * C::PER_WAVE + i;
@@ -240,7 +243,12 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   // rows, so a tile at row 32u is the same offsets plus 32u rows -- an immediate of the LDS instruction
   int koff[C::KS];
 #pragma unroll
-  for (int ks = 0; ks < C::KS; ++ks) koff[ks] = tile_off<D>(ql, 2 * ks + h);
+  for (int ks = 0; ks < C::KS; ++ks) {
+    koff[ks] = tile_off<D>(ql, 2 * ks + h);
+    // the compiler must not know the value's range: it would turn "offset + constant" into an OR computed by a
+    // vector instruction per read; as a plain sum the constant stays the read's immediate offset
+    asm volatile("" : "+v"(koff[ks]));
+  }
   int voff[C::DC][2];
   {
     const int i = lane & 15, g2 = (lane >> 4) & 1;
@@ -248,11 +256,70 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     for (int dc = 0; dc < C::DC; ++dc) {
       const int col = 32 * dc + 16 * g2 + 4 * (i & 3);
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf)
+      for (int hf = 0; hf < 2; ++hf) {
         voff[dc][hf] = tile_off<D>(4 * h + (i >> 2) + 8 * hf, col >> 3) + ((col >> 2) & 1) * 8;
+        asm volatile("" : "+v"(voff[dc][hf]));             // as for koff
+      }
     }
   }
-  auto row_tile = [&](int tile_bytes, const u32x4_t* bf) {   // (32 rows of the LDS tile) x (this wave's 32 queries)
+  // The wave issues in order, so in the earlier blocks' code the instruction stream is the schedule: every LDS
+  // operand is asked for two MFMAs ahead of its use and the order is pinned.
+  // (32 rows each of NTL consecutive LDS tiles) x (this wave's 32 queries)
+  auto row_tiles = [&](int tile_bytes, const u32x4_t* bf, f32x16_t* out, auto ntl_c) __attribute__((always_inline)) {
+    constexpr int NX = decltype(ntl_c)::value * C::KS, PFX = 2;
+    u32x4_t fk[NX];
+#pragma unroll
+    for (int n = 0; n < PFX; ++n) fk[n] = lds_ld128(tile_bytes + 32 * (n / C::KS) * C::ROWB + koff[n % C::KS]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < NX; ++n) {
+      if (n + PFX < NX) fk[n + PFX] = lds_ld128(tile_bytes + 32 * ((n + PFX) / C::KS) * C::ROWB + koff[(n + PFX) % C::KS]);
+      const int u = n / C::KS, ks = n % C::KS;
+      if (ks == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) out[u][r] = 0.f;
+      }
+      out[u] = mfma32<T>(fk[n], bf[ks], out[u]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // dQ^T += (K tiles)^T dS^T for NTL consecutive tiles, dS = e f (dP - nD) in slices of 16 keys: a slice is formed
+  // and packed under the MFMAs of the one before.  u0: first tile's index in the block (the landmark is the last
+  // tile's last key); dP of tile u0 + i is d[d_stride * i].
+  auto dq_tiles = [&](int tile_bytes, int u0, const f32x16_t* e, const f32x16_t* d, int d_stride, float f, float nD,
+                      float dslm, auto ntl_c) __attribute__((always_inline)) {
+    constexpr int NTL = decltype(ntl_c)::value, NZ = NTL * 2 * C::DC, PFZ = 2;
+    auto zload = [&](int n) __attribute__((always_inline)) {
+      const int sl = n / C::DC, dc = n % C::DC;
+      const int base = tile_bytes + 16 * sl * C::ROWB;
+      const u32x2_t a0 = lds_ld_tr(base + voff[dc][0]), a1 = lds_ld_tr(base + voff[dc][1]);
+      const u32x4_t a = {a0[0], a0[1], a1[0], a1[1]};
+      return a;
+    };
+    auto slice = [&](int sl) __attribute__((always_inline)) {
+      const int i = sl >> 1, j = sl & 1;
+      float ds[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) ds[r] = e[i][8 * j + r] * f * (d[d_stride * i][8 * j + r] - nD);
+      if (j == 1 && u0 + i == C::NT - 1 && h == 1) ds[7] = dslm;
+      const u32x4_t wf = {pack2<T>(ds[0], ds[1]), pack2<T>(ds[2], ds[3]), pack2<T>(ds[4], ds[5]), pack2<T>(ds[6], ds[7])};
+      return wf;
+    };
+    u32x4_t zf[NZ], wf[2];
+#pragma unroll
+    for (int n = 0; n < PFZ; ++n) zf[n] = zload(n);
+    wf[0] = slice(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < NZ; ++n) {
+      if (n + PFZ < NZ) zf[n + PFZ] = zload(n + PFZ);
+      const int sl = n / C::DC, dc = n % C::DC;
+      acc[dc] = mfma32<T>(zf[n], wf[sl & 1], acc[dc]);
+      if (dc == 0 && sl + 1 < 2 * NTL) wf[(sl + 1) & 1] = slice(sl + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto row_tile = [&](int tile_bytes, const u32x4_t* bf) __attribute__((always_inline)) {   // one tile, the compiler's order
     f32x16_t s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.f;
@@ -260,7 +327,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     for (int ks = 0; ks < C::KS; ++ks) s = mfma32<T>(lds_ld128(tile_bytes + koff[ks]), bf[ks], s);
     return s;
   };
-  auto dq_tile = [&](int tile_bytes, const float* ds) {      // dQ^T += (K tile)^T dS^T
+  auto dq_tile = [&](int tile_bytes, const float* ds) __attribute__((always_inline)) {   // dQ^T += (K tile)^T dS^T
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       u32x4_t wf = {pack2<T>(ds[8 * j + 0], ds[8 * j + 1]), pack2<T>(ds[8 * j + 2], ds[8 * j + 3]),
@@ -275,83 +342,106 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     }
   };
 
-  request(0);
-  for (int s = 0; s < n_stages; ++s) {
-    const int buf = s & 1;
-    __builtin_amdgcn_s_waitcnt(0x0f70);                    // vmcnt(0): this wave's share of stage s has landed
-    __syncthreads();                                       // ... and everyone's; stage s-1 has been consumed
-    if (s + 1 < n_stages) request(buf ^ 1);
-    const int kb = buf * C::STAGE_BYTES, vb = kb + C::TILE_BYTES;   // LDS byte addresses (the dynamic array starts at 0)
-    if (!active) continue;
+  const uint32_t stat_row = 4u * (uint32_t)qrow;
+  // ---------------- earlier block s at LDS byte addresses kb (K rows) / vb (V rows)
+  auto earlier_block = [&](const int kb, const int vb, const int s) __attribute__((always_inline)) {
     int n_norm = n_norm_all;
-    if constexpr (SEG)
-      if (s <= cblk) n_norm = block_normal_keys<BS>(s, p.n_real, nfull_k, seg_k);
-    if (s < cblk) {
-      float gscale = 1.f;                                  // group dropout: this block's factor for this query row
-      if constexpr (VIRT)
-        if (p.group_scale != nullptr && qtok >= 0) gscale = p.group_scale[(int64_t)bh * p.gs_bh + (int64_t)s * p.gs_blk + qtok];
-      f32x16_t sc[C::NT], dp[C::KEEP_DP ? C::NT : 1];
-#pragma unroll
-      for (int u = 0; u < C::NT; ++u) sc[u] = row_tile(kb + 32 * u * C::ROWB, qf);
-      if (padded) {                                        // padding slots leave the local softmax
-#pragma unroll
-        for (int u = 0; u < C::NT; ++u)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int kl = 32 * u + 8 * (r >> 2) + 4 * h + (r & 3);
-            if (kl >= n_norm && kl < BS - 1) sc[u][r] = -INFINITY;
-          }
-      }
-      const float s_last = sc[C::NT - 1][15];
-      float mx = (h == 0) ? s_last : -INFINITY;
+    if constexpr (SEG) n_norm = block_normal_keys<BS>(s, p.n_real, nfull_k, seg_k);
+    float gscale = 1.f;                                    // group dropout: this block's factor for this query row
+    if constexpr (VIRT)
+      if (p.group_scale != nullptr && qtok >= 0) gscale = p.group_scale[(int64_t)bh * p.gs_bh + (int64_t)s * p.gs_blk + qtok];
+    f32x16_t sc[C::NT], dp[C::KEEP_DP ? C::NT : 1];
+    row_tiles(kb, qf, sc, std::integral_constant<int, C::NT>{});
+    if constexpr (C::KEEP_DP) row_tiles(vb, gf, dp, std::integral_constant<int, C::NT>{});
+    if (padded) {                                          // padding slots leave the local softmax
 #pragma unroll
       for (int u = 0; u < C::NT; ++u)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (!(u == C::NT - 1 && r == 15)) mx = fmaxf(mx, sc[u][r]);
-      mx = pair_max(mx);
-      const float t_lm = pair_hi(s_last) * c2;
-      const float mloc = mx * c2;
-      float den = 0.f, spd = 0.f;
-#pragma unroll
-      for (int u = 0; u < C::NT; ++u) {
-        f32x16_t& d = dp[C::KEEP_DP ? u : 0];
-        d = row_tile(vb + 32 * u * C::ROWB, gf);
-#pragma unroll
         for (int r = 0; r < 16; ++r) {
-          float e = fast_exp2(__builtin_fmaf(sc[u][r], c2, -mloc));
-          if (u == C::NT - 1 && r == 15) e = (h == 0) ? e : 0.f;
-          sc[u][r] = e;
-          den += e;
-          spd = __builtin_fmaf(e, d[r], spd);
+          const int kl = 32 * u + 8 * (r >> 2) + 4 * h + (r & 3);
+          if (kl >= n_norm && kl < BS - 1) sc[u][r] = -INFINITY;
         }
+    }
+    const float s_last = sc[C::NT - 1][15];
+    float mx = (h == 0) ? s_last : -INFINITY;
+#pragma unroll
+    for (int u = 0; u < C::NT; ++u)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (!(u == C::NT - 1 && r == 15)) mx = fmaxf(mx, sc[u][r]);
+    mx = pair_max(mx);
+    const float t_lm = pair_hi(s_last) * c2;
+    const float mloc = mx * c2;
+    float den = 0.f, spd = 0.f;
+#pragma unroll
+    for (int u = 0; u < C::NT; ++u) {
+      if constexpr (!C::KEEP_DP) row_tiles(vb + 32 * u * C::ROWB, gf, dp, std::integral_constant<int, 1>{});
+      const f32x16_t& d = dp[C::KEEP_DP ? u : 0];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float e = fast_exp2(__builtin_fmaf(sc[u][r], c2, -mloc));
+        if (u == C::NT - 1 && r == 15) e = (h == 0) ? e : 0.f;
+        sc[u][r] = e;
+        den += e;
+        spd = __builtin_fmaf(e, d[r], spd);
       }
-      den = pair_sum(den);
-      spd = pair_sum(spd);
-      const float invden = fast_rcp(den);
-      const float nD = spd * invden;
-      const float glog = t_lm - mhat;                      // log2 of the normalised gate
-      const float g = fast_exp2(glog);
-      // out_i = .. + gscale * g * (P V): the weights carry the factor, the landmark's dS sees it through nD
-      const float f = g * invden * gscale;
-      const float dslm = g * (gscale * nD - delta);        // dS at the block's landmark key
-      if (h == 0) {
-        const int64_t si = ((int64_t)bh * p.n_blocks + s) * p.Lq + qrow;
-        p.stat_a[si] = gscale > 0.f ? mloc + fast_log2(den) - glog - fast_log2(gscale) : 1e30f;
-        p.stat_n[si] = nD;
-        p.stat_l[si] = dslm;
-      }
+    }
+    den = pair_sum(den);
+    spd = pair_sum(spd);
+    const float invden = fast_rcp(den);
+    const float nD = spd * invden;
+    const float glog = t_lm - mhat;                        // log2 of the normalised gate
+    const float g = fast_exp2(glog);
+    // out_i = .. + gscale * g * (P V): the weights carry the factor, the landmark's dS sees it through nD
+    const float f = g * invden * gscale;
+    const float dslm = g * (gscale * nD - delta);          // dS at the block's landmark key
+    if (h == 0) {                                          // a scalar base per (head, block) plus the row's 32-bit offset
+      const int64_t sb = 4 * ((int64_t)bh * p.n_blocks + s) * p.Lq;
+      *(float*)((char*)p.stat_a + sb + stat_row) = gscale > 0.f ? mloc + fast_log2(den) - glog - fast_log2(gscale) : 1e30f;
+      *(float*)((char*)p.stat_n + sb + stat_row) = nD;
+      *(float*)((char*)p.stat_l + sb + stat_row) = dslm;
+    }
+    if constexpr (C::KEEP_DP) {
+      dq_tiles(kb, 0, sc, dp, 1, f, nD, dslm, std::integral_constant<int, C::NT>{});
+    } else {
 #pragma unroll
       for (int u = 0; u < C::NT; ++u) {
-        if (!C::KEEP_DP) dp[0] = row_tile(vb + 32 * u * C::ROWB, gf);
-        const f32x16_t& d = dp[C::KEEP_DP ? u : 0];
-        float ds[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) ds[r] = sc[u][r] * f * (d[r] - nD);
-        if (u == C::NT - 1 && h == 1) ds[15] = dslm;
-        dq_tile(kb + 32 * u * C::ROWB, ds);
+        row_tiles(vb + 32 * u * C::ROWB, gf, dp, std::integral_constant<int, 1>{});
+        dq_tiles(kb + 32 * u * C::ROWB, u, sc + u, dp, 0, f, nD, dslm, std::integral_constant<int, 1>{});
       }
+    }
+  };
+
+  // Stages in front of the workgroup's first query block are earlier blocks for every wave: they run two at a
+  // time without a branch, the LDS addresses of both buffers as immediates of the instructions.
+  const int first_cblk = (p.n_prefix * C::NT + qt * 8) / C::NT;   // wave 0's own block: the least of the workgroup's
+  const int s_uniform = min(first_cblk, n_stages - 1);
+  auto uniform_stage = [&](auto buf_c, int s) __attribute__((always_inline)) {
+    constexpr int buf = decltype(buf_c)::value;
+    __builtin_amdgcn_s_waitcnt(0x0f70);                    // vmcnt(0): this wave's share of stage s has landed
+    __syncthreads();                                       // ... and everyone's; stage s-1 has been consumed
+    request(buf ^ 1);
+    if (active) earlier_block(buf * C::STAGE_BYTES, buf * C::STAGE_BYTES + C::TILE_BYTES, s);
+  };
+
+  request(0);
+  int s = 0;
+  for (; s + 2 <= s_uniform; s += 2) {
+    uniform_stage(std::integral_constant<int, 0>{}, s);
+    uniform_stage(std::integral_constant<int, 1>{}, s + 1);
+  }
+  for (; s < n_stages; ++s) {
+    const int buf = s & 1;
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    if (s + 1 < n_stages) request(buf ^ 1);
+    const int kb = buf * C::STAGE_BYTES, vb = kb + C::TILE_BYTES;   // LDS byte addresses (the dynamic array starts at 0)
+    if (!active) continue;
+    if (s < cblk) {
+      earlier_block(kb, vb, s);
     } else if (s == cblk) {
+      int n_norm = n_norm_all;
+      if constexpr (SEG) n_norm = block_normal_keys<BS>(s, p.n_real, nfull_k, seg_k);
       const int lim = ql - ((tsub == C::NT - 1 && ql == 31) ? 1 : 0);
 #pragma unroll
       for (int u = 0; u < C::NT; ++u) {
