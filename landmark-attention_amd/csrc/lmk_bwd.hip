@@ -352,7 +352,6 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
       if (p.group_scale != nullptr && qtok >= 0) gscale = p.group_scale[(int64_t)bh * p.gs_bh + (int64_t)s * p.gs_blk + qtok];
     f32x16_t sc[C::NT], dp[C::KEEP_DP ? C::NT : 1];
     row_tiles(kb, qf, sc, std::integral_constant<int, C::NT>{});
-    if constexpr (C::KEEP_DP) row_tiles(vb, gf, dp, std::integral_constant<int, C::NT>{});
     if (padded) {                                          // padding slots leave the local softmax
 #pragma unroll
       for (int u = 0; u < C::NT; ++u)
@@ -364,26 +363,78 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     }
     const float s_last = sc[C::NT - 1][15];
     float mx = (h == 0) ? s_last : -INFINITY;
+    float t_lm = 0.f, mloc = 0.f, den = 0.f, spd = 0.f;
+    if constexpr (C::KEEP_DP) {
+      // dP^T does not depend on S^T: at head dim 64 its MFMAs carry the local softmax of the scores, a slice behind
+      // each -- first the maximum (one slice per tile), then the exponentials and their sum.  (At head dim 128 the
+      // same placement measured 7 % slower than the softmax behind the MFMAs, in the compiler's order.)
+      constexpr bool UNDER = D == 64;
+      constexpr int NX = C::NT * C::KS, PFX = 2, NEXP = NX - C::NT, PER = (16 * C::NT + NEXP - 1) / NEXP;
+      auto ywork = [&](int n) __attribute__((always_inline)) {
+        if (n < C::NT) {
 #pragma unroll
-    for (int u = 0; u < C::NT; ++u)
+          for (int r = 0; r < 16; ++r)
+            if (!(n == C::NT - 1 && r == 15)) mx = fmaxf(mx, sc[n][r]);
+          if (n == C::NT - 1) {
+            mx = pair_max(mx);
+            t_lm = pair_hi(s_last) * c2;
+            mloc = mx * c2;
+          }
+        } else {
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        if (!(u == C::NT - 1 && r == 15)) mx = fmaxf(mx, sc[u][r]);
-    mx = pair_max(mx);
-    const float t_lm = pair_hi(s_last) * c2;
-    const float mloc = mx * c2;
-    float den = 0.f, spd = 0.f;
+          for (int i = (n - C::NT) * PER; i < (n - C::NT + 1) * PER && i < 16 * C::NT; ++i) {
+            const int u = i >> 4, r = i & 15;
+            float e = fast_exp2(__builtin_fmaf(sc[u][r], c2, -mloc));
+            if (u == C::NT - 1 && r == 15) e = (h == 0) ? e : 0.f;
+            sc[u][r] = e;
+            den += e;
+          }
+        }
+      };
+      u32x4_t fk[NX];
 #pragma unroll
-    for (int u = 0; u < C::NT; ++u) {
-      if constexpr (!C::KEEP_DP) row_tiles(vb + 32 * u * C::ROWB, gf, dp, std::integral_constant<int, 1>{});
-      const f32x16_t& d = dp[C::KEEP_DP ? u : 0];
+      for (int n = 0; n < PFX; ++n) fk[n] = lds_ld128(vb + 32 * (n / C::KS) * C::ROWB + koff[n % C::KS]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float e = fast_exp2(__builtin_fmaf(sc[u][r], c2, -mloc));
-        if (u == C::NT - 1 && r == 15) e = (h == 0) ? e : 0.f;
-        sc[u][r] = e;
-        den += e;
-        spd = __builtin_fmaf(e, d[r], spd);
+      for (int n = 0; n < NX; ++n) {
+        if (n + PFX < NX) fk[n + PFX] = lds_ld128(vb + 32 * ((n + PFX) / C::KS) * C::ROWB + koff[(n + PFX) % C::KS]);
+        const int u = n / C::KS, ks = n % C::KS;
+        if (ks == 0) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) dp[u][r] = 0.f;
+        }
+        dp[u] = mfma32<T>(fk[n], gf[ks], dp[u]);
+        if constexpr (UNDER) ywork(n);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (!UNDER) {
+#pragma unroll
+        for (int n = 0; n < NX; ++n) ywork(n);
+      }
+#pragma unroll
+      for (int u = 0; u < C::NT; ++u)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) spd = __builtin_fmaf(sc[u][r], dp[u][r], spd);
+    } else {
+#pragma unroll
+      for (int u = 0; u < C::NT; ++u)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (!(u == C::NT - 1 && r == 15)) mx = fmaxf(mx, sc[u][r]);
+      mx = pair_max(mx);
+      t_lm = pair_hi(s_last) * c2;
+      mloc = mx * c2;
+#pragma unroll
+      for (int u = 0; u < C::NT; ++u) {
+        row_tiles(vb + 32 * u * C::ROWB, gf, dp, std::integral_constant<int, 1>{});
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float e = fast_exp2(__builtin_fmaf(sc[u][r], c2, -mloc));
+          if (u == C::NT - 1 && r == 15) e = (h == 0) ? e : 0.f;
+          sc[u][r] = e;
+          den += e;
+          spd = __builtin_fmaf(e, dp[0][r], spd);
+        }
       }
     }
     den = pair_sum(den);
