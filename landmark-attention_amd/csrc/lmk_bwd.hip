@@ -108,9 +108,12 @@ __device__ __forceinline__ void dq_dma16(const void* base_uniform, uint32_t voff
 // VIRT: tensors in token layout (p.Lq_real > 0); a template parameter because the slot arithmetic costs the
 // slot-layout instantiations registers they do not have.
 // SEG (with VIRT): blocks of unequal length, looked up in p.seg -- a template parameter for the same reason.
-template <class T, int D, int BS, bool VIRT, bool SEG = false>
+// PLAIN (without VIRT): every block has BS tokens in its BS slots -- no padding slots to mask; the masks' scalar
+// registers and the branch are what it saves the common case.
+template <class T, int D, int BS, bool VIRT, bool SEG = false, bool PLAIN = false>
 __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   static_assert(VIRT || !SEG, "the table describes tensors in token layout");
+  static_assert(!PLAIN || !VIRT, "plain: the tensors' rows are the kernel's rows");
   using C = DqCfg<T, D, BS>;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -237,7 +240,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
   // last slot and padding in between: slots n_norm .. BS-2 hold no key and no query may see them.
   // With blocks of unequal length n_norm is the stage's block's (uniform over the workgroup).
   const int n_norm_all = p.n_real - 1;
-  const bool padded = n_norm_all < BS - 1 || seg_k != nullptr;   // uniform over the launch
+  const bool padded = !PLAIN && (n_norm_all < BS - 1 || seg_k != nullptr);   // uniform over the launch
 
   // LDS byte offsets of this lane's operand fragments inside a 32-row tile: the swizzle repeats every 16
   // rows, so a tile at row 32u is the same offsets plus 32u rows -- an immediate of the LDS instruction
@@ -553,6 +556,11 @@ static int launch_bwd_t(const BwdParams& p, int phases, hipStream_t stream) {
         hipLaunchKernelGGL(kern, grid, dim3(64 * C::NW), C::LDS_BYTES, stream, p);
       } else if (p.Lq_real > 0) {
         auto kern = lmk_bwd_dq_kernel<T, D, BS, true>;
+        static std::atomic<uint64_t> lds_ok{0};
+        if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
+        hipLaunchKernelGGL(kern, grid, dim3(64 * C::NW), C::LDS_BYTES, stream, p);
+      } else if (p.n_real == BS) {
+        auto kern = lmk_bwd_dq_kernel<T, D, BS, false, false, true>;
         static std::atomic<uint64_t> lds_ok{0};
         if ((rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok))) return rc;
         hipLaunchKernelGGL(kern, grid, dim3(64 * C::NW), C::LDS_BYTES, stream, p);

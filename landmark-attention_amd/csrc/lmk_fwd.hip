@@ -54,8 +54,12 @@ __device__ __forceinline__ void fwd_dma16(const void* base_uniform, uint32_t vof
 // the lookup costs the other launches 7 %).
 // GS: group dropout factors in p.group_scale (a template parameter as well: the load's wait for the memory counter
 // would otherwise sit in every launch's loop, where it also waits for the next stage's requests).
-template <class T, int D, int BS, bool SEG = false, bool GS = false>
+// PLAIN: every block has BS tokens in BS slots and the tensors' rows are the kernel's rows (the common case: the
+// token-layout and padding paths, decided at run time, cost it 5 % -- 24 registers and the scalar registers of
+// their masks).
+template <class T, int D, int BS, bool SEG = false, bool GS = false, bool PLAIN = false>
 __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
+  static_assert(!PLAIN || (!SEG && !GS), "the plain variant has no table and no factors");
   using C = FwdCfg<T, D, BS>;
   const int* const seg_k = SEG ? p.seg : nullptr;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -91,7 +95,7 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   const bool active = q0 < p.Lq;
   const int qrow = q0 + ql;
   // token layout: the tensors' rows are tokens, the kernel's rows are slots
-  const bool virt = p.Lq_real > 0;                      // uniform over the launch
+  const bool virt = !PLAIN && p.Lq_real > 0;            // uniform over the launch
   const int nfull_q = p.n_full_q, nfull_k = p.n_full_k;
   const int* seg_q = SEG ? p.seg + p.n_prefix : nullptr;   // the queries' first block
   const int qtok = !virt ? (qrow < p.Lq ? qrow : -1) : (qrow < p.Lq ? slot_to_token_row<BS>(qrow, p.n_real, nfull_q, seg_q) : -1);
@@ -167,7 +171,7 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   // last slot and padding in between: slots n_norm .. BS-2 hold no key and no query may see them.
   // With blocks of unequal length n_norm is the block's at hand (uniform over the workgroup).
   const int n_norm_all = p.n_real - 1;
-  const bool padded = n_norm_all < BS - 1 || SEG;      // uniform over the launch
+  const bool padded = !PLAIN && (n_norm_all < BS - 1 || SEG);   // uniform over the launch
 
   // LDS byte offsets of this lane's operand fragments inside a 32-row tile: the swizzle repeats every 16
   // rows, so a tile at row 32u is the same offsets plus 32u rows -- an immediate of the LDS instruction
@@ -454,10 +458,10 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   }
 }
 
-template <class T, int D, int BS, bool SEG, bool GS>
+template <class T, int D, int BS, bool SEG, bool GS, bool PLAIN = false>
 static int launch_fwd_s(const FwdParams& p, hipStream_t stream) {
   using C = FwdCfg<T, D, BS>;
-  auto kern = lmk_fwd_kernel<T, D, BS, SEG, GS>;
+  auto kern = lmk_fwd_kernel<T, D, BS, SEG, GS, PLAIN>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_dynamic_lds(kern, C::LDS_BYTES, lds_ok)) return rc;
   const int grid = ((p.Lq + 255) / 256) * p.B * p.H;
@@ -468,7 +472,9 @@ static int launch_fwd_s(const FwdParams& p, hipStream_t stream) {
 template <class T, int D, int BS>
 static int launch_fwd_t(const FwdParams& p, hipStream_t stream) {
   if (p.seg != nullptr) return p.group_scale != nullptr ? LMK_ERR_UNSUPPORTED : launch_fwd_s<T, D, BS, true, false>(p, stream);
-  return p.group_scale != nullptr ? launch_fwd_s<T, D, BS, false, true>(p, stream) : launch_fwd_s<T, D, BS, false, false>(p, stream);
+  if (p.group_scale != nullptr) return launch_fwd_s<T, D, BS, false, true>(p, stream);
+  if (p.Lq_real <= 0 && p.n_real == BS) return launch_fwd_s<T, D, BS, false, false, true>(p, stream);
+  return launch_fwd_s<T, D, BS, false, false>(p, stream);
 }
 
 template <class T>
