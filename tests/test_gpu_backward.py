@@ -319,3 +319,19 @@ def test_gradients_at_8192_tokens():
         err = (g.float().cpu() - r).abs().max().item()
         print("L8192", name, "max abs err", err, flush=True)
         assert err <= TOL, (name, err)
+
+
+@pytest.mark.parametrize("L,block,D", [(8960, 64, 64), (6885, 51, 64)])
+def test_gradients_beyond_128_blocks_of_64_slots(L, block, D):
+    # 140 blocks of 64 / 135 blocks of 51 in 64 slots: the 64-slot forward's first pass takes its landmark keys in
+    # two rounds, and the dQ kernel's straight-line stages run for most of the sequence
+    B, H = 1, 1
+    print(f"case L{L} block{block}", flush=True)
+    q, k, v = make_qkv(B, H, L, L, D, seed=L)
+    do = torch.randn(B, H, L, D, generator=torch.Generator().manual_seed(L + 1)).bfloat16()
+    rq, rk, rv = oracle_grads(q, k, v, do, block, chunk=1)
+    gq, gk, gv = _grads(q, k, v, do, block)
+    for name, g, r in (("dq", gq, rq), ("dk", gk, rk), ("dv", gv, rv)):
+        err = (g.float().cpu() - r).abs().max().item()
+        print(f"L{L} block{block}", name, "max abs err", err, flush=True)
+        assert err <= TOL, (name, err)

@@ -88,6 +88,24 @@ def test_long_history_streams_the_landmark_tiles(Lq, Lk):
     assert ((L[:, rows] - L_ref).abs() / L_ref).max() < 1e-3
 
 
+@pytest.mark.parametrize("Lq,Lk,block,D", [(8960, 8960, 64, 128), (256, 9600, 64, 64), (6885, 6885, 51, 64),
+                                            (17024, 17024, 128, 64)])
+def test_more_than_128_earlier_blocks_in_64_and_128_slots(Lq, Lk, block, D):
+    # the 64/128-slot kernel's first pass takes the landmark keys 128 at a time: sequences whose last rows see
+    # more than that, plain, with history, in token layout (blocks of 51 in 64 slots) and at 128 slots
+    from oracle import s1
+    B, H = 1, 2
+    print(f"case first-pass chunks Lq{Lq} Lk{Lk} block{block} D{D}", flush=True)
+    q, k, v = make_qkv(B, H, Lq, Lk, D, seed=Lq + block)
+    rows = sorted({0, 1, block - 1, block, Lq // 2, Lq - block - 1, Lq - block, Lq - 2, Lq - 1})
+    out = _run(q, k, v, block).float().cpu()[0]
+    qf, kf, vf = (t.float()[0] for t in (q, k, v))
+    ref = s1.s1_attention(qf, kf, vf, block, rows=rows)
+    assert (out[:, rows] - ref).abs().max().item() <= TOL
+    ones = torch.ones_like(v)                              # every row: the weights sum to one
+    assert (_run(q, k, ones, block).float() - 1).abs().max().item() <= 1e-2
+
+
 def test_statistics_L_and_M_match_oracle():
     from landmark_hip.attention import _launch_fwd
     B, H, Lq, Lk, D, block = 1, 4, 192, 256, 128, 32
