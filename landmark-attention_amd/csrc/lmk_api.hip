@@ -682,28 +682,43 @@ static int gather_attend_impl(const lmk_tensor4* q, const lmk_tensor4* kcache, c
                               const void* cos_table, const void* sin_table, int64_t table_stride_row, int64_t n_pos,
                               const lmk_tensor4* o_loc, const float* L_loc, const float* M_loc, int64_t stat_stride,
                               const lmk_tensor4* out, int B, int H, int T, int S, int D, float sm_scale, int block,
-                              int top_k, int dtype, void* stream, const lmk::RetrParams* candidates) {
+                              int top_k, int dtype, void* stream, const lmk::RetrParams* candidates,
+                              const lmk_tensor4* k_new = nullptr, const lmk_tensor4* v_new = nullptr) {
+  // k_new, v_new: the gather kernel attends to the rows' local window itself (gather_takes_local_window) and
+  // o_loc, L_loc, M_loc are not read
+  const bool local = k_new != nullptr;
   int rc;
-  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache)) || (rc = check_tensor(vcache)) ||
-      (rc = check_tensor(o_loc)) || (rc = check_tensor(out)))
+  if ((rc = check_tensor(q)) || (rc = check_tensor(kcache)) || (rc = check_tensor(vcache)) || (rc = check_tensor(out)))
     return rc;
-  if (cos_table == nullptr || sin_table == nullptr || idx == nullptr || L_loc == nullptr || M_loc == nullptr)
+  if (local ? ((rc = check_tensor(k_new)) || (rc = check_tensor(v_new))) : (rc = check_tensor(o_loc))) return rc;
+  if (cos_table == nullptr || sin_table == nullptr || idx == nullptr || (!local && (L_loc == nullptr || M_loc == nullptr)))
     return LMK_ERR_NULL;
   if (!aligned16(cos_table) || !aligned16(sin_table) || !stride_ok(table_stride_row)) return LMK_ERR_ALIGN;
   if ((rc = check_retrieval(B, H, T, S, D, block, top_k, dtype, n_pos))) return rc;
   if (!(block == 32 || block == 64 || block == 128)) return LMK_ERR_UNSUPPORTED;
-  if (stat_stride < T) return LMK_ERR_SHAPE;
+  if (!local && stat_stride < T) return LMK_ERR_SHAPE;
+  if (local && !lmk::gather_takes_local_window(T, S, block)) return LMK_ERR_UNSUPPORTED;
   if (!std::isfinite(sm_scale) || !(sm_scale > 0.f)) return LMK_ERR_SCALE;
   lmk::RetrParams p = {};
   fill_retr_common(p, B, H, T, S, D, block, top_k);
   p.q = q->ptr; p.kcache = kcache->ptr; p.vcache = vcache->ptr; p.cos = cos_table; p.sin = sin_table;
   p.idx = const_cast<int64_t*>(idx);
   p.idx_st = p.k; p.idx_sh = (int64_t)T * p.k; p.idx_sb = (int64_t)H * T * p.k;
-  p.o_loc = o_loc->ptr; p.L_loc = L_loc; p.M_loc = M_loc; p.stat_stride = stat_stride; p.out = out->ptr;
+  p.out = out->ptr;
+  if (local) {
+    p.local = 1;
+    p.local_inc = S % block;
+    p.local_row0 = S - S % block;                               // the cache's rows are its positions (llama_mem.py:336-338)
+    p.local_pos0 = p.local_row0;
+    p.k_new = k_new->ptr; p.kns_b = k_new->stride_b; p.kns_h = k_new->stride_h; p.kns_r = k_new->stride_row;
+    p.v_new = v_new->ptr; p.vns_b = v_new->stride_b; p.vns_h = v_new->stride_h; p.vns_r = v_new->stride_row;
+  } else {
+    p.o_loc = o_loc->ptr; p.L_loc = L_loc; p.M_loc = M_loc; p.stat_stride = stat_stride;
+    p.ols_b = o_loc->stride_b; p.ols_h = o_loc->stride_h; p.ols_r = o_loc->stride_row;
+  }
   p.qs_b = q->stride_b; p.qs_h = q->stride_h; p.qs_r = q->stride_row;
   p.kcs_b = kcache->stride_b; p.kcs_h = kcache->stride_h; p.kcs_r = kcache->stride_row;
   p.vcs_b = vcache->stride_b; p.vcs_h = vcache->stride_h; p.vcs_r = vcache->stride_row;
-  p.ols_b = o_loc->stride_b; p.ols_h = o_loc->stride_h; p.ols_r = o_loc->stride_row;
   p.outs_b = out->stride_b; p.outs_h = out->stride_h; p.outs_r = out->stride_row;
   p.cs_r = table_stride_row;
   p.scale_log2 = sm_scale * 1.4426950408889634f;
@@ -1022,6 +1037,9 @@ int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor
   const int inc = S % block;
   const AttendLayout l = attend_layout(B, H, T, S, D, block);
   if (workspace_bytes < l.total) return LMK_ERR_WORKSPACE;
+  if (lmk::gather_takes_local_window(T, S, block))             // a handful of new tokens: one launch, nothing staged
+    return gather_attend_impl(q, kcache, vcache, idx, cos_table, sin_table, table_stride_row, n_pos, nullptr, nullptr,
+                              nullptr, 0, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream, nullptr, k_loc, v_loc);
   char* w = static_cast<char*>(workspace);
   const int64_t W = l.W;
   auto win = [&](size_t off) { return lmk_tensor4{w + off, (int64_t)H * W * D, W * D, (int64_t)D}; };
@@ -1077,6 +1095,19 @@ int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, con
     if ((rc = retrieve_topk_impl(false, q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, retrieve_workspace,
                                  retrieve_workspace_bytes, B, H, T, S, D, block, top_k, dtype, stream, &pr)))
       return rc;
+    if (lmk::gather_takes_local_window(T, S, block)) {
+      // decode: the selection (slice step where it serves, else the fused top-k), then a gather that merges the
+      // slices' candidates and attends to the local window itself -- no window, no forward launch
+      if (lmk::topk_slices(pr) > 0) {
+        if (!reuse_landmark_keys && (rc = lmk::launch_landmark_keys(pr, D, dtype, (hipStream_t)stream))) return rc;
+        if ((rc = lmk::launch_topk_slices(pr, D, dtype, (hipStream_t)stream))) return rc;
+        return gather_attend_impl(q, kcache, vcache, idx_out, cos_table, sin_table, table_stride_row, n_pos, nullptr, nullptr,
+                                  nullptr, 0, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream, &pr, k_loc, v_loc);
+      }
+      if ((rc = lmk::launch_retrieve_topk(pr, D, dtype, reuse_landmark_keys != 0, (hipStream_t)stream))) return rc;
+      return gather_attend_impl(q, kcache, vcache, idx_out, cos_table, sin_table, table_stride_row, n_pos, nullptr, nullptr,
+                                nullptr, 0, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream, nullptr, k_loc, v_loc);
+    }
     lmk::FwdParams pf;
     if (inc) {
       if ((rc = attn_fwd_impl(&q_win, &k_win, &v_win, &o_win, L, M, B, H, (int)W, (int)W, D, sm_scale, block, block, 0, dtype,

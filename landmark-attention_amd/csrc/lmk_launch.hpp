@@ -140,6 +140,11 @@ struct RetrParams {
   int merge_slices;                               // gather step: > 0 = approx / exact hold the candidates of so many slices per row (k each),
                                                   // the k best of which are picked first and written to idx
   int64_t prefix_len;                             // full_len - (k + 1) * block, may be -block
+  // gather step with the rows' local window inside (local != 0): the new tokens' keys and values (rotated by the
+  // caller), the number of cached tokens behind the last complete block, their first row in the cache and its position
+  int local, local_inc;
+  const void *k_new, *v_new;
+  int64_t kns_b, kns_h, kns_r, vns_b, vns_h, vns_r, local_row0, local_pos0;
   int64_t qs_b, qs_h, qs_r, kcs_b, kcs_h, kcs_r, vcs_b, vcs_h, vcs_r, cs_r;
   int64_t ols_b, ols_h, ols_r, outs_b, outs_h, outs_r;
   float sqrt_hd, scale_log2;
@@ -208,6 +213,12 @@ int launch_fwd32_landmark_keys(const FwdParams& pf, const RetrParams& pr, int D,
 // are left in pr.approx / pr.exact for a gather step with merge_slices set
 int launch_fwd32_topk_slices(const FwdParams& pf, const RetrParams& pr, int D, int dtype, hipStream_t stream);
 int launch_landmark_keys(const RetrParams& p, int D, int dtype, hipStream_t stream);   // the rotation alone
+int launch_topk_slices(const RetrParams& p, int D, int dtype, hipStream_t stream);     // the selection's slice step alone
+// rows whose local window the gather kernel attends to itself: block 32, window inside one block, a handful of new tokens
+constexpr int kLocalMaxT = 4;
+inline bool gather_takes_local_window(int T, int S, int block) {
+  return block == 32 && T <= kLocalMaxT && S % block + T <= block;
+}
 // BS: slots per block (32, 64 or 128); p.block <= BS tokens per block in the cache
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream);
 

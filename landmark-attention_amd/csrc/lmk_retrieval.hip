@@ -665,9 +665,17 @@ template <> struct PieceVec<4> { using type = u32x2_t; };
 
 // MERGE: the row's blocks are picked from the slices' candidates first (p.merge_slices > 0); a template parameter
 // because the four registers it holds on to would cost the plain kernel its third wave per SIMD (172 against 168).
-template <class T, int D, int BS, bool SPLIT, bool PADDED, bool MERGE = false>
-__global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
+// LOCAL: the row's local window -- the tokens of the cache behind its last complete block and the new tokens up to
+// the row's own, at most one block together -- is attended to here as well, as one more item of the row's online
+// softmax, instead of coming in as (o_loc, L_loc, M_loc) from a forward launch over a window another launch built:
+// a decode step is then the selection and this kernel.  Its keys join the global bucket directly (own-block rule:
+// causal, the landmark token does not see itself; flash_landmark_attention.py:78-100).
+// With SPLIT the window has a fifth wave of its own.
+template <class T, int D, int BS, bool SPLIT, bool PADDED, bool MERGE = false, bool LOCAL = false>
+__global__ __launch_bounds__((SPLIT && LOCAL) ? 320 : 256) void lmk_gather_attend_kernel(RetrParams p) {
+  constexpr int NWV = (SPLIT && LOCAL) ? 5 : 4;                   // waves of a workgroup
   static_assert((D == 128 || D == 64) && (BS == 32 || BS % 64 == 0), "8 lanes x 2 pieces per row; whole chunks of keys");
+  static_assert(!LOCAL || (BS == 32 && !PADDED), "the local window is one chunk of 32 keys");
   constexpr int E = D / 16;                                       // head dims per lane and rotary half: 8 or 4
   constexpr int PB = 2 * E;                                       // bytes of one piece
   using vec_t = typename PieceVec<E>::type;                       // one piece: E 16-bit values
@@ -680,7 +688,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
   // selected blocks the four waves share out (block js goes to wave js % 4) and merge at the end
   const int64_t row = SPLIT ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
   if (row >= (int64_t)p.B * p.H * p.T) return;                    // SPLIT: the whole workgroup leaves
-  const int js0 = SPLIT ? wave : 0, jstep = SPLIT ? 4 : 1;
+  const int js0 = SPLIT ? (wave < 4 ? wave : p.k) : 0, jstep = SPLIT ? 4 : 1;   // (the window's wave takes no block)
   const int bh = (int)(row / p.T), t = (int)(row % p.T);
   const int b = bh / p.H, hh = bh % p.H;
 
@@ -751,6 +759,70 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       chi[i] = nhi[i];
     }
   };
+  if constexpr (LOCAL) {
+    if (!SPLIT || wave == 4) {
+      const int inc = p.local_inc, own = inc + t;                 // window rows: inc of the cache, then the new tokens
+      const char* kn = (const char*)p.k_new + 2 * (b * p.kns_b + hh * p.kns_h);
+      const char* vn = (const char*)p.v_new + 2 * (b * p.vns_b + hh * p.vns_h);
+      float s_loc[KPG];
+      vec_t vlo[KPG], vhi[KPG];
+#pragma unroll
+      for (int i = 0; i < KPG; ++i) {
+        const int r = g + 8 * i;
+        const bool visible = r <= own && !(r == BS - 1 && own == BS - 1);
+        const int rc = min(r, own);                               // rows behind the row's own are never read
+        const bool cached = rc < inc;
+        const char* kr = (cached ? kc + 2 * ((p.local_row0 + rc) * p.kcs_r) : kn + 2 * ((int64_t)(rc - inc) * p.kns_r)) + PB * j;
+        const char* vr = (cached ? vc + 2 * ((p.local_row0 + rc) * p.vcs_r) : vn + 2 * ((int64_t)(rc - inc) * p.vns_r)) + PB * j;
+        const int64_t pos = inc > 0 ? p.local_pos0 + min(rc, inc - 1) : 0;   // a position the tables hold, used by cached rows only
+        const char* cr = (const char*)p.cos + 2 * (pos * p.cs_r) + PB * j;
+        const char* sr = (const char*)p.sin + 2 * (pos * p.cs_r) + PB * j;
+        float kl[E], kh[E], cl[E], ch[E], sl[E], sh[E];
+        unpack8(*(const vec_t*)(kr), kl);
+        unpack8(*(const vec_t*)(kr + D), kh);
+        unpack8(*(const vec_t*)(cr), cl);
+        unpack8(*(const vec_t*)(cr + D), ch);
+        unpack8(*(const vec_t*)(sr), sl);
+        unpack8(*(const vec_t*)(sr + D), sh);
+        vlo[i] = *(const vec_t*)(vr);
+        vhi[i] = *(const vec_t*)(vr + D);
+        float d = 0.f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {                             // cached keys are rotated in the model dtype, as the cache's
+          const float rl = cached ? round_to<T>(__builtin_fmaf(kl[e], cl[e], -kh[e] * sl[e])) : kl[e];   // window is (llama_mem.py:336-338)
+          const float rh = cached ? round_to<T>(__builtin_fmaf(kh[e], ch[e], kl[e] * sh[e])) : kh[e];
+          d = __builtin_fmaf(qlo[e], rl, d);
+          d = __builtin_fmaf(qhi[e], rh, d);
+        }
+        s_loc[i] = visible ? sum8(d) * c2 : -INFINITY;
+      }
+      float mx = s_loc[0];                                        // row 0 is always visible
+#pragma unroll
+      for (int i = 1; i < KPG; ++i) mx = fmaxf(mx, s_loc[i]);
+      mx = fmaxf(mx, dpp_f<0x128>(mx));
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      float den = 0.f;
+#pragma unroll
+      for (int i = 0; i < KPG; ++i) {
+        const float e = fast_exp2(s_loc[i] - mx);
+        den += e;
+        const float w = round_to<T>(e);                           // weights enter PV in the model dtype
+#pragma unroll
+        for (int e2 = 0; e2 < E / 2; ++e2) {
+          alo[2 * e2] = __builtin_fmaf(w, unpack_lo<T>(vlo[i][e2]), alo[2 * e2]);
+          alo[2 * e2 + 1] = __builtin_fmaf(w, unpack_hi<T>(vlo[i][e2]), alo[2 * e2 + 1]);
+          ahi[2 * e2] = __builtin_fmaf(w, unpack_lo<T>(vhi[i][e2]), ahi[2 * e2]);
+          ahi[2 * e2 + 1] = __builtin_fmaf(w, unpack_hi<T>(vhi[i][e2]), ahi[2 * e2 + 1]);
+        }
+      }
+      den += dpp_f<0x128>(den);
+      den += __shfl_xor(den, 16, 64);
+      den += __shfl_xor(den, 32, 64);
+      Mrun = mx;
+      lrun = den;
+    }
+  }
   int blk = 0;
   if (js0 < p.k) {
     blk = picked(js0);
@@ -852,8 +924,8 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     ahi[e] += __shfl_xor(ahi[e], 32, 64);
   }
   if constexpr (SPLIT) {                                          // the four waves' partial (M, l, acc) -> wave 0
-    __shared__ float part_acc[4][D];
-    __shared__ float part_ml[4][2];
+    __shared__ float part_acc[NWV][D];
+    __shared__ float part_ml[NWV][2];
     if (g == 0) {
 #pragma unroll
       for (int e = 0; e < E; ++e) {
@@ -869,7 +941,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
     if (wave != 0) return;
     float Mall = part_ml[0][0];                                   // wave 0 always has a block (k >= 1)
 #pragma unroll
-    for (int w = 1; w < 4; ++w) Mall = fmaxf(Mall, part_ml[w][0]);
+    for (int w = 1; w < NWV; ++w) Mall = fmaxf(Mall, part_ml[w][0]);
     lrun = 0.f;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -877,7 +949,7 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       ahi[e] = 0.f;
     }
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NWV; ++w) {
       const float sw = fast_exp2(part_ml[w][0] - Mall);           // 0 for a wave without blocks (M = -inf)
       lrun = __builtin_fmaf(part_ml[w][1], sw, lrun);
 #pragma unroll
@@ -887,6 +959,20 @@ __global__ __launch_bounds__(256) void lmk_gather_attend_kernel(RetrParams p) {
       }
     }
     Mrun = Mall;
+  }
+  if constexpr (LOCAL) {                                          // the local window is in the sums already
+    const float inv = 1.0f / lrun;
+    if (g == 0) {
+      char* outp = (char*)p.out + 2 * (b * p.outs_b + hh * p.outs_h + (int64_t)t * p.outs_r) + PB * j;
+      vec_t ov;
+#pragma unroll
+      for (int i = 0; i < E / 2; ++i) ov[i] = pack2<T>(alo[2 * i] * inv, alo[2 * i + 1] * inv);
+      *(vec_t*)(outp) = ov;
+#pragma unroll
+      for (int i = 0; i < E / 2; ++i) ov[i] = pack2<T>(ahi[2 * i] * inv, ahi[2 * i + 1] * inv);
+      *(vec_t*)(outp + D) = ov;
+    }
+    return;
   }
   // merge with the local chunk: out_loc (normalised), L_loc, M_loc (natural-log units)
   const int64_t srow = (int64_t)bh * p.stat_stride + t;
@@ -989,6 +1075,28 @@ static int launch_lk_t(const RetrParams& p, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
+// The slice step of the selection alone (topk_slices(p) > 0): a row's candidates stay in p.approx / p.exact for a
+// gather step that merges them (RetrParams::merge_slices).
+template <class T, int D>
+static int launch_slices_t(const RetrParams& p, hipStream_t stream) {
+  const int n_slices = topk_slices(p);
+  if (n_slices <= 0) return LMK_ERR_UNSUPPORTED;
+  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  hipLaunchKernelGGL((lmk_topk_slice_kernel<T, D>), dim3((unsigned)(rows * n_slices)), dim3(64 * kSliceWaves), 0, stream, p, n_slices);
+  return (int)hipGetLastError();
+}
+
+int launch_topk_slices(const RetrParams& p, int D, int dtype, hipStream_t stream) {
+  if (dtype == LMK_DTYPE_BF16) {
+    if (D == 128) return launch_slices_t<bf16_t, 128>(p, stream);
+    if (D == 64) return launch_slices_t<bf16_t, 64>(p, stream);
+  } else if (dtype == LMK_DTYPE_F16) {
+    if (D == 128) return launch_slices_t<f16_t, 128>(p, stream);
+    if (D == 64) return launch_slices_t<f16_t, 64>(p, stream);
+  }
+  return LMK_ERR_UNSUPPORTED;
+}
+
 int launch_landmark_keys(const RetrParams& p, int D, int dtype, hipStream_t stream) {
   if (dtype == LMK_DTYPE_BF16) {
     if (D == 128) return launch_lk_t<bf16_t, 128>(p, stream);
@@ -1014,6 +1122,22 @@ int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landm
 template <class T, int D, int BS, bool PADDED>
 static int launch_gather_b(const RetrParams& p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.B * p.H * p.T;
+  if (p.local) {                          // with the row's local window: blocks of 32 as they are only
+    if constexpr (BS == 32 && !PADDED) {
+      const bool split = rows <= 1024 && p.k > 1;
+      const dim3 grid((unsigned)(split ? rows : (rows + 3) / 4));
+      if (p.merge_slices > 0) {
+        if (split) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, true, PADDED, true, true>), grid, dim3(320), 0, stream, p);
+        else hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, false, PADDED, true, true>), grid, dim3(256), 0, stream, p);
+      } else {
+        if (split) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, true, PADDED, false, true>), grid, dim3(320), 0, stream, p);
+        else hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, false, PADDED, false, true>), grid, dim3(256), 0, stream, p);
+      }
+      return (int)hipGetLastError();
+    } else {
+      return LMK_ERR_UNSUPPORTED;
+    }
+  }
   if (p.merge_slices > 0) {               // the selection stopped after its slice step: blocks of 32 as they are only
     if constexpr (BS == 32 && !PADDED) {
       if (rows <= 1024 && p.k > 1)
