@@ -215,7 +215,7 @@ def retrieval_bench(n=20, warm=3):
                          "algorithmic_MB_per_launch": k_alg / 1e6}}
 
 
-def decode_bench(n=50, warm=5):
+def decode_bench(n=200, warm=10):
     """One decode step of the mem-cache path: a single new token against a 32768 + 7 token cache
     (1024 complete blocks and a tail of 7), top-4; per-call latency of the two host-level calls."""
     import torch
@@ -239,9 +239,10 @@ def decode_bench(n=50, warm=5):
     retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws)
     t_reuse = _time_launches(lambda: retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws,
                                                    reuse_landmark_keys=True), n, warm)
-    # the step a decode loop makes as its one host call (selection with reused keys + attend: window, forward beside
-    # the slice step of the selection, gather that merges the slices first -- three launches), eagerly and recorded
-    # once into a HIP graph and replayed; and the same work as the two separate calls above (five launches) from a graph
+    # the step a decode loop makes as its one host call (selection with reused keys + attend: the slice step of the
+    # selection, then a gather that merges the slices and attends to the local window itself -- two launches), eagerly
+    # and recorded once into a HIP graph and replayed; and the same work as the two separate calls above (three
+    # launches) from a graph
     from landmark_hip.retrieval import retrieve_and_attend
     one_call = lambda: retrieve_and_attend(q, (kc, vc), kl, vl, cos, sin, block, top_k, workspace=ws,
                                            reuse_landmark_keys=True)

@@ -290,7 +290,11 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
  * in `workspace` (at least lmk_attend_workspace_bytes(...) bytes, 16-byte aligned).  Same result as
  * the three calls -- llama_mem.py:321-342 (window), :386-412 and :447-477 (gather, scores, grouped
  * softmax, output) -- for callers whose per-call host cost matters: a decode step spends more time
- * in the binding than on the GPU.  k_loc, v_loc: the new chunk (B,H,T,D), keys rotated. */
+ * in the binding than on the GPU.  k_loc, v_loc: the new chunk (B,H,T,D), keys rotated.
+ * With blocks of 32, at most four new tokens and a window inside one block (S % block + T <= block: decoding)
+ * the call is ONE launch: the gather kernel attends to the window itself -- cached tail keys rotated at their
+ * positions in the model dtype, the new keys as they are, causal, the landmark token not seeing itself -- as one
+ * more item of each row's online softmax; nothing is written to `workspace` (its size is still checked). */
 size_t lmk_attend_workspace_bytes(int B, int H, int T, int S, int D, int block);
 int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache, const int64_t* idx,
                const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table, const void* sin_table,
@@ -302,8 +306,9 @@ int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor
  * when reuse_landmark_keys != 0) followed by lmk_attend on the indices it wrote -- llama_mem.py:321-412
  * and :447-477.  Same results as the two calls; idx_out (B,H,T,k) int64 is an output.  With blocks of 32 the
  * call takes fewer launches than the two: the forward over the local window shares one with a step of the
- * selection (the rotation of the landmark keys when there are many query rows; the slice step when there are a
- * handful, as in decoding, in which case the gather picks a row's k best from the slices' candidates itself). */
+ * selection (the rotation of the landmark keys) when there are many query rows; with a handful, as in decoding
+ * (the case lmk_attend serves in one launch), the call is two launches -- the slice step of the selection, then a
+ * gather that picks a row's k best from the slices' candidates and attends to the row's local window itself. */
 int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,
                             const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table,
                             const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,

@@ -157,6 +157,38 @@ def test_incomplete_cached_block(n_mems, inc, T, block, top_k, D):
         assert (out[b, h, t] - o).abs().max().item() <= 2e-2, (b, h, t)
 
 
+# A handful of new tokens whose window stays inside one block: the gather kernel attends to the window itself
+# (no window, no forward launch).  Window filling the block with the last new token its landmark; a fresh block;
+# one block per row (no split over waves); more than 1024 rows (a wave per row); fp16; head dim 64.
+@pytest.mark.parametrize("n_mems,inc,T,top_k,B,H,D,dtype", [
+    (20, 28, 4, 4, 2, 3, 128, torch.bfloat16),
+    (20, 0, 4, 4, 2, 3, 128, torch.bfloat16),
+    (10, 29, 3, 1, 2, 3, 128, torch.bfloat16),
+    (10, 13, 3, 4, 12, 32, 128, torch.bfloat16),
+    (20, 30, 2, 4, 1, 2, 128, torch.float16),
+    (20, 27, 4, 5, 2, 3, 64, torch.bfloat16),
+])
+def test_decode_rows_attend_to_their_local_window_inside_the_gather(n_mems, inc, T, top_k, B, H, D, dtype):
+    from landmark_hip.retrieval import gather_attend, retrieve_and_attend
+    block = 32
+    S = n_mems * block + inc
+    print(f"case local n_mems{n_mems} inc{inc} T{T} k{top_k} B{B} H{H} D{D} {dtype}", flush=True)
+    q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=S + T + 5, dtype=dtype)
+    is_mem = ((torch.arange(T) + inc) % block == block - 1)[None].expand(B, T)
+    ref, idx_ref = oret.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, block, top_k)
+    dev = lambda t: t.cuda()
+    out, idx = retrieve_and_attend(dev(q), (dev(kc), dev(vc)), dev(kl), dev(vl), dev(cos), dev(sin), block, top_k)
+    out2 = gather_attend(dev(q), dev(kc), dev(vc), idx, dev(kl), dev(vl), dev(cos), dev(sin), block, top_k)
+    torch.cuda.synchronize()
+    assert torch.equal(idx.cpu(), idx_ref)
+    assert (out.float().cpu() - ref.float()).abs().max().item() <= 2e-2
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))     # the attend step by itself: same kernel
+    ref32 = oret.retrieve_and_attend_s1(q, kc, vc, kl, vl, cos, sin, block, top_k, idx_ref,
+                                        heads=[0, H - 1], tokens=sorted({0, T - 1}))
+    for (b, h, t), o in ref32.items():
+        assert (out.float().cpu()[b, h, t] - o).abs().max().item() <= 2e-2, (b, h, t)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_local_window_rows_bit_exact(dtype):
     # the window builder alone: rotated tail keys bit for bit, values and new rows copied, zero query rows
@@ -339,9 +371,9 @@ def test_gather_clamps_indices_outside_the_cache():
     assert torch.equal(got, want)
 
 
-# The one-call step of a decode loop runs the selection's slice step beside the local forward and lets the gather
-# pick a row's k best from the slices' candidates; the separate calls run slice step, merge and gather as three
-# launches.  Same indices, same output bits -- with a candidate per lane (<= 64) and with several per lane.
+# The one-call step of a decode loop runs the selection's slice step and lets the gather pick a row's k best from the
+# slices' candidates (and attend to the row's local window); the separate calls run slice step, merge and gather as
+# three launches.  Same indices, same output bits -- with a candidate per lane (<= 64) and with several per lane.
 @pytest.mark.parametrize("n_mems,inc,T,top_k,reuse", [(1024, 7, 1, 4, True), (1024, 0, 3, 32, False),
                                                       (700, 31, 1, 40, True), (40, 5, 2, 4, False)])
 def test_one_call_decode_step_equals_the_separate_calls(n_mems, inc, T, top_k, reuse):
