@@ -291,7 +291,7 @@ int lmk_gather_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk
  * the three calls -- llama_mem.py:321-342 (window), :386-412 and :447-477 (gather, scores, grouped
  * softmax, output) -- for callers whose per-call host cost matters: a decode step spends more time
  * in the binding than on the GPU.  k_loc, v_loc: the new chunk (B,H,T,D), keys rotated.
- * With blocks of 32, at most four new tokens and a window inside one block (S % block + T <= block: decoding)
+ * With at most four new tokens and a window inside one block (S % block + T <= block: decoding)
  * the call is ONE launch: the gather kernel attends to the window itself -- cached tail keys rotated at their
  * positions in the model dtype, the new keys as they are, causal, the landmark token not seeing itself -- as one
  * more item of each row's online softmax; nothing is written to `workspace` (its size is still checked). */
@@ -304,11 +304,11 @@ int lmk_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor
 
 /* One inference step of the mem-cache path in one call: lmk_retrieve_topk (or lmk_retrieve_topk_reuse
  * when reuse_landmark_keys != 0) followed by lmk_attend on the indices it wrote -- llama_mem.py:321-412
- * and :447-477.  Same results as the two calls; idx_out (B,H,T,k) int64 is an output.  With blocks of 32 the
- * call takes fewer launches than the two: the forward over the local window shares one with a step of the
- * selection (the rotation of the landmark keys) when there are many query rows; with a handful, as in decoding
- * (the case lmk_attend serves in one launch), the call is two launches -- the slice step of the selection, then a
- * gather that picks a row's k best from the slices' candidates and attends to the row's local window itself. */
+ * and :447-477.  Same results as the two calls; idx_out (B,H,T,k) int64 is an output.  The call takes fewer
+ * launches than the two: in decoding (the case lmk_attend serves in one launch) it is two launches -- the slice
+ * step of the selection, then a gather that picks a row's k best from the slices' candidates and attends to the
+ * row's local window itself; with blocks of 32 and more query rows the forward over the local window shares a
+ * launch with a step of the selection (the slice step up to 1024 rows, else the rotation of the landmark keys). */
 int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, const lmk_tensor4* vcache,
                             const lmk_tensor4* k_loc, const lmk_tensor4* v_loc, const void* cos_table,
                             const void* sin_table, int64_t table_stride_row, int64_t n_pos, int64_t* idx_out,

@@ -1076,11 +1076,29 @@ int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, con
   if (retrieve_workspace == nullptr) return LMK_ERR_NULL;
   if (!aligned16(retrieve_workspace)) return LMK_ERR_ALIGN;
   if (retrieve_workspace_bytes < retr_layout(B, H, T, S, D, block).total) return LMK_ERR_WORKSPACE;
+  if (lmk::gather_takes_local_window(T, S, block)) {
+    // decode: the selection (slice step where it serves, else the fused top-k), then a gather that merges the
+    // slices' candidates and attends to the local window itself -- no window, no forward launch
+    int rc;
+    lmk::RetrParams pr;
+    if ((rc = retrieve_topk_impl(false, q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, retrieve_workspace,
+                                 retrieve_workspace_bytes, B, H, T, S, D, block, top_k, dtype, stream, &pr)))
+      return rc;
+    if (lmk::topk_slices(pr) > 0) {
+      if (!reuse_landmark_keys && (rc = lmk::launch_landmark_keys(pr, D, dtype, (hipStream_t)stream))) return rc;
+      if ((rc = lmk::launch_topk_slices(pr, D, dtype, (hipStream_t)stream))) return rc;
+      return gather_attend_impl(q, kcache, vcache, idx_out, cos_table, sin_table, table_stride_row, n_pos, nullptr, nullptr,
+                                nullptr, 0, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream, &pr, k_loc, v_loc);
+    }
+    if ((rc = lmk::launch_retrieve_topk(pr, D, dtype, reuse_landmark_keys != 0, (hipStream_t)stream))) return rc;
+    return gather_attend_impl(q, kcache, vcache, idx_out, cos_table, sin_table, table_stride_row, n_pos, nullptr, nullptr,
+                              nullptr, 0, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream, nullptr, k_loc, v_loc);
+  }
   if (block == 32) {
     // The forward over the local window needs nothing from the selection and alone fills a fraction of the chip, so
     // it shares a launch with a step of the selection that is as small:
     //   many query rows   window, forward || rotation of the landmark keys, fused top-k, gather
-    //   a handful (decode) window, [rotation,] forward || slice step of the selection, gather that first picks a row's
+    //   up to 1024 rows   window, [rotation,] forward || slice step of the selection, gather that first picks a row's
     //                     k best from the slices' candidates
     int rc;
     const int inc = S % block;
@@ -1095,19 +1113,6 @@ int lmk_retrieve_and_attend(const lmk_tensor4* q, const lmk_tensor4* kcache, con
     if ((rc = retrieve_topk_impl(false, q, kcache, cos_table, sin_table, table_stride_row, n_pos, idx_out, retrieve_workspace,
                                  retrieve_workspace_bytes, B, H, T, S, D, block, top_k, dtype, stream, &pr)))
       return rc;
-    if (lmk::gather_takes_local_window(T, S, block)) {
-      // decode: the selection (slice step where it serves, else the fused top-k), then a gather that merges the
-      // slices' candidates and attends to the local window itself -- no window, no forward launch
-      if (lmk::topk_slices(pr) > 0) {
-        if (!reuse_landmark_keys && (rc = lmk::launch_landmark_keys(pr, D, dtype, (hipStream_t)stream))) return rc;
-        if ((rc = lmk::launch_topk_slices(pr, D, dtype, (hipStream_t)stream))) return rc;
-        return gather_attend_impl(q, kcache, vcache, idx_out, cos_table, sin_table, table_stride_row, n_pos, nullptr, nullptr,
-                                  nullptr, 0, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream, &pr, k_loc, v_loc);
-      }
-      if ((rc = lmk::launch_retrieve_topk(pr, D, dtype, reuse_landmark_keys != 0, (hipStream_t)stream))) return rc;
-      return gather_attend_impl(q, kcache, vcache, idx_out, cos_table, sin_table, table_stride_row, n_pos, nullptr, nullptr,
-                                nullptr, 0, out, B, H, T, S, D, sm_scale, block, top_k, dtype, stream, nullptr, k_loc, v_loc);
-    }
     lmk::FwdParams pf;
     if (inc) {
       if ((rc = attn_fwd_impl(&q_win, &k_win, &v_win, &o_win, L, M, B, H, (int)W, (int)W, D, sm_scale, block, block, 0, dtype,

@@ -214,10 +214,10 @@ int launch_fwd32_landmark_keys(const FwdParams& pf, const RetrParams& pr, int D,
 int launch_fwd32_topk_slices(const FwdParams& pf, const RetrParams& pr, int D, int dtype, hipStream_t stream);
 int launch_landmark_keys(const RetrParams& p, int D, int dtype, hipStream_t stream);   // the rotation alone
 int launch_topk_slices(const RetrParams& p, int D, int dtype, hipStream_t stream);     // the selection's slice step alone
-// rows whose local window the gather kernel attends to itself: block 32, window inside one block, a handful of new tokens
+// rows whose local window the gather kernel attends to itself: window inside one block, a handful of new tokens
 constexpr int kLocalMaxT = 4;
 inline bool gather_takes_local_window(int T, int S, int block) {
-  return block == 32 && T <= kLocalMaxT && S % block + T <= block;
+  return (block == 32 || block == 64 || block == 128) && T <= kLocalMaxT && S % block + T <= block;
 }
 // BS: slots per block (32, 64 or 128); p.block <= BS tokens per block in the cache
 int launch_gather_attend(const RetrParams& p, int D, int BS, int dtype, hipStream_t stream);

@@ -670,12 +670,13 @@ template <> struct PieceVec<4> { using type = u32x2_t; };
 // softmax, instead of coming in as (o_loc, L_loc, M_loc) from a forward launch over a window another launch built:
 // a decode step is then the selection and this kernel.  Its keys join the global bucket directly (own-block rule:
 // causal, the landmark token does not see itself; flash_landmark_attention.py:78-100).
-// With SPLIT the window has a fifth wave of its own.
+// With SPLIT the window has a fifth wave of its own (blocks of 128 keep four waves, whose registers the kernel needs:
+// there the window goes to the wave next in turn behind the blocks).
 template <class T, int D, int BS, bool SPLIT, bool PADDED, bool MERGE = false, bool LOCAL = false>
-__global__ __launch_bounds__((SPLIT && LOCAL) ? 320 : 256) void lmk_gather_attend_kernel(RetrParams p) {
-  constexpr int NWV = (SPLIT && LOCAL) ? 5 : 4;                   // waves of a workgroup
+__global__ __launch_bounds__((SPLIT && LOCAL && BS <= 64) ? 320 : 256) void lmk_gather_attend_kernel(RetrParams p) {
+  constexpr int NWV = (SPLIT && LOCAL && BS <= 64) ? 5 : 4;      // waves of a workgroup
   static_assert((D == 128 || D == 64) && (BS == 32 || BS % 64 == 0), "8 lanes x 2 pieces per row; whole chunks of keys");
-  static_assert(!LOCAL || (BS == 32 && !PADDED), "the local window is one chunk of 32 keys");
+  static_assert(!LOCAL || !PADDED, "the local window sits in a block of BS tokens");
   constexpr int E = D / 16;                                       // head dims per lane and rotary half: 8 or 4
   constexpr int PB = 2 * E;                                       // bytes of one piece
   using vec_t = typename PieceVec<E>::type;                       // one piece: E 16-bit values
@@ -760,60 +761,72 @@ __global__ __launch_bounds__((SPLIT && LOCAL) ? 320 : 256) void lmk_gather_atten
     }
   };
   if constexpr (LOCAL) {
-    if (!SPLIT || wave == 4) {
+    if (!SPLIT || wave == (NWV == 5 ? 4 : (p.k & 3))) {
       const int inc = p.local_inc, own = inc + t;                 // window rows: inc of the cache, then the new tokens
       const char* kn = (const char*)p.k_new + 2 * (b * p.kns_b + hh * p.kns_h);
       const char* vn = (const char*)p.v_new + 2 * (b * p.vns_b + hh * p.vns_h);
-      float s_loc[KPG];
-      vec_t vlo[KPG], vhi[KPG];
+      float s_loc[KPG * NC];
 #pragma unroll
-      for (int i = 0; i < KPG; ++i) {
-        const int r = g + 8 * i;
-        const bool visible = r <= own && !(r == BS - 1 && own == BS - 1);
-        const int rc = min(r, own);                               // rows behind the row's own are never read
-        const bool cached = rc < inc;
-        const char* kr = (cached ? kc + 2 * ((p.local_row0 + rc) * p.kcs_r) : kn + 2 * ((int64_t)(rc - inc) * p.kns_r)) + PB * j;
-        const char* vr = (cached ? vc + 2 * ((p.local_row0 + rc) * p.vcs_r) : vn + 2 * ((int64_t)(rc - inc) * p.vns_r)) + PB * j;
-        const int64_t pos = inc > 0 ? p.local_pos0 + min(rc, inc - 1) : 0;   // a position the tables hold, used by cached rows only
-        const char* cr = (const char*)p.cos + 2 * (pos * p.cs_r) + PB * j;
-        const char* sr = (const char*)p.sin + 2 * (pos * p.cs_r) + PB * j;
-        float kl[E], kh[E], cl[E], ch[E], sl[E], sh[E];
-        unpack8(*(const vec_t*)(kr), kl);
-        unpack8(*(const vec_t*)(kr + D), kh);
-        unpack8(*(const vec_t*)(cr), cl);
-        unpack8(*(const vec_t*)(cr + D), ch);
-        unpack8(*(const vec_t*)(sr), sl);
-        unpack8(*(const vec_t*)(sr + D), sh);
-        vlo[i] = *(const vec_t*)(vr);
-        vhi[i] = *(const vec_t*)(vr + D);
-        float d = 0.f;
+      for (int c = 0; c < NC; ++c) {
+        if (CK * c > own) {                                       // a chunk behind the row's own token (wave-uniform)
 #pragma unroll
-        for (int e = 0; e < E; ++e) {                             // cached keys are rotated in the model dtype, as the cache's
-          const float rl = cached ? round_to<T>(__builtin_fmaf(kl[e], cl[e], -kh[e] * sl[e])) : kl[e];   // window is (llama_mem.py:336-338)
-          const float rh = cached ? round_to<T>(__builtin_fmaf(kh[e], ch[e], kl[e] * sh[e])) : kh[e];
-          d = __builtin_fmaf(qlo[e], rl, d);
-          d = __builtin_fmaf(qhi[e], rh, d);
+          for (int i = 0; i < KPG; ++i) s_loc[KPG * c + i] = -INFINITY;
+          continue;
         }
-        s_loc[i] = visible ? sum8(d) * c2 : -INFINITY;
+#pragma unroll
+        for (int i = 0; i < KPG; ++i) {
+          const int r = CK * c + g + 8 * i;
+          const bool visible = r <= own && !(r == BS - 1 && own == BS - 1);
+          const int rc = min(r, own);                             // rows behind the row's own are never read
+          const bool cached = rc < inc;
+          const char* kr = (cached ? kc + 2 * ((p.local_row0 + rc) * p.kcs_r) : kn + 2 * ((int64_t)(rc - inc) * p.kns_r)) + PB * j;
+          const int64_t pos = inc > 0 ? p.local_pos0 + min(rc, inc - 1) : 0;   // a position the tables hold, used by cached rows only
+          const char* cr = (const char*)p.cos + 2 * (pos * p.cs_r) + PB * j;
+          const char* sr = (const char*)p.sin + 2 * (pos * p.cs_r) + PB * j;
+          float kl[E], kh[E], cl[E], ch[E], sl[E], sh[E];
+          unpack8(*(const vec_t*)(kr), kl);
+          unpack8(*(const vec_t*)(kr + D), kh);
+          unpack8(*(const vec_t*)(cr), cl);
+          unpack8(*(const vec_t*)(cr + D), ch);
+          unpack8(*(const vec_t*)(sr), sl);
+          unpack8(*(const vec_t*)(sr + D), sh);
+          float d = 0.f;
+#pragma unroll
+          for (int e = 0; e < E; ++e) {                           // cached keys are rotated in the model dtype, as the cache's
+            const float rl = cached ? round_to<T>(__builtin_fmaf(kl[e], cl[e], -kh[e] * sl[e])) : kl[e];   // window is (llama_mem.py:336-338)
+            const float rh = cached ? round_to<T>(__builtin_fmaf(kh[e], ch[e], kl[e] * sh[e])) : kh[e];
+            d = __builtin_fmaf(qlo[e], rl, d);
+            d = __builtin_fmaf(qhi[e], rh, d);
+          }
+          s_loc[KPG * c + i] = visible ? sum8(d) * c2 : -INFINITY;
+        }
       }
       float mx = s_loc[0];                                        // row 0 is always visible
 #pragma unroll
-      for (int i = 1; i < KPG; ++i) mx = fmaxf(mx, s_loc[i]);
+      for (int i = 1; i < KPG * NC; ++i) mx = fmaxf(mx, s_loc[i]);
       mx = fmaxf(mx, dpp_f<0x128>(mx));
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       float den = 0.f;
 #pragma unroll
-      for (int i = 0; i < KPG; ++i) {
-        const float e = fast_exp2(s_loc[i] - mx);
-        den += e;
-        const float w = round_to<T>(e);                           // weights enter PV in the model dtype
+      for (int c = 0; c < NC; ++c) {
+        if (CK * c > own) continue;
 #pragma unroll
-        for (int e2 = 0; e2 < E / 2; ++e2) {
-          alo[2 * e2] = __builtin_fmaf(w, unpack_lo<T>(vlo[i][e2]), alo[2 * e2]);
-          alo[2 * e2 + 1] = __builtin_fmaf(w, unpack_hi<T>(vlo[i][e2]), alo[2 * e2 + 1]);
-          ahi[2 * e2] = __builtin_fmaf(w, unpack_lo<T>(vhi[i][e2]), ahi[2 * e2]);
-          ahi[2 * e2 + 1] = __builtin_fmaf(w, unpack_hi<T>(vhi[i][e2]), ahi[2 * e2 + 1]);
+        for (int i = 0; i < KPG; ++i) {
+          const int rc = min(CK * c + g + 8 * i, own);
+          const bool cached = rc < inc;
+          const char* vr = (cached ? vc + 2 * ((p.local_row0 + rc) * p.vcs_r) : vn + 2 * ((int64_t)(rc - inc) * p.vns_r)) + PB * j;
+          const vec_t vlo = *(const vec_t*)(vr), vhi = *(const vec_t*)(vr + D);
+          const float e = fast_exp2(s_loc[KPG * c + i] - mx);
+          den += e;
+          const float w = round_to<T>(e);                         // weights enter PV in the model dtype
+#pragma unroll
+          for (int e2 = 0; e2 < E / 2; ++e2) {
+            alo[2 * e2] = __builtin_fmaf(w, unpack_lo<T>(vlo[e2]), alo[2 * e2]);
+            alo[2 * e2 + 1] = __builtin_fmaf(w, unpack_hi<T>(vlo[e2]), alo[2 * e2 + 1]);
+            ahi[2 * e2] = __builtin_fmaf(w, unpack_lo<T>(vhi[e2]), ahi[2 * e2]);
+            ahi[2 * e2 + 1] = __builtin_fmaf(w, unpack_hi<T>(vhi[e2]), ahi[2 * e2 + 1]);
+          }
         }
       }
       den += dpp_f<0x128>(den);
@@ -1122,15 +1135,15 @@ int launch_retrieve_topk(const RetrParams& p, int D, int dtype, bool reuse_landm
 template <class T, int D, int BS, bool PADDED>
 static int launch_gather_b(const RetrParams& p, hipStream_t stream) {
   const int64_t rows = (int64_t)p.B * p.H * p.T;
-  if (p.local) {                          // with the row's local window: blocks of 32 as they are only
-    if constexpr (BS == 32 && !PADDED) {
+  if (p.local) {                          // with the row's local window: blocks as they are only
+    if constexpr (!PADDED) {
       const bool split = rows <= 1024 && p.k > 1;
       const dim3 grid((unsigned)(split ? rows : (rows + 3) / 4));
       if (p.merge_slices > 0) {
-        if (split) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, true, PADDED, true, true>), grid, dim3(320), 0, stream, p);
+        if (split) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, true, PADDED, true, true>), grid, dim3(BS <= 64 ? 320 : 256), 0, stream, p);
         else hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, false, PADDED, true, true>), grid, dim3(256), 0, stream, p);
       } else {
-        if (split) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, true, PADDED, false, true>), grid, dim3(320), 0, stream, p);
+        if (split) hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, true, PADDED, false, true>), grid, dim3(BS <= 64 ? 320 : 256), 0, stream, p);
         else hipLaunchKernelGGL((lmk_gather_attend_kernel<T, D, BS, false, PADDED, false, true>), grid, dim3(256), 0, stream, p);
       }
       return (int)hipGetLastError();

@@ -160,19 +160,25 @@ def test_incomplete_cached_block(n_mems, inc, T, block, top_k, D):
 # A handful of new tokens whose window stays inside one block: the gather kernel attends to the window itself
 # (no window, no forward launch).  Window filling the block with the last new token its landmark; a fresh block;
 # one block per row (no split over waves); more than 1024 rows (a wave per row); fp16; head dim 64.
-@pytest.mark.parametrize("n_mems,inc,T,top_k,B,H,D,dtype", [
-    (20, 28, 4, 4, 2, 3, 128, torch.bfloat16),
-    (20, 0, 4, 4, 2, 3, 128, torch.bfloat16),
-    (10, 29, 3, 1, 2, 3, 128, torch.bfloat16),
-    (10, 13, 3, 4, 12, 32, 128, torch.bfloat16),
-    (20, 30, 2, 4, 1, 2, 128, torch.float16),
-    (20, 27, 4, 5, 2, 3, 64, torch.bfloat16),
+# Blocks of 64 (the reference's default) and 128: the window is one or two chunks of 64 keys.
+@pytest.mark.parametrize("n_mems,inc,T,top_k,B,H,D,dtype,block", [
+    (20, 28, 4, 4, 2, 3, 128, torch.bfloat16, 32),
+    (20, 0, 4, 4, 2, 3, 128, torch.bfloat16, 32),
+    (10, 29, 3, 1, 2, 3, 128, torch.bfloat16, 32),
+    (10, 13, 3, 4, 12, 32, 128, torch.bfloat16, 32),
+    (20, 30, 2, 4, 1, 2, 128, torch.float16, 32),
+    (20, 27, 4, 5, 2, 3, 64, torch.bfloat16, 32),
+    (12, 60, 4, 3, 2, 3, 128, torch.bfloat16, 64),     # fills the block: the last new token is its landmark
+    (12, 0, 2, 3, 2, 3, 128, torch.bfloat16, 64),
+    (12, 33, 1, 3, 12, 32, 64, torch.float16, 64),     # a wave per row
+    (300, 41, 1, 4, 1, 4, 128, torch.bfloat16, 64),    # two slices to merge
+    (7, 125, 3, 2, 2, 3, 128, torch.bfloat16, 128),    # second chunk of the window, ends on the landmark
+    (7, 40, 2, 4, 1, 2, 64, torch.bfloat16, 128),      # window inside the first chunk
 ])
-def test_decode_rows_attend_to_their_local_window_inside_the_gather(n_mems, inc, T, top_k, B, H, D, dtype):
+def test_decode_rows_attend_to_their_local_window_inside_the_gather(n_mems, inc, T, top_k, B, H, D, dtype, block):
     from landmark_hip.retrieval import gather_attend, retrieve_and_attend
-    block = 32
     S = n_mems * block + inc
-    print(f"case local n_mems{n_mems} inc{inc} T{T} k{top_k} B{B} H{H} D{D} {dtype}", flush=True)
+    print(f"case local n_mems{n_mems} inc{inc} T{T} k{top_k} B{B} H{H} D{D} {dtype} bs{block}", flush=True)
     q, kc, vc, kl, vl, cos, sin = _inputs(B, H, T, S, D, seed=S + T + 5, dtype=dtype)
     is_mem = ((torch.arange(T) + inc) % block == block - 1)[None].expand(B, T)
     ref, idx_ref = oret.retrieve_and_attend(q, kc, vc, kl, vl, is_mem, cos, sin, block, top_k)
