@@ -438,9 +438,11 @@ __global__ __launch_bounds__(64 * NW, 2) void lmk_fwd32_landmark_keys_kernel(Fwd
 }
 
 // Workgroups of 8 waves (256 query rows) share one K/V stream among the most rows; when that many rows per
-// workgroup would leave compute units without one, workgroups of 4 waves (128 rows, one wave per SIMD) are used.
+// workgroup would leave compute units without one, workgroups of 4 waves (128 rows, one wave per SIMD, two
+// workgroups per compute unit) are used -- and for sequences up to 512 keys, where the blocks a workgroup's waves
+// do not all see (its last 8, or 4) are half or all of its stream: 5-11 % faster there, the same from 1024 on.
 static bool fwd32_small_workgroups(const FwdParams& p) {
-  return (int64_t)((p.Lq + 255) / 256) * p.B * p.H < cu_count();
+  return p.Lk <= 512 || (int64_t)((p.Lq + 255) / 256) * p.B * p.H < cu_count();
 }
 
 template <class T, int D, int NW>
