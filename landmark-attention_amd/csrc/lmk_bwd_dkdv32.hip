@@ -455,44 +455,20 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   // finishes in the last.  The ring slot of tile i is a wave-uniform counter that runs on from item to item: the
   // slots behind an item's last tile already hold the next item's first tiles.
   auto wrap = [](int x) LMK_INL { return x >= C::NBUF ? x - C::NBUF : x; };
-  // An accumulator holds (dim 32 dc + 8 g + 4 h + e, key ql) in register 4 g + e of chunk dc: stored from there a
-  // wave's every store instruction would touch 32 rows, 16 bytes each, and the eight waves' 128 of them at an item's
-  // end keep the compute unit's memory pipeline busy for 4 us.  So each 32-dim chunk goes through this wave's 2 KB of
-  // the W hand-over area (the first role uses parity 0, the second parity 1: behind the item's last barrier nobody
-  // reads W there, and the next item's first W goes to parity 0 behind the first role's own stores) and leaves as
-  // 64-byte row segments, 16 rows per store instruction.
+  // An item's accumulators leave as row segments (store_tile_rows) through this wave's 2 KB of the W hand-over
+  // area: the first role uses parity 0, the second parity 1 -- behind the item's last barrier nobody reads W there,
+  // and the next item's first W goes to parity 0 behind the first role's own stores.  (Stored straight from the
+  // registers the eight waves' 128 store instructions at an item's end took 4 us.)
   auto store_acc = [&](const f32x16_t* acc, char* dst, int64_t rs, float scl) LMK_INL {
-    unsigned char* xb = smem + C::XCH_OFF + ((role_k ? 1 : 0) * C::NKT + tile) * C::XCH_TILE;
-    // everything per lane is formed here from the lane id, not ahead of the loops: a value kept across them (the
-    // thread index included) is spilled, and its reload's wait for the memory counter also waits for the ring's tiles in flight
-    int ln;                                                // lane id without a long-lived register
-    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
-    const int rk = ln >> 2, rq = ln & 3;
-    const int ql_now = ln & 31, h_now = ln >> 5;
-    unsigned char* wr = xb + ql_now * 64 + 8 * h_now;
-    char* out[2];
-    bool ok[2];
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      int kr = kt * 32 + rk + 16 * k;
-      if constexpr (VIRT) kr = slot_to_token_row<BS>(kr, p.n_real, nfull_k, seg_k);   // -1: a slot without a token, nothing to store
-      ok[k] = !VIRT || kr >= 0;
-      out[k] = dst + 2 * ((int64_t)(ok[k] ? kr : 0) * rs + 8 * rq);
-    }
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * scl, acc[dc][4 * g + 1] * scl),
-                            pack2<T>(acc[dc][4 * g + 2] * scl, acc[dc][4 * g + 3] * scl)};
-        *(u32x2_t*)(wr + 16 * g) = o2;
+    store_tile_rows<T, C::DC>(acc, scl, C::XCH_OFF + ((role_k ? 1 : 0) * C::NKT + tile) * C::XCH_TILE,
+                              [&](int r) LMK_INL -> char* {
+      int kr = kt * 32 + r;
+      if constexpr (VIRT) {                                // a slot without a token: nothing to store
+        kr = slot_to_token_row<BS>(kr, p.n_real, nfull_k, seg_k);
+        if (kr < 0) return nullptr;
       }
-#pragma unroll
-      for (int k = 0; k < 2; ++k) {
-        const u32x4_t v = *(const u32x4_t*)(xb + (rk + 16 * k) * 64 + 16 * rq);
-        if (ok[k]) *(u32x4_t*)(out[k] + 64 * dc) = v;
-      }
-    }
+      return dst + 2 * ((int64_t)kr * rs);
+    });
   };
   if (!role_k) {
     f32x16_t acc[C::DC];                                   // dV^T: rows = d, lane = key

@@ -460,17 +460,11 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq32_kernel(BwdParams p) {
   }
   dq_wait_vmcnt<0>();                                      // nothing may still be writing LDS when the wave ends
 
-  if (rowok) {
-    const float scl = p.scale;
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * scl, acc[dc][4 * g + 1] * scl),
-                      pack2<T>(acc[dc][4 * g + 2] * scl, acc[dc][4 * g + 3] * scl)};
-        *(u32x2_t*)(dqp + 2 * ((int64_t)qrow * p.dqs_r + 32 * dc + 8 * g + 4 * h)) = o2;
-      }
-  }
+  // dQ leaves as row segments through the LDS that held the wave's dO rows, which it no longer needs
+  if (q0 < p.Lq)                                           // (all or none of a wave's rows exist)
+    store_tile_rows<T, C::DC>(acc, p.scale, C::GO_OFF + wave * C::BLK_BYTES, [&](int r) __attribute__((always_inline)) -> char* {
+      return dqp + 2 * ((int64_t)(q0 + r) * p.dqs_r);
+    });
 }
 
 template <class T, int D, bool HO>

@@ -132,6 +132,7 @@ __device__ __forceinline__ u32x2_t lds_read_tr(const unsigned char* p) {
 // every address with a vector instruction.
 typedef __attribute__((address_space(3))) u32x4_t* lds_u32x4_ptr;
 typedef __attribute__((address_space(3))) float* lds_f32_ptr;
+typedef __attribute__((address_space(3))) u32x2_t* lds_u32x2_ptr;
 __device__ __forceinline__ u32x4_t lds_ld128(int addr) { return *(lds_u32x4_ptr)(uintptr_t)(uint32_t)addr; }
 __device__ __forceinline__ void lds_st128(int addr, u32x4_t v) { *(lds_u32x4_ptr)(uintptr_t)(uint32_t)addr = v; }
 __device__ __forceinline__ void lds_st32(int addr, float v) { *(lds_f32_ptr)(uintptr_t)(uint32_t)addr = v; }
@@ -203,6 +204,42 @@ template <int BS>
 __device__ __forceinline__ int block_normal_keys(int blk, int n, int n_full, const int* seg) {
   if (seg == nullptr) return n - 1;
   return blk < n_full ? seg[blk + 1] - seg[blk] - 1 : BS - 1;
+}
+
+// A wave's 32 x (32 DC) accumulator tile in the MFMA C layout -- register 4 g + e of chunk dc holds (row ql,
+// column 32 dc + 8 g + 4 h + e), ql = lane % 32, h = lane / 32 -- scaled per lane, rounded to T and stored as rows.
+// Stored straight from the registers every store instruction touches 32 rows, 16 bytes each, and a workgroup's
+// waves doing that together keep the compute unit's memory pipeline busy for microseconds; so each 32-column chunk
+// goes through 2 KB of LDS that belong to this wave alone (at LDS byte address `xb`; the kernels' dynamic array
+// starts at address 0) and leaves as 64-byte row segments, 16 rows per store instruction.  row_ptr(r): where row r of the tile (r = 0..31) starts in memory, or null to skip it.
+// Everything per lane is formed here from the lane id: kept across a kernel's loops such values are spilled, and a
+// reload's wait for the memory counter also waits for whatever the kernel has in flight.
+template <class T, int DC, class RowPtr>
+__device__ __forceinline__ void store_tile_rows(const f32x16_t* acc, float scl, int xb, RowPtr row_ptr) {
+  int ln;                                                  // lane id without a long-lived register
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+  const int rk = ln >> 2, rq = ln & 3;
+  const int wr = xb + (ln & 31) * 64 + 8 * (ln >> 5);
+  char* out[2];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    out[k] = row_ptr(rk + 16 * k);
+    if (out[k] != nullptr) out[k] += 16 * rq;
+  }
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * scl, acc[dc][4 * g + 1] * scl),
+                          pack2<T>(acc[dc][4 * g + 2] * scl, acc[dc][4 * g + 3] * scl)};
+      *(lds_u32x2_ptr)(uintptr_t)(uint32_t)(wr + 16 * g) = o2;
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const u32x4_t v = lds_ld128(xb + (rk + 16 * k) * 64 + 16 * rq);
+      if (out[k] != nullptr) *(u32x4_t*)(out[k] + 64 * dc) = v;
+    }
+  }
 }
 
 template <class T>
