@@ -517,16 +517,16 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dq_kernel(BwdParams p) {
     }
   }
 
-  if (qtok >= 0) {
-    const float sc = p.scale;
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * sc, acc[dc][4 * g + 1] * sc),
-                      pack2<T>(acc[dc][4 * g + 2] * sc, acc[dc][4 * g + 3] * sc)};
-        *(u32x2_t*)(dqp + 2 * ((int64_t)qtok * p.dqs_r + 32 * dc + 8 * g + 4 * h)) = o2;
-      }
+  // dQ leaves as row segments through the wave's share of the stage buffer the last stage did not use: every wave
+  // is past the barrier in front of the last stage, so nobody reads that buffer and no request targets it
+  if (active) {
+    static_assert(C::STAGE_BYTES / C::NW >= 2048, "32 rows x 32 columns of 16 bits per wave");
+    const int free_buf = (n_stages & 1) * C::STAGE_BYTES;  // the last stage sits in buffer (n_stages - 1) & 1
+    store_tile_rows<T, C::DC>(acc, p.scale, free_buf + wave * (C::STAGE_BYTES / C::NW),
+                              [&](int r) __attribute__((always_inline)) -> char* {
+      const int tok = virt ? slot_to_token_row<BS>(q0 + r, p.n_real, p.n_full_q, seg_q) : q0 + r;
+      return tok < 0 ? nullptr : dqp + 2 * ((int64_t)tok * p.dqs_r);
+    });
   }
 }
 

@@ -34,6 +34,7 @@ struct FwdCfg {
   static constexpr int DC = D / 32;                     // 32-wide output chunks of the head dim
   static constexpr int LM_BASE = 2 * STAGE_BYTES;       // behind the two stages: 128 landmark keys for the first pass
   static constexpr int LDS_BYTES = LM_BASE + 128 * ROWB;
+  static_assert(128 * ROWB / NW >= 2048, "a wave's share of that area also takes its output tile, 32 columns at a time");
   static constexpr int RPD = 1024 / ROWB;               // rows covered by one 1 KB request
   static constexpr int NREQ = 2 * SK / RPD;             // requests per stage
   static constexpr int PER_WAVE = NREQ / NW;
@@ -440,16 +441,17 @@ __global__ __launch_bounds__(512, 2) void lmk_fwd_kernel(FwdParams p) {
   }
 
   // ---- epilogue: out = acc / l, statistics in natural-log units like the reference
+  // the output leaves as row segments through the wave's share of the first pass's LDS area, which nothing has
+  // touched since (a slot without a token, or past the last row, stores nothing)
+  if (active)
+    store_tile_rows<T, C::DC>(acc, 1.0f / lrun, C::LM_BASE + wave * (128 * C::ROWB / C::NW),
+                              [&](int r) __attribute__((always_inline)) -> char* {
+      const int qr = q0 + r;
+      if (qr >= p.Lq) return nullptr;
+      const int tok = virt ? slot_to_token_row<BS>(qr, p.n_real, nfull_q, seg_q) : qr;
+      return tok < 0 ? nullptr : op + 2 * ((int64_t)tok * p.os_r);
+    });
   if (active && qtok >= 0) {
-    const float inv = 1.0f / lrun;
-#pragma unroll
-    for (int dc = 0; dc < C::DC; ++dc)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * inv, acc[dc][4 * g + 1] * inv),
-                      pack2<T>(acc[dc][4 * g + 2] * inv, acc[dc][4 * g + 3] * inv)};
-        *(u32x2_t*)(op + 2 * ((int64_t)qtok * p.os_r + 32 * dc + 8 * g + 4 * h)) = o2;
-      }
     if (h == 0) {                                       // statistics follow the tensors' layout
       const int64_t si = (int64_t)bh * (virt ? p.Lq_real : p.Lq) + qtok;
       p.L[si] = lrun;
