@@ -29,11 +29,14 @@ MAX_BLOCK = 128
 SUPPORTED_HEAD_DIMS = (64, 128)
 # Two backward paths exist for block 32.  With a workspace of lmk_attn_bwd_handover_workspace_bytes() the dQ kernel
 # leaves dS behind for the dK/dV kernel (2 bytes per visible (query, key) pair), which then forms neither dP nor dS
-# again.  That pays while the tiles stay in the GPU's 256 MB last-level cache between the two kernels (measured:
-# backward 4 % faster at B1 H32 L2048, 154 MB) and loses once they have to travel through HBM (7 % slower at
-# B2 H32 L2048, 307 MB), so workspaces above this many bytes are not allocated and the recomputing kernels run
-# in 4 * (2 + 3 * Lk / block) bytes per query row.
+# again.  That can only pay while the tiles stay in the GPU's 256 MB last-level cache between the two kernels (it
+# loses once they have to travel through HBM: 7 % slower at B2 H32 L2048, 307 MB), so workspaces above this many
+# bytes are not allocated and the recomputing kernels run in 4 * (2 + 3 * Lk / block) bytes per query row ...
 HANDOVER_MAX_BYTES = int(os.environ.get("LMK_BWD_HANDOVER_MAX_MB", "160")) << 20
+# ... and only for sequences from this many keys on: below, the recomputing pair is as fast or faster (B4 H32 L512:
+# 112 against 114 us for forward + backward; B2 H32 L1024: 159 against 160) in a fraction of the workspace, while a
+# few long heads gain 3-4 % (B1 H16 L2048: 188 against 193 us, B1 H8 L4096: 330 against 345).
+HANDOVER_MIN_KEYS = int(os.environ.get("LMK_BWD_HANDOVER_MIN_KEYS", "2048"))
 PADDED_HEAD_DIMS = (16, 32)          # accepted by fused_landmark_attention, zero-padded to 64
 
 
@@ -113,7 +116,7 @@ def _launch_bwd(q, k, v, o, do, L, M, n_prefix, sm_scale, block, block_real=None
     nbytes = lib.lmk_attn_bwd_workspace_bytes(B, H, Lq, Lk, int(block))
     if block_real == block:
         ho = lib.lmk_attn_bwd_handover_workspace_bytes(B, H, Lq, Lk, int(block))
-        if 0 < ho <= HANDOVER_MAX_BYTES:
+        if 0 < ho <= HANDOVER_MAX_BYTES and Lk >= HANDOVER_MIN_KEYS:
             nbytes = ho          # the library picks the hand-over kernels from the size it is handed
     ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
     rc = lib.lmk_attn_bwd_padded(_lib.tensor4(q), _lib.tensor4(k), _lib.tensor4(v), _lib.tensor4(o),

@@ -59,6 +59,7 @@ def test_forward_backward_replays_from_a_graph(path, monkeypatch):
     from landmark_hip import attention
     from landmark_hip.attention import _launch_bwd, _launch_fwd
     monkeypatch.setattr(attention, "HANDOVER_MAX_BYTES", 0 if path == "recompute" else 1 << 40)
+    monkeypatch.setattr(attention, "HANDOVER_MIN_KEYS", 0)
     B, H, L, D, block = 1, 4, 256, 128, 32
     gen = torch.Generator().manual_seed(6)
     mk = lambda: (torch.randn(B, H, L, D, generator=gen) * 0.5).bfloat16().cuda()
