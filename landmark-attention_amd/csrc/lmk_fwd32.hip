@@ -51,7 +51,9 @@ struct Fwd32Cfg {
   static constexpr int LM_OFF = NBUF * BUF_BYTES;          // two tiles of 32 landmark keys for the first pass
   static constexpr int LM_TILES = 2;
   static constexpr int LM_REQ = (32 / RPD + NW - 1) / NW;  // requests per wave and landmark tile
-  static constexpr int LDS_BYTES = LM_OFF + LM_TILES * BLK_BYTES;
+  static constexpr int OUT_SHARE = 2048;                   // per wave: its output tile leaves through here, 32 columns at a time
+  static constexpr int LM_BYTES = LM_TILES * BLK_BYTES > NW * OUT_SHARE ? LM_TILES * BLK_BYTES : NW * OUT_SHARE;
+  static constexpr int LDS_BYTES = LM_OFF + LM_BYTES;
 };
 
 __device__ __forceinline__ void fw_dma16(const void* base_uniform, uint32_t voff, uint32_t lds_off) {
@@ -399,26 +401,12 @@ __device__ __forceinline__ void fwd32_body(const FwdParams& p, const int bid_) {
   fw_wait_vmcnt<0>();                                      // nothing may still be writing LDS when the wave ends
 
   // the output leaves as row segments through the wave's share of the landmark tiles' LDS, which nothing has
-  // touched since the first pass (a share of 2 KB: all but head dim 64 in workgroups of 8 waves)
-  constexpr int LM_SHARE = C::LM_TILES * C::BLK_BYTES / C::NW;
-  if constexpr (LM_SHARE >= 2048) {
-    if (waveok)
-      store_tile_rows<T, C::DC>(acc, 1.0f / lsum, C::LM_OFF + wave * LM_SHARE, [&](int r) LMK_INL -> char* {
-        return q0 + r < p.Lq ? op + 2 * ((int64_t)(q0 + r) * p.os_r) : nullptr;
-      });
-  }
+  // touched since the first pass
+  if (waveok)
+    store_tile_rows<T, C::DC>(acc, 1.0f / lsum, C::LM_OFF + wave * C::OUT_SHARE, [&](int r) LMK_INL -> char* {
+      return q0 + r < p.Lq ? op + 2 * ((int64_t)(q0 + r) * p.os_r) : nullptr;
+    });
   if (rowok) {
-    if constexpr (LM_SHARE < 2048) {
-      const float inv = 1.0f / lsum;
-#pragma unroll
-      for (int dc = 0; dc < C::DC; ++dc)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          u32x2_t o2 = {pack2<T>(acc[dc][4 * g + 0] * inv, acc[dc][4 * g + 1] * inv),
-                        pack2<T>(acc[dc][4 * g + 2] * inv, acc[dc][4 * g + 3] * inv)};
-          *(u32x2_t*)(op + 2 * ((int64_t)qrow * p.os_r + 32 * dc + 8 * g + 4 * h)) = o2;
-        }
-    }
     if (h == 0) {                                          // statistics of the global bucket, relative to its maximum
       p.L[(int64_t)bh * p.Lq + qrow] = lsum;
       p.M[(int64_t)bh * p.Lq + qrow] = Mfin * kLn2;
