@@ -84,27 +84,34 @@ __global__ __launch_bounds__(256) void lmk_fill_u32_kernel(uint32_t* dst, int64_
   if (i < n) dst[i] = value;
 }
 
-// One wave per (batch, head, query): scores -> softmax -> 16-bit probabilities -> maximum per block
-// into agg (B*H, num_mems), which holds zeros on entry.  A lane owns the blocks m = lane, lane + 64, ...;
-// the row's sum is each lane's running sum in that order, folded across lanes by halves.
-// A workgroup is four queries of one (batch, head): 128 rotated landmark keys at a time are staged
-// through LDS, fetched once in memory order and shared by the four waves; the query sits in registers.
+// Scores of every query against every landmark key, in the contract's order, into p.approx (B*H*T, num_mems).
+// A lane owns a query row (its 16-bit values unpacked once into registers), a wave 64 rows and 16 keys (137
+// registers leave three waves per SIMD, and every fma of a score waits for the one before it: pieces this small keep
+// three waves at work until the end; with 32 keys a wave the last of four per SIMD ran alone for half the time).  The key is the same for all lanes: its chunks come in through scalar loads and are
+// unpacked on the scalar side, so a score costs one vector fma per dimension (with a key per lane every fma had an
+// unpack beside it).  The kernel stores nothing before its last load, which is what lets the loads be scalar ones;
+// the 64 x 16 scores cross through LDS on their way out and leave as 64-byte row segments.
+constexpr int kScoreKeys = 16;                                    // keys per wave: half a tile of the rotated keys
+
 template <class T, int D>
-__global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
-  constexpr int ROWB = 2 * D + 16;                                // padded key row: a 16-lane group reads 16 B each, all banks
+__global__ __launch_bounds__(256) void lmk_block_score_kernel(RetrParams p) {
   constexpr int CPR = D / 8;                                      // 16-byte chunks per key row
-  constexpr int TM = 128;                                         // landmark keys per tile: two per lane
-  constexpr int NCH = TM * CPR / 256;                             // chunks per thread and tile
-  __shared__ __align__(16) unsigned char tile[TM * ROWB];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n_rg = (p.T + 3) / 4;
-  const int bh = blockIdx.x / n_rg, t = (blockIdx.x % n_rg) * 4 + wave;
-  const bool active = t < p.T;                                    // idle waves still help with the tiles
-  const int b = bh / p.H, hh = bh % p.H;
+  __shared__ float xs[4][kScoreKeys][64];                         // [wave][key][row]
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int NM = p.num_mems;
+  const int n_qg = (p.T + 63) / 64, n_kc = (NM + kScoreKeys - 1) / kScoreKeys;
+  // wave -> (query group, key tile, head), query group first: the waves that run side by side read the same tile
+  // against different rows, and all but the first find it in the scalar cache
+  const int64_t wid = (int64_t)blockIdx.x * 4 + wave;
+  const int qg = (int)(wid % n_qg), kc = (int)((wid / n_qg) % n_kc);
+  const int64_t bh64 = wid / n_qg / n_kc;
+  if (bh64 >= (int64_t)p.B * p.H) return;                         // no workgroup-wide barrier below
+  const int bh = (int)bh64;
+  const int b = bh / p.H, hh = bh % p.H;
+  const int t = qg * 64 + lane;
   float qf[D];
   {
-    const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)(active ? t : 0) * p.qs_r);
+    const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)min(t, p.T - 1) * p.qs_r);
 #pragma unroll
     for (int c = 0; c < CPR; ++c) {
       const u32x4_t u = *(const u32x4_t*)(qp + 16 * c);
@@ -115,54 +122,131 @@ __global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
       }
     }
   }
-  const int64_t row = (int64_t)bh * p.T + (active ? t : 0);
-  float* sc = p.approx + row * NM;                                // this row's scores, then its exponentials
-  const char* lk = (const char*)p.lk_rot + (int64_t)bh * lk_tiles(NM) * lk_tile_bytes(D);
-
-  auto fetch = [&](int m0, u32x4_t* r) {
+  const int m0 = kc * kScoreKeys;
+  const u32x4_t* tile = (const u32x4_t*)((const char*)p.lk_rot + (int64_t)bh * lk_tiles(NM) * lk_tile_bytes(D) + lk_key_offset(m0, D));
+  const int n_keys = min(kScoreKeys, NM - m0);
+  // A key's chunks arrive in two halves, each asked for while the half before it is being used (a whole key ahead
+  // would not fit the scalar registers beside the current one).
+  constexpr int HC = CPR / 2;                                     // chunks per half
+  auto fetch_half = [&](int j, int half, u32x4_t* r) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int c = i * 256 + tid;                                  // the tile's chunks in memory order: m0 is a multiple of 32
-      u32x4_t z = {0, 0, 0, 0};
-      r[i] = (m0 + 32 * (c / (32 * CPR)) < NM) ? *(const u32x4_t*)(lk + lk_key_offset(m0, D) + 16 * (int64_t)c) : z;
-    }
+    for (int c = 0; c < HC; ++c) r[c] = tile[32 * (half * HC + c) + j];   // chunk c of key j: the same address in every lane
   };
-  u32x4_t nxt[NCH];
-  fetch(0, nxt);
-  float mx = -INFINITY;
-  for (int m0 = 0; m0 < NM; m0 += TM) {
-    __syncthreads();                                              // the previous tile has been read by every wave
+  auto use_half = [&](int half, const u32x4_t* r, float acc) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int c = i * 256 + tid, kr = 32 * (c / (32 * CPR)) + (c & 31), col = (c >> 5) % CPR;
-      *(u32x4_t*)(tile + kr * ROWB + 16 * col) = nxt[i];
-    }
-    __syncthreads();
-    if (m0 + TM < NM) fetch(m0 + TM, nxt);                        // in flight during the arithmetic below
-#pragma unroll 1
-    for (int half = 0; half < TM / 64; ++half) {
-      const int m = m0 + 64 * half + lane;
-      if (!(active && m < NM)) continue;
-      const unsigned char* kr = tile + (64 * half + lane) * ROWB;
-      float acc = 0.f;
+    for (int c = 0; c < HC; ++c) {
 #pragma unroll
-      for (int d8 = 0; d8 < CPR; ++d8) {
-        const u32x4_t kk = *(const u32x4_t*)(kr + 16 * d8);
-        acc = __builtin_fmaf(qf[8 * d8 + 0], unpack_lo<T>(kk[0]), acc);
-        acc = __builtin_fmaf(qf[8 * d8 + 1], unpack_hi<T>(kk[0]), acc);
-        acc = __builtin_fmaf(qf[8 * d8 + 2], unpack_lo<T>(kk[1]), acc);
-        acc = __builtin_fmaf(qf[8 * d8 + 3], unpack_hi<T>(kk[1]), acc);
-        acc = __builtin_fmaf(qf[8 * d8 + 4], unpack_lo<T>(kk[2]), acc);
-        acc = __builtin_fmaf(qf[8 * d8 + 5], unpack_hi<T>(kk[2]), acc);
-        acc = __builtin_fmaf(qf[8 * d8 + 6], unpack_lo<T>(kk[3]), acc);
-        acc = __builtin_fmaf(qf[8 * d8 + 7], unpack_hi<T>(kk[3]), acc);
+      for (int i = 0; i < 4; ++i) {
+        uint32_t w = r[c][i];
+        // the word is unpacked here, next to its two fmas: unpacked ahead of time the key's values do not fit the
+        // scalar registers.  (Not a scheduling barrier: behind one the loads are no longer scalar ones.)
+        if constexpr (std::is_same<T, bf16_t>::value) asm("" : "+s"(w), "+v"(acc));   // (fp16 words are unpacked inside the fma)
+        acc = __builtin_fmaf(qf[8 * (half * HC + c) + 2 * i], unpack_lo<T>(w), acc);
+        acc = __builtin_fmaf(qf[8 * (half * HC + c) + 2 * i + 1], unpack_hi<T>(w), acc);
       }
-      const float x = contract<T>(acc, p.sqrt_hd);
-      sc[m] = x;                                                  // read back below by the same lane only
-      mx = fmaxf(mx, x);
+    }
+    return acc;
+  };
+  u32x4_t ha[HC], hb[HC];
+  fetch_half(0, 0, ha);
+#pragma unroll 1
+  for (int j = 0; j < n_keys; ++j) {
+    fetch_half(j, 1, hb);
+    float acc = use_half(0, ha, 0.f);
+    fetch_half(min(j + 1, n_keys - 1), 0, ha);                    // behind the last key: a re-read nobody uses
+    acc = use_half(1, hb, acc);
+    xs[wave][j][lane] = contract<T>(acc, p.sqrt_hd);
+  }
+  // rows r = lane / CPL + (64 / CPL) i, keys 4 (lane % CPL) .. + 3: a row's scores are contiguous bytes
+  constexpr int CPL = kScoreKeys / 4;                             // lanes per row
+  const int64_t row0 = (int64_t)bh * p.T + qg * 64;
+  const int c4 = 4 * (lane % CPL);
+#pragma unroll
+  for (int i = 0; i < CPL; ++i) {
+    const int r = lane / CPL + (64 / CPL) * i;
+    float4 v = {xs[wave][c4][r], xs[wave][c4 + 1][r], xs[wave][c4 + 2][r], xs[wave][c4 + 3][r]};
+    if (qg * 64 + r >= p.T) continue;
+    float* dst = p.approx + (row0 + r) * NM + m0 + c4;
+    if (c4 + 3 < n_keys && (NM & 3) == 0) *(float4*)dst = v;      // rows of whole 16-byte chunks
+    else {
+      if (c4 < n_keys) dst[0] = v.x;
+      if (c4 + 1 < n_keys) dst[1] = v.y;
+      if (c4 + 2 < n_keys) dst[2] = v.z;
+      if (c4 + 3 < n_keys) dst[3] = v.w;
     }
   }
-  if (!active) return;                                            // no block-wide barrier below
+}
+
+// The rows' scores (p.approx) -> softmax -> 16-bit probabilities -> maximum per block into agg, which holds zeros on
+// entry: one vector per (batch, head), maxima over the queries -- or per (batch, query), maxima over the heads.
+// A lane owns the blocks m = lane, lane + 64, ...; a row's sum is each lane's running sum in that order, folded
+// across lanes by halves.  A wave takes `rows_per_wave` rows that share a vector one after the other with the row in
+// registers (NPL values per lane: num_mems <= 64 NPL) and the running maxima too, so a row is read once, nothing is
+// written back and the vector sees one atomic per block and wave.  fp32 probabilities are positive, so their bit
+// patterns order like the values.
+template <int NPL>
+__global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p, int model_is_bf16, int rows_per_wave) {
+  const int lane = threadIdx.x & 63;
+  const int NM = p.num_mems;
+  // rows that share a vector: the T queries of a (batch, head), or the H heads of a (batch, query)
+  const int group = p.agg_over_heads ? p.H : p.T;
+  const int per_group = (group + rows_per_wave - 1) / rows_per_wave;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (w >= (int64_t)per_group * (p.agg_over_heads ? p.B * p.T : p.B * p.H)) return;
+  const int64_t vec = w / per_group;                              // (batch, query) or (batch, head)
+  const int first = (int)(w % per_group) * rows_per_wave, last = min(first + rows_per_wave, group);
+  uint32_t best[NPL];
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) best[i] = 0u;
+  for (int g = first; g < last; ++g) {
+    // over heads: vec = b T + t, row (b H + g) T + t; over queries: vec = b H + h, row vec T + g
+    const int64_t row = p.agg_over_heads ? ((vec / p.T) * p.H + g) * p.T + vec % p.T : vec * p.T + g;
+    const float* sc = p.approx + row * NM;
+    float x[NPL];
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) x[i] = (lane + 64 * i < NM) ? sc[lane + 64 * i] : -INFINITY;
+    float mx = x[0];
+#pragma unroll
+    for (int i = 1; i < NPL; ++i) mx = fmaxf(mx, x[i]);
+#pragma unroll
+    for (int msk = 32; msk >= 1; msk >>= 1) mx = fmaxf(mx, __shfl_xor(mx, msk, 64));
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      if (lane + 64 * i < NM) {
+        float d = x[i] - mx;
+        asm volatile("" : "+v"(d));                               // the product below stays a product
+        x[i] = exp2_contract(d * kLog2e);
+        sum += x[i];
+      }
+    }
+#pragma unroll
+    for (int msk = 32; msk >= 1; msk >>= 1) sum = sum + __shfl_xor(sum, msk, 64);
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      if (lane + 64 * i < NM) {
+        const float pr = __fdiv_rn(x[i], sum);
+        const uint32_t bits = p.prob32 ? __float_as_uint(pr) : (model_is_bf16 ? prob_bits<bf16_t>(pr) : prob_bits<f16_t>(pr));
+        best[i] = max(best[i], bits);
+      }
+    }
+  }
+  uint32_t* agg = p.agg + vec * NM;
+#pragma unroll
+  for (int i = 0; i < NPL; ++i)
+    if (lane + 64 * i < NM) atomicMax(agg + lane + 64 * i, best[i]);
+}
+
+// The same for vectors of any length: one wave per row, the row's exponentials written back over its scores.
+__global__ __launch_bounds__(256) void lmk_block_prob_long_kernel(RetrParams p, int model_is_bf16) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= (int64_t)p.B * p.H * p.T) return;
+  const int bh = (int)(row / p.T), t = (int)(row % p.T), b = bh / p.H;
+  const int NM = p.num_mems;
+  float* sc = p.approx + row * NM;                                // this row's scores, then its exponentials
+  float mx = -INFINITY;
+  for (int m = lane; m < NM; m += 64) mx = fmaxf(mx, sc[m]);
 #pragma unroll
   for (int msk = 32; msk >= 1; msk >>= 1) mx = fmaxf(mx, __shfl_xor(mx, msk, 64));
   float sum = 0.f;
@@ -175,12 +259,11 @@ __global__ __launch_bounds__(256) void lmk_block_prob_kernel(RetrParams p) {
   }
 #pragma unroll
   for (int msk = 32; msk >= 1; msk >>= 1) sum = sum + __shfl_xor(sum, msk, 64);
-  // one vector per (batch, head), maxima over the queries -- or per (batch, query), maxima over the heads;
-  // fp32 probabilities are positive, so their bit patterns order like the values
   uint32_t* agg = p.agg + (int64_t)(p.agg_over_heads ? b * p.T + t : bh) * NM;
   for (int m = lane; m < NM; m += 64) {
     const float pr = __fdiv_rn(sc[m], sum);
-    atomicMax(agg + m, p.prob32 ? __float_as_uint(pr) : prob_bits<T>(pr));
+    const uint32_t bits = p.prob32 ? __float_as_uint(pr) : (model_is_bf16 ? prob_bits<bf16_t>(pr) : prob_bits<f16_t>(pr));
+    atomicMax(agg + m, bits);
   }
 }
 
@@ -1063,7 +1146,24 @@ static int launch_topk_shared_t(const RetrParams& p, hipStream_t stream) {
   const int64_t agg_words = sel_rows * p.num_mems;
   hipLaunchKernelGGL(lmk_fill_u32_kernel, dim3((unsigned)((agg_words + 255) / 256)), dim3(256), 0, stream, p.agg, agg_words, 0u);
   if ((rc = (int)hipGetLastError())) return rc;
-  hipLaunchKernelGGL((lmk_block_prob_kernel<T, D>), dim3((unsigned)(p.B * p.H * ((p.T + 3) / 4))), dim3(256), 0, stream, p);
+  const int64_t score_waves = (int64_t)p.B * p.H * ((p.T + 63) / 64) * ((p.num_mems + kScoreKeys - 1) / kScoreKeys);
+  hipLaunchKernelGGL((lmk_block_score_kernel<T, D>), dim3((unsigned)((score_waves + 3) / 4)), dim3(256), 0, stream, p);
+  if ((rc = (int)hipGetLastError())) return rc;
+  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  const int is_bf16 = std::is_same<T, bf16_t>::value ? 1 : 0;
+  if (p.num_mems <= 64 * 32) {
+    // rows per wave: as many as leave the chip a few thousand waves, at most 8
+    const int group = p.agg_over_heads ? p.H : p.T;
+    const int rpw = (int)std::max<int64_t>(1, std::min<int64_t>(std::min(8, group), rows / 4096));
+    const int64_t waves = (int64_t)((group + rpw - 1) / rpw) * sel_rows;
+    const dim3 grid((unsigned)((waves + 3) / 4));
+    if (p.num_mems <= 64) hipLaunchKernelGGL(lmk_block_prob_kernel<1>, grid, dim3(256), 0, stream, p, is_bf16, rpw);
+    else if (p.num_mems <= 64 * 4) hipLaunchKernelGGL(lmk_block_prob_kernel<4>, grid, dim3(256), 0, stream, p, is_bf16, rpw);
+    else if (p.num_mems <= 64 * 16) hipLaunchKernelGGL(lmk_block_prob_kernel<16>, grid, dim3(256), 0, stream, p, is_bf16, rpw);
+    else hipLaunchKernelGGL(lmk_block_prob_kernel<32>, grid, dim3(256), 0, stream, p, is_bf16, rpw);
+  } else {
+    hipLaunchKernelGGL(lmk_block_prob_long_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p, is_bf16);
+  }
   if ((rc = (int)hipGetLastError())) return rc;
   hipLaunchKernelGGL(lmk_block_select_kernel, dim3((unsigned)sel_rows), dim3(256), 0, stream, p);
   return (int)hipGetLastError();

@@ -229,6 +229,8 @@ SHARED_CASES = [
     (1, 2, 5, 17, 9, 128, 32, 4, torch.bfloat16, 0.5),       # cache ends in an incomplete block
     (1, 3, 1, 33, 31, 128, 32, 2, torch.bfloat16, 0.5),      # decode step that lands on the landmark
     (1, 2, 20, 12, 40, 128, 64, 3, torch.float16, 0.5),
+    (1, 1, 70, 1100, 0, 64, 32, 4, torch.bfloat16, 0.5),     # 32 probabilities per lane; a second, partial group of 64 queries
+    (1, 1, 5, 2100, 0, 64, 32, 4, torch.float16, 0.5),       # more blocks than a wave holds in registers
 ]
 
 
