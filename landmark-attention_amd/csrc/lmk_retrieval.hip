@@ -85,28 +85,51 @@ __global__ __launch_bounds__(256) void lmk_fill_u32_kernel(uint32_t* dst, int64_
 }
 
 // Scores of every query against every landmark key, in the contract's order, into p.approx (B*H*T, num_mems).
-// A lane owns a query row (its 16-bit values unpacked once into registers), a wave 64 rows and 16 keys (137
-// registers leave three waves per SIMD, and every fma of a score waits for the one before it: pieces this small keep
-// three waves at work until the end; with 32 keys a wave the last of four per SIMD ran alone for half the time).  The key is the same for all lanes: its chunks come in through scalar loads and are
-// unpacked on the scalar side, so a score costs one vector fma per dimension (with a key per lane every fma had an
-// unpack beside it).  The kernel stores nothing before its last load, which is what lets the loads be scalar ones;
-// the 64 x 16 scores cross through LDS on their way out and leave as 64-byte row segments.
-constexpr int kScoreKeys = 16;                                    // keys per wave: half a tile of the rotated keys
+// A workgroup is 16 keys of a head against up to 256 query rows: a lane owns a row (its 16-bit values unpacked once
+// into registers), a wave 64 rows.  The keys are unpacked to fp32 once per workgroup into LDS, a wave reads a key from
+// there once (256 bytes per 64 dimensions) and the fmas pick their dimension from the lane that holds it, so a score
+// costs one vector fma per dimension.  (With a key per
+// lane every fma had an unpack beside it.  With the key in scalar registers -- scalar loads, unpacked by scalar
+// instructions or read from an fp32 copy -- the kernel took 58 us at config 4's shapes whatever else changed: taken
+// apart, 32 us of it were the scalar loads, 8 bytes per score, and 9 us the fmas.)
+constexpr int kScoreKeys = 16;                                    // keys per workgroup: half a tile of the rotated keys
+
+// acc += q * (k of lane N of this lane's row of 16 lanes)
+template <int N>
+__device__ __forceinline__ void fma_row_bcast(float& acc, float k, float q) {
+  asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(k), "v"(q), "n"(N));
+}
+// the 64 dimensions of a group in order: dimension 4 n + i sits in component i of lane n
+template <int... N>
+__device__ __forceinline__ void score_fma_group(float& acc, const float4& kv, const float* q, std::integer_sequence<int, N...>) {
+  ((fma_row_bcast<N>(acc, kv.x, q[4 * N]), fma_row_bcast<N>(acc, kv.y, q[4 * N + 1]), fma_row_bcast<N>(acc, kv.z, q[4 * N + 2]),
+    fma_row_bcast<N>(acc, kv.w, q[4 * N + 3])), ...);
+}
 
 template <class T, int D>
 __global__ __launch_bounds__(256) void lmk_block_score_kernel(RetrParams p) {
-  constexpr int CPR = D / 8;                                      // 16-byte chunks per key row
+  constexpr int CPR = D / 8;                                      // 16-byte chunks per row of 16-bit values
+  __shared__ __align__(16) float ks[kScoreKeys][D];               // the workgroup's keys
   __shared__ float xs[4][kScoreKeys][64];                         // [wave][key][row]
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int NM = p.num_mems;
-  const int n_qg = (p.T + 63) / 64, n_kc = (NM + kScoreKeys - 1) / kScoreKeys;
-  // wave -> (query group, key tile, head), query group first: the waves that run side by side read the same tile
-  // against different rows, and all but the first find it in the scalar cache
-  const int64_t wid = (int64_t)blockIdx.x * 4 + wave;
-  const int qg = (int)(wid % n_qg), kc = (int)((wid / n_qg) % n_kc);
-  const int64_t bh64 = wid / n_qg / n_kc;
-  if (bh64 >= (int64_t)p.B * p.H) return;                         // no workgroup-wide barrier below
-  const int bh = (int)bh64;
+  const int n_qg = (p.T + 63) / 64, n_q4 = (n_qg + 3) / 4, n_kc = (NM + kScoreKeys - 1) / kScoreKeys;
+  // workgroup -> (four query groups, keys, head): the grid holds exactly B H n_kc n_q4 of them
+  const int q4 = (int)(blockIdx.x % n_q4), kc = (int)((blockIdx.x / n_q4) % n_kc), bh = (int)(blockIdx.x / n_q4 / n_kc);
+  const int m0 = kc * kScoreKeys;
+  const int n_keys = min(kScoreKeys, NM - m0);
+  const char* lk = (const char*)p.lk_rot + (int64_t)bh * lk_tiles(NM) * lk_tile_bytes(D);
+  for (int c = tid; c < kScoreKeys * CPR; c += 256) {             // chunk c % CPR of key c / CPR
+    const int j = c / CPR, cc = c % CPR;
+    u32x4_t u = {0, 0, 0, 0};
+    if (j < n_keys) u = *(const u32x4_t*)(lk + lk_key_offset(m0 + j, D) + 512 * cc);
+    float4* dst = (float4*)&ks[j][8 * cc];
+    dst[0] = float4{unpack_lo<T>(u[0]), unpack_hi<T>(u[0]), unpack_lo<T>(u[1]), unpack_hi<T>(u[1])};
+    dst[1] = float4{unpack_lo<T>(u[2]), unpack_hi<T>(u[2]), unpack_lo<T>(u[3]), unpack_hi<T>(u[3])};
+  }
+  __syncthreads();
+  const int qg = 4 * q4 + wave;
+  if (qg >= n_qg) return;                                         // no workgroup-wide barrier below
   const int b = bh / p.H, hh = bh % p.H;
   const int t = qg * 64 + lane;
   float qf[D];
@@ -122,39 +145,19 @@ __global__ __launch_bounds__(256) void lmk_block_score_kernel(RetrParams p) {
       }
     }
   }
-  const int m0 = kc * kScoreKeys;
-  const u32x4_t* tile = (const u32x4_t*)((const char*)p.lk_rot + (int64_t)bh * lk_tiles(NM) * lk_tile_bytes(D) + lk_key_offset(m0, D));
-  const int n_keys = min(kScoreKeys, NM - m0);
-  // A key's chunks arrive in two halves, each asked for while the half before it is being used (a whole key ahead
-  // would not fit the scalar registers beside the current one).
-  constexpr int HC = CPR / 2;                                     // chunks per half
-  auto fetch_half = [&](int j, int half, u32x4_t* r) __attribute__((always_inline)) {
-#pragma unroll
-    for (int c = 0; c < HC; ++c) r[c] = tile[32 * (half * HC + c) + j];   // chunk c of key j: the same address in every lane
-  };
-  auto use_half = [&](int half, const u32x4_t* r, float acc) __attribute__((always_inline)) {
-#pragma unroll
-    for (int c = 0; c < HC; ++c) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        uint32_t w = r[c][i];
-        // the word is unpacked here, next to its two fmas: unpacked ahead of time the key's values do not fit the
-        // scalar registers.  (Not a scheduling barrier: behind one the loads are no longer scalar ones.)
-        if constexpr (std::is_same<T, bf16_t>::value) asm("" : "+s"(w), "+v"(acc));   // (fp16 words are unpacked inside the fma)
-        acc = __builtin_fmaf(qf[8 * (half * HC + c) + 2 * i], unpack_lo<T>(w), acc);
-        acc = __builtin_fmaf(qf[8 * (half * HC + c) + 2 * i + 1], unpack_hi<T>(w), acc);
-      }
-    }
-    return acc;
-  };
-  u32x4_t ha[HC], hb[HC];
-  fetch_half(0, 0, ha);
+  // A key reaches the lanes 64 dimensions at a time: lane l reads dimensions 4 (l % 16) .. + 3 of the group (one
+  // 16-byte LDS read per lane, the four rows of 16 lanes reading the same 256 bytes), and the fma takes dimension
+  // 4 n + i from lane n of its own row of 16 (row_newbcast).  Reading every value into every lane instead costs 16
+  // times the LDS traffic, and LDS then bounds the kernel (52 us).
+  const int koff = 4 * (lane & 15);
 #pragma unroll 1
   for (int j = 0; j < n_keys; ++j) {
-    fetch_half(j, 1, hb);
-    float acc = use_half(0, ha, 0.f);
-    fetch_half(min(j + 1, n_keys - 1), 0, ha);                    // behind the last key: a re-read nobody uses
-    acc = use_half(1, hb, acc);
+    float acc = 0.f;
+#pragma unroll
+    for (int c = 0; c < D / 64; ++c) {
+      const float4 kv = *(const float4*)&ks[j][64 * c + koff];
+      score_fma_group(acc, kv, qf + 64 * c, std::make_integer_sequence<int, 16>{});
+    }
     xs[wave][j][lane] = contract<T>(acc, p.sqrt_hd);
   }
   // rows r = lane / CPL + (64 / CPL) i, keys 4 (lane % CPL) .. + 3: a row's scores are contiguous bytes
@@ -1146,8 +1149,8 @@ static int launch_topk_shared_t(const RetrParams& p, hipStream_t stream) {
   const int64_t agg_words = sel_rows * p.num_mems;
   hipLaunchKernelGGL(lmk_fill_u32_kernel, dim3((unsigned)((agg_words + 255) / 256)), dim3(256), 0, stream, p.agg, agg_words, 0u);
   if ((rc = (int)hipGetLastError())) return rc;
-  const int64_t score_waves = (int64_t)p.B * p.H * ((p.T + 63) / 64) * ((p.num_mems + kScoreKeys - 1) / kScoreKeys);
-  hipLaunchKernelGGL((lmk_block_score_kernel<T, D>), dim3((unsigned)((score_waves + 3) / 4)), dim3(256), 0, stream, p);
+  const int64_t score_wgs = (int64_t)p.B * p.H * (((p.T + 63) / 64 + 3) / 4) * ((p.num_mems + kScoreKeys - 1) / kScoreKeys);
+  hipLaunchKernelGGL((lmk_block_score_kernel<T, D>), dim3((unsigned)score_wgs), dim3(256), 0, stream, p);
   if ((rc = (int)hipGetLastError())) return rc;
   const int64_t rows = (int64_t)p.B * p.H * p.T;
   const int is_bf16 = std::is_same<T, bf16_t>::value ? 1 : 0;

@@ -231,6 +231,8 @@ SHARED_CASES = [
     (1, 2, 20, 12, 40, 128, 64, 3, torch.float16, 0.5),
     (1, 1, 70, 1100, 0, 64, 32, 4, torch.bfloat16, 0.5),     # 32 probabilities per lane; a second, partial group of 64 queries
     (1, 1, 5, 2100, 0, 64, 32, 4, torch.float16, 0.5),       # more blocks than a wave holds in registers
+    (1, 2, 140, 40, 0, 128, 32, 4, torch.float16, 0.5),      # enough queries for the fp32 copy of the keys (as the 70 above)
+    (2, 2, 200, 70, 0, 128, 64, 4, torch.bfloat16, 0.5),
 ]
 
 
