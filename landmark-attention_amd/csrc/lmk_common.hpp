@@ -21,6 +21,7 @@ typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
 typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(32 * sizeof(float)))) float f32x32_t;
 typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;

@@ -85,98 +85,64 @@ __global__ __launch_bounds__(256) void lmk_fill_u32_kernel(uint32_t* dst, int64_
 }
 
 // Scores of every query against every landmark key, in the contract's order, into p.approx (B*H*T, num_mems).
-// A workgroup is 16 keys of a head against up to 256 query rows: a lane owns a row (its 16-bit values unpacked once
-// into registers), a wave 64 rows.  The keys are unpacked to fp32 once per workgroup into LDS, a wave reads a key from
-// there once (256 bytes per 64 dimensions) and the fmas pick their dimension from the lane that holds it, so a score
-// costs one vector fma per dimension.  (With a key per
-// lane every fma had an unpack beside it.  With the key in scalar registers -- scalar loads, unpacked by scalar
-// instructions or read from an fp32 copy -- the kernel took 58 us at config 4's shapes whatever else changed: taken
-// apart, 32 us of it were the scalar loads, 8 bytes per score, and 9 us the fmas.)
-constexpr int kScoreKeys = 16;                                    // keys per workgroup: half a tile of the rotated keys
-
-// acc += q * (k of lane N of this lane's row of 16 lanes)
-template <int N>
-__device__ __forceinline__ void fma_row_bcast(float& acc, float k, float q) {
-  asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(k), "v"(q), "n"(N));
-}
-// the 64 dimensions of a group in order: dimension 4 n + i sits in component i of lane n
-template <int... N>
-__device__ __forceinline__ void score_fma_group(float& acc, const float4& kv, const float* q, std::integer_sequence<int, N...>) {
-  ((fma_row_bcast<N>(acc, kv.x, q[4 * N]), fma_row_bcast<N>(acc, kv.y, q[4 * N + 1]), fma_row_bcast<N>(acc, kv.z, q[4 * N + 2]),
-    fma_row_bcast<N>(acc, kv.w, q[4 * N + 3])), ...);
-}
+// The contract's dot product is a chain of fp32 fmas over d ascending, and v_mfma_f32_32x32x1_2b_f32 is 2 x 32 x 32 of
+// exactly that step: C[i][j] = fma(A[i], B[j], C[i][j]).  A wave takes 64 query rows (a lane holds its row, packed) and
+// 64 keys (lanes 0..31 hold keys 0..31, lanes 32..63 keys 32..63, packed, 16 bytes per lane and chunk straight from the
+// tiles of the rotated keys); per dimension one unpack each and two MFMAs -- the 64 rows as two blocks of 32 against
+// the keys of the first 32 lanes (BLGP 1), then against those of the other 32 (BLGP 2) -- 4 matrix-pipe cycles per
+// score.  (On the vector unit a score is 128 fmas plus whatever brings the key's value to every lane -- an unpack per
+// fma with a key per lane, scalar loads of 8 bytes per score with the key in scalar registers, 16 times the LDS
+// traffic with every lane reading the value, half-rate cross-lane fmas -- and every such kernel took 50-60 us at
+// config 4's shapes.)
+constexpr int kScoreRows = 64, kScoreKeys = 64;                   // per wave
 
 template <class T, int D>
 __global__ __launch_bounds__(256) void lmk_block_score_kernel(RetrParams p) {
   constexpr int CPR = D / 8;                                      // 16-byte chunks per row of 16-bit values
-  __shared__ __align__(16) float ks[kScoreKeys][D];               // the workgroup's keys
-  __shared__ float xs[4][kScoreKeys][64];                         // [wave][key][row]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int NM = p.num_mems;
-  const int n_qg = (p.T + 63) / 64, n_q4 = (n_qg + 3) / 4, n_kc = (NM + kScoreKeys - 1) / kScoreKeys;
-  // workgroup -> (four query groups, keys, head): the grid holds exactly B H n_kc n_q4 of them
-  const int q4 = (int)(blockIdx.x % n_q4), kc = (int)((blockIdx.x / n_q4) % n_kc), bh = (int)(blockIdx.x / n_q4 / n_kc);
-  const int m0 = kc * kScoreKeys;
-  const int n_keys = min(kScoreKeys, NM - m0);
-  const char* lk = (const char*)p.lk_rot + (int64_t)bh * lk_tiles(NM) * lk_tile_bytes(D);
-  for (int c = tid; c < kScoreKeys * CPR; c += 256) {             // chunk c % CPR of key c / CPR
-    const int j = c / CPR, cc = c % CPR;
-    u32x4_t u = {0, 0, 0, 0};
-    if (j < n_keys) u = *(const u32x4_t*)(lk + lk_key_offset(m0 + j, D) + 512 * cc);
-    float4* dst = (float4*)&ks[j][8 * cc];
-    dst[0] = float4{unpack_lo<T>(u[0]), unpack_hi<T>(u[0]), unpack_lo<T>(u[1]), unpack_hi<T>(u[1])};
-    dst[1] = float4{unpack_lo<T>(u[2]), unpack_hi<T>(u[2]), unpack_lo<T>(u[3]), unpack_hi<T>(u[3])};
-  }
-  __syncthreads();
-  const int qg = 4 * q4 + wave;
-  if (qg >= n_qg) return;                                         // no workgroup-wide barrier below
+  const int n_qg = (p.T + kScoreRows - 1) / kScoreRows, n_kc = (NM + kScoreKeys - 1) / kScoreKeys;
+  // wave -> (query group, keys, head), query group first: the waves that run side by side read the same keys
+  const int64_t wid = (int64_t)blockIdx.x * 4 + wave;
+  const int qg = (int)(wid % n_qg), kc = (int)((wid / n_qg) % n_kc);
+  const int64_t bh64 = wid / n_qg / n_kc;
+  if (bh64 >= (int64_t)p.B * p.H) return;                         // no workgroup-wide barrier in this kernel
+  const int bh = (int)bh64;
   const int b = bh / p.H, hh = bh % p.H;
-  const int t = qg * 64 + lane;
-  float qf[D];
+  const int m0 = kc * kScoreKeys;
+  u32x4_t qp[CPR], kp[CPR];                                       // this lane's query row and key, packed
   {
-    const char* qp = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)min(t, p.T - 1) * p.qs_r);
+    const int t = min(qg * kScoreRows + lane, p.T - 1);           // rows behind the last one: a re-read, never stored
+    const char* src = (const char*)p.q + 2 * (b * p.qs_b + hh * p.qs_h + (int64_t)t * p.qs_r);
 #pragma unroll
-    for (int c = 0; c < CPR; ++c) {
-      const u32x4_t u = *(const u32x4_t*)(qp + 16 * c);
+    for (int c = 0; c < CPR; ++c) qp[c] = *(const u32x4_t*)(src + 16 * c);
+    const int m = min(m0 + lane, (int)(32 * lk_tiles(NM)) - 1);   // keys behind the last tile: likewise
+    const char* lk = (const char*)p.lk_rot + (int64_t)bh * lk_tiles(NM) * lk_tile_bytes(D) + lk_key_offset(m, D);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        qf[8 * c + 2 * i] = unpack_lo<T>(u[i]);
-        qf[8 * c + 2 * i + 1] = unpack_hi<T>(u[i]);
-      }
-    }
+    for (int c = 0; c < CPR; ++c) kp[c] = *(const u32x4_t*)(lk + 512 * c);
   }
-  // A key reaches the lanes 64 dimensions at a time: lane l reads dimensions 4 (l % 16) .. + 3 of the group (one
-  // 16-byte LDS read per lane, the four rows of 16 lanes reading the same 256 bytes), and the fma takes dimension
-  // 4 n + i from lane n of its own row of 16 (row_newbcast).  Reading every value into every lane instead costs 16
-  // times the LDS traffic, and LDS then bounds the kernel (52 us).
-  const int koff = 4 * (lane & 15);
-#pragma unroll 1
-  for (int j = 0; j < n_keys; ++j) {
-    float acc = 0.f;
+  f32x32_t lo, hi;                                                // scores against keys m0 .. +31 and m0 + 32 .. + 63
 #pragma unroll
-    for (int c = 0; c < D / 64; ++c) {
-      const float4 kv = *(const float4*)&ks[j][64 * c + koff];
-      score_fma_group(acc, kv, qf + 64 * c, std::make_integer_sequence<int, 16>{});
-    }
-    xs[wave][j][lane] = contract<T>(acc, p.sqrt_hd);
-  }
-  // rows r = lane / CPL + (64 / CPL) i, keys 4 (lane % CPL) .. + 3: a row's scores are contiguous bytes
-  constexpr int CPL = kScoreKeys / 4;                             // lanes per row
-  const int64_t row0 = (int64_t)bh * p.T + qg * 64;
-  const int c4 = 4 * (lane % CPL);
+  for (int r = 0; r < 32; ++r) lo[r] = hi[r] = 0.f;
 #pragma unroll
-  for (int i = 0; i < CPL; ++i) {
-    const int r = lane / CPL + (64 / CPL) * i;
-    float4 v = {xs[wave][c4][r], xs[wave][c4 + 1][r], xs[wave][c4 + 2][r], xs[wave][c4 + 3][r]};
-    if (qg * 64 + r >= p.T) continue;
-    float* dst = p.approx + (row0 + r) * NM + m0 + c4;
-    if (c4 + 3 < n_keys && (NM & 3) == 0) *(float4*)dst = v;      // rows of whole 16-byte chunks
-    else {
-      if (c4 < n_keys) dst[0] = v.x;
-      if (c4 + 1 < n_keys) dst[1] = v.y;
-      if (c4 + 2 < n_keys) dst[2] = v.z;
-      if (c4 + 3 < n_keys) dst[3] = v.w;
+  for (int c = 0; c < CPR; ++c)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {                                 // dimension 8 c + i
+      const float qv = (i & 1) ? unpack_hi<T>(qp[c][i >> 1]) : unpack_lo<T>(qp[c][i >> 1]);
+      const float kv = (i & 1) ? unpack_hi<T>(kp[c][i >> 1]) : unpack_lo<T>(kp[c][i >> 1]);
+      lo = __builtin_amdgcn_mfma_f32_32x32x1f32(qv, kv, lo, 0, 0, 1);
+      hi = __builtin_amdgcn_mfma_f32_32x32x1f32(qv, kv, hi, 0, 0, 2);
     }
+  // register 16 blk + r of lane l: row 32 blk + 8 (r / 4) + 4 (l / 32) + r % 4, key l % 32 of the accumulator's 32
+  const int key = lane & 31, rsub = 4 * (lane >> 5);
+  const int64_t row0 = (int64_t)bh * p.T;
+#pragma unroll
+  for (int r = 0; r < 32; ++r) {
+    const int t = qg * kScoreRows + 32 * (r >> 4) + 8 * ((r & 15) >> 2) + rsub + (r & 3);
+    if (t >= p.T) continue;
+    float* dst = p.approx + (row0 + t) * NM + m0 + key;
+    if (m0 + key < NM) dst[0] = contract<T>(lo[r], p.sqrt_hd);
+    if (m0 + 32 + key < NM) dst[32] = contract<T>(hi[r], p.sqrt_hd);
   }
 }
 
@@ -1149,8 +1115,8 @@ static int launch_topk_shared_t(const RetrParams& p, hipStream_t stream) {
   const int64_t agg_words = sel_rows * p.num_mems;
   hipLaunchKernelGGL(lmk_fill_u32_kernel, dim3((unsigned)((agg_words + 255) / 256)), dim3(256), 0, stream, p.agg, agg_words, 0u);
   if ((rc = (int)hipGetLastError())) return rc;
-  const int64_t score_wgs = (int64_t)p.B * p.H * (((p.T + 63) / 64 + 3) / 4) * ((p.num_mems + kScoreKeys - 1) / kScoreKeys);
-  hipLaunchKernelGGL((lmk_block_score_kernel<T, D>), dim3((unsigned)score_wgs), dim3(256), 0, stream, p);
+  const int64_t score_waves = (int64_t)p.B * p.H * ((p.T + kScoreRows - 1) / kScoreRows) * ((p.num_mems + kScoreKeys - 1) / kScoreKeys);
+  hipLaunchKernelGGL((lmk_block_score_kernel<T, D>), dim3((unsigned)((score_waves + 3) / 4)), dim3(256), 0, stream, p);
   if ((rc = (int)hipGetLastError())) return rc;
   const int64_t rows = (int64_t)p.B * p.H * p.T;
   const int is_bf16 = std::is_same<T, bf16_t>::value ? 1 : 0;
