@@ -108,6 +108,22 @@ def _time_launches(fn, n, warm):
     return e0.elapsed_time(e1) / n
 
 
+def _time_from_graph(step, n, warm):
+    """Average duration in ms of `step` replayed from a HIP graph (one warm run on a side stream, then the capture):
+    the device's time for it, whatever the host needs to issue its launches."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    return _time_launches(graph.replay, n, warm)
+
+
 def config0_inputs(seed=0):
     """Benchmark config 0 exactly as specified: q, k, v ~ N(0,1) fp32 (2,8,510,128), a landmark at every
     51st position (50 regular tokens + 1 landmark per block)."""
@@ -249,19 +265,8 @@ def decode_bench(n=200, warm=10):
     def two_calls():
         i = retrieve_topk(q, kc, cos, sin, block, top_k, workspace=ws, reuse_landmark_keys=True)
         return gather_attend(q, kc, vc, i, kl, vl, cos, sin, block, top_k)
-    def from_graph(step):
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            step()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step()
-        return _time_launches(graph.replay, n, warm)
-    t_graph = from_graph(one_call)
-    t_graph2 = from_graph(two_calls)
+    t_graph = _time_from_graph(one_call, n, warm)
+    t_graph2 = _time_from_graph(two_calls, n, warm)
     t_eager = _time_launches(one_call, n, warm)
     return {"workload": "decode: 1 new token, H32 D128, cache 32775 tok (1024 blocks of 32 + tail of 7), top-4",
             "topk_ms": t_topk, "topk_reusing_landmark_keys_ms": t_reuse, "gather_attend_ms": t_att,
@@ -324,7 +329,8 @@ def side_legs(n=30, warm=5):
         torch.autograd.grad(out, [q0, k0, v0], do0)
     with torch.no_grad():
         t_c0_fwd = _time_launches(lambda: fused_landmark_attention(q0, k0, v0, None, block_size=block0), n, warm)
-    t_c0_step = _time_launches(config0_step, n, warm)
+    t_c0_step = _time_launches(config0_step, n, warm)          # eager: three launches and the autograd machinery, host-bound
+    t_c0_graph = _time_from_graph(config0_step, n, warm)
     # the offloaded cache (keys and values of config 4's cache in pinned host memory, landmark keys on the GPU): one
     # chunk of 256 queries and one single token, selection per head + attention over blocks read from host memory
     from landmark_hip.cache import OffloadedLandmarkCache
@@ -369,7 +375,8 @@ def side_legs(n=30, warm=5):
                                             "one selection per head; 256 queries / 1 query", "chunk_step_ms": t_off_chunk,
                                 "token_step_ms": t_off_token},
             "config0_on_hip": {"workload": "benchmark config 0 (B2 H8 L510 D128, block 51) in bf16, blocks of 51 tokens worked on in 64 slots and read in place",
-                               "forward_ms": t_c0_fwd, "forward_backward_ms": t_c0_step},
+                               "forward_ms": t_c0_fwd, "forward_backward_ms": t_c0_step,
+                               "forward_backward_from_hip_graph_ms": t_c0_graph},
             "per_head_selection": {"workload": "config 4 shapes, aggregate=max_over_tokens", "topk_ms": t_sel,
                                    "attend_ms": t_att},
             "rotary": {"workload": "q and k of config 2, (2,32,2048,128) bf16 each, one launch for both", "ms": t_rot,
