@@ -72,10 +72,10 @@ def traffic_summary(fetch_csv, write_csv):
     f_scale = COPY_BYTES / 1024 / fetch[COPY_KERNEL][0]
     w_scale = COPY_BYTES / 1024 / write[COPY_KERNEL][0]
     lines = ["# HBM bytes per launch of each kernel, from two counter runs on an MI355X (one counter per run):",
-             "#   rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/pmc_fetch -o p -- python3 bench.py --traffic-probe",
-             "#   rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/pmc_write -o p -- python3 bench.py --traffic-probe",
-             "#   python3 bench.py --traffic-summary gpurun_out/pmc_fetch/p_counter_collection.csv "
-             "gpurun_out/pmc_write/p_counter_collection.csv",
+             "#   rocprofv3 --pmc FETCH_SIZE --output-format csv -d out/pmc_fetch -o p -- python3 bench.py --traffic-probe",
+             "#   rocprofv3 --pmc WRITE_SIZE --output-format csv -d out/pmc_write -o p -- python3 bench.py --traffic-probe",
+             "#   python3 bench.py --traffic-summary out/pmc_fetch/p_counter_collection.csv "
+             "out/pmc_write/p_counter_collection.csv",
              f"# calibration: the 256 MiB device copy ({COPY_KERNEL}) reads {fetch[COPY_KERNEL][0]:.0f} KiB on FETCH_SIZE and "
              f"{write[COPY_KERNEL][0]:.0f} KiB on WRITE_SIZE for 262144 KiB each way:",
              f"#   FETCH_SIZE is scaled by {f_scale:.3f}, WRITE_SIZE by {w_scale:.3f}",
