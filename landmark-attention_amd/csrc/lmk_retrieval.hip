@@ -92,8 +92,8 @@ __global__ __launch_bounds__(256) void lmk_fill_u32_kernel(uint32_t* dst, int64_
 // the keys of the first 32 lanes (BLGP 1), then against those of the other 32 (BLGP 2) -- 4 matrix-pipe cycles per
 // score.  (On the vector unit a score is 128 fmas plus whatever brings the key's value to every lane -- an unpack per
 // fma with a key per lane, scalar loads of 8 bytes per score with the key in scalar registers, 16 times the LDS
-// traffic with every lane reading the value, fmas that take the value from the lane that holds it (row_newbcast) -- and every such kernel took 50-60 us at
-// config 4's shapes.)
+// traffic with every lane reading the value, fmas that take the value from the lane that holds it (row_newbcast) --
+// and every such kernel took 50-60 us at config 4's shapes.)
 constexpr int kScoreRows = 64, kScoreKeys = 64;                   // per wave
 
 template <class T, int D>
