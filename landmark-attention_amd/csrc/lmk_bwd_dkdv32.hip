@@ -123,13 +123,12 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   const int PT = p.n_prefix * C::TPB;                      // history tiles in front of the queries
   const int nq = p.Lq >> 5;
   // the item being computed
-  int kt, krow, kt_end, j_first;
+  int kt, kt_end, j_first;
   bool active, lm_lane;
   auto set_item = [&](int c) LMK_INL {
     kvt = item_kvt(c);
     kt = kvt * C::NKT + tile;
     active = kt < nkt;
-    krow = kt * 32 + ql;
     lm_lane = (ql == 31) && (kt % C::TPB == C::TPB - 1);   // this lane's key is its block's landmark
     kt_end = (kt / C::TPB + 1) * C::TPB;                   // first tile behind this key tile's block
     j_first = max(0, kvt * C::NKT - PT);                   // first query tile any wave here can see
@@ -408,40 +407,72 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     sync();
   };
 
-  // this wave's stationary operand of the current item: K fragments (V role) or V fragments (K role), lane = key
-  auto load_stationary = [&]() LMK_INL {
+  // this wave's stationary operand for key tile kt_i: K fragments (V role) or V fragments (K role), lane = key.
+  // An item's operand is asked for at the end of the item before it, in front of that item's stores: behind them
+  // the wait for it would also be the wait for the stores' acknowledgements.
+  auto load_stationary = [&](int kt_i) LMK_INL {
     const char* src = role_k ? (const char*)p.v + 2 * (b_ * p.vs_b + hh * p.vs_h)
                              : (const char*)p.k + 2 * (b_ * p.ks_b + hh * p.ks_h);
     const int64_t rs = role_k ? p.vs_r : p.ks_r;
-    int kr = krow, h8 = 8 * h;
-    asm volatile("" : "+v"(kr), "+v"(h8));                 // the address is formed here, not ahead of the loops (and spilled)
-    if constexpr (VIRT) kr = slot_to_token_row_clamped<BS>(active ? kr : 0, p.n_real, nfull_k, seg_k);
-    const char* row = src + 2 * ((int64_t)kr * rs + h8);
+    const bool act = kt_i < nkt;
+    int ln;                                                // the address is formed here from the lane id, not from values
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));   // kept across the loops (and spilled)
+    int kr = kt_i * 32 + (ln & 31);
+    if constexpr (VIRT) kr = slot_to_token_row_clamped<BS>(act ? kr : 0, p.n_real, nfull_k, seg_k);
+    const char* row = src + 2 * ((int64_t)kr * rs + 8 * (ln >> 5));
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) {
       u32x4_t z = {0, 0, 0, 0};
       bf[ks] = z;
-      if (active) bf[ks] = *(const u32x4_t*)(row + 32 * ks);
+      if (act) bf[ks] = *(const u32x4_t*)(row + 32 * ks);
     }
   };
   // consume the operand at once: no wait for these loads can then end up inside the loop, where it would
-  // drain the ring; the explicit wait covers everything this wave has in flight, which the compiler does not count
-  auto await_stationary = [&]() LMK_INL {
-    wait_vmcnt<0>();
+  // drain the ring; the explicit wait covers everything this wave asked for up to and including the operand, which
+  // the compiler does not count.  newer: what the wave has issued behind the operand's loads (an item's stores).
+  // (await_stationary: wait_vmcnt<newer operations>() in front of this)
+  auto use_stationary = [&]() LMK_INL {
 #pragma unroll
     for (int ks = 0; ks < C::KS; ++ks) asm volatile("" : "+v"(bf[ks]));
+  };
+  // an item's stores, issued behind the next item's loads: without rows that have no token their number is fixed
+  // (such rows' stores are skipped lane by lane)
+  constexpr int kStoresNewer = VIRT ? 0 : 2 * C::DC;
+  // The end of item c: its accumulators leave, and the wave turns to the item behind it, if there is one (the ring
+  // already holds that item's first tiles).  Returns that item's index, or n_c.
+  auto finish_item = [&](int c, const f32x16_t* acc, char* dst, int64_t rs, float scl, auto store_acc) LMK_INL {
+    const int c_nx = next_item(c + 1);
+    if (c_nx < n_c) {
+      // the wait stands in each branch, behind a known number of newer operations: the compiler puts its own wait for
+      // these loads where their registers are first used, counted along the path with the fewest newer operations
+      load_stationary(item_kvt(c_nx) * C::NKT + tile);
+      if (active) {
+        store_acc(acc, dst, rs, scl);
+        wait_vmcnt<kStoresNewer>();
+        use_stationary();
+      } else {
+        wait_vmcnt<0>();
+        use_stationary();
+      }
+      set_item(c_nx);
+      announce_next(c_nx);
+    } else if (active) {
+      store_acc(acc, dst, rs, scl);
+    }
+    return c_nx;
   };
 
   // ---- prologue of the first item.  The stationary operand and the first two tiles are asked for first and
   // awaited; tiles j_first+2, +3 go out behind that wait, so the workgroup does not sit through four tiles'
   // worth of traffic (every workgroup of a launch round starts at the same moment) before its first product.
-  load_stationary();
+  load_stationary(kt);
   if (!role_k) {
     request(0);
     request(C::BUF_BYTES);
   }
   if (tid < 64) ((float*)(smem + C::CONST_OFF))[tid] = (tid < 32) ? 1e30f : 0.f;
-  await_stationary();
+  wait_vmcnt<0>();
+  use_stationary();
   if (!role_k) {
     request(2 * C::BUF_BYTES);
     request(3 * C::BUF_BYTES);
@@ -460,7 +491,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
   // and the next item's first W goes to parity 0 behind the first role's own stores.  (Stored straight from the
   // registers the eight waves' 128 store instructions at an item's end took 4 us.)
   auto store_acc = [&](const f32x16_t* acc, char* dst, int64_t rs, float scl) LMK_INL {
-    store_tile_rows<T, C::DC>(acc, scl, C::XCH_OFF + ((role_k ? 1 : 0) * C::NKT + tile) * C::XCH_TILE,
+    store_tile_rows<T, C::DC, VIRT>(acc, scl, C::XCH_OFF + ((role_k ? 1 : 0) * C::NKT + tile) * C::XCH_TILE,
                               [&](int r) LMK_INL -> char* {
       int kr = kt * 32 + r;
       if constexpr (VIRT) {                                // a slot without a token: nothing to store
@@ -474,13 +505,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
     f32x16_t acc[C::DC];                                   // dV^T: rows = d, lane = key
     f32x16_t cur, nxt;                                      // S of tiles i and i+1
     int sc = 0;                                            // slot of the item's tile i
-    for (int c = 0; c < n_c; c = next_item(c + 1)) {
-      if (c > 0) {                                         // the ring already holds this item's first tiles
-        set_item(c);
-        announce_next(c);
-        load_stationary();
-        await_stationary();
-      }
+    for (int c = 0; c < n_c;) {
 #pragma unroll
       for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
       row_tile(sc * C::BUF_BYTES, cur);                     // S of the first tile
@@ -505,20 +530,14 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
       // that iteration is the one its first iteration of the next item leaves out)
       wait_vmcnt<2 * C::PER_TILE_V>();
       __syncthreads();
-      if (active) store_acc(acc, (char*)p.dv + 2 * (b_ * p.dvs_b + hh * p.dvs_h), p.dvs_r, 1.f);
+      c = finish_item(c, acc, (char*)p.dv + 2 * (b_ * p.dvs_b + hh * p.dvs_h), p.dvs_r, 1.f, store_acc);
     }
     wait_vmcnt<0>();                                       // nothing may still be writing LDS when the wave ends
   } else {
     f32x16_t acc[C::DC];                                   // dK^T: rows = d, lane = key
     f32x16_t prv, cur;                                      // dP of tiles i-1 and i
     int sc = 0;                                            // slot of the item's first tile, then of tile i
-    for (int c = 0; c < n_c; c = next_item(c + 1)) {
-      if (c > 0) {
-        set_item(c);
-        announce_next(c);
-        load_stationary();
-        await_stationary();
-      }
+    for (int c = 0; c < n_c;) {
 #pragma unroll
       for (int dc = 0; dc < C::DC; ++dc) zero16(acc[dc]);
       int cs = sc * C::BUF_BYTES, ps;                       // byte offsets of the slots of tiles i and i-1
@@ -553,7 +572,7 @@ __global__ __launch_bounds__(512, 2) void lmk_bwd_dkdv32_kernel(BwdParams p) {
         advance();
       }
       sc = ps / C::BUF_BYTES;                               // the slot behind the last tile: the next item's first tile
-      if (active) store_acc(acc, (char*)p.dk + 2 * (b_ * p.dks_b + hh * p.dks_h), p.dks_r, p.scale);
+      c = finish_item(c, acc, (char*)p.dk + 2 * (b_ * p.dks_b + hh * p.dks_h), p.dks_r, p.scale, store_acc);
     }
     wait_vmcnt<0>();
   }

@@ -215,7 +215,9 @@ __device__ __forceinline__ int block_normal_keys(int blk, int n, int n_full, con
 // starts at address 0) and leaves as 64-byte row segments, 16 rows per store instruction.  row_ptr(r): where row r of the tile (r = 0..31) starts in memory, or null to skip it.
 // Everything per lane is formed here from the lane id: kept across a kernel's loops such values are spilled, and a
 // reload's wait for the memory counter also waits for whatever the kernel has in flight.
-template <class T, int DC, class RowPtr>
+// MAY_SKIP = false: row_ptr never returns null, and the tile's 2 DC store instructions are issued unconditionally
+// (a caller that counts its memory operations needs that).
+template <class T, int DC, bool MAY_SKIP = true, class RowPtr>
 __device__ __forceinline__ void store_tile_rows(const f32x16_t* acc, float scl, int xb, RowPtr row_ptr) {
   int ln;                                                  // lane id without a long-lived register
   asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
@@ -225,7 +227,7 @@ __device__ __forceinline__ void store_tile_rows(const f32x16_t* acc, float scl, 
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
     out[k] = row_ptr(rk + 16 * k);
-    if (out[k] != nullptr) out[k] += 16 * rq;
+    if (!MAY_SKIP || out[k] != nullptr) out[k] += 16 * rq;
   }
 #pragma unroll
   for (int dc = 0; dc < DC; ++dc) {
@@ -238,7 +240,7 @@ __device__ __forceinline__ void store_tile_rows(const f32x16_t* acc, float scl, 
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       const u32x4_t v = lds_ld128(xb + (rk + 16 * k) * 64 + 16 * rq);
-      if (out[k] != nullptr) *(u32x4_t*)(out[k] + 64 * dc) = v;
+      if (!MAY_SKIP || out[k] != nullptr) *(u32x4_t*)(out[k] + 64 * dc) = v;
     }
   }
 }
