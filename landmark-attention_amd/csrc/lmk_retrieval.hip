@@ -79,11 +79,6 @@ __device__ __forceinline__ uint32_t prob_bits<bf16_t>(float x) {
 template <>
 __device__ __forceinline__ uint32_t prob_bits<f16_t>(float x) { return pack2<f16_t>(x, 0.f) & 0xffffu; }
 
-__global__ __launch_bounds__(256) void lmk_fill_u32_kernel(uint32_t* dst, int64_t n, uint32_t value) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) dst[i] = value;
-}
-
 // Scores of every query against every landmark key, in the contract's order, into p.approx (B*H*T, num_mems).
 // The contract's dot product is a chain of fp32 fmas over d ascending, and v_mfma_f32_32x32x1_2b_f32 is 2 x 32 x 32 of
 // exactly that step: C[i][j] = fma(A[i], B[j], C[i][j]).  A wave takes 64 query rows (a lane holds its row, packed) and
@@ -104,6 +99,12 @@ __global__ __launch_bounds__(256) void lmk_block_score_kernel(RetrParams p) {
   const int n_qg = (p.T + kScoreRows - 1) / kScoreRows, n_kc = (NM + kScoreKeys - 1) / kScoreKeys;
   // wave -> (query group, keys, head), query group first: the waves that run side by side read the same keys
   const int64_t wid = (int64_t)blockIdx.x * 4 + wave;
+  {
+    // the vectors the next kernel takes its maxima into start at zero: every wave of this one clears its share
+    const int64_t words = (int64_t)(p.agg_over_heads ? p.B * p.T : p.B * p.H) * NM, n_waves = (int64_t)gridDim.x * 4;
+    const int64_t per = (words + n_waves - 1) / n_waves, end = min(words, (wid + 1) * per);
+    for (int64_t i = wid * per + lane; i < end; i += 64) p.agg[i] = 0u;
+  }
   const int qg = (int)(wid % n_qg), kc = (int)((wid / n_qg) % n_kc);
   const int64_t bh64 = wid / n_qg / n_kc;
   if (bh64 >= (int64_t)p.B * p.H) return;                         // no workgroup-wide barrier in this kernel
@@ -1112,9 +1113,6 @@ static int launch_topk_shared_t(const RetrParams& p, hipStream_t stream) {
   hipLaunchKernelGGL((lmk_landmark_keys_kernel<T, D>), dim3((unsigned)((lkrows + RPW - 1) / RPW)), dim3(256), 0, stream, p);
   if ((rc = (int)hipGetLastError())) return rc;
   const int64_t sel_rows = p.agg_over_heads ? (int64_t)p.B * p.T : (int64_t)p.B * p.H;   // vectors to pick from
-  const int64_t agg_words = sel_rows * p.num_mems;
-  hipLaunchKernelGGL(lmk_fill_u32_kernel, dim3((unsigned)((agg_words + 255) / 256)), dim3(256), 0, stream, p.agg, agg_words, 0u);
-  if ((rc = (int)hipGetLastError())) return rc;
   const int64_t score_waves = (int64_t)p.B * p.H * ((p.T + kScoreRows - 1) / kScoreRows) * ((p.num_mems + kScoreKeys - 1) / kScoreKeys);
   hipLaunchKernelGGL((lmk_block_score_kernel<T, D>), dim3((unsigned)((score_waves + 3) / 4)), dim3(256), 0, stream, p);
   if ((rc = (int)hipGetLastError())) return rc;
